@@ -1,0 +1,128 @@
+/* libtfmi: MI355X (gfx950) kernels for TensorFold's quantized routed-expert matmul path, C ABI.
+ *
+ * Every entry point takes raw device pointers, sizes and a hipStream_t (passed as void*), launches on that stream
+ * without synchronising or allocating, and returns 0 on success or a non-zero status; tf_last_error() then holds a
+ * sentence naming the offending argument (thread-local).  All buffers are caller-owned.  Launches are safe to
+ * capture in a hipGraph: no host reads of device data, grid sizes come from host-side upper bounds.
+ *
+ * Each declaration cites the binding of the reference's CUDA extension it replaces (paths relative to
+ * src/tensorfold/cuda/ in the reference tree).
+ *
+ * Packed layouts (ours; callers only rely on the outer dimensions):
+ *   experts table  int32 [E, N/32, K/gs, M, 32*gs/8 + 32]   M = 2 (gate, up) or 1
+ *       block (32 columns x one group): gs/32 chunks of [32 columns][4 words], then [32 columns] (scale | bias << 16)
+ *       word j of a column's chunk holds inputs 8 j .. 8 j + 7; nibble slot p (bits 4p..4p+3) holds input
+ *       2 (p % 4) + p / 4, so (word >> 4 i) & 0x000F000F is the pair (input 2 i, input 2 i + 1)
+ *   lane weight Q4 int32 [npad/64, K/gs, gs/32, 64, 4]  (same chunk and nibble order, 64 columns a tile),
+ *       scales and biases bf16 [K/gs, npad], npad = n rounded up to 128
+ */
+#ifndef TFMI_H
+#define TFMI_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* tf_stream_t; /* hipStream_t */
+
+/* dtype codes for EXL3 inputs and outputs (exl3/linear.cu:16 `enum DType`) */
+enum { TF_F16 = 0, TF_BF16 = 1, TF_F32 = 2 };
+
+/* ---- library ------------------------------------------------------------------------------------------------- */
+
+/* The message of the last failing call on this thread ("" if none). */
+const char* tf_last_error(void);
+/* ABI version of this header. */
+int tf_version(void);
+/* 0 when the current HIP device is gfx950; otherwise non-zero with a message naming the device.
+ * Replaces build.py:20-32 `arch_flags` (refusal of a GPU the kernels were not built for). */
+int tf_check_device(void);
+
+/* ---- affine 4-bit lane matmul (kernels/qmm.cpp:151-157, module tensorfold_qmm_v5) --------------------------------- */
+
+/* MLX (n, k/8) words and (n, k/gs) bf16 scales/biases -> Q4 weight, (k/gs, npad) scales and biases.
+ * Replaces kernels/qmm.py:72-99 `pack` (torch ops in the reference, one kernel here). */
+int tf_qmm_pack(const uint32_t* words, const uint16_t* scales, const uint16_t* biases, int n, int k, int gs,
+                uint32_t* weight, uint16_t* scales_t, uint16_t* biases_t, tf_stream_t stream);
+/* The inverse: kernels/qmm.py:102-119 `unpack`. */
+int tf_qmm_unpack(const uint32_t* weight, const uint16_t* scales_t, const uint16_t* biases_t, int n, int k, int gs,
+                  uint32_t* words, uint16_t* scales, uint16_t* biases, tf_stream_t stream);
+/* xs[m, g] = fp32 sum of x[m, g*gs .. (g+1)*gs).  Replaces kernels/qmm.py:139-154 `group_sums` (Triton). */
+int tf_group_sums(const uint16_t* x, int64_t ldx, int m, int k, int gs, float* xs, tf_stream_t stream);
+/* Decode-form matmul: per group in order acc = fma(xs, b, fma(P, s, acc)), P = sum x*q with exact q; K in `sk`
+ * slices summed in slice order; one rounding to bf16 (or fp32 with f32).  `part` fp32 [sk, m, n] is required when
+ * sk > 1 (with reduce == 0 the slices are left there unadded).  sb_stride = elements between scale rows (>= npad).
+ * Replaces kernels/qmm.cpp:18-48 `qmm`. */
+int tf_qmm(const uint16_t* x, int64_t ldx, const float* xs, const uint32_t* weight, const uint16_t* scales,
+           const uint16_t* biases, int64_t sb_stride, void* out, float* part, int m, int n, int k, int sk, int gs,
+           int bm, int f32, int reduce, tf_stream_t stream);
+/* Prefill-form matmul: w = bf16(fma(q, s, b)), one fp32 chain over K on bf16 MFMA.
+ * Replaces kernels/qmm.cpp:83-102 `qmm_prefill`. */
+int tf_qmm_prefill(const uint16_t* x, int64_t ldx, const uint32_t* weight, const uint16_t* scales,
+                   const uint16_t* biases, void* out, int m, int n, int k, int gs, int f32, int tile,
+                   tf_stream_t stream);
+
+/* ---- routed experts (experts.cpp:77-82, module tensorfold_experts_v7) ---------------------------------------------- */
+
+/* MLX words [E, N, K/8], scales/biases [E, N, K/gs] -> blocks [E, N/32, K/gs, 32*gs/8 + 32].
+ * Replaces experts.cpp:57-75 `pack`. */
+int tf_experts_pack(const uint32_t* words, const uint16_t* scales, const uint16_t* biases, int e, int n, int k,
+                    int gs, uint32_t* out, tf_stream_t stream);
+/* The inverse (experts.py:43-59 `unpack`, torch ops in the reference).  `blocks` may be one matrix of a stacked
+ * table: block_stride = int32 elements between consecutive (column block, group) blocks. */
+int tf_experts_unpack(const uint32_t* blocks, int64_t block_stride, int e, int n, int k, int gs, uint32_t* words,
+                      uint16_t* scales, uint16_t* biases, tf_stream_t stream);
+/* Stable grouping of pairs p = row*slots + slot by expert: members [pairs], items [(expert, first, count<=tile)],
+ * counts = {items, distinct experts}.  rank [pairs] and hist [ceil(pairs/1024) * experts] are scratch, used when
+ * pairs > 1024.  tile is 16 (decode), 64 or 128 (prefill).  Replaces experts.cpp:33-41 `plan`. */
+int tf_experts_plan(const int32_t* picks, int64_t pairs, int experts, int tile, int32_t* members, int32_t* items,
+                    int32_t* counts, int32_t* rank, int32_t* hist, tf_stream_t stream);
+/* Decode form.  epi 0: fp32 out; 1: bf16 relu(bf16 a)^2; 2: bf16 SwiGLU(matrix 0, matrix 1) with clip `limit`.
+ * Pair p reads x row p / slots when slots > 0, row p when slots == 0.  max_units = max items * nb bounds the grid;
+ * the live item count is read on the device.  Replaces experts.cpp:43-48 `run`. */
+int tf_experts_run(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg, int nb,
+                   const int32_t* items, const int32_t* counts, const int32_t* members, void* out, int n, float limit,
+                   int64_t max_units, tf_stream_t stream);
+/* Prefill form on bf16 MFMA, w = bf16(fma(q, s, b)); epi 3: bf16 out.  `tile` is the plan's item size (16, 64 or
+ * 128).  Replaces experts.cpp:50-55 `prefill`. */
+int tf_experts_prefill(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg,
+                       int nb, const int32_t* items, const int32_t* counts, const int32_t* members, void* out, int n,
+                       float limit, int64_t max_items, int tile, tf_stream_t stream);
+
+/* ---- MoE glue (moe.py:23-151; Triton kernels in the reference) ------------------------------------------------------ */
+
+/* logits[m, e] = fp32 x[m] . rows[e]  (bf16 inputs).  Replaces moe.py:23-55 `_router` / `router`. */
+int tf_moe_router(const uint16_t* x, int64_t ldx, const uint16_t* rows, float* logits, int m, int d, int ne,
+                  tf_stream_t stream);
+/* Per row: top_k of logits[r, 0..experts) (largest first, lower id on ties), weights bf16(exp(l_k - l_0)/sum) as
+ * fp32; with shared != 0 slot top_k is expert id `experts` weighted bf16(sigmoid(bf16(logits[r, experts]))).
+ * pick int32 and wts fp32 are [rows, top_k + (shared ? 1 : 0)].  Replaces moe.py:58-108 `_topk_rows` / `select_rows`. */
+int tf_moe_topk(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared, int32_t* pick,
+                float* wts, tf_stream_t stream);
+/* out[r] = bf16(sum_k wts[r, k] * y[r, k]) in slot order, fp32; y is fp32 (y_bf16 == 0) or bf16.
+ * Replaces moe.py:131-151 `_combine` / `combine`. */
+int tf_moe_combine(const void* y, int y_bf16, const float* wts, uint16_t* out, int rows, int slots, int d,
+                   tf_stream_t stream);
+
+/* ---- EXL3 linear (exl3/linear.cpp:70-74, module tensorfold_exl3_linear_v3) ---------------------------------------- */
+
+/* xh[m, k] fp16 = fp16(((x * suh) @ H) / sqrt(128)) per block of 128; x is fp16, bf16 or fp32 (TF_* code).
+ * Replaces exl3/linear.cpp:24-33 `rot_in`. */
+int tf_exl3_rot_in(const void* x, int x_dtype, const uint16_t* suh, uint16_t* xh, int m, int k, tf_stream_t stream);
+/* y[m, n] = ((xh @ W_q) @ H / sqrt(128)) * svh + bias, 1 <= m <= 128.  T: trellis words, tile (kt, nt) at
+ * kt*stride_k + (nt/8)*stride_nb + (nt%8)*4*k2 words; k2 = 2*bits; cb 0 3inst, 1 mcg, 2 mul1; sk K splits (Z fp32
+ * [sk, m, n] and zeroed int32 counters [8 * n/128] needed when sk > 1; counters are left zero); wk waves a block.
+ * Replaces exl3/linear.cpp:36-58 `linear`. */
+int tf_exl3_linear(const uint16_t* xh, const uint32_t* T, int64_t stride_k, int64_t stride_nb, const uint16_t* svh,
+                   const uint16_t* bias, void* y, int y_dtype, float* Z, int32_t* counters, int m, int k, int n,
+                   int k2, int cb, int sk, int wk, tf_stream_t stream);
+/* W[k, n] fp16 = the decoded trellis (bit-exact codebook values).  Replaces exl3/linear.cpp:61-68 `unpack`. */
+int tf_exl3_unpack(const uint32_t* T, uint16_t* W, int k, int n, int64_t stride_k, int64_t stride_nb, int k2, int cb,
+                   tf_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TFMI_H */

@@ -1,0 +1,135 @@
+"""Oracle: MLX 4-bit affine weights, dequant-then-matmul and the expert epilogues, in numpy.  Test infrastructure only.
+
+Conventions: bf16 tensors travel as float32 arrays whose values are bf16-representable (or as uint16 bit patterns
+where a function says so); packed codes travel as uint32 arrays ``[..., K/8]``.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+
+# -- bf16 ---------------------------------------------------------------------------------------------------------
+
+def bf16_bits(x: np.ndarray) -> np.ndarray:
+    """float32 -> bf16 bit patterns (uint16), round to nearest even (what ``.to(torch.bfloat16)`` does)."""
+
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    bias = ((u >> np.uint32(16)) & np.uint32(1)) + np.uint32(0x7FFF)
+    return ((u + bias) >> np.uint32(16)).astype(np.uint16)
+
+
+def bf16_from_bits(b: np.ndarray) -> np.ndarray:
+    return (np.ascontiguousarray(b).astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def bf16(x: np.ndarray) -> np.ndarray:
+    """Round float32 values to bf16 and return them as float32."""
+
+    return bf16_from_bits(bf16_bits(x))
+
+
+# -- the format (families/qwen3_5/cuda/qmm.py:132-149; tests/cuda/test_qmm.py:22-26) ---------------------------------
+
+def nibbles(words: np.ndarray) -> np.ndarray:
+    """uint32 words [..., K/8] -> codes uint8 [..., K]: element 8 w + i is bits [4 i, 4 i + 4) of word w."""
+
+    w = np.ascontiguousarray(words).view(np.uint32)
+    q = (w[..., None] >> (np.arange(8, dtype=np.uint32) * np.uint32(4))) & np.uint32(15)
+    return q.reshape(*w.shape[:-1], w.shape[-1] * 8).astype(np.uint8)
+
+
+def words_from_nibbles(q: np.ndarray) -> np.ndarray:
+    """The inverse of ``nibbles``."""
+
+    q = np.ascontiguousarray(q).astype(np.uint32).reshape(*q.shape[:-1], q.shape[-1] // 8, 8)
+    return (q << (np.arange(8, dtype=np.uint32) * np.uint32(4))).sum(-1, dtype=np.uint64).astype(np.uint32)
+
+
+def dequantize(words: np.ndarray, scales: np.ndarray, biases: np.ndarray, gs: int) -> np.ndarray:
+    """W[..., n, k] = scale[n, k // gs] * q[n, k] + bias[n, k // gs] in float32 (a product, then a sum)."""
+
+    q = nibbles(words).astype(np.float32)
+    s = np.repeat(np.asarray(scales, dtype=np.float32), gs, axis=-1)
+    b = np.repeat(np.asarray(biases, dtype=np.float32), gs, axis=-1)
+    return q * s + b
+
+
+def linear(x: np.ndarray, words: np.ndarray, scales: np.ndarray, biases: np.ndarray, gs: int, *,
+           f32: bool = False, prefill: bool = False) -> np.ndarray:
+    """(x.float() @ dequantize(...).T).to(bf16)  (families/qwen3_5/cuda/reference.py:11-15).
+
+    ``prefill`` rounds each dequantized weight to bf16 first (cuda/kernels/qmm_prefill.cu:1)."""
+
+    w = dequantize(words, scales, biases, gs)
+    if prefill:
+        w = bf16(w)
+    y = np.asarray(x, dtype=np.float32) @ w.T
+    return y if f32 else bf16(y)
+
+
+def group_sums(x: np.ndarray, gs: int) -> np.ndarray:
+    """xs[m, g] = sum of x[m, g*gs:(g+1)*gs] in float32 (cuda/kernels/qmm.py:139-154)."""
+
+    x = np.asarray(x, dtype=np.float32)
+    return x.reshape(x.shape[0], -1, gs).sum(-1, dtype=np.float32)
+
+
+# -- expert epilogues (cuda/experts.cuh:53-103) -----------------------------------------------------------------------
+
+def relu2(a: np.ndarray) -> np.ndarray:
+    """bf16(max(bf16(a), 0)^2)."""
+
+    u = np.maximum(bf16(a), np.float32(0))
+    return bf16(u * u)
+
+
+def swiglu(g: np.ndarray, u: np.ndarray, limit: float = 0.0) -> np.ndarray:
+    """bf16(bf16(silu(g')) * u') on bf16 g and u; with limit > 0, g' = min(g, limit), u' = clip(u, -limit, limit)."""
+
+    gv, uv = bf16(g), bf16(u)
+    if limit > 0:
+        gv = np.minimum(gv, np.float32(limit))
+        uv = np.clip(uv, np.float32(-limit), np.float32(limit))
+    silu = gv / (np.float32(1) + np.exp(-gv, dtype=np.float32))
+    return bf16(bf16(silu.astype(np.float32)) * uv)
+
+
+def expert_pairs(x: np.ndarray, picks: np.ndarray, up: list, down: tuple, gs: int, *, limit: float = 0.0,
+                 prefill: bool = False, y_bf16: bool = False) -> tuple[np.ndarray, np.ndarray]:
+    """Every (row, slot) pair through its expert: act [R*S, NI] (bf16 values) and y [R*S, D] (fp32, or bf16 values).
+
+    ``up`` is [gate, up] (SwiGLU) or [up] (relu^2), each (words [E, NI, D/8], scales, biases); ``down`` likewise
+    [E, D, NI/8].  Weights are dequantized per used expert; ``prefill`` rounds them to bf16 first
+    (cuda/experts_prefill.cu:130-131)."""
+
+    x = np.asarray(x, dtype=np.float32)
+    rows, slots = picks.shape
+    ni, d = up[0][0].shape[1], down[0].shape[1]
+    act = np.zeros((rows * slots, ni), dtype=np.float32)
+    y = np.zeros((rows * slots, d), dtype=np.float32)
+    flat = picks.reshape(-1)
+
+    def weight(m, e):
+        w = dequantize(m[0][e], m[1][e], m[2][e], gs)
+        return bf16(w) if prefill else w
+
+    for e in np.unique(flat):
+        pairs = np.nonzero(flat == e)[0]
+        xe = x[pairs // slots]
+        projs = [xe @ weight(m, e).T for m in up]
+        a = swiglu(projs[0], projs[1], limit) if len(up) == 2 else relu2(projs[0])
+        act[pairs] = a
+        ye = a @ weight(down, e).T
+        y[pairs] = bf16(ye) if y_bf16 else ye
+    return act, y
+
+
+def combine(y: np.ndarray, wts: np.ndarray) -> np.ndarray:
+    """out[r] = bf16(sum over slots, in slot order, of fp32 w[r, k] * y[r, k])  (cuda/moe.py:131-142)."""
+
+    rows, slots, _ = y.shape
+    acc = np.zeros((rows, y.shape[2]), dtype=np.float32)
+    for k in range(slots):
+        acc = acc + wts[:, k:k + 1].astype(np.float32) * y[:, k].astype(np.float32)
+    return bf16(acc)

@@ -1,0 +1,83 @@
+"""Build and load ``libtfmi.so``: hipcc for gfx950, nothing else (the counterpart of the reference's cuda/build.py).
+
+The reference JIT-builds one pybind11 module per kernel family for whatever NVIDIA GPU is present and refuses GPUs
+under compute capability 8.9 (cuda/build.py:20-69).  Here one shared library with a C ABI is compiled ahead of
+time, in the tree, for the one target this package supports, and a GPU that is not gfx950 is refused by name.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import shutil
+import subprocess
+import sys
+from functools import lru_cache
+from pathlib import Path
+
+ARCH = "gfx950"
+HERE = Path(__file__).resolve().parent
+CSRC = HERE / "csrc"
+LIB = HERE / "libtfmi.so"
+SOURCES = ("api.hip", "pack.hip", "decode.hip", "route.hip", "prefill.hip", "exl3.hip")
+# packed-fp32 VALU forms are switched off for the device pass (the host pass warns that it does not know the feature)
+FLAGS = ("-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops")
+
+
+def say(text: str) -> None:
+    print(f"[tensorfold-amd] {text}", file=sys.stderr, flush=True)
+
+
+def hipcc() -> str | None:
+    return shutil.which("hipcc") or (str(Path("/opt/rocm/bin/hipcc")) if Path("/opt/rocm/bin/hipcc").exists() else None)
+
+
+def stale() -> bool:
+    if not LIB.exists():
+        return True
+    built = LIB.stat().st_mtime
+    deps = [CSRC / s for s in SOURCES] + [CSRC / "tf_common.h", HERE.parent / "include" / "tfmi.h"]
+    return any(d.stat().st_mtime > built for d in deps)
+
+
+def compile(verbose: bool = False) -> Path:
+    """Compile every kernel for gfx950 into ``libtfmi.so`` (cross-compiles without a GPU)."""
+
+    cc = hipcc()
+    if cc is None:
+        raise RuntimeError("tensorfold-amd: hipcc was not found; ROCm's compiler is needed to build libtfmi.so")
+    cmd = [cc, *FLAGS, "-o", str(LIB), *(str(CSRC / s) for s in SOURCES)]
+    say(f"building {LIB.name} for {ARCH} (about a minute)")
+    done = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "packed-fp32-ops"
+    err = "\n".join(line for line in done.stderr.splitlines() if noise not in line)
+    if done.returncode:
+        raise RuntimeError(f"tensorfold-amd: hipcc failed:\n{err}")
+    if verbose and err:
+        say(err)
+    return LIB
+
+
+@lru_cache(maxsize=1)
+def load() -> ctypes.CDLL:
+    """The library, built first if it is missing and hipcc is here; a missing library never falls back to anything."""
+
+    if not LIB.exists():
+        if hipcc() is None:
+            raise RuntimeError(f"tensorfold-amd: {LIB} is missing and there is no hipcc to build it; "
+                               "run `python -c 'import __graft_entry__ as g; g.build()'` where ROCm is installed")
+        compile()
+    return ctypes.CDLL(str(LIB))
+
+
+def refuse_other_gpu() -> None:
+    """With a GPU present, refuse by name one the kernels were not built for (cuda/build.py:35-46 in spirit)."""
+
+    import torch
+
+    if not torch.cuda.is_available():
+        return
+    lib = load()
+    lib.tf_last_error.restype = ctypes.c_char_p
+    if lib.tf_check_device():
+        raise ValueError(lib.tf_last_error().decode())

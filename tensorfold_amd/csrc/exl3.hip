@@ -1,0 +1,332 @@
+// EXL3 trellis-coded linear layers: tf_exl3_rot_in, tf_exl3_linear, tf_exl3_unpack.
+//
+// A tile holds 256 values of k2/2 bits in a circular bitstream (most significant bit of each little-endian 32-bit
+// word first); value p is the 16-bit window ending at bit E(p), pushed through a procedural codebook to an fp16
+// value, and lands at row 2 (l % 4) + (j & 1) + 8 ((j >> 1) & 1), column l / 4 + 8 (j >> 2) of the 16 x 16 tile
+// (l = p / 8, j = p % 8)  (reference: docs/recipes/exl3.md:43-63, cuda/exl3/format.py:31-110).
+//
+// On a 64-lane wave the B operand of v_mfma_f32_16x16x32_f16 is 32 inputs x 16 columns, 8 values a lane: lane
+// (column c, quarter kq) takes, from each of two consecutive k tiles, the four stream-consecutive values
+// p0 .. p0 + 3 with p0 = 8 (4 (c % 8) + kq) + 4 (c / 8).  They sit in rows {2 kq, 2 kq + 1, 2 kq + 8, 2 kq + 9} of
+// column c, so the A operand reads the rotated activations at the same eight inputs and no value moves across
+// lanes.  Rows of the call are MFMA rows: independent by construction.  K is split over waves and blocks as a
+// function of the shape only and every sum runs in a fixed order.
+
+#include <hip/hip_fp16.h>
+
+#include "tf_common.h"
+
+namespace tf {
+namespace {
+
+constexpr float HAD_SCALE = 0.08838834764831845f;   // 1 / sqrt(128)
+
+template <int K2>
+__host__ __device__ constexpr int tile_words() {
+  return 4 * K2;
+}
+
+// E(p): one past the last stream bit of value p's window
+template <int K2>
+__host__ __device__ constexpr int stream_end(int p) {
+  return (K2 & 1) ? ((p + 1) * K2 - ((p + 1) & 1)) / 2 : (p + 1) * (K2 / 2);
+}
+
+// bit distance from value p0's window to value p0 + j's, p0 a multiple of 4
+template <int K2>
+__host__ __device__ constexpr int delta(int j) {
+  return stream_end<K2>(j) - stream_end<K2>(0);
+}
+
+// The 16-bit states of values p0 .. p0 + 3 (p0 = 8 L + 4 h) of the tile at `tile` (global or LDS words).
+template <int K2>
+__device__ __forceinline__ void states4(const uint32_t* tile, int L, int h, uint32_t (&s)[4]) {
+  constexpr int TW = tile_words<K2>(), R = 32 * TW;
+  constexpr bool NEED_LO = delta<K2>(3) + 16 > 32;      // a window reaches past the first aligned word
+  constexpr bool NEED_W2 = 31 + delta<K2>(3) + 16 > 64; // ... and past the second stored word
+  const int p0 = 8 * L + 4 * h;
+  const int first = (stream_end<K2>(0) + p0 * K2 / 2 - 16 + R) % R;   // E(p0) - 16, p0 even so p0 * K2 / 2 is whole
+  const int wi = first >> 5, o = first & 31;
+  const uint32_t w0 = tile[wi], w1 = tile[(wi + 1) % TW];
+  const uint32_t hi = __funnelshift_l(w1, w0, o);       // the stream from the first window on, 32 bits
+  uint32_t lo = 0;
+  if constexpr (NEED_LO) {
+    const uint32_t w2 = NEED_W2 ? tile[(wi + 2) % TW] : 0u;
+    lo = __funnelshift_l(w2, w1, o);
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int d = delta<K2>(j);
+    if (d + 16 <= 32) s[j] = (hi >> (16 - d)) & 0xFFFFu;
+    else if (d < 32) s[j] = __funnelshift_l(lo, hi, d) >> 16;
+    else s[j] = (lo >> (48 - d)) & 0xFFFFu;
+  }
+}
+
+// fp16 bits of the codebook value of state s
+template <int CB>
+__device__ __forceinline__ uint16_t code_value(uint32_t s) {
+  if constexpr (CB == 2) {
+    const uint32_t x = s * 0x83DCD12Du;
+    const uint32_t hs = 1024u + (x & 255u) + ((x >> 8) & 255u) + ((x >> 16) & 255u) + (x >> 24);
+    const __half hv = __ushort_as_half((unsigned short)(0x6400u + (hs - 1024u)));   // fp16 of 1024 + byte sum (< 2048)
+    const __half r = __hfma(hv, __ushort_as_half((unsigned short)0x1EEE), __ushort_as_half((unsigned short)0xC931));
+    return __half_as_ushort(r);
+  } else {
+    uint32_t x = CB == 1 ? s * 0xCBAC1FEDu : s * 89226354u + 64248484u;
+    x = (x & 0x8FFF8FFFu) ^ 0x3B603B60u;
+    const __half r = __hadd(__ushort_as_half((unsigned short)(x & 0xFFFFu)), __ushort_as_half((unsigned short)(x >> 16)));
+    return __half_as_ushort(r);
+  }
+}
+
+template <int K2, int CB>
+__device__ __forceinline__ void values4(const uint32_t* tile, int L, int h, uint16_t (&v)[4]) {
+  uint32_t s[4];
+  states4<K2>(tile, L, h, s);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) v[j] = code_value<CB>(s[j]);
+}
+
+// Unscaled Walsh-Hadamard transform of 128 values, two a lane (elements 2 lane, 2 lane + 1), fixed butterfly order.
+__device__ __forceinline__ void fwht128(float& a, float& b, int lane) {
+  const float s = a + b, d = a - b;
+  a = s;
+  b = d;
+#pragma unroll
+  for (int m = 1; m < 64; m <<= 1) {
+    const float oa = __shfl_xor(a, m), ob = __shfl_xor(b, m);
+    a = (lane & m) ? oa - a : a + oa;
+    b = (lane & m) ? ob - b : b + ob;
+  }
+}
+
+__device__ __forceinline__ void load2(const void* p, int dtype, size_t i, float& a, float& b) {
+  if (dtype == TF_F32) {
+    const float2 u = *reinterpret_cast<const float2*>(static_cast<const float*>(p) + i);
+    a = u.x;
+    b = u.y;
+  } else if (dtype == TF_BF16) {
+    const uint32_t u = *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(p) + i);
+    a = bf16_lo(u);
+    b = bf16_hi(u);
+  } else {
+    const __half2 u = *reinterpret_cast<const __half2*>(static_cast<const __half*>(p) + i);
+    a = __low2float(u);
+    b = __high2float(u);
+  }
+}
+
+__device__ __forceinline__ void store2(void* p, int dtype, size_t i, float a, float b) {
+  if (dtype == TF_F32) {
+    *reinterpret_cast<float2*>(static_cast<float*>(p) + i) = make_float2(a, b);
+  } else if (dtype == TF_BF16) {
+    *reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(p) + i) = pack_bf16(a, b);
+  } else {
+    *reinterpret_cast<__half2*>(static_cast<__half*>(p) + i) = __floats2half2_rn(a, b);
+  }
+}
+
+// xh = fp16(((x * suh) H) / sqrt(128)), a wave a (row, block of 128)
+__global__ void __launch_bounds__(256)
+    rot_in_kernel(const void* __restrict__ x, int x_dtype, const uint16_t* __restrict__ suh, uint16_t* __restrict__ xh,
+                  int K) {
+  const int blk = blockIdx.x * 4 + (threadIdx.x >> 6), row = blockIdx.y, lane = threadIdx.x & 63;
+  if (blk * 128 >= K) return;
+  const int k = blk * 128 + 2 * lane;
+  float a, b, sa, sb;
+  load2(x, x_dtype, (size_t)row * K + k, a, b);
+  load2(suh, TF_F16, k, sa, sb);
+  a *= sa;
+  b *= sb;
+  fwht128(a, b, lane);
+  store2(xh, TF_F16, (size_t)row * K + k, a * HAD_SCALE, b * HAD_SCALE);
+}
+
+// the finished outputs of one row's 128 columns from their fp32 sums: H / sqrt(128), * svh, + bias
+__device__ __forceinline__ void finish_row(float a, float b, int lane, const uint16_t* svh, const uint16_t* bias,
+                                           int col, void* y, int y_dtype, size_t at) {
+  fwht128(a, b, lane);
+  float sa, sb;
+  load2(svh, TF_F16, col, sa, sb);
+  a = a * HAD_SCALE * sa;
+  b = b * HAD_SCALE * sb;
+  if (bias) {
+    float ba, bb;
+    load2(bias, TF_F16, col, ba, bb);
+    a += ba;
+    b += bb;
+  }
+  store2(y, y_dtype, at, a, b);
+}
+
+// grid (N / 128, SK); WK waves a block; each wave walks its range of k-tile pairs over the block's eight column tiles
+template <int K2, int CB, int WK>
+__global__ void __launch_bounds__(WK * 64)
+    linear_kernel(const uint16_t* __restrict__ xh, const uint32_t* __restrict__ T, int64_t stride_k, int64_t stride_nb,
+                  const uint16_t* __restrict__ svh, const uint16_t* __restrict__ bias, void* __restrict__ y, int y_dtype,
+                  float* __restrict__ Z, int* __restrict__ counters, int M, int K, int N, int SK) {
+  constexpr int TW = tile_words<K2>();
+  extern __shared__ __align__(16) float red[];              // [WK][16][128]
+  __shared__ int last;
+  const int nb = blockIdx.x, split = blockIdx.y, NB = gridDim.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c = lane & 15, kq = lane >> 4;
+  const int L = 4 * (c & 7) + kq, h = c >> 3;
+  const int pairs = K >> 5, slot = split * WK + wave, nslots = SK * WK;
+  const int pr0 = (int)((long long)slot * pairs / nslots), pr1 = (int)((long long)(slot + 1) * pairs / nslots);
+  const uint32_t* tiles = T + (size_t)nb * stride_nb;
+  const int col0 = nb * 128;
+
+  for (int m0 = 0, pass = 0; m0 < M; m0 += 16, ++pass) {
+    const int R = min(16, M - m0);
+    f32x4_t acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    // the A operand's row: lane (row c, quarter kq); rows past the pass read a valid row and are dropped later
+    const uint16_t* xr = xh + (size_t)(m0 + (c < R ? c : R - 1)) * K + 2 * kq;
+    for (int pr = pr0; pr < pr1; ++pr) {
+      const uint32_t* xk = reinterpret_cast<const uint32_t*>(xr + 32 * pr);
+      const u32x4_t av = {xk[0], xk[4], xk[8], xk[12]};
+      const f16x8_t a = __builtin_bit_cast(f16x8_t, av);
+      const uint32_t* t0 = tiles + (size_t)(2 * pr) * stride_k;
+      const uint32_t* t1 = t0 + stride_k;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        uint16_t v0[4], v1[4];
+        values4<K2, CB>(t0 + j * TW, L, h, v0);
+        values4<K2, CB>(t1 + j * TW, L, h, v1);
+        const u32x4_t bw = {(uint32_t)v0[0] | ((uint32_t)v0[1] << 16), (uint32_t)v0[2] | ((uint32_t)v0[3] << 16),
+                            (uint32_t)v1[0] | ((uint32_t)v1[1] << 16), (uint32_t)v1[2] | ((uint32_t)v1[3] << 16)};
+        const f16x8_t b = __builtin_bit_cast(f16x8_t, bw);
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[j], 0, 0, 0);
+      }
+    }
+    // D[row 4 kq + i][column c] of column tile j -> red[wave][row][16 j + c]
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[(wave * 16 + 4 * kq + i) * 128 + 16 * j + c] = acc[j][i];
+    __syncthreads();
+    // a wave a row: the waves' sums in wave order, two columns a lane
+    for (int r = wave; r < R; r += WK) {
+      float2 s = *reinterpret_cast<const float2*>(red + r * 128 + 2 * lane);
+      for (int w = 1; w < WK; ++w) {
+        const float2 q = *reinterpret_cast<const float2*>(red + (w * 16 + r) * 128 + 2 * lane);
+        s.x += q.x;
+        s.y += q.y;
+      }
+      const size_t at = (size_t)(m0 + r) * N + col0 + 2 * lane;
+      if (SK == 1) finish_row(s.x, s.y, lane, svh, bias, col0 + 2 * lane, y, y_dtype, at);
+      else *reinterpret_cast<float2*>(Z + (size_t)split * M * N + at) = s;
+    }
+    if (SK > 1) {
+      __threadfence();
+      __syncthreads();
+      if (threadIdx.x == 0) last = atomicAdd(counters + pass * NB + nb, 1) == SK - 1;
+      __syncthreads();
+      if (last) {
+        __threadfence();
+        for (int r = wave; r < R; r += WK) {
+          const size_t at = (size_t)(m0 + r) * N + col0 + 2 * lane;
+          float sx = __hip_atomic_load(Z + at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          float sy = __hip_atomic_load(Z + at + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          for (int q = 1; q < SK; ++q) {
+            sx += __hip_atomic_load(Z + (size_t)q * M * N + at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            sy += __hip_atomic_load(Z + (size_t)q * M * N + at + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+          finish_row(sx, sy, lane, svh, bias, col0 + 2 * lane, y, y_dtype, at);
+        }
+        if (threadIdx.x == 0) counters[pass * NB + nb] = 0;     // every block of the column has arrived
+      }
+    }
+  }
+}
+
+// W_q [K, N] fp16: a wave a tile
+template <int K2, int CB>
+__global__ void __launch_bounds__(64)
+    unpack_kernel(const uint32_t* __restrict__ T, uint16_t* __restrict__ W, int N, int64_t stride_k, int64_t stride_nb) {
+  const int kt = blockIdx.y, nt = blockIdx.x, lane = threadIdx.x, L = lane & 31, h = lane >> 5;
+  const uint32_t* tile = T + (size_t)kt * stride_k + (size_t)(nt >> 3) * stride_nb + (nt & 7) * tile_words<K2>();
+  uint16_t v[4];
+  values4<K2, CB>(tile, L, h, v);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int row = 2 * (L & 3) + (j & 1) + 8 * (j >> 1), col = (L >> 2) + 8 * h;
+    W[(size_t)(kt * 16 + row) * N + nt * 16 + col] = v[j];
+  }
+}
+
+// every width ExLlamaV3 writes: k2 = 2 * bits; half-integer widths exist with the mul1 codebook only
+#define TF_EXL3_WIDTHS(X, CB) X(2, CB) X(4, CB) X(6, CB) X(8, CB) X(10, CB) X(12, CB) X(14, CB) X(16, CB)
+#define TF_EXL3_ALL(X) TF_EXL3_WIDTHS(X, 0) TF_EXL3_WIDTHS(X, 1) TF_EXL3_WIDTHS(X, 2) X(3, 2) X(5, 2) X(7, 2)
+
+}  // namespace
+}  // namespace tf
+
+using namespace tf;
+
+extern "C" int tf_exl3_rot_in(const void* x, int x_dtype, const uint16_t* suh, uint16_t* xh, int m, int k,
+                              tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(x && suh && xh, "rot_in: null pointer argument");
+  TF_REQUIRE(x_dtype == TF_F16 || x_dtype == TF_BF16 || x_dtype == TF_F32, "x: expected fp16, bf16 or fp32");
+  TF_REQUIRE(m >= 1 && k >= 128 && k % 128 == 0, "x and xh must be [M, K], K a multiple of 128, suh [K]");
+  TF_REQUIRE(aligned16(x) && aligned16(xh), "x: must be 16-byte aligned");
+  TF_REQUIRE(m <= 65535, "rot_in: at most 65535 rows");
+  rot_in_kernel<<<dim3((k / 128 + 3) / 4, m), 256, 0, as_stream(stream)>>>(x, x_dtype, suh, xh, k);
+  TF_LAUNCH_OK("tf_exl3_rot_in");
+  return 0;
+}
+
+extern "C" int tf_exl3_linear(const uint16_t* xh, const uint32_t* T, int64_t stride_k, int64_t stride_nb,
+                              const uint16_t* svh, const uint16_t* bias, void* y, int y_dtype, float* Z,
+                              int32_t* counters, int m, int k, int n, int k2, int cb, int sk, int wk,
+                              tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(xh && T && svh && y, "linear: null pointer argument");
+  TF_REQUIRE(y_dtype == TF_F16 || y_dtype == TF_BF16 || y_dtype == TF_F32, "y: expected fp16, bf16 or fp32");
+  TF_REQUIRE(m >= 1 && m <= 128, "xh and y must have the same 1 to 128 rows");
+  TF_REQUIRE(k >= 128 && n >= 128 && k % 128 == 0 && n % 128 == 0, "K and N must be multiples of 128");
+  TF_REQUIRE(aligned16(T) && aligned16(xh) && aligned16(y), "T must be 16-byte aligned");
+  TF_REQUIRE(wk == 2 || wk == 4 || wk == 8, "WK must be 2, 4 or 8");
+  TF_REQUIRE(sk >= 1 && sk <= 64 && (int64_t)sk * wk <= k / 32, "K / 32 = %d tile pairs do not split over %d x %d waves",
+             k / 32, sk, wk);
+  TF_REQUIRE(sk == 1 || (Z && counters), "Z and counters are needed with more than one split");
+  const dim3 grid((unsigned)(n / 128), (unsigned)sk);
+  hipStream_t s = as_stream(stream);
+  const size_t smem = (size_t)wk * 16 * 128 * sizeof(float);
+#define TF_LAUNCH(K2_, CB_)                                                                                             \
+  if (k2 == K2_ && cb == CB_) {                                                                                         \
+    if (wk == 2) linear_kernel<K2_, CB_, 2><<<grid, 128, smem, s>>>(xh, T, stride_k, stride_nb, svh, bias, y, y_dtype, Z, counters, m, k, n, sk); \
+    else if (wk == 4) linear_kernel<K2_, CB_, 4><<<grid, 256, smem, s>>>(xh, T, stride_k, stride_nb, svh, bias, y, y_dtype, Z, counters, m, k, n, sk); \
+    else linear_kernel<K2_, CB_, 8><<<grid, 512, smem, s>>>(xh, T, stride_k, stride_nb, svh, bias, y, y_dtype, Z, counters, m, k, n, sk); \
+    TF_LAUNCH_OK("tf_exl3_linear");                                                                                     \
+    return 0;                                                                                                           \
+  }
+  TF_EXL3_ALL(TF_LAUNCH)
+#undef TF_LAUNCH
+  set_error("unsupported EXL3 width/codebook: K2=%d codebook=%d", k2, cb);
+  return 1;
+}
+
+extern "C" int tf_exl3_unpack(const uint32_t* T, uint16_t* W, int k, int n, int64_t stride_k, int64_t stride_nb, int k2,
+                              int cb, tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(T && W, "unpack: null pointer argument");
+  TF_REQUIRE(k >= 128 && n >= 128 && k % 128 == 0 && n % 128 == 0, "W must be [K, N], multiples of 128");
+  TF_REQUIRE(k / 16 <= 65535, "unpack: K too large for one launch");
+  const dim3 grid((unsigned)(n / 16), (unsigned)(k / 16));
+  hipStream_t s = as_stream(stream);
+#define TF_LAUNCH(K2_, CB_)                                                          \
+  if (k2 == K2_ && cb == CB_) {                                                      \
+    unpack_kernel<K2_, CB_><<<grid, 64, 0, s>>>(T, W, n, stride_k, stride_nb);       \
+    TF_LAUNCH_OK("tf_exl3_unpack");                                                  \
+    return 0;                                                                        \
+  }
+  TF_EXL3_ALL(TF_LAUNCH)
+#undef TF_LAUNCH
+  set_error("unsupported EXL3 width/codebook: K2=%d codebook=%d", k2, cb);
+  return 1;
+}

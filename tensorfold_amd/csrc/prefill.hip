@@ -1,0 +1,366 @@
+// Prefill-form 4-bit matmuls on bf16 MFMA: the token-sorted grouped expert GEMM (tf_experts_prefill) and the dense
+// prompt matmul (tf_qmm_prefill).  w = bf16(fma(q, s, b)) and one fp32 chain over K in order, so a row's bits depend
+// neither on its item nor on its chunk (reference: experts_prefill.cu:1, qmm_prefill.cu:1).
+//
+// A workgroup of four waves takes (item of up to 16*RT rows) x (128 columns); each wave owns 32 columns and all the
+// item's rows.  The gathered activation rows are staged through LDS (64 inputs a step, double-buffered); the
+// weights never touch LDS: lane (column c, quarter kq) of v_mfma_f32_16x16x32_bf16's B operand needs the eight
+// inputs 8 kq .. 8 kq + 7 of column c, which is exactly one packed word, so each lane loads its word and
+// dequantizes it in registers.
+
+#include "tf_common.h"
+
+namespace tf {
+namespace {
+
+constexpr int KSTEP = 64;                      // inputs staged a step
+constexpr int AROW = KSTEP * 2 + 16;           // bytes of an LDS row: 128 of data, 16 of padding against conflicts
+
+// one packed word -> the B operand: inputs in order, each bf16(fma(q, s, b))
+__device__ __forceinline__ bf16x8_t dequant8(uint32_t w, float s, float b) {
+  const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
+  // slot p holds input 2 (p % 4) + p / 4: lo bytes are inputs 0, 4, 1, 5; hi bytes are inputs 2, 6, 3, 7
+  float f[8];
+  f[0] = (float)(lo & 0xFFu);
+  f[4] = (float)((lo >> 8) & 0xFFu);
+  f[1] = (float)((lo >> 16) & 0xFFu);
+  f[5] = (float)(lo >> 24);
+  f[2] = (float)(hi & 0xFFu);
+  f[6] = (float)((hi >> 8) & 0xFFu);
+  f[3] = (float)((hi >> 16) & 0xFFu);
+  f[7] = (float)(hi >> 24);
+  bf16x8_t r;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) r[j] = (__bf16)fmaf(f[j], s, b);
+  return r;
+}
+
+// EPI 0: fp32; 1: bf16 relu(bf16 a)^2; 2: bf16 SwiGLU(matrix 0, matrix 1); 3: bf16
+template <int EPI>
+__device__ __forceinline__ void store_out(void* out, size_t at, float a, float u, float limit) {
+  if constexpr (EPI == 0) reinterpret_cast<float*>(out)[at] = a;
+  else if constexpr (EPI == 1) reinterpret_cast<uint16_t*>(out)[at] = (uint16_t)f32_bf16_bits(relu2(a));
+  else if constexpr (EPI == 2) reinterpret_cast<uint16_t*>(out)[at] = (uint16_t)f32_bf16_bits(swiglu(a, u, limit));
+  else reinterpret_cast<uint16_t*>(out)[at] = (uint16_t)f32_bf16_bits(a);
+}
+
+// The shared body.  SRC gives, for the workgroup's item: rows(), src_row(r), dst_row(r); WSRC gives the lane's
+// packed word and its column's scale and bias.
+//   word(g, m, i, t): group g, matrix m, chunk i (32 inputs) of the group, column tile t (16 columns) of the wave
+//   sb(g, m, t, s, b)
+template <int GS, int NM, int EPI, int RT, class WSRC>
+__device__ __forceinline__ void mfma_body(const uint16_t* __restrict__ X, int64_t x_stride, int K, const WSRC& ws,
+                                          const int* src_rows, int cnt, void* out, int N, int col0, int wave_cols_ok,
+                                          const int* dst_rows, float limit, unsigned char* smem) {
+  constexpr int ROWS = 16 * RT;
+  constexpr int CPS = KSTEP / 32;              // chunks a step
+  constexpr int GPS = KSTEP / GS;              // groups a step (1 or 2)
+  constexpr int PIECES = ROWS * 8;             // 16-byte pieces of a staged tile
+  constexpr int PPT = (PIECES + 255) / 256;
+  const int tid = threadIdx.x, lane = tid & 63, c = lane & 15, kq = lane >> 4;
+  const int steps = (K + KSTEP - 1) / KSTEP;
+
+  // this thread's pieces of the activation tile
+  const uint16_t* asrc[PPT];
+  int adst[PPT];
+#pragma unroll
+  for (int j = 0; j < PPT; ++j) {
+    const int q = tid + j * 256, r = q >> 3, ch = q & 7;
+    adst[j] = -1;
+    asrc[j] = X;
+    if (q < PIECES) {
+      adst[j] = r * AROW + ch * 16;
+      asrc[j] = X + (size_t)src_rows[r < cnt ? r : cnt - 1] * x_stride + ch * 8;
+    }
+  }
+  auto load_a = [&](int step, uint4 (&v)[PPT]) {
+#pragma unroll
+    for (int j = 0; j < PPT; ++j) {
+      const int q = tid + j * 256, ch = q & 7;
+      v[j] = make_uint4(0u, 0u, 0u, 0u);
+      if (adst[j] >= 0 && step * KSTEP + ch * 8 < K) v[j] = *reinterpret_cast<const uint4*>(asrc[j] + (size_t)step * KSTEP);
+    }
+  };
+  auto store_a = [&](int buf, const uint4 (&v)[PPT]) {
+#pragma unroll
+    for (int j = 0; j < PPT; ++j)
+      if (adst[j] >= 0) *reinterpret_cast<uint4*>(smem + buf * (ROWS * AROW) + adst[j]) = v[j];
+  };
+
+  uint32_t wcur[NM][CPS][2], wnxt[NM][CPS][2];
+  float scur[NM][GPS][2], bcur[NM][GPS][2], snxt[NM][GPS][2], bnxt[NM][GPS][2];
+  auto load_w = [&](int step, uint32_t (&w)[NM][CPS][2], float (&s)[NM][GPS][2], float (&b)[NM][GPS][2]) {
+#pragma unroll
+    for (int m = 0; m < NM; ++m)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+#pragma unroll
+        for (int i = 0; i < CPS; ++i) {
+          const int k0 = step * KSTEP + 32 * i;
+          w[m][i][t] = k0 < K ? ws.word(k0 / GS, m, (k0 % GS) / 32, t) : 0u;
+        }
+#pragma unroll
+        for (int gi = 0; gi < GPS; ++gi) {
+          const int k0 = step * KSTEP + GS * gi;
+          s[m][gi][t] = 0.f;
+          b[m][gi][t] = 0.f;
+          if (k0 < K) ws.sb(k0 / GS, m, t, s[m][gi][t], b[m][gi][t]);
+        }
+      }
+  };
+
+  f32x4_t acc[NM][RT][2];
+#pragma unroll
+  for (int m = 0; m < NM; ++m)
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) acc[m][r][t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+
+  const int nt = (cnt + 15) >> 4;              // row tiles in use
+  uint4 areg[PPT];
+  load_a(0, areg);
+  load_w(0, wcur, scur, bcur);
+  store_a(0, areg);
+  __syncthreads();
+  for (int step = 0; step < steps; ++step) {
+    const bool more = step + 1 < steps;
+    if (more) {
+      load_a(step + 1, areg);
+      load_w(step + 1, wnxt, snxt, bnxt);
+    }
+    const unsigned char* abuf = smem + (step & 1) * (ROWS * AROW);
+#pragma unroll
+    for (int i = 0; i < CPS; ++i) {
+      if (step * KSTEP + 32 * i >= K) break;
+      bf16x8_t bfrag[NM][2];
+#pragma unroll
+      for (int m = 0; m < NM; ++m)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          const int gi = (32 * i) / GS;
+          bfrag[m][t] = dequant8(wcur[m][i][t], scur[m][gi][t], bcur[m][gi][t]);
+        }
+#pragma unroll
+      for (int r = 0; r < RT; ++r) {
+        if (r >= nt) break;
+        const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(abuf + (16 * r + c) * AROW + i * 64 + kq * 16);
+#pragma unroll
+        for (int m = 0; m < NM; ++m)
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+            acc[m][r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bfrag[m][t], acc[m][r][t], 0, 0, 0);
+      }
+    }
+    if (more) {
+      store_a((step + 1) & 1, areg);
+#pragma unroll
+      for (int m = 0; m < NM; ++m) {
+#pragma unroll
+        for (int i = 0; i < CPS; ++i)
+#pragma unroll
+          for (int t = 0; t < 2; ++t) wcur[m][i][t] = wnxt[m][i][t];
+#pragma unroll
+        for (int gi = 0; gi < GPS; ++gi)
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            scur[m][gi][t] = snxt[m][gi][t];
+            bcur[m][gi][t] = bnxt[m][gi][t];
+          }
+      }
+    }
+    __syncthreads();
+  }
+  if (!wave_cols_ok) return;
+  // D[row 4 kq + i][column c] of each 16 x 16 tile
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    if (r >= nt) break;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 16 * r + 4 * kq + i;
+      if (row >= cnt) continue;
+      const size_t base = (size_t)dst_rows[row] * N;
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const int col = col0 + 16 * t + c;
+        if (col < N) store_out<EPI>(out, base + col, acc[0][r][t][i], acc[NM - 1][r][t][i], limit);
+      }
+    }
+  }
+}
+
+// ---- routed experts ----------------------------------------------------------------------------------------------------
+
+template <int GS, int NM>
+struct ExpertWords {
+  const uint32_t* base;      // the lane's (expert, column block): + c * 4 + kq applied
+  const uint32_t* sbase;
+  __device__ __forceinline__ uint32_t word(int g, int m, int i, int t) const {
+    return base[((size_t)g * NM + m) * block_words(GS) + i * 128 + t * 64];
+  }
+  __device__ __forceinline__ void sb(int g, int m, int t, float& s, float& b) const {
+    const uint32_t v = sbase[((size_t)g * NM + m) * block_words(GS) + t * 16];
+    s = bf16_lo(v);
+    b = bf16_hi(v);
+  }
+};
+
+template <int GS, int NM, int EPI, int RT>
+__global__ void __launch_bounds__(256)
+    experts_prefill_kernel(const uint16_t* __restrict__ X, int64_t x_stride, int slots, const uint32_t* __restrict__ W,
+                           int KG, int NB, const int* __restrict__ items, const int* __restrict__ counts,
+                           const int* __restrict__ members, void* __restrict__ out, int N, float limit) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  __shared__ int src_rows[16 * RT], dst_rows[16 * RT];
+  const int nbt = (NB + 3) >> 2;
+  const int it = blockIdx.x / nbt, cbt = blockIdx.x - it * nbt;
+  if (it >= counts[0]) return;
+  const int e = items[3 * it], first = items[3 * it + 1], cnt = min(items[3 * it + 2], 16 * RT);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, kq = lane >> 4;
+  if (tid < 16 * RT) {
+    const int p = members[first + (tid < cnt ? tid : 0)];
+    dst_rows[tid] = p;
+    src_rows[tid] = slots ? p / slots : p;
+  }
+  __syncthreads();
+  const int nb = cbt * 4 + wave;
+  const bool ok = nb < NB;
+  ExpertWords<GS, NM> ws;
+  const uint32_t* blk = W + (((size_t)e * NB + (ok ? nb : NB - 1)) * KG) * (size_t)(NM * block_words(GS));
+  ws.base = blk + c * 4 + kq;
+  ws.sbase = blk + 32 * GS / 8 + c;
+  mfma_body<GS, NM, EPI, RT>(X, x_stride, KG * GS, ws, src_rows, cnt, out, N, nb * 32, ok, dst_rows, limit, smem);
+}
+
+// ---- dense prompt matmul --------------------------------------------------------------------------------------------
+
+template <int GS>
+struct LaneWords {
+  const uint32_t* base;      // the lane's 64-column tile: + (32 * half + c) * 4 + kq applied
+  const uint16_t* S;
+  const uint16_t* B;
+  int64_t stride;
+  int KG;
+  __device__ __forceinline__ uint32_t word(int g, int, int i, int t) const {
+    return base[((size_t)g * (GS / 32) + i) * 256 + t * 64];
+  }
+  __device__ __forceinline__ void sb(int g, int, int t, float& s, float& b) const {
+    s = bf16_f32(S[(size_t)g * stride + t * 16]);
+    b = bf16_f32(B[(size_t)g * stride + t * 16]);
+  }
+};
+
+template <int GS, int EPI, int RT>
+__global__ void __launch_bounds__(256)
+    qmm_prefill_kernel(const uint16_t* __restrict__ X, int64_t ldx, const uint32_t* __restrict__ W,
+                       const uint16_t* __restrict__ S, const uint16_t* __restrict__ B, void* __restrict__ out, int M,
+                       int N, int KG, int npad) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  __shared__ int rows[16 * RT];
+  const int ct = (N + 127) >> 7;
+  const int rt = blockIdx.x / ct, cbt = blockIdx.x - rt * ct;
+  const int m0 = rt * 16 * RT, cnt = min(16 * RT, M - m0);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, kq = lane >> 4;
+  if (tid < 16 * RT) rows[tid] = m0 + (tid < cnt ? tid : 0);
+  __syncthreads();
+  const int col0 = cbt * 128 + wave * 32;
+  const bool ok = col0 < N;                      // columns up to npad are stored zeros, safe to read
+  const int tile = (ok ? col0 : 0) >> 6, half = (col0 >> 5) & 1;
+  LaneWords<GS> ws;
+  ws.base = W + ((size_t)tile * KG) * (size_t)(GS / 32 * 256) + (32 * half + c) * 4 + kq;
+  ws.S = S + (ok ? col0 : 0) + c;
+  ws.B = B + (ok ? col0 : 0) + c;
+  ws.stride = npad;
+  ws.KG = KG;
+  mfma_body<GS, 1, EPI, RT>(X, ldx, KG * GS, ws, rows, cnt, out, N, col0, ok, rows, 0.f, smem);
+}
+
+template <int RT>
+constexpr size_t stage_bytes() {
+  return 2 * (size_t)(16 * RT) * AROW;
+}
+
+template <int GS, int NM, int EPI>
+int launch_experts_prefill(int tile, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg, int nb,
+                           const int* items, const int* counts, const int* members, void* out, int n, float limit,
+                           int64_t max_items, hipStream_t s) {
+  const int64_t grid = max_items * ((nb + 3) / 4);
+  if (grid < 1) return 0;
+  TF_REQUIRE(grid <= 0x7FFFFFFF, "experts: %lld workgroups exceed the grid limit", (long long)grid);
+  const dim3 g((unsigned)grid), b(256);
+  if (tile == 16)
+    experts_prefill_kernel<GS, NM, EPI, 1><<<g, b, stage_bytes<1>(), s>>>(x, x_stride, slots, w, kg, nb, items, counts,
+                                                                         members, out, n, limit);
+  else if (tile == 64)
+    experts_prefill_kernel<GS, NM, EPI, 4><<<g, b, stage_bytes<4>(), s>>>(x, x_stride, slots, w, kg, nb, items, counts,
+                                                                         members, out, n, limit);
+  else
+    experts_prefill_kernel<GS, NM, EPI, 8><<<g, b, stage_bytes<8>(), s>>>(x, x_stride, slots, w, kg, nb, items, counts,
+                                                                         members, out, n, limit);
+  TF_LAUNCH_OK("tf_experts_prefill");
+  return 0;
+}
+
+template <int GS, int EPI>
+int launch_qmm_prefill(const uint16_t* x, int64_t ldx, const uint32_t* w, const uint16_t* s, const uint16_t* b,
+                       void* out, int m, int n, int kg, hipStream_t st) {
+  const int npad = (n + 127) / 128 * 128;
+  const int ct = (n + 127) / 128;
+  if (m <= 16) {
+    qmm_prefill_kernel<GS, EPI, 1><<<(unsigned)(((m + 15) / 16) * ct), 256, stage_bytes<1>(), st>>>(x, ldx, w, s, b, out,
+                                                                                                   m, n, kg, npad);
+  } else if (m <= 64) {
+    qmm_prefill_kernel<GS, EPI, 4><<<(unsigned)(((m + 63) / 64) * ct), 256, stage_bytes<4>(), st>>>(x, ldx, w, s, b, out,
+                                                                                                   m, n, kg, npad);
+  } else {
+    const int64_t grid = (int64_t)((m + 127) / 128) * ct;
+    TF_REQUIRE(grid <= 0x7FFFFFFF, "qmm_prefill: grid too large");
+    qmm_prefill_kernel<GS, EPI, 8><<<(unsigned)grid, 256, stage_bytes<8>(), st>>>(x, ldx, w, s, b, out, m, n, kg, npad);
+  }
+  TF_LAUNCH_OK("tf_qmm_prefill");
+  return 0;
+}
+
+}  // namespace
+}  // namespace tf
+
+using namespace tf;
+
+extern "C" int tf_experts_prefill(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w,
+                                  int kg, int nb, const int32_t* items, const int32_t* counts, const int32_t* members,
+                                  void* out, int n, float limit, int64_t max_items, int tile, tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(gs == 32 || gs == 64, "experts: groups of 32 or 64 inputs, not %d", gs);
+  TF_REQUIRE(x && w && items && counts && members && out, "experts: null pointer argument");
+  TF_REQUIRE(kg >= 1 && nb >= 1 && n == nb * 32, "experts: n (%d) must be the column blocks (%d) times 32", n, nb);
+  TF_REQUIRE(aligned16(x) && x_stride % 8 == 0, "x: rows of K = groups * group size inputs, 16-byte aligned");
+  TF_REQUIRE(tile == 16 || tile == 64 || tile == 128, "prefill items hold 16, 64 or 128 pairs, not %d", tile);
+  TF_REQUIRE(slots >= 0 && max_items >= 0, "experts: negative slots or max_items");
+  hipStream_t s = as_stream(stream);
+#define TF_PRE(GS_, NM_, EPI_) \
+  if (gs == GS_ && epi == EPI_) \
+    return launch_experts_prefill<GS_, NM_, EPI_>(tile, x, x_stride, slots, w, kg, nb, items, counts, members, out, n, limit, max_items, s);
+  TF_PRE(32, 1, 0) TF_PRE(32, 1, 1) TF_PRE(32, 1, 3) TF_PRE(32, 2, 2)
+  TF_PRE(64, 1, 0) TF_PRE(64, 1, 1) TF_PRE(64, 1, 3) TF_PRE(64, 2, 2)
+#undef TF_PRE
+  set_error("experts: no prefill kernel for group %d and epilogue %d", gs, epi);
+  return 1;
+}
+
+extern "C" int tf_qmm_prefill(const uint16_t* x, int64_t ldx, const uint32_t* weight, const uint16_t* scales,
+                              const uint16_t* biases, void* out, int m, int n, int k, int gs, int f32, int tile,
+                              tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(gs == 32 || gs == 64, "groups of 32 or 64");
+  TF_REQUIRE(tile >= 0 && tile <= 11, "tile 0-11");
+  TF_REQUIRE(x && weight && scales && biases && out && m >= 1 && n >= 1, "qmm_prefill: null pointer or empty shape");
+  TF_REQUIRE(aligned16(x) && (m == 1 || ldx % 8 == 0), "x rows must start on 16-byte boundaries");
+  TF_REQUIRE(k >= gs && k % gs == 0, "K splits into whole groups");
+  hipStream_t s = as_stream(stream);
+  const int kg = k / gs;
+  if (gs == 64) return f32 ? launch_qmm_prefill<64, 0>(x, ldx, weight, scales, biases, out, m, n, kg, s)
+                           : launch_qmm_prefill<64, 3>(x, ldx, weight, scales, biases, out, m, n, kg, s);
+  return f32 ? launch_qmm_prefill<32, 0>(x, ldx, weight, scales, biases, out, m, n, kg, s)
+             : launch_qmm_prefill<32, 3>(x, ldx, weight, scales, biases, out, m, n, kg, s);
+}

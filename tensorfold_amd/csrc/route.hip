@@ -1,0 +1,311 @@
+// MoE glue around the expert kernels: router logits, per-row top-k, the stable grouping of pairs by expert, and the
+// weighted combine.  All integer results (ids, members, items) are deterministic and independent of the row count.
+
+#include "tf_common.h"
+
+namespace tf {
+namespace {
+
+// ---- router: logits[m, e] = x[m] . rows[e], bf16 MFMA, K in steps of 32 in order ------------------------------------
+
+__global__ void __launch_bounds__(64)
+    router_kernel(const uint16_t* __restrict__ X, int64_t ldx, const uint16_t* __restrict__ R, float* __restrict__ out,
+                  int M, int D, int NE) {
+  const int lane = threadIdx.x, r = lane & 15, kq = lane >> 4;
+  const int m0 = blockIdx.x * 16, e0 = blockIdx.y * 16;
+  const uint16_t* xa = X + (size_t)min(m0 + r, M - 1) * ldx + kq * 8;
+  const uint16_t* wb = R + (size_t)min(e0 + r, NE - 1) * D + kq * 8;
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < D; k0 += 32) {
+    const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(xa + k0);
+    const bf16x8_t b = *reinterpret_cast<const bf16x8_t*>(wb + k0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0);
+  }
+  const int col = e0 + r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = m0 + 4 * kq + i;
+    if (row < M && col < NE) out[(size_t)row * NE + col] = acc[i];
+  }
+}
+
+// ---- top-k: one wave a row ------------------------------------------------------------------------------------------
+
+constexpr int TOPK_VPL = 16;     // values a lane: up to 1024 experts
+
+__global__ void __launch_bounds__(64)
+    topk_kernel(const float* __restrict__ L, int64_t ldl, int NE, int TOPK, int shared, int* __restrict__ pick,
+                float* __restrict__ wts) {
+  const int r = blockIdx.x, lane = threadIdx.x, slots = TOPK + (shared ? 1 : 0);
+  const float* row = L + (size_t)r * ldl;
+  const float NEG = -__builtin_inff();
+  float v[TOPK_VPL];
+#pragma unroll
+  for (int i = 0; i < TOPK_VPL; ++i) {
+    const int e = lane + 64 * i;
+    v[i] = e < NE ? row[e] : NEG;
+  }
+  float top = 0.f, total = 0.f, mine_ex = 0.f;
+  int mine_id = 0;
+  for (int k = 0; k < TOPK; ++k) {
+    float bv = v[0];
+    int bi = lane;
+#pragma unroll
+    for (int i = 1; i < TOPK_VPL; ++i)
+      if (v[i] > bv) {
+        bv = v[i];
+        bi = lane + 64 * i;
+      }
+    float m = bv;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+    int idx = bv == m ? bi : 0x7FFFFFFF;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) idx = min(idx, __shfl_xor(idx, o));
+    if (k == 0) top = m;
+    const float ex = expf(m - top);
+    total += ex;
+    if (lane == k) {
+      mine_ex = ex;
+      mine_id = idx;
+    }
+    if ((idx & 63) == lane) {
+#pragma unroll
+      for (int i = 0; i < TOPK_VPL; ++i)
+        if (i == (idx >> 6)) v[i] = NEG;
+    }
+  }
+  if (lane < TOPK) {
+    pick[(size_t)r * slots + lane] = mine_id;
+    wts[(size_t)r * slots + lane] = round_bf16(mine_ex / total);
+  }
+  if (shared && lane == 0) {
+    const float sg = round_bf16(row[NE]);
+    pick[(size_t)r * slots + TOPK] = NE;
+    wts[(size_t)r * slots + TOPK] = round_bf16(1.f / (1.f + expf(-sg)));
+  }
+}
+
+// ---- plan: stable counting sort of pairs by expert -------------------------------------------------------------------
+
+constexpr int PLAN_THREADS = 1024;
+constexpr int EMAX = 1024;
+
+// Block-wide exclusive prefix sums of three per-thread values (1024 threads = 16 waves of 64); totals in tot[3].
+__device__ void scan3(int (&val)[3], int (&excl)[3], int (&tot)[3]) {
+  __shared__ int wsum[3][16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int inc[3];
+#pragma unroll
+  for (int s = 0; s < 3; ++s) {
+    int a = val[s];
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int u = __shfl_up(a, o);
+      if (lane >= o) a += u;
+    }
+    inc[s] = a;
+    if (lane == 63) wsum[s][wave] = a;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int s = 0; s < 3; ++s) {
+    int base = 0, all = 0;
+    for (int w = 0; w < 16; ++w) {
+      const int t = wsum[s][w];
+      if (w < wave) base += t;
+      all += t;
+    }
+    excl[s] = base + inc[s] - val[s];
+    tot[s] = all;
+  }
+  __syncthreads();
+}
+
+// thread e: expert e's pair count c -> its first member; writes the items (expert order) and counts
+__device__ int place_items(int c, int E, int T, int* __restrict__ items, int* __restrict__ counts) {
+  const int tid = threadIdx.x;
+  const int tiles = (c + T - 1) / T;
+  int val[3] = {c, tiles, c > 0 ? 1 : 0}, excl[3], tot[3];
+  scan3(val, excl, tot);
+  if (tid == 0) {
+    counts[0] = tot[1];
+    counts[1] = tot[2];
+  }
+  if (tid < E)
+    for (int j = 0; j < tiles; ++j) {
+      int* it = items + 3 * (excl[1] + j);
+      it[0] = tid;
+      it[1] = excl[0] + T * j;
+      it[2] = min(T, c - T * j);
+    }
+  return excl[0];
+}
+
+// up to 1024 pairs: one block does everything
+__global__ void __launch_bounds__(PLAN_THREADS)
+    plan_small_kernel(const int* __restrict__ picks, int P, int E, int T, int* __restrict__ members,
+                      int* __restrict__ items, int* __restrict__ counts) {
+  __shared__ int pk[PLAN_THREADS];
+  __shared__ int cnt[EMAX];
+  __shared__ int off[EMAX];
+  const int tid = threadIdx.x;
+  cnt[tid] = 0;
+  __syncthreads();
+  int e = -1;
+  if (tid < P) {
+    e = picks[tid];
+    if ((unsigned)e >= (unsigned)E) e = -1;          // an id outside the table joins no expert (and faults nothing)
+    pk[tid] = e;
+    if (e >= 0) atomicAdd(&cnt[e], 1);
+  }
+  __syncthreads();
+  const int o = place_items(tid < E ? cnt[tid] : 0, E, T, items, counts);
+  off[tid] = o;
+  __syncthreads();
+  if (tid < P && e >= 0) {
+    int rank = 0;
+    for (int q = 0; q < tid; ++q) rank += pk[q] == e;
+    members[off[e] + rank] = tid;
+  }
+}
+
+// wide plans, pass 1: block b ranks its 1024 pairs within each expert (pair order) and leaves its counts in hist[b]
+__global__ void __launch_bounds__(PLAN_THREADS)
+    plan_rank_kernel(const int* __restrict__ picks, int P, int E, int* __restrict__ rank, int* __restrict__ hist) {
+  __shared__ int pk[PLAN_THREADS];
+  __shared__ int cnt[EMAX];
+  const int tid = threadIdx.x, p = blockIdx.x * PLAN_THREADS + tid;
+  cnt[tid] = 0;
+  __syncthreads();
+  int e = -1;
+  if (p < P) {
+    e = picks[p];
+    if ((unsigned)e >= (unsigned)E) e = -1;
+    if (e >= 0) atomicAdd(&cnt[e], 1);
+  }
+  pk[tid] = e;
+  __syncthreads();
+  if (p < P && e >= 0) {
+    int rk = 0;
+    for (int q = 0; q < tid; ++q) rk += pk[q] == e;
+    rank[p] = rk;
+  }
+  if (tid < E) hist[(size_t)blockIdx.x * E + tid] = cnt[tid];
+}
+
+// pass 2, one block: hist[b][e] becomes block b's first member of expert e; items and counts are written
+__global__ void __launch_bounds__(PLAN_THREADS)
+    plan_offsets_kernel(int nblk, int E, int T, int* __restrict__ hist, int* __restrict__ items,
+                        int* __restrict__ counts) {
+  const int tid = threadIdx.x;
+  int c = 0;
+  if (tid < E)
+    for (int b = 0; b < nblk; ++b) {
+      int* h = hist + (size_t)b * E + tid;
+      const int v = *h;
+      *h = c;
+      c += v;
+    }
+  const int off = place_items(c, E, T, items, counts);
+  if (tid < E)
+    for (int b = 0; b < nblk; ++b) hist[(size_t)b * E + tid] += off;
+}
+
+// pass 3: every pair to its place
+__global__ void plan_scatter_kernel(const int* __restrict__ picks, int P, int E, const int* __restrict__ rank,
+                                    const int* __restrict__ hist, int* __restrict__ members) {
+  const int p = blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= P) return;
+  const int e = picks[p];
+  if ((unsigned)e < (unsigned)E) members[hist[(size_t)(p / PLAN_THREADS) * E + e] + rank[p]] = p;
+}
+
+// ---- combine ---------------------------------------------------------------------------------------------------------
+
+template <bool YBF16>
+__global__ void __launch_bounds__(256)
+    combine_kernel(const void* __restrict__ Y, const float* __restrict__ Wt, uint16_t* __restrict__ out, int S, int D) {
+  const int r = blockIdx.x;
+  const int d = (blockIdx.y * 256 + threadIdx.x) * 2;
+  if (d >= D) return;
+  float a0 = 0.f, a1 = 0.f;
+  for (int k = 0; k < S; ++k) {
+    const float w = Wt[(size_t)r * S + k];
+    const size_t at = ((size_t)r * S + k) * D + d;
+    if (YBF16) {
+      const uint32_t v = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(Y) + at);
+      a0 = fmaf(w, bf16_lo(v), a0);
+      a1 = fmaf(w, bf16_hi(v), a1);
+    } else {
+      const float2 v = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(Y) + at);
+      a0 = fmaf(w, v.x, a0);
+      a1 = fmaf(w, v.y, a1);
+    }
+  }
+  *reinterpret_cast<uint32_t*>(out + (size_t)r * D + d) = pack_bf16(a0, a1);
+}
+
+}  // namespace
+}  // namespace tf
+
+using namespace tf;
+
+extern "C" int tf_moe_router(const uint16_t* x, int64_t ldx, const uint16_t* rows, float* logits, int m, int d, int ne,
+                             tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(x && rows && logits && m >= 1 && ne >= 1, "router: null pointer or empty shape");
+  TF_REQUIRE(d >= 32 && d % 32 == 0, "router: the hidden size (%d) must be a multiple of 32", d);
+  TF_REQUIRE(aligned16(x) && aligned16(rows) && ldx % 8 == 0, "router: x and rows must be 16-byte aligned");
+  router_kernel<<<dim3((m + 15) / 16, (ne + 15) / 16), 64, 0, as_stream(stream)>>>(x, ldx, rows, logits, m, d, ne);
+  TF_LAUNCH_OK("tf_moe_router");
+  return 0;
+}
+
+extern "C" int tf_moe_topk(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared,
+                           int32_t* pick, float* wts, tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(logits && pick && wts && rows >= 1, "topk: null pointer or empty shape");
+  TF_REQUIRE(experts >= 1 && experts <= 64 * TOPK_VPL, "topk: 1 to %d experts, not %d", 64 * TOPK_VPL, experts);
+  TF_REQUIRE(top_k >= 1 && top_k <= 64 && top_k <= experts, "topk: 1 to 64 experts a row, not %d", top_k);
+  TF_REQUIRE(ldl >= experts + (shared ? 1 : 0), "topk: logits rows hold %lld values, %d are read", (long long)ldl,
+             experts + (shared ? 1 : 0));
+  topk_kernel<<<rows, 64, 0, as_stream(stream)>>>(logits, ldl, experts, top_k, shared, pick, wts);
+  TF_LAUNCH_OK("tf_moe_topk");
+  return 0;
+}
+
+extern "C" int tf_experts_plan(const int32_t* picks, int64_t pairs, int experts, int tile, int32_t* members,
+                               int32_t* items, int32_t* counts, int32_t* rank, int32_t* hist, tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(picks && members && items && counts, "plan: null pointer argument");
+  TF_REQUIRE(experts >= 1 && experts <= EMAX, "experts: at most %d experts", EMAX);
+  TF_REQUIRE(tile == 16 || tile == 64 || tile == 128, "items hold 16 pairs (decode) or 64 or 128 (prefill)");
+  TF_REQUIRE(pairs >= 0 && pairs <= 0x7FFFFFFF, "plan: pair count out of range");
+  hipStream_t s = as_stream(stream);
+  const int P = (int)pairs;
+  if (P <= PLAN_THREADS) {
+    plan_small_kernel<<<1, PLAN_THREADS, 0, s>>>(picks, P, experts, tile, members, items, counts);
+    TF_LAUNCH_OK("tf_experts_plan");
+    return 0;
+  }
+  TF_REQUIRE(rank && hist, "experts: plan scratch (rank, hist) is needed past %d pairs", PLAN_THREADS);
+  const int nblk = (P + PLAN_THREADS - 1) / PLAN_THREADS;
+  plan_rank_kernel<<<nblk, PLAN_THREADS, 0, s>>>(picks, P, experts, rank, hist);
+  plan_offsets_kernel<<<1, PLAN_THREADS, 0, s>>>(nblk, experts, tile, hist, items, counts);
+  plan_scatter_kernel<<<(P + 255) / 256, 256, 0, s>>>(picks, P, experts, rank, hist, members);
+  TF_LAUNCH_OK("tf_experts_plan");
+  return 0;
+}
+
+extern "C" int tf_moe_combine(const void* y, int y_bf16, const float* wts, uint16_t* out, int rows, int slots, int d,
+                              tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(y && wts && out && rows >= 1 && slots >= 1, "combine: null pointer or empty shape");
+  TF_REQUIRE(d >= 2 && d % 2 == 0, "combine: the hidden size (%d) must be even", d);
+  const dim3 grid(rows, (d / 2 + 255) / 256);
+  if (y_bf16) combine_kernel<true><<<grid, 256, 0, as_stream(stream)>>>(y, wts, out, slots, d);
+  else combine_kernel<false><<<grid, 256, 0, as_stream(stream)>>>(y, wts, out, slots, d);
+  TF_LAUNCH_OK("tf_moe_combine");
+  return 0;
+}

@@ -1,0 +1,94 @@
+// Shared by every translation unit of libtfmi: status/error plumbing, bf16 helpers, the 4-bit block geometry.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "../../include/tfmi.h"
+
+namespace tf {
+
+// ---- status -------------------------------------------------------------------------------------------------------
+
+void set_error(const char* fmt, ...);
+void clear_error();
+
+#define TF_REQUIRE(cond, ...)      \
+  do {                             \
+    if (!(cond)) {                 \
+      ::tf::set_error(__VA_ARGS__); \
+      return 1;                    \
+    }                              \
+  } while (0)
+
+// after a launch: a sticky or launch-time error becomes a status
+#define TF_LAUNCH_OK(what)                                                        \
+  do {                                                                            \
+    hipError_t e_ = hipGetLastError();                                            \
+    if (e_ != hipSuccess) {                                                       \
+      ::tf::set_error("%s: launch failed: %s", what, hipGetErrorString(e_));      \
+      return 2;                                                                   \
+    }                                                                             \
+  } while (0)
+
+inline hipStream_t as_stream(tf_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- vector types ------------------------------------------------------------------------------------------------
+
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+// ---- bf16 ----------------------------------------------------------------------------------------------------------
+
+__device__ __forceinline__ float bf16_lo(uint32_t v) { return __uint_as_float(v << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t v) { return __uint_as_float(v & 0xFFFF0000u); }
+__device__ __forceinline__ float bf16_f32(uint16_t v) { return __uint_as_float(static_cast<uint32_t>(v) << 16); }
+
+// round to nearest even (finite inputs; NaN stays NaN because the payload's top bit survives the add for quiet NaNs)
+__device__ __forceinline__ uint32_t f32_bf16_bits(float f) {
+  const uint32_t u = __float_as_uint(f);
+  return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ float round_bf16(float f) { return __uint_as_float(f32_bf16_bits(f) << 16); }
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  return f32_bf16_bits(lo) | (f32_bf16_bits(hi) << 16);
+}
+
+// ---- epilogues (rounding points of the reference's experts.cuh:53-70) ---------------------------------------------
+
+__device__ __forceinline__ float relu2(float a) {
+  const float u = fmaxf(round_bf16(a), 0.f);
+  return u * u;
+}
+
+__device__ __forceinline__ float swiglu(float g, float u, float limit) {
+  float gv = round_bf16(g), uv = round_bf16(u);
+  if (limit > 0.f) {
+    gv = fminf(gv, limit);
+    uv = fminf(fmaxf(uv, -limit), limit);
+  }
+  return round_bf16(gv / (1.f + __expf(-gv))) * uv;
+}
+
+// ---- 4-bit blocks -------------------------------------------------------------------------------------------------
+
+constexpr uint32_t NIB_MASK = 0x000F000Fu;
+constexpr uint32_t BF16_128 = 0x43004300u;   // the bf16 pair (128, 128): OR-ing a nibble into the mantissa gives 128 + q
+
+// (word >> 4 i) & mask | 128.0: the bf16 pair (128 + q[2 i], 128 + q[2 i + 1]) of a packed word
+__device__ __forceinline__ uint32_t nib_pair(uint32_t word, int i) {
+  return ((word >> (4 * i)) & NIB_MASK) | BF16_128;
+}
+
+// int32 words of an experts block: 32 columns x gs inputs of codes, then 32 (scale | bias << 16) words
+__host__ __device__ constexpr int block_words(int gs) { return 32 * gs / 8 + 32; }
+
+}  // namespace tf

@@ -1,0 +1,172 @@
+"""EXL3 linear layers on MI355X: y = x @ W + bias for 1 to 128 rows, any codebook and width, row-invariant.
+
+Host side of ``tf_exl3_*``; the class and function names follow the reference's operator module
+(src/tensorfold/cuda/exl3/linear.py:30-204).  W = diag(suh) H W_q H diag(svh): ``rot_in`` rotates the input once a
+call (fp16 out), ``linear`` decodes each pair of k tiles straight into f16 MFMA operands, sums in fp32 in a fixed
+order and applies the output Hadamard, svh and the bias.
+"""
+
+from __future__ import annotations
+
+import dataclasses
+
+import torch
+
+from .. import _lib
+from . import format as fmt
+
+CODEBOOK_IDS = fmt.CODEBOOK_IDS
+_DTYPES = {torch.float16: 0, torch.bfloat16: 1, torch.float32: 2}
+
+
+def k2_of(bits: float) -> int:
+    """Twice the width: the integer the kernels are specialised on."""
+
+    return int(2 * fmt.check_bits(bits))
+
+
+def plan(k: int, n: int, blocks: int = 512, min_pairs: int = 4) -> tuple[int, int]:
+    """(K splits, waves a workgroup) of a K x N layer, from the shape alone so that a layer keeps one reduction
+    order at every row count.  An MI355X wants about two workgroups on each of its 256 CUs: K is split until
+    N/128 * splits reaches ``blocks`` while every wave keeps ``min_pairs`` pairs of k tiles."""
+
+    pairs, nb = k // 32, n // 128
+    wk = 4
+    while wk > 2 and pairs // wk < min_pairs:
+        wk //= 2
+    sk = 1
+    while sk < 64 and nb * sk < blocks and pairs // (2 * sk * wk) >= min_pairs:
+        sk *= 2
+    return sk, wk
+
+
+def strips(words: torch.Tensor) -> torch.Tensor:
+    """Trellis words [K/16, N/16, W] -> [N/128, K/16, 8, W] (a copy): each 128-column block's tiles in k order, the
+    order a workgroup walks."""
+
+    kt, nt, w = words.shape
+    return words.reshape(kt, nt // 8, 8, w).transpose(0, 1).contiguous()
+
+
+@dataclasses.dataclass
+class Exl3Linear:
+    """One EXL3 layer resident on the GPU."""
+
+    words: torch.Tensor           # int32 [N/128, K/16, 8, 8 * bits] ("strips") or [K/16, N/16, 8 * bits] ("stored")
+    suh: torch.Tensor             # fp16 [K]
+    svh: torch.Tensor             # fp16 [N]
+    bias: torch.Tensor | None     # fp16 [N]
+    bits: float
+    codebook: str
+    k: int
+    n: int
+    layout: str = "strips"
+    split: tuple[int, int] | None = None     # (K splits, waves); plan(k, n) when None
+
+    def __post_init__(self) -> None:
+        if self.split is None:
+            self.split = plan(self.k, self.n)
+        self._counters: torch.Tensor | None = None
+
+    @classmethod
+    def from_tensors(cls, trellis: torch.Tensor, suh: torch.Tensor, svh: torch.Tensor, codebook: str,
+                     bias: torch.Tensor | None = None, device: str | torch.device = "cuda",
+                     layout: str = "strips") -> "Exl3Linear":
+        """Build from a checkpoint group: trellis int16 [K/16, N/16, 16 * bits]; suh / svh fp16, or the int16 sign
+        words of older checkpoints; the codebook's name."""
+
+        bits = fmt.bits_of(trellis.shape)
+        fmt.check_pair(bits, codebook)
+        k, n = 16 * int(trellis.shape[0]), 16 * int(trellis.shape[1])
+        if k % fmt.HAD or n % fmt.HAD:
+            raise ValueError(f"K={k} and N={n} must be multiples of 128")
+        if layout not in ("strips", "stored"):
+            raise ValueError(f"layout must be 'strips' or 'stored', got {layout!r}")
+
+        def vector(t: torch.Tensor, size: int) -> torch.Tensor:
+            if t.dtype == torch.int16 and t.numel() * 16 == size:
+                t = torch.from_numpy(fmt.unpack_signs(t))
+            if t.dtype != torch.float16 or t.numel() != size:
+                raise ValueError(f"scales must be fp16 [{size}] or int16 sign words [{size // 16}]")
+            return t.reshape(size).to(device).contiguous()
+
+        words = trellis.to(device).contiguous().view(torch.int32)
+        if layout == "strips":
+            words = strips(words)
+        b = None if bias is None else bias.to(device=device, dtype=torch.float16).contiguous()
+        return cls(words, vector(suh, k), vector(svh, n), b, bits, codebook, k, n, layout)
+
+    @property
+    def k2(self) -> int:
+        return k2_of(self.bits)
+
+    @property
+    def strides(self) -> tuple[int, int]:
+        """int32 words from one k tile to the next, and from one 128-column block to the next."""
+
+        tile = 4 * self.k2
+        if self.layout == "strips":
+            return 8 * tile, (self.k // 16) * 8 * tile
+        return (self.n // 16) * tile, 8 * tile
+
+    def nbytes(self) -> int:
+        return self.words.numel() * 4
+
+    @property
+    def counters(self) -> torch.Tensor:
+        """Arrival counters of the K splits, zero between calls."""
+
+        if self._counters is None:
+            self._counters = torch.zeros((8 * (self.n // 128),), dtype=torch.int32, device=self.words.device)
+        return self._counters
+
+    def __call__(self, x: torch.Tensor, out: torch.Tensor | None = None, out_dtype: torch.dtype | None = None,
+                 xh: torch.Tensor | None = None, z: torch.Tensor | None = None) -> torch.Tensor:
+        """y [M, N] for x [M, K], M = 1..128 (fp16, bf16 or fp32 in and out).  ``xh`` (fp16 [M, K]) and ``z`` (fp32
+        [splits * M * N]) are scratch, allocated here when not passed."""
+
+        if x.dim() != 2 or x.shape[1] != self.k or not 1 <= x.shape[0] <= 128:
+            raise ValueError(f"x must be [1..128, {self.k}], got {tuple(x.shape)}")
+        if x.dtype not in _DTYPES:
+            raise ValueError("x: expected fp16, bf16 or fp32")
+        _lib.on_gpu(x)
+        x = x.contiguous()
+        m = int(x.shape[0])
+        if out is None:
+            out = x.new_empty((m, self.n), dtype=out_dtype or x.dtype)
+        sk, wk = self.split
+        if xh is None:
+            xh = x.new_empty((m, self.k), dtype=torch.float16)
+        if sk > 1 and z is None:
+            z = x.new_empty((sk * m * self.n,), dtype=torch.float32)
+        stride_k, stride_nb = self.strides
+        _lib.call("tf_exl3_rot_in", _lib.ptr(x), _DTYPES[x.dtype], _lib.ptr(self.suh), _lib.ptr(xh), m, self.k)
+        _lib.call("tf_exl3_linear", _lib.ptr(xh), _lib.ptr(self.words), stride_k, stride_nb, _lib.ptr(self.svh),
+                  _lib.ptr(self.bias), _lib.ptr(out), _DTYPES[out.dtype], _lib.ptr(z) if sk > 1 else None,
+                  _lib.ptr(self.counters), m, self.k, self.n, self.k2, CODEBOOK_IDS[self.codebook], sk, wk)
+        return out
+
+    def unpack(self, out: torch.Tensor | None = None) -> torch.Tensor:
+        """W_q [K, N] fp16, decoded on the GPU from either layout."""
+
+        w = out if out is not None else self.words.new_empty((self.k, self.n), dtype=torch.float16)
+        _lib.call("tf_exl3_unpack", _lib.ptr(self.words), _lib.ptr(w), self.k, self.n, *self.strides, self.k2,
+                  CODEBOOK_IDS[self.codebook])
+        return w
+
+
+def unpack_gpu(trellis: torch.Tensor, codebook: str) -> torch.Tensor:
+    """W_q [K, N] fp16 from trellis int16 [K/16, N/16, 16 * bits], decoded on the GPU from the stored order."""
+
+    bits = fmt.bits_of(trellis.shape)
+    fmt.check_pair(bits, codebook)
+    words = trellis.cuda().contiguous().view(torch.int32)
+    k, n = 16 * int(trellis.shape[0]), 16 * int(trellis.shape[1])
+    w = words.new_empty((k, n), dtype=torch.float16)
+    tile = 4 * k2_of(bits)
+    _lib.call("tf_exl3_unpack", _lib.ptr(words), _lib.ptr(w), k, n, (n // 16) * tile, 8 * tile, k2_of(bits),
+              CODEBOOK_IDS[codebook])
+    return w
+
+
+unpack_cuda = unpack_gpu      # the name the reference's callers use (torch keeps the "cuda" device name on ROCm)

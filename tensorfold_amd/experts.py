@@ -1,0 +1,190 @@
+"""Routed-expert matmuls over 4-bit affine tables (MI355X).
+
+Host side of ``tf_experts_*`` in ``include/tfmi.h``.  The function names, argument order and error behaviour follow
+the operator interface the reference's engines call (reference: src/tensorfold/cuda/experts.py:28-150), so an
+engine can swap the import; everything below the signatures is this package's own.
+
+Contract kept from the reference: the bits computed for a (row, slot) pair are a function of that row and that
+expert only - not of the other rows in the call, of the item the pair lands in, or of the row count.
+"""
+
+from __future__ import annotations
+
+import dataclasses
+
+import torch
+
+from . import _lib
+
+COLS = 32             # columns of one weight block
+TILE = 16             # largest decode item, in pairs
+PREFILL_TILE = 64     # default prompt item; the MFMA kernel also takes 16 and 128
+SMALL = 1024          # a plan up to this many pairs is sorted by one workgroup
+_GROUPS = (32, 64)
+
+
+def block_words(gs: int) -> int:
+    """Size in int32 of the block covering 32 columns and one group: gs/8 code words a column plus one
+    (scale | bias << 16) word a column."""
+
+    return COLS * gs // 8 + COLS
+
+
+def _group_ok(gs: int) -> None:
+    if gs not in _GROUPS:
+        raise ValueError(f"groups of 32 or 64 inputs, not {gs}")
+
+
+def pack(words: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, gs: int) -> torch.Tensor:
+    """Stored MLX tensors of E experts -> kernel blocks.
+
+    words int32/uint32 [E, N, K/8]; scales, biases bf16 [E, N, K/gs]  ->  int32 [E, N/32, K/gs, block_words(gs)].
+    ``unpack`` is the exact inverse."""
+
+    _group_ok(gs)
+    e, n, k8 = words.shape
+    k = 8 * k8
+    want = (e, n, k // gs)
+    if n % COLS or k % gs or tuple(scales.shape) != want or tuple(biases.shape) != want:
+        raise ValueError(f"experts: shape {tuple(words.shape)} with scales {tuple(scales.shape)} does not pack")
+    _lib.on_gpu(words, scales, biases)
+    blocks = words.new_empty((e, n // COLS, k // gs, block_words(gs)), dtype=torch.int32)
+    _lib.call("tf_experts_pack", _lib.ptr(words.contiguous()), _lib.ptr(scales.contiguous()),
+              _lib.ptr(biases.contiguous()), e, n, k, gs, _lib.ptr(blocks))
+    return blocks
+
+
+def unpack(blocks: torch.Tensor, gs: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Kernel blocks [E, N/32, K/gs, block] -> (words [E, N, K/8], scales, biases [E, N, K/gs]).
+
+    ``blocks`` may be a view selecting one matrix of a stacked table (``table[:, :, :, m]``); it is copied only if
+    its strides are not those of such a view."""
+
+    _group_ok(gs)
+    e, nb, kg, bw = blocks.shape
+    if bw != block_words(gs):
+        raise ValueError(f"experts: blocks of {bw} words are not groups of {gs}")
+    s0, s1, s2, s3 = blocks.stride()
+    if not (s3 == 1 and s1 == kg * s2 and s0 == nb * s1):
+        blocks = blocks.contiguous()
+        s2 = blocks.stride(2)
+    n, k = nb * COLS, kg * gs
+    words = blocks.new_empty((e, n, k // 8), dtype=torch.int32)
+    scales = blocks.new_empty((e, n, kg), dtype=torch.bfloat16)
+    biases = torch.empty_like(scales)
+    _lib.call("tf_experts_unpack", _lib.ptr(blocks), s2, e, n, k, gs, _lib.ptr(words), _lib.ptr(scales),
+              _lib.ptr(biases))
+    return words, scales, biases
+
+
+@dataclasses.dataclass
+class Experts:
+    """The packed experts of one layer.
+
+    up   int32 [E, NI/32, D/gs, M, block]  M = 2: gate then up (SwiGLU); M = 1: up alone (relu^2)
+    down int32 [E, D/32, NI/gs, 1, block]
+    """
+
+    up: torch.Tensor
+    down: torch.Tensor
+    gs: int
+    width: int           # NI
+    dims: int            # D
+    limit: float = 0.0   # SwiGLU clip, 0 for none
+
+    @property
+    def count(self) -> int:
+        return int(self.up.shape[0])
+
+    @property
+    def swiglu(self) -> bool:
+        return int(self.up.shape[3]) == 2
+
+    def bytes_per_expert(self) -> int:
+        return 4 * (self.up[0].numel() + self.down[0].numel())
+
+
+def make(up: list[tuple], down: tuple, gs: int, *, limit: float = 0.0) -> Experts:
+    """Pack a layer.  ``up`` = [(words, scales, biases)] for relu^2 or [gate, up] for SwiGLU; ``down`` one triple."""
+
+    if len(up) not in (1, 2):
+        raise ValueError("experts take a gate and an up projection, or an up projection alone")
+    ni, d = int(up[0][0].shape[1]), 8 * int(up[0][0].shape[2])
+    table_up = torch.stack([pack(w, s, b, gs) for (w, s, b) in up], dim=3)
+    table_down = pack(*down, gs).unsqueeze(3)
+    return Experts(table_up, table_down, gs, ni, d, float(limit))
+
+
+def max_items(pairs: int, experts: int, tile: int = TILE) -> int:
+    """Upper bound on the items of any plan over ``pairs`` pairs: each used expert opens one item and every full
+    ``tile`` pairs can open one more.  Grids are sized with it; the live count stays on the device."""
+
+    return min(pairs, experts) + pairs // tile
+
+
+class Plan:
+    """Device scratch of the pair sort: ``members`` (pairs ordered by expert), ``items`` rows of
+    (expert, first member, count) and ``counts`` = (items, distinct experts).  Sized once for ``rows`` x ``slots``."""
+
+    def __init__(self, rows: int, slots: int, experts: int, device: torch.device | str, *,
+                 prefill: bool = False) -> None:
+        self.rows, self.slots, self.experts, self.prefill = rows, slots, experts, prefill
+        self.tile = PREFILL_TILE if prefill else TILE
+        pairs = rows * slots
+
+        def ints(*shape: int) -> torch.Tensor:
+            return torch.zeros(shape, dtype=torch.int32, device=device)
+
+        self.members = ints(pairs)
+        self.items = ints(max_items(pairs, experts, TILE), 3)     # sized for the narrowest item any consumer takes
+        self.counts = ints(2)
+        blocks = -(-pairs // SMALL)
+        self.rank = ints(pairs if pairs > SMALL else 1)            # the multi-workgroup sort's scratch
+        self.hist = ints(blocks * experts if pairs > SMALL else 1)
+
+
+def route(picks: torch.Tensor, plan: Plan, tile: int = PREFILL_TILE) -> None:
+    """Sort the pairs of ``picks`` (int32 [R, slots], contiguous) into ``plan``.  ``tile`` is honoured by prompt
+    plans only; decode plans always use items of 16."""
+
+    rows, slots = picks.shape
+    if slots != plan.slots or rows > plan.rows:
+        raise ValueError(f"picks {tuple(picks.shape)} do not fit a plan of {plan.rows} x {plan.slots}")
+    if picks.dtype != torch.int32 or not picks.is_contiguous():
+        raise ValueError("picks: contiguous int32, one id a pair")
+    _lib.on_gpu(picks)
+    plan.tile = tile if plan.prefill else TILE
+    _lib.call("tf_experts_plan", _lib.ptr(picks), rows * slots, plan.experts, plan.tile, _lib.ptr(plan.members),
+              _lib.ptr(plan.items), _lib.ptr(plan.counts), _lib.ptr(plan.rank), _lib.ptr(plan.hist))
+
+
+def _launch(x: torch.Tensor, slots: int, table: torch.Tensor, gs: int, k: int, n: int, epi: int, plan: Plan,
+            out: torch.Tensor, limit: float, rows: int) -> None:
+    if x.dtype != torch.bfloat16 or x.dim() != 2 or x.stride(1) != 1 or x.stride(0) % 8 or x.shape[1] != k:
+        raise RuntimeError("x: rows of K = groups * group size inputs, 16-byte aligned")
+    if not out.is_contiguous() or out.shape[-1] != n:
+        raise RuntimeError("out: contiguous rows of n columns")
+    if out.dtype != (torch.float32 if epi == 0 else torch.bfloat16):
+        raise RuntimeError("out has the wrong dtype")
+    _lib.on_gpu(x, out)
+    bound = max_items(rows * plan.slots, plan.experts, plan.tile)
+    common = (gs, epi, _lib.ptr(x), x.stride(0), slots, _lib.ptr(table), k // gs, n // COLS, _lib.ptr(plan.items),
+              _lib.ptr(plan.counts), _lib.ptr(plan.members), _lib.ptr(out), n, limit)
+    if plan.prefill:
+        _lib.call("tf_experts_prefill", *common, bound, plan.tile)
+    else:
+        _lib.call("tf_experts_run", *common, bound * (n // COLS))
+
+
+def gate_up(x: torch.Tensor, ex: Experts, plan: Plan, out: torch.Tensor, rows: int) -> None:
+    """Token rows x bf16 [R, D] -> the activation of every pair, out bf16 [R * slots, NI]."""
+
+    _launch(x, plan.slots, ex.up, ex.gs, ex.dims, ex.width, 2 if ex.swiglu else 1, plan, out, ex.limit, rows)
+
+
+def down(act: torch.Tensor, ex: Experts, plan: Plan, out: torch.Tensor, rows: int) -> None:
+    """Pair activations bf16 [R * slots, NI] -> every pair's output [R * slots, D]: fp32, or bf16 when a prompt plan
+    is given a bf16 ``out``."""
+
+    epi = 3 if (plan.prefill and out.dtype == torch.bfloat16) else 0
+    _launch(act, 0, ex.down, ex.gs, ex.width, ex.dims, epi, plan, out, 0.0, rows)

@@ -1,0 +1,138 @@
+"""MoE layer glue (MI355X): router logits, per-row top-k with softmax-over-selected weights, the expert calls and the
+weighted combine.
+
+Host side of ``tf_moe_*``.  Names and signatures follow the reference's operator module
+(src/tensorfold/cuda/moe.py:41-186), whose Triton kernels the HIP ones replace.  Rules kept: fp32 logits, ties go
+to the lower expert id, weights are bf16-rounded values held in fp32, each row is routed and run independently, and
+the optional shared expert rides in the last slot with a sigmoid gate.
+"""
+
+from __future__ import annotations
+
+import dataclasses
+
+import torch
+
+from . import _lib
+from . import experts as grouped
+
+
+def router(x: torch.Tensor, rows: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """fp32 logits [R, rows.shape[0]] = x [R, D] @ rows.T, both bf16.  ``rows`` holds the router's rows followed, when
+    the layer has a shared expert, by that expert's gate row."""
+
+    _lib.on_gpu(x, rows)
+    if x.dtype != torch.bfloat16 or rows.dtype != torch.bfloat16 or x.stride(1) != 1 or not rows.is_contiguous():
+        raise ValueError("router: x and rows must be bf16 with unit-stride rows")
+    r, d = x.shape
+    ne = int(rows.shape[0])
+    if out is None:
+        out = x.new_empty((r, ne), dtype=torch.float32)
+    elif not out.is_contiguous() or tuple(out.shape) != (r, ne) or out.dtype != torch.float32:
+        raise ValueError("router: out must be contiguous [R, E + 1] fp32")
+    _lib.call("tf_moe_router", _lib.ptr(x), x.stride(0), _lib.ptr(rows), _lib.ptr(out), r, d, ne)
+    return out
+
+
+class MoEBuffers:
+    """Preallocated scratch of a layer for at most ``rows`` rows, so that a captured graph can replay it.
+
+    ``prefill`` selects the prompt arithmetic of the experts (and bf16 pair outputs); ``shared=False`` is for layers
+    without a shared expert: no extra logit column, no extra slot."""
+
+    def __init__(self, rows: int, cfg, device: torch.device | str, *, prefill: bool = False,
+                 shared: bool = True) -> None:
+        extra = int(shared)
+        self.rows, self.shared = rows, shared
+        self.slots = cfg.num_experts_per_tok + extra
+        f32 = dict(dtype=torch.float32, device=device)
+        self.logits = torch.empty((rows, cfg.num_experts + extra), **f32)
+        self.pick = torch.empty((rows, self.slots), dtype=torch.int32, device=device)
+        self.wts = torch.empty((rows, self.slots), **f32)
+        self.plan = grouped.Plan(rows, self.slots, cfg.num_experts + extra, device, prefill=prefill)
+        self.act = torch.empty((rows, self.slots, cfg.moe_intermediate_size), dtype=torch.bfloat16, device=device)
+        self.y = torch.empty((rows, self.slots, cfg.hidden_size), device=device,
+                             dtype=torch.bfloat16 if prefill else torch.float32)
+
+
+def select_rows(logits: torch.Tensor, buf: MoEBuffers, top_k: int, experts: int) -> None:
+    """Fill ``buf.pick`` / ``buf.wts`` for the rows of ``logits`` (one wave a row)."""
+
+    _lib.on_gpu(logits)
+    if logits.dtype != torch.float32 or logits.stride(1) != 1:
+        raise ValueError("select: logits must be fp32 with unit-stride rows")
+    _lib.call("tf_moe_topk", _lib.ptr(logits), logits.stride(0), int(logits.shape[0]), experts, top_k,
+              int(buf.shared), _lib.ptr(buf.pick), _lib.ptr(buf.wts))
+
+
+def select(logits: torch.Tensor, buf: MoEBuffers, top_k: int, experts: int,
+           tile: int = grouped.PREFILL_TILE) -> None:
+    """``select_rows`` followed by the pair sort into ``buf.plan`` (``tile``: a prompt plan's item size)."""
+
+    select_rows(logits, buf, top_k, experts)
+    grouped.route(buf.pick[:logits.shape[0]], buf.plan, tile)
+
+
+def moe(x: torch.Tensor, router_rows: torch.Tensor, ex: grouped.Experts, buf: MoEBuffers, top_k: int,
+        experts: int) -> MoEBuffers:
+    """Router, selection and both expert matmuls for x [R, D]; the pair outputs are left in ``buf.y`` [R, slots, D]
+    (the caller combines them, often fused with its residual add)."""
+
+    n = int(x.shape[0])
+    router(x, router_rows, buf.logits[:n])
+    select(buf.logits[:n], buf, top_k, experts)
+    act = buf.act.view(-1, ex.width)
+    grouped.gate_up(x, ex, buf.plan, act, n)
+    grouped.down(act, ex, buf.plan, buf.y.view(-1, ex.dims), n)
+    return buf
+
+
+def combine(y: torch.Tensor, wts: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """bf16 [R, D] = sum over slots, in slot order and in fp32, of wts[r, k] * y[r, k]; y is fp32 or bf16 [R, S, D]."""
+
+    _lib.on_gpu(y, wts)
+    if not y.is_contiguous() or not wts.is_contiguous() or wts.dtype != torch.float32:
+        raise ValueError("combine: y and wts must be contiguous, wts fp32")
+    r, s, d = y.shape
+    if out is None:
+        out = y.new_empty((r, d), dtype=torch.bfloat16)
+    _lib.call("tf_moe_combine", _lib.ptr(y), int(y.dtype == torch.bfloat16), _lib.ptr(wts), _lib.ptr(out), r, s, d)
+    return out
+
+
+@dataclasses.dataclass
+class Routed:
+    """What ``run`` needs of a layer: router rows bf16 [E + 1, D] (gate row of the shared expert last), the packed
+    E + 1 experts, and k."""
+
+    router: torch.Tensor
+    experts: grouped.Experts
+    top_k: int
+
+    @property
+    def count(self) -> int:
+        return int(self.router.shape[0]) - 1
+
+
+class _Dims:
+    """The four sizes MoEBuffers reads, taken from a ``Routed``."""
+
+    def __init__(self, m: Routed) -> None:
+        self.num_experts, self.num_experts_per_tok = m.count, m.top_k
+        self.hidden_size, self.moe_intermediate_size = m.experts.dims, m.experts.width
+
+
+_pool: dict[tuple, MoEBuffers] = {}
+
+
+def run(x: torch.Tensor, m: Routed, *, prefill: bool = False) -> torch.Tensor:
+    """The whole layer: bf16 [R, D] in, bf16 [R, D] out.  Scratch is pooled by the row count rounded up to a power
+    of two (16 at least), so every layer of a model shares it."""
+
+    n = int(x.shape[0])
+    cap = max(16, 1 << (n - 1).bit_length())
+    key = (cap, m.count, m.top_k, m.experts.width, m.experts.dims, prefill, x.device)
+    if key not in _pool:
+        _pool[key] = MoEBuffers(cap, _Dims(m), x.device, prefill=prefill)
+    buf = moe(x.contiguous(), m.router, m.experts, _pool[key], m.top_k, m.count)
+    return combine(buf.y[:n], buf.wts[:n])

@@ -1,0 +1,150 @@
+"""Dense 4-bit affine matmul ("lane matmul") on MI355X.
+
+Host side of ``tf_qmm*`` / ``tf_group_sums``.  The public names and signatures are the operator interface of the
+reference (src/tensorfold/cuda/kernels/qmm.py:41-219); the packed layout, the K split and the kernels are this
+package's.  Invariant kept: groups and K slices are walked identically at every row count, so a row's output bits
+do not depend on its neighbours.
+"""
+
+from __future__ import annotations
+
+import dataclasses
+
+import torch
+
+from . import _lib
+
+
+@dataclasses.dataclass
+class Q4:
+    """A packed (n, k) weight.
+
+    weight int32 [npad/64, k/gs, gs/32, 64, 4]  (64-column tiles; chunks of 32 inputs; 4 words a column a chunk)
+    scales, biases bf16 [k/gs, npad]            (npad = n rounded up to 128; padding is zero)
+    """
+
+    weight: torch.Tensor
+    scales: torch.Tensor
+    biases: torch.Tensor
+    n: int
+    k: int
+    gs: int
+
+    def nbytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in (self.weight, self.scales, self.biases))
+
+
+def pack(weight: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, gs: int) -> Q4:
+    """MLX layout (words [n, k/8] int32 or uint32, scales and biases [n, k/gs]) -> ``Q4``, in one kernel."""
+
+    if gs not in (32, 64):
+        raise ValueError(f"groups of 32 or 64 inputs, not {gs}")
+    words = weight if weight.dtype == torch.int32 else weight.view(torch.int32)
+    n, k8 = words.shape
+    k = 8 * k8
+    if k % gs or tuple(scales.shape) != (n, k // gs) or tuple(biases.shape) != (n, k // gs):
+        raise ValueError(f"qmm: shape {tuple(words.shape)} with scales {tuple(scales.shape)} does not pack")
+    _lib.on_gpu(words, scales, biases)
+    kg, npad = k // gs, 128 * -(-n // 128)
+    q = Q4(words.new_empty((npad // 64, kg, gs // 32, 64, 4)),
+           words.new_empty((kg, npad), dtype=torch.bfloat16), words.new_empty((kg, npad), dtype=torch.bfloat16),
+           n, k, gs)
+    _lib.call("tf_qmm_pack", _lib.ptr(words.contiguous()), _lib.ptr(scales.to(torch.bfloat16).contiguous()),
+              _lib.ptr(biases.to(torch.bfloat16).contiguous()), n, k, gs, _lib.ptr(q.weight), _lib.ptr(q.scales),
+              _lib.ptr(q.biases))
+    return q
+
+
+def unpack(q: Q4) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``pack`` inverted: (words [n, k/8], scales [n, k/gs], biases [n, k/gs])."""
+
+    kg = q.k // q.gs
+    words = q.weight.new_empty((q.n, q.k // 8))
+    scales = q.scales.new_empty((q.n, kg))
+    biases = q.scales.new_empty((q.n, kg))
+    _lib.call("tf_qmm_unpack", _lib.ptr(q.weight), _lib.ptr(q.scales.contiguous()), _lib.ptr(q.biases.contiguous()),
+              q.n, q.k, q.gs, _lib.ptr(words), _lib.ptr(scales), _lib.ptr(biases))
+    return words, scales, biases
+
+
+def split_k(n: int, k: int, gs: int = 64, target: int = 1024) -> int:
+    """Number of K slices of an (n, k) weight - from the shape alone, never the row count.
+
+    Doubles while there are fewer than ``target`` workgroups (64-column tiles x slices; an MI355X has 256 CUs and
+    wants a few workgroups on each), the groups still divide evenly and a slice keeps at least 4 groups."""
+
+    tiles, groups = -(-n // 64), k // gs
+    sk = 1
+    while sk < 16 and tiles * sk < target and groups % (2 * sk) == 0 and groups // (2 * sk) >= 4:
+        sk *= 2
+    return sk
+
+
+def bucket(m: int) -> int:
+    """Rows a workgroup walks: 16, 32 or 64.  Purely a scheduling choice; bits do not change with it."""
+
+    if m < 1:
+        raise ValueError("the lane matmul takes at least one row")
+    return 16 if m <= 16 else (32 if m <= 32 else 64)
+
+
+def _aligned_rows(x: torch.Tensor) -> torch.Tensor:
+    """The kernels read rows in 16-byte pieces: copy x when its rows are not laid out for that."""
+
+    bad = x.stride(1) != 1 or x.data_ptr() % 16 or (x.shape[0] > 1 and x.stride(0) % 8)
+    return x.clone(memory_format=torch.contiguous_format) if bad else x
+
+
+def group_sums(x: torch.Tensor, gs: int = 64) -> torch.Tensor:
+    """fp32 [M, K/gs]: the sum of every group of ``gs`` inputs of x (bf16 [M, K], rows may be strided)."""
+
+    _lib.on_gpu(x)
+    x = _aligned_rows(x)
+    m, k = x.shape
+    xs = x.new_empty((m, k // gs), dtype=torch.float32)
+    _lib.call("tf_group_sums", _lib.ptr(x), x.stride(0), m, k, gs, _lib.ptr(xs))
+    return xs
+
+
+def _check_x(x: torch.Tensor, q: Q4, who: str) -> torch.Tensor:
+    if x.dtype != torch.bfloat16 or x.dim() != 2 or x.shape[1] != q.k:
+        raise ValueError(f"{who}: x must be (M, {q.k}) bf16")
+    _lib.on_gpu(x)
+    return _aligned_rows(x)
+
+
+def matmul(x: torch.Tensor, q: Q4, xs: torch.Tensor | None = None, *, sk: int | None = None, f32: bool = False,
+           out: torch.Tensor | None = None, part: torch.Tensor | None = None, reduce: bool = True) -> torch.Tensor:
+    """Decode-form x @ W.T -> (M, n) bf16, or fp32 without the final rounding when ``f32``.
+
+    With ``reduce=False`` the fp32 K slices come back unadded as (sk, M, n); adding them in order and rounding once
+    reproduces the reduced result bit for bit."""
+
+    x = _check_x(x, q, "matmul")
+    m = int(x.shape[0])
+    xs = group_sums(x, q.gs) if xs is None else xs
+    sk = split_k(q.n, q.k, q.gs) if not sk else sk
+    if out is None:
+        out = x.new_empty((m, q.n), dtype=torch.float32 if f32 else torch.bfloat16)
+    if sk > 1 and part is None:
+        part = x.new_empty((sk, m, q.n), dtype=torch.float32)
+    _lib.call("tf_qmm", _lib.ptr(x), x.stride(0), _lib.ptr(xs), _lib.ptr(q.weight), _lib.ptr(q.scales),
+              _lib.ptr(q.biases), q.scales.stride(0), _lib.ptr(out), _lib.ptr(part), m, q.n, q.k, sk, q.gs, bucket(m),
+              int(f32), int(reduce))
+    if reduce or sk == 1:
+        return out
+    return part.reshape(-1)[:sk * m * q.n].view(sk, m, q.n)
+
+
+def prefill_matmul(x: torch.Tensor, q: Q4, *, f32: bool = False, tile: int = 0,
+                   out: torch.Tensor | None = None) -> torch.Tensor:
+    """Prompt-form x @ W.T on bf16 MFMA: every weight is rounded to bf16 once and K is one fp32 chain, so chunking a
+    prompt never changes a row's bits (they differ from ``matmul``'s)."""
+
+    x = _check_x(x, q, "prefill_matmul")
+    m = int(x.shape[0])
+    if out is None:
+        out = x.new_empty((m, q.n), dtype=torch.float32 if f32 else torch.bfloat16)
+    _lib.call("tf_qmm_prefill", _lib.ptr(x), x.stride(0), _lib.ptr(q.weight), _lib.ptr(q.scales.contiguous()),
+              _lib.ptr(q.biases.contiguous()), _lib.ptr(out), m, q.n, q.k, q.gs, int(f32), tile)
+    return out

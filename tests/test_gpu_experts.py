@@ -1,0 +1,253 @@
+"""Routed-expert kernels on the GPU, decode and prefill forms, against the CPU oracle (properties after the
+reference's tests/cuda/test_experts.py; tensors are seeded on the CPU so the oracle sees the same bits)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import affine as ora
+from oracle import routing as orr
+from tensorfold_amd import experts, synthetic
+from tests.helpers import f32, max_abs, rel_l2, u32
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+# (group size, SwiGLU, limit, experts incl. shared, D, NI, shared slots)
+CASES = [(32, True, 0.0, 41, 256, 96, 1), (64, True, 10.0, 19, 512, 128, 1), (64, False, 0.0, 12, 384, 192, 2)]
+
+
+def build(case, seed):
+    gs, swiglu, limit, e, d, ni, _ = case
+    up = [synthetic.affine_general(ni, d, gs, seed + i, (e,)) for i in range(2 if swiglu else 1)]
+    down = synthetic.affine_general(d, ni, gs, seed + 7, (e,))
+    ex = experts.make([tuple(t.to(DEV) for t in m) for m in up], tuple(t.to(DEV) for t in down), gs, limit=limit)
+    return ex, up, down
+
+
+def picks_for(rows, case, seed, hot=None):
+    """Each row: distinct routed experts (the first ones when ``hot``, so every row shares them), then the shared."""
+
+    e, shared = case[3], case[6]
+    routed = e - shared
+    k = min(6, routed)
+    g = torch.Generator().manual_seed(seed)
+    out = []
+    for _ in range(rows):
+        r = torch.arange(k) if hot is not None else torch.randperm(routed, generator=g)[:k]
+        out.append(torch.cat([r, torch.arange(routed, e)]))
+    return torch.stack(out).to(torch.int32)
+
+
+def run(ex, x, picks, prefill=False, y_dtype=torch.float32, tile=None):
+    rows, slots = picks.shape
+    plan = experts.Plan(rows, slots, ex.count, DEV, prefill=prefill)
+    experts.route(picks.to(DEV).contiguous(), plan, *(() if tile is None else (tile,)))
+    act = torch.empty((rows * slots, ex.width), dtype=torch.bfloat16, device=DEV)
+    y = torch.empty((rows * slots, ex.dims), dtype=y_dtype, device=DEV)
+    experts.gate_up(x, ex, plan, act, rows)
+    experts.down(act, ex, plan, y, rows)
+    return act, y, plan
+
+
+def np_tables(ms):
+    return [(u32(w), f32(s), f32(b)) for (w, s, b) in ms]
+
+
+@pytest.mark.parametrize("gs", [32, 64])
+def test_pack_round_trip(gs):
+    w = tuple(t.to(DEV) for t in synthetic.affine_general(96, 256, gs, 61, (3,)))
+    blocks = experts.pack(*w, gs)
+    assert blocks.shape == (3, 3, 256 // gs, experts.block_words(gs))
+    back = experts.unpack(blocks, gs)
+    assert all(torch.equal(a, b) for a, b in zip(back, w))
+    stacked = torch.stack([blocks, blocks.flip(0)], dim=3)             # one matrix of a stacked table, as a view
+    back = experts.unpack(stacked[1:2, :, :, 0], gs)
+    assert all(torch.equal(a, b[1:2]) for a, b in zip(back, w))
+
+
+@pytest.mark.parametrize("rows,prefill,tile", [(1, False, 64), (23, False, 64), (23, True, 64), (300, False, 64),
+                                              (300, True, 64), (1500, True, 64), (1500, True, 16), (1500, True, 128)])
+def test_plan_groups_pairs_by_expert(rows, prefill, tile):
+    """Bit-exact members, items and counts against the oracle: one workgroup up to 1,024 pairs, several past it."""
+
+    slots, e = 7, 50
+    g = torch.Generator().manual_seed(9)
+    picks = torch.stack([torch.randperm(e, generator=g)[:slots] for _ in range(rows)]).to(torch.int32)
+    picks[:, 0] = 3                                            # one expert with a pair in every row
+    plan = experts.Plan(rows, slots, e, DEV, prefill=prefill)
+    experts.route(picks.to(DEV), plan, tile)
+    assert plan.tile == (tile if prefill else experts.TILE)
+    items, members, distinct = orr.plan(picks.numpy(), e, plan.tile)
+    n = int(plan.counts[0])
+    assert n == len(items) and int(plan.counts[1]) == distinct
+    assert n <= experts.max_items(rows * slots, e, plan.tile)
+    assert np.array_equal(plan.items[:n].cpu().numpy(), items)
+    assert np.array_equal(plan.members.cpu().numpy(), members)
+
+
+def test_an_expert_shared_by_many_rows_makes_items_of_16():
+    picks = torch.full((37, 1), 5, dtype=torch.int32)
+    plan = experts.Plan(37, 1, 8, DEV)
+    experts.route(picks.to(DEV), plan)
+    assert int(plan.counts[0]) == 3 and int(plan.counts[1]) == 1
+    assert plan.items[:3].cpu().tolist() == [[5, 0, 16], [5, 16, 16], [5, 32, 5]]
+
+
+@pytest.mark.parametrize("prefill", [False, True])
+@pytest.mark.parametrize("case", CASES)
+def test_matches_the_oracle(case, prefill):
+    """act and y of every pair against dequant-then-matmul with the reference's rounding points (prefill: weights
+    rounded to bf16 first).  Bounds: the reference's own (act 2^-6, y 1e-5 of the largest value) and rel-L2 2e-3."""
+
+    gs, swiglu, limit = case[0], case[1], case[2]
+    ex, up, down = build(case, 31)
+    rows = 5
+    x = synthetic.activations(rows, ex.dims, 77, 0.5)
+    picks = picks_for(rows, case, 6)
+    act, y, _ = run(ex, x.to(DEV), picks, prefill=prefill)
+    act_ref, _ = ora.expert_pairs(f32(x), picks.numpy(), np_tables(up), np_tables([down])[0], gs, limit=limit,
+                                  prefill=prefill)
+    assert max_abs(f32(act), act_ref) <= 2 ** -6 * np.abs(act_ref).max()
+    assert rel_l2(f32(act), act_ref) <= 2e-3
+    # down from the GPU's own activations, so that only the down matmul is measured
+    slots = picks.shape[1]
+    pe = picks.reshape(-1).numpy()
+    wd = ora.dequantize(u32(down[0]), f32(down[1]), f32(down[2]), gs)
+    if prefill:
+        wd = ora.bf16(wd)
+    y_ref = np.einsum("pk,pnk->pn", f32(act).astype(np.float64), wd[pe].astype(np.float64))
+    assert max_abs(f32(y), y_ref) <= 1e-5 * np.abs(y_ref).max()
+    assert rel_l2(f32(y), y_ref) <= 1e-5
+    assert slots == picks.shape[1]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_pairs_do_not_depend_on_the_window(case):
+    ex, _, _ = build(case, 11)
+    rows = 40
+    x = synthetic.activations(rows, ex.dims, 5, 0.5).to(DEV)
+    picks = picks_for(rows, case, 3)
+    slots = picks.shape[1]
+    act, y, _ = run(ex, x, picks)
+    alone = [run(ex, x[r:r + 1], picks[r:r + 1]) for r in range(rows)]
+    assert torch.equal(act, torch.cat([a[0] for a in alone])) and torch.equal(y, torch.cat([a[1] for a in alone]))
+    for m in (2, 3, 8, 9, 16, 17, 33):
+        a_m, y_m, _ = run(ex, x[:m], picks[:m])
+        assert torch.equal(a_m, act[:m * slots]) and torch.equal(y_m, y[:m * slots]), m
+    perm = torch.randperm(rows, generator=torch.Generator().manual_seed(5))
+    a_p, y_p, _ = run(ex, x[perm.to(DEV)], picks[perm])
+    idx = (perm[:, None] * slots + torch.arange(slots)).reshape(-1).to(DEV)
+    assert torch.equal(a_p, act[idx]) and torch.equal(y_p, y[idx])
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_an_expert_shared_by_many_rows(case):
+    """Every row picks the same experts: items of 16 pairs, several an expert, same bits as alone."""
+
+    ex, _, _ = build(case, 21)
+    rows = 37
+    x = synthetic.activations(rows, ex.dims, 8, 0.5).to(DEV)
+    picks = picks_for(rows, case, 4, hot=0)
+    _, y, plan = run(ex, x, picks)
+    slots = picks.shape[1]
+    alone = torch.cat([run(ex, x[r:r + 1], picks[r:r + 1])[1] for r in range(rows)])
+    assert torch.equal(y, alone)
+    assert int(plan.counts[1]) == slots and int(plan.counts[0]) == slots * 3
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_a_pairs_bits_never_depend_on_its_item(case):
+    """A prompt plan grouped in items of 16, 64 and 128 pairs gives every pair the same bits."""
+
+    ex, _, _ = build(case, 31)
+    rows = 300
+    x = synthetic.activations(rows, ex.dims, 12, 0.5).to(DEV)
+    picks = picks_for(rows, case, 6)
+    got = {t: run(ex, x, picks, prefill=True, y_dtype=torch.bfloat16, tile=t) for t in (16, 64, 128)}
+    for t in (64, 128):
+        assert torch.equal(got[16][0], got[t][0]) and torch.equal(got[16][1], got[t][1]), t
+    assert int(got[128][2].counts[0]) <= int(got[64][2].counts[0]) < int(got[16][2].counts[0])
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_prefill_rows_do_not_depend_on_the_chunk(case):
+    """Prefill form past 1,024 pairs: any chunk or row order keeps each row's bits; bf16 down is fp32 rounded."""
+
+    ex, _, _ = build(case, 71)
+    rows = 200
+    x = synthetic.activations(rows, ex.dims, 15, 0.5).to(DEV)
+    picks = picks_for(rows, case, 13)
+    slots = picks.shape[1]
+    assert rows * slots > experts.SMALL
+    act, y, _ = run(ex, x, picks, prefill=True)
+    for a, b in ((0, 1), (77, 78), (199, 200), (0, 7), (5, 22), (0, 64), (100, 200)):
+        a1, y1, _ = run(ex, x[a:b], picks[a:b], prefill=True)
+        assert torch.equal(a1, act[a * slots:b * slots]) and torch.equal(y1, y[a * slots:b * slots]), (a, b)
+    perm = torch.randperm(rows, generator=torch.Generator().manual_seed(5))
+    a_p, y_p, _ = run(ex, x[perm.to(DEV)], picks[perm], prefill=True)
+    idx = (perm[:, None] * slots + torch.arange(slots)).reshape(-1).to(DEV)
+    assert torch.equal(a_p, act[idx]) and torch.equal(y_p, y[idx])
+    _, y16, _ = run(ex, x, picks, prefill=True, y_dtype=torch.bfloat16)
+    assert torch.equal(y16, y.to(torch.bfloat16))
+
+
+def test_graph_replay_follows_the_picks():
+    """A captured route + gate_up + down replays on new picks (no host reads of the plan); replayed three times with
+    eager work in between."""
+
+    case = CASES[1]
+    ex, _, _ = build(case, 41)
+    rows = 9
+    picks = picks_for(rows, case, 7).to(DEV).contiguous()
+    slots = picks.shape[1]
+    plan = experts.Plan(rows, slots, ex.count, DEV)
+    x = synthetic.activations(rows, ex.dims, 2, 0.5).to(DEV)
+    act = torch.empty((rows * slots, ex.width), dtype=torch.bfloat16, device=DEV)
+    y = torch.empty((rows * slots, ex.dims), dtype=torch.float32, device=DEV)
+
+    def step():
+        experts.route(picks, plan)
+        experts.gate_up(x, ex, plan, act, rows)
+        experts.down(act, ex, plan, y, rows)
+
+    step()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        step()
+    for seed in (8, 9, 10):
+        picks.copy_(picks_for(rows, case, seed))
+        g.replay()
+        torch.cuda.synchronize()
+        _, want, _ = run(ex, x, picks.cpu())
+        assert torch.equal(y, want), seed
+
+
+def test_many_units_keep_the_bits():
+    """Far more workgroups than the chip holds at once, against rows alone."""
+
+    case = (64, True, 0.0, 257, 2048, 128, 1)
+    ex, _, _ = build(case, 81)
+    rows = 64
+    x = synthetic.activations(rows, ex.dims, 4, 0.5).to(DEV)
+    g = torch.Generator().manual_seed(12)
+    picks = torch.stack([torch.cat([torch.randperm(256, generator=g)[:8], torch.tensor([256])])
+                         for _ in range(rows)]).to(torch.int32)
+    _, y, plan = run(ex, x, picks)
+    assert int(plan.counts[0]) * (ex.dims // experts.COLS) > 8192
+    for r in (0, 31, 63):
+        assert torch.equal(run(ex, x[r:r + 1], picks[r:r + 1])[1], y[9 * r:9 * r + 9]), r
+
+
+def test_bad_arguments_raise():
+    w = tuple(t.to(DEV) for t in synthetic.affine_general(96, 256, 64, 1, (2,)))
+    with pytest.raises(ValueError):
+        experts.pack(*w, 16)
+    with pytest.raises(ValueError):
+        experts.pack(w[0], w[1][:, :, :2], w[2], 64)
+    plan = experts.Plan(4, 3, 8, DEV)
+    with pytest.raises(ValueError):
+        experts.route(torch.zeros((5, 3), dtype=torch.int32, device=DEV), plan)
+    with pytest.raises(ValueError):
+        experts.make([w, w, w], w, 64)

@@ -1,0 +1,202 @@
+"""The MoE layer on the GPU (router, top-k, plan, experts, combine) against the CPU oracle, at the BASELINE shapes
+(configs 1 and 2) and in small; ids are checked bit for bit."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import affine as ora
+from oracle import native
+from oracle import routing as orr
+from tensorfold_amd import experts, moe, synthetic
+from tests.helpers import bits16, f32, max_abs, rel_l2, u32
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+TOL = 2e-3
+
+
+class Cfg:
+    def __init__(self, shape):
+        self.num_experts_per_tok, self.num_experts = shape.top_k, shape.experts
+        self.moe_intermediate_size, self.hidden_size = shape.width, shape.hidden
+
+
+def test_topk_ids_are_bit_exact_and_weights_are_the_softmax():
+    for rows, ne, k, shared in ((1, 128, 6, False), (8, 128, 6, False), (32, 512, 10, True), (5, 1000, 8, True),
+                                (3, 64, 64, False)):
+        l = synthetic.logits(rows, ne + int(shared), 100 + rows)
+        buf = moe.MoEBuffers(rows, type("c", (), dict(num_experts_per_tok=k, num_experts=ne, moe_intermediate_size=32,
+                                                      hidden_size=32)), DEV, shared=shared)
+        moe.select_rows(l.to(DEV), buf, k, ne)
+        picks, wts = orr.topk_rows(l.numpy(), ne, k, shared=shared)
+        assert np.array_equal(buf.pick.cpu().numpy(), picks)
+        # brute force, independent of the oracle's loop: sort by (-logit, id)
+        for r in range(rows):
+            order = sorted(range(ne), key=lambda e: (-float(l[r, e]), e))[:k]
+            assert buf.pick[r, :k].cpu().tolist() == order
+        got = buf.wts.cpu().numpy()
+        assert np.abs(got - wts).max() <= 2 ** -8 * np.abs(wts).max()      # bf16-rounded values: at most one step
+        assert (got == wts).mean() > 0.9
+        assert np.allclose(got[:, :k].sum(1), 1.0, atol=2e-2)
+
+
+def test_ties_go_to_the_lower_expert():
+    l = torch.zeros((3, 129), dtype=torch.float32)
+    buf = moe.MoEBuffers(3, type("c", (), dict(num_experts_per_tok=6, num_experts=128, moe_intermediate_size=32,
+                                               hidden_size=32)), DEV)
+    moe.select_rows(l.to(DEV), buf, 6, 128)
+    assert buf.pick.cpu().tolist() == [[0, 1, 2, 3, 4, 5, 128]] * 3
+    w = buf.wts.cpu()
+    assert torch.equal(w[:, :6], torch.full((3, 6), 1 / 6).bfloat16().float()) and torch.all(w[:, 6] == 0.5)
+
+
+def test_router_logits():
+    g = torch.Generator().manual_seed(4)
+    x = synthetic.activations(37, 2048, 1)
+    rows = (torch.randn((513, 2048), generator=g) * 0.02).bfloat16()
+    got = f32(moe.router(x.to(DEV), rows.to(DEV)))
+    want = f32(x).astype(np.float64) @ f32(rows).astype(np.float64).T
+    assert rel_l2(got, want) < 1e-5
+
+
+def test_combine_is_the_slot_ordered_sum():
+    g = torch.Generator().manual_seed(5)
+    y = torch.randn((9, 7, 2688), generator=g)
+    w = torch.rand((9, 7), generator=g)
+    want = ora.combine(y.numpy(), w.numpy())
+    got = f32(moe.combine(y.to(DEV), w.to(DEV)))
+    assert max_abs(got, want) <= 2 ** -7 * np.abs(want).max() and rel_l2(got, want) < 1e-3
+    got16 = f32(moe.combine(y.bfloat16().to(DEV), w.to(DEV)))
+    want16 = ora.combine(f32(y.bfloat16()), w.numpy())
+    assert rel_l2(got16, want16) < 1e-3
+
+
+def layer_tables(shape, seed, experts_built):
+    """MLX tensors of the first ``experts_built`` experts (a full table is hundreds of MB; ids are drawn below it)."""
+
+    e = experts_built + int(shape.shared)
+    up = [synthetic.affine(shape.width, shape.hidden, shape.gs, seed + i, (e,)) for i in range(2 if shape.swiglu else 1)]
+    down = synthetic.affine(shape.hidden, shape.width, shape.gs, seed + 5, (e,))
+    return up, down
+
+
+def run_layer(shape, up, down, x, l, ne, prefill=False):
+    """The layer through the host API on logits ``l`` ([R, ne (+1)])."""
+
+    ex = experts.make([tuple(t.to(DEV) for t in m) for m in up], tuple(t.to(DEV) for t in down), shape.gs)
+    rows = x.shape[0]
+    cfg = type("c", (), dict(num_experts_per_tok=shape.top_k, num_experts=ne, moe_intermediate_size=shape.width,
+                             hidden_size=shape.hidden))
+    buf = moe.MoEBuffers(rows, cfg, DEV, prefill=prefill, shared=shape.shared)
+    moe.select(l.to(DEV), buf, shape.top_k, ne)
+    xd = x.to(DEV)
+    experts.gate_up(xd, ex, buf.plan, buf.act.view(-1, ex.width), rows)
+    experts.down(buf.act.view(-1, ex.width), ex, buf.plan, buf.y.view(-1, ex.dims), rows)
+    return moe.combine(buf.y, buf.wts), buf
+
+
+@pytest.mark.parametrize("tokens", [1, 4, 8])
+def test_config1_decode_layer(tokens):
+    """BASELINE config 1: D 2688, NI 1856, relu^2, top-6, g64, tokens 1 / 4 / 8 (ids drawn over the first 24 of the
+    128 experts so the CPU oracle's table stays small; every other shape is the config's)."""
+
+    shape, ne = synthetic.C1, 24
+    up, down = layer_tables(shape, 1100, ne)
+    x = synthetic.activations(tokens, shape.hidden, 1101)
+    l = synthetic.logits(tokens, ne, 1102)
+    out, buf = run_layer(shape, up, down, x, l, ne)
+    picks, wts = orr.topk_rows(l.numpy(), ne, shape.top_k, shared=False)
+    assert np.array_equal(buf.pick.cpu().numpy(), picks)
+    want_bits, act_bits, y_ref = native.moe_layer(
+        bits16(x), picks, buf.wts.cpu().numpy(), None, (u32(up[0][0]), bits16(up[0][1]), bits16(up[0][2])),
+        (u32(down[0]), bits16(down[1]), bits16(down[2])), shape.gs, want_pairs=True)
+    want = ora.bf16_from_bits(want_bits)
+    err = rel_l2(f32(out), want)
+    print(f"config 1, {tokens} tokens: rel-L2 {err:.2e}, max-abs {max_abs(f32(out), want):.3e}")
+    assert err <= TOL
+    assert rel_l2(f32(buf.act).reshape(-1, shape.width), ora.bf16_from_bits(act_bits)) <= TOL
+    assert rel_l2(f32(buf.y).reshape(-1, shape.hidden), y_ref) <= TOL
+
+
+@pytest.mark.parametrize("prefill", [False, True])
+def test_config2_verify_layer(prefill):
+    """BASELINE config 2: D 2048, NI 512, SwiGLU, top-10 + shared, g32, 32 rows (8 lanes x 4 draft tokens); ids over
+    the first 48 experts.  Both arithmetic forms: decode, and the prefill form the reference runs this window in."""
+
+    shape, ne = synthetic.C2, 48
+    up, down = layer_tables(shape, 1200, ne)
+    x = synthetic.activations(32, shape.hidden, 1201)
+    l = synthetic.logits(32, ne + 1, 1202)
+    out, buf = run_layer(shape, up, down, x, l, ne, prefill=prefill)
+    picks, wts = orr.topk_rows(l.numpy(), ne, shape.top_k, shared=True)
+    assert np.array_equal(buf.pick.cpu().numpy(), picks)
+    items, members, distinct = orr.plan(picks, ne + 1, buf.plan.tile)
+    n = int(buf.plan.counts[0])
+    assert np.array_equal(buf.plan.items[:n].cpu().numpy(), items)
+    assert np.array_equal(buf.plan.members.cpu().numpy(), members)
+    want_bits = native.moe_layer(bits16(x), picks, buf.wts.cpu().numpy(),
+                                 (u32(up[0][0]), bits16(up[0][1]), bits16(up[0][2])),
+                                 (u32(up[1][0]), bits16(up[1][1]), bits16(up[1][2])),
+                                 (u32(down[0]), bits16(down[1]), bits16(down[2])), shape.gs)
+    want = ora.bf16_from_bits(want_bits)
+    err = rel_l2(f32(out), want)
+    print(f"config 2 ({'prefill' if prefill else 'decode'} form): rel-L2 {err:.2e}, max-abs {max_abs(f32(out), want):.3e}")
+    assert err <= TOL
+
+
+def test_config3_prefill_chunk_small():
+    """BASELINE config 3 in small: Zipf(1.1) picks over 64 experts, 512 tokens, SwiGLU g32, bf16 MFMA path, items of
+    64 and 128; weighted scatter-add back to token order.  Sort permutation bit-exact, output within 2e-3."""
+
+    shape, ne, rows = synthetic.C2, 64, 512
+    up, down = layer_tables(shape, 1300, ne)
+    x = synthetic.activations(rows, shape.hidden, 1301)
+    ids = synthetic.zipf_picks(rows, ne, shape.top_k, 1302)
+    sel = synthetic.logits(rows, shape.top_k + 1, 1303)
+    # weights: softmax over the chosen ten (bf16-rounded), shared slot sigmoid-gated, as the reference's rule
+    wts = torch.cat([torch.softmax(sel[:, :-1], 1).bfloat16().float(),
+                     torch.sigmoid(sel[:, -1:].bfloat16().float()).bfloat16().float()], 1).contiguous()
+    picks = torch.cat([ids, torch.full((rows, 1), ne, dtype=torch.int32)], 1).contiguous()
+    ex = experts.make([tuple(t.to(DEV) for t in m) for m in up], tuple(t.to(DEV) for t in down), shape.gs)
+    outs = {}
+    for tile in (64, 128):
+        plan = experts.Plan(rows, picks.shape[1], ne + 1, DEV, prefill=True)
+        experts.route(picks.to(DEV), plan, tile)
+        items, members, _ = orr.plan(picks.numpy(), ne + 1, tile)
+        assert np.array_equal(plan.members.cpu().numpy(), members)
+        assert np.array_equal(plan.items[:int(plan.counts[0])].cpu().numpy(), items)
+        act = torch.empty((rows * picks.shape[1], shape.width), dtype=torch.bfloat16, device=DEV)
+        y = torch.empty((rows * picks.shape[1], shape.hidden), dtype=torch.bfloat16, device=DEV)
+        experts.gate_up(x.to(DEV), ex, plan, act, rows)
+        experts.down(act, ex, plan, y, rows)
+        outs[tile] = moe.combine(y.view(rows, -1, shape.hidden), wts.to(DEV))
+    assert torch.equal(outs[64], outs[128])
+    sample = list(range(0, rows, 37))
+    want_bits = native.moe_layer(bits16(x[sample]), picks[sample].numpy(), wts[sample].numpy(),
+                                 (u32(up[0][0]), bits16(up[0][1]), bits16(up[0][2])),
+                                 (u32(up[1][0]), bits16(up[1][1]), bits16(up[1][2])),
+                                 (u32(down[0]), bits16(down[1]), bits16(down[2])), shape.gs)
+    want = ora.bf16_from_bits(want_bits)
+    err = rel_l2(f32(outs[64][sample]), want)
+    print(f"config 3 (small): rel-L2 {err:.2e}, max-abs {max_abs(f32(outs[64][sample]), want):.3e}")
+    assert err <= TOL
+
+
+def test_moe_run_rows_do_not_depend_on_the_window():
+    shape = synthetic.MoEShape("small", 512, 16, 128, 4, 32, True, True)
+    up, down = layer_tables(shape, 7, 16)
+    ex = experts.make([tuple(t.to(DEV) for t in m) for m in up], tuple(t.to(DEV) for t in down), 32)
+    g = torch.Generator().manual_seed(3)
+    rr = (torch.randn((17, 512), generator=g) * 0.05).bfloat16().to(DEV)
+    layer = moe.Routed(rr, ex, 4)
+    x = synthetic.activations(8, 512, 9).to(DEV)
+    whole = moe.run(x, layer)
+    for r in range(8):
+        assert torch.equal(moe.run(x[r:r + 1], layer)[0], whole[r]), r
+    for m in (2, 3, 5):
+        assert torch.equal(moe.run(x[:m], layer), whole[:m]), m
+    whole_p = moe.run(x, layer, prefill=True)
+    for r in (0, 7):
+        assert torch.equal(moe.run(x[r:r + 1], layer, prefill=True)[0], whole_p[r]), r
+    assert rel_l2(f32(whole_p), f32(whole)) < 1e-2

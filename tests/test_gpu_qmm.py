@@ -1,0 +1,144 @@
+"""Dense 4-bit lane matmul on the GPU against the CPU oracle (properties after the reference's tests/cuda/test_qmm.py)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import affine as ora
+from oracle import native
+from tensorfold_amd import qmm, synthetic
+from tests.helpers import bits16, f32, max_abs, rel_l2, u32
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+TOL = 2e-3          # relative L2 bound on bf16 outputs (fp32 accumulation), as BASELINE states
+
+
+def gpu(*ts):
+    return tuple(t.to(DEV) for t in ts)
+
+
+@pytest.mark.parametrize("n,k,gs", [(48, 5120, 64), (1024, 5120, 64), (200, 1024, 32), (1536, 2048, 32)])
+def test_pack_round_trip(n, k, gs):
+    w = gpu(*synthetic.affine_general(n, k, gs, n + k))
+    back = qmm.unpack(qmm.pack(*w, gs))
+    assert all(torch.equal(a, b) for a, b in zip(back, w))
+
+
+@pytest.mark.parametrize("n,k,gs", [(128, 5120, 64), (200, 1024, 32)])
+def test_every_nibble_decodes_exactly(n, k, gs):
+    """One-hot rows read back each stored nibble (scale 1, bias 0), through every K split, decode and prefill form."""
+
+    words = synthetic.affine_general(n, k, gs, 29)[0].to(DEV)
+    ones = torch.ones((n, k // gs), device=DEV).bfloat16()
+    zeros = torch.zeros_like(ones)
+    q = qmm.pack(words, ones, zeros, gs)
+    want = torch.from_numpy(ora.nibbles(u32(words)).astype(np.float32).T.copy())            # (k, n): every code
+    assert set(want.unique().tolist()) == set(range(16))
+    eye = torch.eye(k, device=DEV).bfloat16()
+    for f in (False, True):
+        assert torch.equal(qmm.matmul(eye, q, f32=f).float().cpu(), want), f
+        assert torch.equal(qmm.matmul(eye, q, f32=f, sk=1).float().cpu(), want), f
+        assert torch.equal(qmm.prefill_matmul(eye, q, f32=f).float().cpu(), want), f
+
+
+def test_config0_single_linear_matches_the_oracle():
+    """BASELINE config 0: N = K = 4096, g64, one row; bf16 out against dequant-then-matmul."""
+
+    n = k = 4096
+    w = synthetic.affine(n, k, 64, 1000)
+    x = synthetic.activations(1, k, 1001)
+    q = qmm.pack(*gpu(*w), 64)
+    y = qmm.matmul(x.to(DEV), q)
+    ref = native.affine_linear(bits16(x), u32(w[0]), bits16(w[1]), bits16(w[2]), 64)
+    want = ora.bf16(ref)
+    err = rel_l2(f32(y), want)
+    print(f"config 0 decode: rel-L2 {err:.2e}, max-abs {max_abs(f32(y), want):.3e}")
+    assert err <= TOL
+    yp = qmm.prefill_matmul(x.to(DEV), q)
+    errp = rel_l2(f32(yp), want)
+    print(f"config 0 prefill form: rel-L2 {errp:.2e}, max-abs {max_abs(f32(yp), want):.3e}")
+    assert errp <= TOL
+    # numpy statement of the same oracle agrees with the C one
+    assert rel_l2(ora.linear(f32(x), u32(w[0]), f32(w[1]), f32(w[2]), 64, f32=True), ref) < 1e-5
+
+
+@pytest.mark.parametrize("n,k,gs", [(1024, 5120, 64), (512, 2048, 32), (200, 1024, 32)])
+def test_accuracy_matches_fp32_reference(n, k, gs):
+    w = synthetic.affine_general(n, k, gs, 11 * n + k)
+    x = synthetic.activations(16, k, 5)
+    q = qmm.pack(*gpu(*w), gs)
+    ref = native.affine_linear(bits16(x), u32(w[0]), bits16(w[1]), bits16(w[2]), gs)
+    y = f32(qmm.matmul(x.to(DEV), q))
+    assert max_abs(y, ref) <= np.abs(ref).max() * 2 ** -7          # the reference's own bound (test_qmm.py:64-70)
+    assert rel_l2(y, ref) <= TOL
+    y32 = f32(qmm.matmul(x.to(DEV), q, f32=True))
+    assert rel_l2(y32, ref) <= 1e-5
+    refp = native.affine_linear(bits16(x), u32(w[0]), bits16(w[1]), bits16(w[2]), gs, prefill=True)
+    yp = f32(qmm.prefill_matmul(x.to(DEV), q, f32=True))
+    assert rel_l2(yp, refp) <= 1e-5                                  # same bf16-rounded weights, fp32 chain
+    assert rel_l2(f32(qmm.prefill_matmul(x.to(DEV), q)), ref) <= TOL
+
+
+ROWS = [1, 2, 3, 4, 5, 7, 15, 16, 17, 31, 32, 33, 63, 64, 65, 100, 129, 200]
+
+
+@pytest.mark.parametrize("n,k,gs", [(48, 5120, 64), (1024, 2048, 64), (200, 1024, 32)])
+def test_rows_do_not_depend_on_row_count(n, k, gs):
+    q = qmm.pack(*gpu(*synthetic.affine_general(n, k, gs, 3 * n + k)), gs)
+    x = synthetic.activations(max(ROWS), k, 7).to(DEV)
+    alone = torch.cat([qmm.matmul(x[r:r + 1], q) for r in range(max(ROWS))])
+    alone_p = torch.cat([qmm.prefill_matmul(x[r:r + 1], q) for r in range(max(ROWS))])
+    for m in ROWS:
+        assert torch.equal(qmm.matmul(x[:m], q), alone[:m]), f"{n}x{k}: rows differ at M={m}"
+        assert torch.equal(qmm.prefill_matmul(x[:m], q), alone_p[:m]), f"{n}x{k}: prefill rows differ at M={m}"
+    perm = torch.randperm(max(ROWS), generator=torch.Generator().manual_seed(3)).to(DEV)
+    assert torch.equal(qmm.matmul(x[perm], q), alone[perm])
+    f32_ = qmm.matmul(x[:40], q, f32=True)
+    assert torch.equal(torch.cat([qmm.matmul(x[r:r + 1], q, f32=True) for r in range(40)]), f32_)
+
+
+def test_split_depends_only_on_shape():
+    for n, k in [(48, 5120), (1024, 5120), (5120, 6144), (17408, 5120), (5120, 17408), (248320, 5120), (4096, 4096)]:
+        sk = qmm.split_k(n, k)
+        assert sk == qmm.split_k(n, k) and (k // 64) % sk == 0
+
+
+def test_strided_rows_buffers_and_unreduced_slices():
+    n, k, gs = 640, 8192, 64
+    q = qmm.pack(*gpu(*synthetic.affine_general(n, k, gs, 17)), gs)
+    wide = synthetic.activations(24, k + 64, 9).to(DEV)
+    x = wide[:, :k]                                   # rows 16-byte aligned, stride k + 64
+    want = qmm.matmul(x.contiguous(), q)
+    assert torch.equal(qmm.matmul(x, q), want)
+    out = torch.empty_like(want)
+    assert qmm.matmul(x, q, out=out) is out and torch.equal(out, want)
+    sk = qmm.split_k(n, k)
+    assert sk > 1
+    slices = qmm.matmul(x, q, reduce=False, f32=True)
+    assert slices.shape == (sk, 24, n)
+    total = slices[0]
+    for s in range(1, sk):
+        total = total + slices[s]
+    assert torch.equal(total, qmm.matmul(x, q, f32=True))
+
+
+def test_group_sums():
+    x = synthetic.activations(5, 2048, 3).to(DEV)
+    for gs in (32, 64):
+        got = f32(qmm.group_sums(x, gs))
+        want = ora.group_sums(f32(x), gs)
+        assert np.allclose(got, want, rtol=1e-5, atol=1e-5)
+
+
+def test_bad_arguments_raise():
+    w = gpu(*synthetic.affine_general(64, 256, 64, 1))
+    with pytest.raises(ValueError):
+        qmm.pack(*w, 48)
+    q = qmm.pack(*w, 64)
+    with pytest.raises(ValueError):
+        qmm.matmul(torch.zeros((1, 128), device=DEV).bfloat16(), q)
+    with pytest.raises(ValueError):
+        qmm.matmul(torch.zeros((1, 256), device=DEV), q)
+    with pytest.raises(RuntimeError, match="whole groups"):
+        qmm.matmul(torch.zeros((1, 256), device=DEV).bfloat16(), q, sk=3)

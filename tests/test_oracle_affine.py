@@ -1,0 +1,120 @@
+"""Pins of the affine-4-bit oracle (CPU only): hand-built words, the one-hot identity, three independent statements
+(numpy, C, pure Python), float64 textbook products, closed forms of the epilogues."""
+
+import math
+
+import numpy as np
+import pytest
+
+from oracle import affine as ora
+from oracle import native
+
+
+def rng_tables(n, k, gs, seed, lead=()):
+    rng = np.random.default_rng(seed)
+    words = rng.integers(0, 2 ** 32, size=(*lead, n, k // 8), dtype=np.uint64).astype(np.uint32)
+    scales = ora.bf16((rng.random((*lead, n, k // gs)) * 0.02 + 0.001).astype(np.float32))
+    biases = ora.bf16((rng.standard_normal((*lead, n, k // gs)) * 0.02).astype(np.float32))
+    return words, scales, biases
+
+
+def test_nibble_order_known_answer():
+    """Element 8 w + i is bits [4 i, 4 i + 4) of word w: 0x76543210 reads 0, 1, .. 7; 0xF0000001 reads 1, 0.., 15."""
+
+    got = ora.nibbles(np.array([[0x76543210, 0xF0000001]], dtype=np.uint32))
+    assert got.tolist() == [[0, 1, 2, 3, 4, 5, 6, 7, 1, 0, 0, 0, 0, 0, 0, 15]]
+    assert np.array_equal(ora.words_from_nibbles(got), np.array([[0x76543210, 0xF0000001]], dtype=np.uint32))
+
+
+def test_bf16_rounding_known_answers():
+    """Round to nearest even on the 16 dropped bits: 1 + 2^-8 is a tie and goes down to 1, 1 + 3 * 2^-8 goes up."""
+
+    x = np.array([1.0, 1 + 2 ** -8, 1 + 2 ** -8 + 2 ** -20, 1 + 3 * 2 ** -8, -2.5, 3.140625], dtype=np.float32)
+    assert ora.bf16(x).tolist() == [1.0, 1.0, 1.0078125, 1.015625, -2.5, 3.140625]
+    assert ora.bf16_bits(np.array([1.0, -2.0], dtype=np.float32)).tolist() == [0x3F80, 0xC000]
+
+
+def test_one_hot_rows_read_back_every_nibble():
+    """eye(K) @ W.T with scale 1 and bias 0 is the table of codes (the reference's tests/cuda/test_qmm.py:98-111)."""
+
+    words, _, _ = rng_tables(24, 128, 32, 1)
+    ones, zeros = np.ones((24, 4), np.float32), np.zeros((24, 4), np.float32)
+    y = ora.linear(np.eye(128, dtype=np.float32), words, ones, zeros, 32, f32=True)
+    assert np.array_equal(y, ora.nibbles(words).astype(np.float32).T)
+    assert set(np.unique(y).tolist()) == set(range(16))
+
+
+@pytest.mark.parametrize("gs", [32, 64])
+def test_three_statements_of_dequantize_agree(gs):
+    words, scales, biases = rng_tables(10, 256, gs, 2)
+    a = ora.dequantize(words, scales, biases, gs)
+    b = native.affine_dequant(words, ora.bf16_bits(scales), ora.bf16_bits(biases), gs)
+    assert np.array_equal(a, b)
+    for n in range(10):                                        # pure Python, element by element
+        for k in (0, 1, 7, 8, 63, 64, 200, 255):
+            q = (int(words[n, k // 8]) >> (4 * (k % 8))) & 15
+            want = np.float32(np.float32(q) * scales[n, k // gs]) + biases[n, k // gs]
+            assert a[n, k] == want
+
+
+def test_linear_is_the_textbook_product():
+    words, scales, biases = rng_tables(48, 512, 64, 3)
+    rng = np.random.default_rng(4)
+    x = ora.bf16(rng.standard_normal((3, 512)).astype(np.float32))
+    w64 = ora.nibbles(words).astype(np.float64) * np.repeat(scales, 64, -1) + np.repeat(biases, 64, -1)
+    want = x.astype(np.float64) @ w64.T
+    got = ora.linear(x, words, scales, biases, 64, f32=True)
+    assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
+    c = native.affine_linear(ora.bf16_bits(x), words, ora.bf16_bits(scales), ora.bf16_bits(biases), 64)
+    assert np.abs(c - want).max() <= 1e-5 * np.abs(want).max()
+    assert np.array_equal(ora.linear(x, words, scales, biases, 64), ora.bf16(got))
+    # prefill: weights rounded to bf16 first
+    wp = ora.bf16(ora.dequantize(words, scales, biases, 64)).astype(np.float64)
+    cp = native.affine_linear(ora.bf16_bits(x), words, ora.bf16_bits(scales), ora.bf16_bits(biases), 64, prefill=True)
+    assert np.abs(cp - x.astype(np.float64) @ wp.T).max() <= 1e-5 * np.abs(want).max()
+
+
+def test_group_sums():
+    x = np.arange(256, dtype=np.float32).reshape(2, 128)
+    assert ora.group_sums(x, 64).tolist() == [[2016.0, 6112.0], [10208.0, 14304.0]]
+
+
+def test_epilogue_closed_forms():
+    """relu^2 on the bf16-rounded input; SwiGLU = bf16(bf16(silu(g)) * u), clipped first when a limit is set."""
+
+    assert ora.relu2(np.array([-3.0, 0.0, 2.0, 1.00390625], np.float32)).tolist() == [0.0, 0.0, 4.0, 1.0]
+    g, u = np.array([0.0, 1.0, -20.0, 12.0], np.float32), np.array([5.0, 2.0, 1.0, -30.0], np.float32)
+    got = ora.swiglu(g, u)
+    silu = [v / (1 + math.exp(-v)) for v in g.tolist()]
+    want = [float(ora.bf16(np.float32(ora.bf16(np.float32(s)) * uu))) for s, uu in zip(silu, u.tolist())]
+    assert got.tolist() == want and got[0] == 0.0 and abs(got[1] - 1.4609375) < 1e-6
+    clipped = ora.swiglu(g, u, limit=10.0)
+    assert clipped[3] == float(ora.bf16(np.float32(ora.bf16(np.float32(10 / (1 + math.exp(-10)))) * -10.0)))
+
+
+def test_combine_is_slot_ordered():
+    y = np.array([[[1.0, 2.0], [10.0, 20.0], [100.0, 200.0]]], np.float32)
+    w = np.array([[0.5, 0.25, 2.0]], np.float32)
+    assert ora.combine(y, w).tolist() == [[203.0, 406.0]]
+
+
+@pytest.mark.parametrize("swiglu,gs", [(True, 32), (False, 64)])
+def test_c_layer_agrees_with_the_numpy_pairs(swiglu, gs):
+    """orc_moe_layer (C) against expert_pairs + combine (numpy): same rounding points, different code."""
+
+    e, d, ni, rows, slots = 6, 256, 128, 4, 3
+    up = [rng_tables(ni, d, gs, 10 + i, (e,)) for i in range(2 if swiglu else 1)]
+    down = rng_tables(d, ni, gs, 20, (e,))
+    rng = np.random.default_rng(5)
+    x = ora.bf16((rng.standard_normal((rows, d)) * 0.5).astype(np.float32))
+    picks = np.stack([rng.permutation(e)[:slots] for _ in range(rows)]).astype(np.int32)
+    wts = rng.random((rows, slots)).astype(np.float32)
+    act, y = ora.expert_pairs(x, picks, up, down, gs, limit=7.0 if swiglu else 0.0)
+    want = ora.combine(y.reshape(rows, slots, d), wts)
+    bits = lambda m: (m[0], ora.bf16_bits(m[1]), ora.bf16_bits(m[2]))
+    out, act_c, y_c = native.moe_layer(ora.bf16_bits(x), picks, wts, bits(up[0]) if swiglu else None, bits(up[-1]),
+                                       bits(down), gs, limit=7.0 if swiglu else 0.0, want_pairs=True)
+    assert np.abs(y_c - y).max() <= 1e-4 * np.abs(y).max()
+    a_c = ora.bf16_from_bits(act_c)
+    assert np.abs(a_c - act).max() <= 2 ** -7 * np.abs(act).max()          # summation order may move a bf16 step
+    assert np.abs(ora.bf16_from_bits(out) - want).max() <= 2 ** -7 * np.abs(want).max()
