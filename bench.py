@@ -1,0 +1,250 @@
+"""Benchmark of the hot path on one MI355X: the 4-bit decode MoE layer of BASELINE config 1.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--tokens T]
+
+A step is one pass of the layer (top-k routing, pair sort, up projection with relu^2, down projection, weighted
+combine) over one batch of T tokens, all inputs resident in HBM.  Steps cycle over several layers' expert tables
+(each 718 MB, together far past the 256 MB Infinity Cache) and over a pool of router logits, so every step streams
+its experts from HBM as a model's forward pass does.  The K timed steps are one hipGraph replay; the dominant
+kernels are then timed by themselves with HIP events around back-to-back launches on the same stream.  Prints one
+JSON line.  Synthetic data, random-init weights (there are no checkpoints here).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+import numpy as np
+import torch
+
+from tensorfold_amd import experts, moe, synthetic
+
+HBM_PEAK_GBS = 8000.0
+SHAPE = synthetic.C1
+LAYERS = 4          # 4 x 718 MB of expert tables
+POOL = 64           # distinct routing draws
+PLANS = 16          # pre-routed plans the kernel timing cycles through
+
+
+def device_tables(shape, layers: int, dev: str):
+    """Random MLX tensors drawn on the GPU and packed; the MLX copies of layer 0 are kept for the CPU baseline."""
+
+    g = torch.Generator(device=dev).manual_seed(1100)
+    out, keep = [], None
+    for layer in range(layers):
+        def table(n, k):
+            words = torch.randint(-(2 ** 31), 2 ** 31, (shape.experts, n, k // 8), generator=g, device=dev,
+                                  dtype=torch.int64).to(torch.int32)
+            scales = (torch.rand((shape.experts, n, k // shape.gs), generator=g, device=dev) * 0.018 + 0.002).bfloat16()
+            return words, scales, (scales.float() * -8).bfloat16()
+        up, down = table(shape.width, shape.hidden), table(shape.hidden, shape.width)
+        out.append(experts.make([up], down, shape.gs))
+        if layer == 0:
+            keep = (up, down)
+        del up, down
+    return out, keep
+
+
+class Layer:
+    """One batch size's buffers and the launch sequence of a step."""
+
+    def __init__(self, tokens: int, tables, dev: str) -> None:
+        s = SHAPE
+        self.tokens, self.tables = tokens, tables
+        cfg = type("cfg", (), dict(num_experts_per_tok=s.top_k, num_experts=s.experts,
+                                   moe_intermediate_size=s.width, hidden_size=s.hidden))
+        self.buf = moe.MoEBuffers(tokens, cfg, dev, shared=False)
+        self.plans = [moe.MoEBuffers(tokens, cfg, dev, shared=False) for _ in range(PLANS)]   # pre-routed, for kernel timing
+        self.x = [synthetic.activations(tokens, s.hidden, 1101 + i).to(dev) for i in range(4)]
+        self.logits = [synthetic.logits(tokens, s.experts, 2000 + i).to(dev) for i in range(POOL)]
+        self.out = torch.empty((tokens, s.hidden), dtype=torch.bfloat16, device=dev)
+
+    def route(self, i: int) -> None:
+        moe.select(self.logits[i % POOL], self.buf, SHAPE.top_k, SHAPE.experts)
+
+    def up(self, i: int, buf=None) -> None:
+        ex, buf = self.tables[i % len(self.tables)], buf or self.buf
+        experts.gate_up(self.x[i % 4], ex, buf.plan, buf.act.view(-1, ex.width), self.tokens)
+
+    def down(self, i: int, buf=None) -> None:
+        ex, buf = self.tables[i % len(self.tables)], buf or self.buf
+        experts.down(buf.act.view(-1, ex.width), ex, buf.plan, buf.y.view(-1, ex.dims), self.tokens)
+
+    def route_plans(self) -> float:
+        """Route every pre-built plan on its own logits; returns the mean number of distinct experts a plan holds."""
+
+        for j, b in enumerate(self.plans):
+            moe.select(self.logits[(7 * j + 3) % POOL], b, SHAPE.top_k, SHAPE.experts)
+            self.up(j, b)                     # fills the plan's activations for the down kernel
+        torch.cuda.synchronize()
+        return float(np.mean([int(b.plan.counts[1]) for b in self.plans]))
+
+    def combine(self) -> None:
+        moe.combine(self.buf.y, self.buf.wts, self.out)
+
+    def step(self, i: int) -> None:
+        self.route(i)
+        self.up(i)
+        self.down(i)
+        self.combine()
+
+    def unique_experts(self, i: int) -> int:
+        self.route(i)
+        torch.cuda.synchronize()
+        return int(self.buf.plan.counts[1])
+
+
+def bytes_per_expert(shape) -> int:
+    """Codes plus scales and biases of one expert's up and down matrices (the algorithmic bytes of a routed expert)."""
+
+    per_matrix = shape.width * shape.hidden // 2 + 2 * 2 * shape.width * shape.hidden // shape.gs
+    return 2 * per_matrix
+
+
+def run_batch(tokens: int, tables, steps: int, warmup: int, dev: str) -> dict:
+    s = SHAPE
+    layer = Layer(tokens, tables, dev)
+    uniq = [layer.unique_experts(i) for i in range(steps)]
+    for i in range(warmup):
+        layer.step(i)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for i in range(steps):
+            layer.step(i)
+    graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    graph.replay()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    layer_us = wall / steps * 1e6
+
+    # the two expert kernels by themselves: HIP events around back-to-back launches on the launch stream
+    def kernel_us(fn) -> float:
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps = 4 * PLANS
+        for i in range(4):
+            fn(i, layer.plans[i % PLANS])
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(reps):
+                fn(i, layer.plans[(i // LAYERS) % PLANS])
+        g.replay()
+        torch.cuda.synchronize()
+        a.record()
+        g.replay()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e3 / reps
+
+    u0 = layer.route_plans()
+    up_us, down_us = kernel_us(layer.up), kernel_us(layer.down)
+    half = bytes_per_expert(s) // 2
+    act_bytes = tokens * s.top_k * (s.hidden + s.width) * 2
+    mean_u = float(np.mean(uniq))
+    algo = mean_u * bytes_per_expert(s) + tokens * s.hidden * 2 * 2 + tokens * s.top_k * 8
+    return {
+        "tokens": tokens, "layer_us": layer_us, "us_per_token": layer_us / tokens, "unique_experts": mean_u,
+        "layer_bytes": algo, "layer_gbs": algo / layer_us * 1e-3, "layer_frac": algo / layer_us * 1e-3 / HBM_PEAK_GBS,
+        "up_kernel_us": up_us, "down_kernel_us": down_us,
+        "up_gbs": (u0 * half + act_bytes / 2) / up_us * 1e-3, "down_gbs": (u0 * half + act_bytes / 2) / down_us * 1e-3,
+        "kernel_unique_experts": u0, "kernel_bytes": u0 * half,
+    }
+
+
+def cpu_baseline(keep, tokens: int, dev: str) -> dict:
+    """The C oracle (dequant-then-matmul per selected expert, OpenMP) on one layer pass of ``tokens`` tokens, and a
+    parity check of the GPU result against it on the same inputs."""
+
+    from oracle import affine as ora
+    from oracle import native
+    from oracle import routing as orr
+
+    s = SHAPE
+    up, down = keep
+    x = synthetic.activations(tokens, s.hidden, 1101)
+    l = synthetic.logits(tokens, s.experts, 2000)
+    picks, wts = orr.topk_rows(l.numpy(), s.experts, s.top_k, shared=False)
+    used = np.unique(picks)
+    remap = np.zeros(s.experts, dtype=np.int32)
+    remap[used] = np.arange(len(used), dtype=np.int32)
+    idx = torch.from_numpy(used.astype(np.int64)).to(dev)
+    b16 = lambda t: t.cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+    cpu = lambda m: (m[0][idx].cpu().numpy().view(np.uint32), b16(m[1][idx]), b16(m[2][idx]))
+    upc, downc = cpu(up), cpu(down)
+    native.moe_layer(b16(x), remap[picks], wts, None, upc, downc, s.gs)             # warm-up
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        out = native.moe_layer(b16(x), remap[picks], wts, None, upc, downc, s.gs)
+        times.append(time.perf_counter() - t0)
+    # the GPU on the same inputs (layer 0's table)
+    ex = experts.make([up], down, s.gs)
+    cfg = type("cfg", (), dict(num_experts_per_tok=s.top_k, num_experts=s.experts, moe_intermediate_size=s.width,
+                               hidden_size=s.hidden))
+    buf = moe.MoEBuffers(tokens, cfg, dev, shared=False)
+    moe.select(l.to(dev), buf, s.top_k, s.experts)
+    experts.gate_up(x.to(dev), ex, buf.plan, buf.act.view(-1, s.width), tokens)
+    experts.down(buf.act.view(-1, s.width), ex, buf.plan, buf.y.view(-1, s.hidden), tokens)
+    got = moe.combine(buf.y, buf.wts).float().cpu().numpy().astype(np.float64)
+    want = ora.bf16_from_bits(out).astype(np.float64)
+    rel = float(np.linalg.norm(got - want) / np.linalg.norm(want))
+    ids_ok = bool(np.array_equal(buf.pick.cpu().numpy(), picks))
+    med = float(np.median(times))
+    return {"value": med / tokens * 1e6, "unit": "us/token", "cores": native.threads(), "kind": "port",
+            "sample": f"one layer pass, {tokens} tokens x top-{s.top_k} ({len(used)} experts), median of 3",
+            "parity_rel_l2": rel, "parity_ids_exact": ids_ok}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--tokens", type=int, default=8, help="batch of the headline value (1, 4 and 8 are all reported)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus above 1 is not supported (the path has no multi-GPU code)",
+              file=sys.stderr)
+        return 2
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    tables, keep = device_tables(SHAPE, LAYERS, dev)
+    results = {t: run_batch(t, tables, args.steps, args.warmup, dev) for t in sorted({1, 4, 8, args.tokens})}
+    head = results[args.tokens]
+    dom = "up" if head["up_kernel_us"] >= head["down_kernel_us"] else "down"
+    dom_us = head[f"{dom}_kernel_us"]
+    achieved = head["kernel_bytes"] / dom_us * 1e-3
+    line = {
+        "metric": "moe_decode_layer_us_per_token", "value": head["us_per_token"], "unit": "us/token", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["layer_us"] * 1e-3,
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 x int4 -> fp32",
+        "data": "synthetic",
+        "config": {"workload": f"BASELINE config 1: {SHAPE.name}; {args.tokens} tokens a step; {LAYERS} layers' tables "
+                               f"cycled", "tokens": args.tokens, "hidden": SHAPE.hidden, "experts": SHAPE.experts,
+                   "intermediate": SHAPE.width, "top_k": SHAPE.top_k, "group_size": SHAPE.gs},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": f"expert_kernel ({dom} projection, {head['kernel_unique_experts']:.1f} experts a launch)",
+                     "kernel_us": dom_us, "bytes_per_launch": head["kernel_bytes"]},
+        "layer_hbm": {"achieved": head["layer_gbs"], "frac": head["layer_frac"], "unit": "GB/s",
+                      "bytes_per_step": head["layer_bytes"]},
+        "batches": {str(t): {k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()}
+                    for t, r in results.items()},
+    }
+    if not args.no_cpu:
+        del tables
+        torch.cuda.empty_cache()
+        line["cpu_baseline"] = cpu_baseline(keep, args.tokens, dev)
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
