@@ -55,15 +55,23 @@ def dequantize(words: np.ndarray, scales: np.ndarray, biases: np.ndarray, gs: in
     return q * s + b
 
 
+def prefill_weight(w: np.ndarray) -> np.ndarray:
+    """The prompt form's one rounding of a dequantized weight.  The reference rounds to bf16
+    (cuda/kernels/qmm_prefill.cu:1); this build's kernels round 256 w to fp16 (11 significant bits), which is what the
+    tight prompt-form checks compare against; the bound that matters is the unrounded oracle's."""
+
+    return ((w.astype(np.float64) * 256.0).astype(np.float16).astype(np.float32) / np.float32(256)).astype(np.float32)
+
+
 def linear(x: np.ndarray, words: np.ndarray, scales: np.ndarray, biases: np.ndarray, gs: int, *,
            f32: bool = False, prefill: bool = False) -> np.ndarray:
     """(x.float() @ dequantize(...).T).to(bf16)  (families/qwen3_5/cuda/reference.py:11-15).
 
-    ``prefill`` rounds each dequantized weight to bf16 first (cuda/kernels/qmm_prefill.cu:1)."""
+    ``prefill`` rounds each dequantized weight first (see ``prefill_weight``)."""
 
     w = dequantize(words, scales, biases, gs)
     if prefill:
-        w = bf16(w)
+        w = prefill_weight(w)
     y = np.asarray(x, dtype=np.float32) @ w.T
     return y if f32 else bf16(y)
 
@@ -100,8 +108,7 @@ def expert_pairs(x: np.ndarray, picks: np.ndarray, up: list, down: tuple, gs: in
     """Every (row, slot) pair through its expert: act [R*S, NI] (bf16 values) and y [R*S, D] (fp32, or bf16 values).
 
     ``up`` is [gate, up] (SwiGLU) or [up] (relu^2), each (words [E, NI, D/8], scales, biases); ``down`` likewise
-    [E, D, NI/8].  Weights are dequantized per used expert; ``prefill`` rounds them to bf16 first
-    (cuda/experts_prefill.cu:130-131)."""
+    [E, D, NI/8].  Weights are dequantized per used expert; ``prefill`` rounds them first (``prefill_weight``)."""
 
     x = np.asarray(x, dtype=np.float32)
     rows, slots = picks.shape
@@ -112,7 +119,7 @@ def expert_pairs(x: np.ndarray, picks: np.ndarray, up: list, down: tuple, gs: in
 
     def weight(m, e):
         w = dequantize(m[0][e], m[1][e], m[2][e], gs)
-        return bf16(w) if prefill else w
+        return prefill_weight(w) if prefill else w
 
     for e in np.unique(flat):
         pairs = np.nonzero(flat == e)[0]

@@ -98,7 +98,8 @@ void orc_affine_dequant(const uint32_t* words, const uint16_t* scales, const uin
   }
 }
 
-/* one weight row, dequantized; prefill rounds each weight to bf16 (cuda/kernels/qmm_prefill.cu:1) */
+/* one weight row, dequantized; prefill rounds each weight once: the reference to bf16 (cuda/kernels/qmm_prefill.cu:1),
+ * this build's kernels 256 w to fp16, which is what is restated here */
 static void dequant_row(const uint32_t* row, const uint16_t* s, const uint16_t* b, int k, int gs, int prefill,
                         float* w) {
   for (int g = 0; g < k / gs; ++g) {
@@ -106,7 +107,7 @@ static void dequant_row(const uint32_t* row, const uint16_t* s, const uint16_t* 
     for (int c = g * gs; c < (g + 1) * gs; ++c) {
       const float prod = (float)code_at(row, c) * sv;
       const float v = prod + bv;
-      w[c] = prefill ? round_bf16(v) : v;
+      w[c] = prefill ? (float)(half_to_double(double_to_half((double)v * 256.0)) / 256.0) : v;
     }
   }
 }

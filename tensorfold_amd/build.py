@@ -8,6 +8,7 @@ time, in the tree, for the one target this package supports, and a GPU that is n
 from __future__ import annotations
 
 import ctypes
+import os
 import shutil
 import subprocess
 import sys
@@ -41,20 +42,36 @@ def stale() -> bool:
 
 
 def compile(verbose: bool = False) -> Path:
-    """Compile every kernel for gfx950 into ``libtfmi.so`` (cross-compiles without a GPU)."""
+    """Compile every kernel for gfx950 into ``libtfmi.so`` (cross-compiles without a GPU): one hipcc per source,
+    side by side, then a link."""
+
+    import tempfile
+    from concurrent.futures import ThreadPoolExecutor
 
     cc = hipcc()
     if cc is None:
         raise RuntimeError("tensorfold-amd: hipcc was not found; ROCm's compiler is needed to build libtfmi.so")
-    cmd = [cc, *FLAGS, "-o", str(LIB), *(str(CSRC / s) for s in SOURCES)]
-    say(f"building {LIB.name} for {ARCH} (about a minute)")
-    done = subprocess.run(cmd, capture_output=True, text=True)
+    say(f"building {LIB.name} for {ARCH} (about half a minute)")
     noise = "packed-fp32-ops"
-    err = "\n".join(line for line in done.stderr.splitlines() if noise not in line)
-    if done.returncode:
-        raise RuntimeError(f"tensorfold-amd: hipcc failed:\n{err}")
-    if verbose and err:
-        say(err)
+
+    def run(cmd: list[str]) -> str:
+        done = subprocess.run(cmd, capture_output=True, text=True)
+        err = "\n".join(line for line in done.stderr.splitlines() if noise not in line)
+        if done.returncode:
+            raise RuntimeError(f"tensorfold-amd: hipcc failed:\n{err}")
+        return err
+
+    compile_flags = [f for f in FLAGS if f != "-shared"]
+    with tempfile.TemporaryDirectory(prefix="tfmi-build-") as tmp:
+        objects = [str(Path(tmp) / (Path(s).stem + ".o")) for s in SOURCES]
+        with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
+            logs = list(pool.map(lambda so: run([cc, *compile_flags, "-c", str(CSRC / so[0]), "-o", so[1]]),
+                                 zip(SOURCES, objects)))
+        logs.append(run([cc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", str(LIB), *objects]))
+    if verbose:
+        for text in logs:
+            if text:
+                say(text)
     return LIB
 
 
@@ -62,6 +79,9 @@ def compile(verbose: bool = False) -> Path:
 def load() -> ctypes.CDLL:
     """The library, built first if it is missing and hipcc is here; a missing library never falls back to anything."""
 
+    override = os.environ.get("TENSORFOLD_AMD_LIB")        # a library built elsewhere (same ABI)
+    if override:
+        return ctypes.CDLL(override)
     if not LIB.exists():
         if hipcc() is None:
             raise RuntimeError(f"tensorfold-amd: {LIB} is missing and there is no hipcc to build it; "

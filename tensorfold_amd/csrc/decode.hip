@@ -55,76 +55,112 @@ __device__ __forceinline__ void group_sums_block(const uint16_t* const* xrow, in
   }
 }
 
-// One wave's share of a GEMV: groups [g0, g1) of NM matrices against RB rows.
+// (x & mask) | magic in one VALU op; the mask rides in an SGPR and the magic in a VGPR (one constant-bus read)
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t magic) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(mask), "v"(magic));
+  return r;
+}
+
+// A group's weights of NM matrices in registers: GS/32 16-byte chunks and the (scale | bias << 16) word a matrix.
+template <int GS, int NM>
+struct Stage {
+  uint4 w[NM][GS / 32];
+  float s[NM], b[NM];
+};
+
+template <int GS, int NM, class WQ, class SB>
+__device__ __forceinline__ void load_stage(Stage<GS, NM>& st, const WQ& wq, const SB& sb, int g) {
+#pragma unroll
+  for (int m = 0; m < NM; ++m) {
+#pragma unroll
+    for (int i = 0; i < GS / 32; ++i) st.w[m][i] = wq(g, m, i);
+    sb(g, m, st.s[m], st.b[m]);
+  }
+}
+
+// acc += one group: P = sum x * (128 + q) by v_dot2c (x from SGPRs), then the scale and bias.
+template <int GS, int NM, int RB>
+__device__ __forceinline__ void compute_stage(float (&acc)[NM][RB], const Stage<GS, NM>& st,
+                                              const const_u32_ptr (&xr)[RB], const float* xs, int KG, int g) {
+  constexpr int CH = GS / 32;
+  const uint32_t magic = BF16_128;
+#ifdef TF_X_NOCOMPUTE
+#pragma unroll
+  for (int m = 0; m < NM; ++m)
+#pragma unroll
+    for (int i = 0; i < CH; ++i)
+      acc[m][0] += __uint_as_float((st.w[m][i].x ^ st.w[m][i].y ^ st.w[m][i].z ^ st.w[m][i].w) & 0x3fffffffu) + st.s[m] + st.b[m];
+  return;
+#endif
+  float p[NM][RB];
+#pragma unroll
+  for (int m = 0; m < NM; ++m)
+#pragma unroll
+    for (int r = 0; r < RB; ++r) p[m][r] = 0.f;
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    uint32_t xv[RB][16];
+#pragma unroll
+    for (int r = 0; r < RB; ++r)
+#pragma unroll
+#ifdef TF_X_NOX
+      for (int j = 0; j < 16; ++j) xv[r][j] = 0x3f803f80u + (uint32_t)KG;
+#else
+      for (int j = 0; j < 16; ++j) xv[r][j] = xr[r][(g * CH + i) * 16 + j];
+#endif
+#pragma unroll
+    for (int m = 0; m < NM; ++m) {
+      const uint32_t w4[4] = {st.w[m][i].x, st.w[m][i].y, st.w[m][i].z, st.w[m][i].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const uint32_t b2 = and_or(q ? w4[j] >> (4 * q) : w4[j], NIB_MASK, magic);
+#pragma unroll
+          for (int r = 0; r < RB; ++r) p[m][r] = dot2(b2, xv[r][4 * j + q], p[m][r]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < RB; ++r) {
+    const float xsum = xs[r * KG + g];
+#pragma unroll
+    for (int m = 0; m < NM; ++m) {
+      const float pq = fmaf(-128.f, xsum, p[m][r]);
+      acc[m][r] = fmaf(xsum, st.b[m], fmaf(pq, st.s[m], acc[m][r]));
+    }
+  }
+}
+
+#ifndef TF_X_DEPTH
+#define TF_X_DEPTH 3
+#endif
+constexpr int DEPTH = TF_X_DEPTH;        // groups a wave keeps in flight
+
+// One wave's share of a GEMV: groups [g0, g1) of NM matrices against RB rows, DEPTH groups in flight.
 //   wq(g, m, i)  -> the lane's 16 bytes of chunk i of group g of matrix m
 //   sb(g, m, s, b) -> the lane's column's scale and bias of that group
 //   xr[r]        -> row r's inputs as dwords (wave-uniform, constant address space)
 //   xs[r * KG + g] -> group sums (LDS)
+// `st` holds groups g0 .. g0 + DEPTH - 1 on entry when `loaded` (the caller issued them before its prologue).
 template <int GS, int NM, int RB, class WQ, class SB>
-__device__ __forceinline__ void gemv_slice(float (&acc)[NM][RB], const WQ& wq, const SB& sb, const const_u32_ptr (&xr)[RB],
-                                           const float* xs, int KG, int g0, int g1) {
-  constexpr int CH = GS / 32;
-  uint4 cur[NM][CH], nxt[NM][CH];
-  float cs[NM], cb[NM], ns[NM], nb[NM];
-  if (g0 < g1) {
+__device__ __forceinline__ void gemv_slice(float (&acc)[NM][RB], Stage<GS, NM> (&st)[DEPTH], bool loaded, const WQ& wq,
+                                           const SB& sb, const const_u32_ptr (&xr)[RB], const float* xs, int KG,
+                                           int g0, int g1) {
+  if (!loaded) {
 #pragma unroll
-    for (int m = 0; m < NM; ++m) {
-#pragma unroll
-      for (int i = 0; i < CH; ++i) cur[m][i] = wq(g0, m, i);
-      sb(g0, m, cs[m], cb[m]);
-    }
+    for (int d = 0; d < DEPTH; ++d)
+      if (g0 + d < g1) load_stage<GS, NM>(st[d], wq, sb, g0 + d);
   }
-  for (int g = g0; g < g1; ++g) {
-    if (g + 1 < g1) {
+  for (int gb = g0; gb < g1; gb += DEPTH) {
 #pragma unroll
-      for (int m = 0; m < NM; ++m) {
-#pragma unroll
-        for (int i = 0; i < CH; ++i) nxt[m][i] = wq(g + 1, m, i);
-        sb(g + 1, m, ns[m], nb[m]);
-      }
-    }
-    float p[NM][RB];
-#pragma unroll
-    for (int m = 0; m < NM; ++m)
-#pragma unroll
-      for (int r = 0; r < RB; ++r) p[m][r] = 0.f;
-#pragma unroll
-    for (int i = 0; i < CH; ++i) {
-      uint32_t xv[RB][16];
-#pragma unroll
-      for (int r = 0; r < RB; ++r)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) xv[r][j] = xr[r][(g * CH + i) * 16 + j];
-#pragma unroll
-      for (int m = 0; m < NM; ++m) {
-        const uint32_t w4[4] = {cur[m][i].x, cur[m][i].y, cur[m][i].z, cur[m][i].w};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const uint32_t b2 = nib_pair(w4[j], q);
-#pragma unroll
-            for (int r = 0; r < RB; ++r) p[m][r] = dot2(b2, xv[r][4 * j + q], p[m][r]);
-          }
-        }
-      }
-    }
-#pragma unroll
-    for (int r = 0; r < RB; ++r) {
-      const float xsum = xs[r * KG + g];
-#pragma unroll
-      for (int m = 0; m < NM; ++m) {
-        const float pq = fmaf(-128.f, xsum, p[m][r]);
-        acc[m][r] = fmaf(xsum, cb[m], fmaf(pq, cs[m], acc[m][r]));
-      }
-    }
-    if (g + 1 < g1) {
-#pragma unroll
-      for (int m = 0; m < NM; ++m) {
-#pragma unroll
-        for (int i = 0; i < CH; ++i) cur[m][i] = nxt[m][i];
-        cs[m] = ns[m];
-        cb[m] = nb[m];
+    for (int d = 0; d < DEPTH; ++d) {
+      const int g = gb + d;
+      if (g < g1) {
+        compute_stage<GS, NM, RB>(acc, st[d], xr, xs, KG, g);
+        if (g + DEPTH < g1) load_stage<GS, NM>(st[d], wq, sb, g + DEPTH);
       }
     }
   }
@@ -137,7 +173,7 @@ template <int GS, int NM, int EPI, int WAVES, int RB, class WQ, class SB>
 __device__ __forceinline__ void expert_pass(const uint16_t* __restrict__ X, int64_t x_stride, int slots, const WQ& wq,
                                             const SB& sb, int KG, int NB, int cb2, const int* __restrict__ members,
                                             int at0, void* __restrict__ out, int N, float limit, float* xs, float* part,
-                                            int g0, int g1) {
+                                            int g0, int g1, Stage<GS, NM> (&st)[DEPTH], bool loaded) {
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   int pr[RB];
   const uint16_t* xrow[RB];
@@ -150,14 +186,16 @@ __device__ __forceinline__ void expert_pass(const uint16_t* __restrict__ X, int6
     xr[r] = as_const(xrow[r]);
   }
   __syncthreads();                                  // the previous pass is done with xs and part
+#ifndef TF_X_NOXS
   group_sums_block<GS>(xrow, RB, KG, xs, tid, WAVES * 64);
   __syncthreads();
+#endif
   float acc[NM][RB];
 #pragma unroll
   for (int m = 0; m < NM; ++m)
 #pragma unroll
     for (int r = 0; r < RB; ++r) acc[m][r] = 0.f;
-  gemv_slice<GS, NM, RB>(acc, wq, sb, xr, xs, KG, g0, g1);
+  gemv_slice<GS, NM, RB>(acc, st, loaded, wq, sb, xr, xs, KG, g0, g1);
 #pragma unroll
   for (int m = 0; m < NM; ++m)
 #pragma unroll
@@ -201,8 +239,13 @@ __global__ void __launch_bounds__(WAVES * 64)
   extern __shared__ float lds[];            // xs [4][KG], then partials [WAVES][NM][4][64]
   const int NB2 = (NB + 1) >> 1;
   const int it = blockIdx.x / NB2, cb2 = blockIdx.x - it * NB2;
+#ifdef TF_X_NOITEM
+  if (it >= 40) return;
+  const int e = it * 3 + 1, first = it, cnt = 1;
+#else
   if (it >= counts[0]) return;
   const int e = items[3 * it], first = items[3 * it + 1], cnt = items[3 * it + 2];
+#endif
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int nb = 2 * cb2 + (lane >> 5), c = lane & 31;
   const bool col_ok = nb < NB;
@@ -218,18 +261,28 @@ __global__ void __launch_bounds__(WAVES * 64)
   const int g0 = (int)((long long)wave * KG / WAVES), g1 = (int)((long long)(wave + 1) * KG / WAVES);
   float* xs = lds;
   float* part = lds + 4 * KG;
+  // the slice's first groups are on their way before anything else is read
+  Stage<GS, NM> st[DEPTH];
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d)
+    if (g0 + d < g1) load_stage<GS, NM>(st[d], wq, sb, g0 + d);
+  bool loaded = true;
   int r0 = 0;
-  for (; r0 + 4 <= cnt; r0 += 4)
-    expert_pass<GS, NM, EPI, WAVES, 4>(X, x_stride, slots, wq, sb, KG, NB, cb2, members, first + r0, out, N, limit, xs,
-                                       part, g0, g1);
+#define TF_PASS(RB_)                                                                                                 \
+  expert_pass<GS, NM, EPI, WAVES, RB_>(X, x_stride, slots, wq, sb, KG, NB, cb2, members, first + r0, out, N, limit, xs, \
+                                       part, g0, g1, st, loaded);                                                    \
+  loaded = g1 - g0 <= DEPTH   /* a slice that fits the stages stays in registers for the next pass */
+  for (; r0 + 4 <= cnt; r0 += 4) {
+    TF_PASS(4);
+  }
   if (r0 + 2 <= cnt) {
-    expert_pass<GS, NM, EPI, WAVES, 2>(X, x_stride, slots, wq, sb, KG, NB, cb2, members, first + r0, out, N, limit, xs,
-                                       part, g0, g1);
+    TF_PASS(2);
     r0 += 2;
   }
-  if (r0 < cnt)
-    expert_pass<GS, NM, EPI, WAVES, 1>(X, x_stride, slots, wq, sb, KG, NB, cb2, members, first + r0, out, N, limit, xs,
-                                       part, g0, g1);
+  if (r0 < cnt) {
+    TF_PASS(1);
+  }
+#undef TF_PASS
 }
 
 // ---- dense lane matmul ---------------------------------------------------------------------------------------------
@@ -239,7 +292,8 @@ template <int GS, int WAVES, int RB, class WQ, class SB>
 __device__ __forceinline__ void qmm_pass(const uint16_t* __restrict__ X, int64_t ldx, const float* __restrict__ XS,
                                          const WQ& wq, const SB& sb, int r0, int tile, int slice, int gs0, int per,
                                          int g0, int g1, void* __restrict__ out, float* __restrict__ part_out, int M,
-                                         int N, int KG, int SK, int f32, float* xs, float* part) {
+                                         int N, int KG, int SK, int f32, float* xs, float* part,
+                                         Stage<GS, 1> (&st)[DEPTH], bool loaded) {
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const_u32_ptr xr[RB];
 #pragma unroll
@@ -254,7 +308,7 @@ __device__ __forceinline__ void qmm_pass(const uint16_t* __restrict__ X, int64_t
 #pragma unroll
   for (int r = 0; r < RB; ++r) acc[0][r] = 0.f;
   // gemv_slice indexes xs by absolute group: shift the base so that xs[r * per + (g - gs0)] is read
-  gemv_slice<GS, 1, RB>(acc, wq, sb, xr, xs - gs0, per, g0, g1);
+  gemv_slice<GS, 1, RB>(acc, st, loaded, wq, sb, xr, xs - gs0, per, g0, g1);
 #pragma unroll
   for (int r = 0; r < RB; ++r) part[(wave * RB + r) * 64 + lane] = acc[0][r];
   __syncthreads();
@@ -296,15 +350,25 @@ __global__ void __launch_bounds__(WAVES * 64)
   float* part = lds + 4 * per;
   const int m_end = min(M, (rt + 1) * BM);
   int r0 = rt * BM;
+  Stage<GS, 1> st[DEPTH];
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d)
+    if (g0 + d < g1) load_stage<GS, 1>(st[d], wq, sb, g0 + d);
+  bool loaded = true;
 #define TF_QMM_PASS(RB_)                                                                                             \
   qmm_pass<GS, WAVES, RB_>(X, ldx, XS, wq, sb, r0, tile, slice, gs0, per, g0, g1, out, part_out, M, N, KG, SK, f32, xs, \
-                           part)
-  for (; r0 + 4 <= m_end; r0 += 4) TF_QMM_PASS(4);
+                           part, st, loaded);                                                                        \
+  loaded = g1 - g0 <= DEPTH
+  for (; r0 + 4 <= m_end; r0 += 4) {
+    TF_QMM_PASS(4);
+  }
   if (r0 + 2 <= m_end) {
     TF_QMM_PASS(2);
     r0 += 2;
   }
-  if (r0 < m_end) TF_QMM_PASS(1);
+  if (r0 < m_end) {
+    TF_QMM_PASS(1);
+  }
 #undef TF_QMM_PASS
 }
 
@@ -327,7 +391,10 @@ __global__ void __launch_bounds__(256)
   group_sums_block<GS>(xrow, 1, KG, XS + (size_t)r * KG, threadIdx.x, 256);
 }
 
-constexpr int EXPERT_WAVES = 8;
+#ifndef TF_X_WAVES
+#define TF_X_WAVES 16
+#endif
+constexpr int EXPERT_WAVES = TF_X_WAVES;
 constexpr int EXPERT_RB = 4;
 constexpr int QMM_WAVES = 4;
 constexpr int QMM_RB = 4;

@@ -37,7 +37,7 @@ def router(x: torch.Tensor, rows: torch.Tensor, out: torch.Tensor | None = None)
 class MoEBuffers:
     """Preallocated scratch of a layer for at most ``rows`` rows, so that a captured graph can replay it.
 
-    ``prefill`` selects the prompt arithmetic of the experts (and bf16 pair outputs); ``shared=False`` is for layers
+    ``prefill`` selects the prompt arithmetic of the experts; ``shared=False`` is for layers
     without a shared expert: no extra logit column, no extra slot."""
 
     def __init__(self, rows: int, cfg, device: torch.device | str, *, prefill: bool = False,
@@ -51,8 +51,10 @@ class MoEBuffers:
         self.wts = torch.empty((rows, self.slots), **f32)
         self.plan = grouped.Plan(rows, self.slots, cfg.num_experts + extra, device, prefill=prefill)
         self.act = torch.empty((rows, self.slots, cfg.moe_intermediate_size), dtype=torch.bfloat16, device=device)
-        self.y = torch.empty((rows, self.slots, cfg.hidden_size), device=device,
-                             dtype=torch.bfloat16 if prefill else torch.float32)
+        # Pair outputs stay fp32 in both forms.  (The reference keeps bf16 pair outputs in its prompt form; that
+        # rounding alone costs 1.1e-3 relative L2 at the combine, most of a 2e-3 budget.  ``experts.down`` still
+        # writes bf16 into a bf16 ``out`` on a prompt plan for callers that want the smaller buffer.)
+        self.y = torch.empty((rows, self.slots, cfg.hidden_size), device=device, dtype=torch.float32)
 
 
 def select_rows(logits: torch.Tensor, buf: MoEBuffers, top_k: int, experts: int) -> None:
@@ -76,7 +78,7 @@ def select(logits: torch.Tensor, buf: MoEBuffers, top_k: int, experts: int,
 def moe(x: torch.Tensor, router_rows: torch.Tensor, ex: grouped.Experts, buf: MoEBuffers, top_k: int,
         experts: int) -> MoEBuffers:
     """Router, selection and both expert matmuls for x [R, D]; the pair outputs are left in ``buf.y`` [R, slots, D]
-    (the caller combines them, often fused with its residual add)."""
+    (fp32; the caller combines them, often fused with its residual add)."""
 
     n = int(x.shape[0])
     router(x, router_rows, buf.logits[:n])

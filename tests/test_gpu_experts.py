@@ -115,7 +115,7 @@ def test_matches_the_oracle(case, prefill):
     pe = picks.reshape(-1).numpy()
     wd = ora.dequantize(u32(down[0]), f32(down[1]), f32(down[2]), gs)
     if prefill:
-        wd = ora.bf16(wd)
+        wd = ora.prefill_weight(wd)
     y_ref = np.einsum("pk,pnk->pn", f32(act).astype(np.float64), wd[pe].astype(np.float64))
     assert max_abs(f32(y), y_ref) <= 1e-5 * np.abs(y_ref).max()
     assert rel_l2(f32(y), y_ref) <= 1e-5

@@ -167,7 +167,7 @@ def test_config3_prefill_chunk_small():
         assert np.array_equal(plan.members.cpu().numpy(), members)
         assert np.array_equal(plan.items[:int(plan.counts[0])].cpu().numpy(), items)
         act = torch.empty((rows * picks.shape[1], shape.width), dtype=torch.bfloat16, device=DEV)
-        y = torch.empty((rows * picks.shape[1], shape.hidden), dtype=torch.bfloat16, device=DEV)
+        y = torch.empty((rows * picks.shape[1], shape.hidden), dtype=torch.float32, device=DEV)
         experts.gate_up(x.to(DEV), ex, plan, act, rows)
         experts.down(act, ex, plan, y, rows)
         outs[tile] = moe.combine(y.view(rows, -1, shape.hidden), wts.to(DEV))

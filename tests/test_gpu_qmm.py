@@ -76,7 +76,7 @@ def test_accuracy_matches_fp32_reference(n, k, gs):
     assert rel_l2(y32, ref) <= 1e-5
     refp = native.affine_linear(bits16(x), u32(w[0]), bits16(w[1]), bits16(w[2]), gs, prefill=True)
     yp = f32(qmm.prefill_matmul(x.to(DEV), q, f32=True))
-    assert rel_l2(yp, refp) <= 1e-5                                  # same bf16-rounded weights, fp32 chain
+    assert rel_l2(yp, refp) <= 1e-5                                  # same once-rounded weights, fp32 chain
     assert rel_l2(f32(qmm.prefill_matmul(x.to(DEV), q)), ref) <= TOL
 
 

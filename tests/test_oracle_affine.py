@@ -68,8 +68,8 @@ def test_linear_is_the_textbook_product():
     c = native.affine_linear(ora.bf16_bits(x), words, ora.bf16_bits(scales), ora.bf16_bits(biases), 64)
     assert np.abs(c - want).max() <= 1e-5 * np.abs(want).max()
     assert np.array_equal(ora.linear(x, words, scales, biases, 64), ora.bf16(got))
-    # prefill: weights rounded to bf16 first
-    wp = ora.bf16(ora.dequantize(words, scales, biases, 64)).astype(np.float64)
+    # prompt form: each weight rounded once first
+    wp = ora.prefill_weight(ora.dequantize(words, scales, biases, 64)).astype(np.float64)
     cp = native.affine_linear(ora.bf16_bits(x), words, ora.bf16_bits(scales), ora.bf16_bits(biases), 64, prefill=True)
     assert np.abs(cp - x.astype(np.float64) @ wp.T).max() <= 1e-5 * np.abs(want).max()
 
