@@ -81,10 +81,13 @@ int tf_experts_plan(const int32_t* picks, int64_t pairs, int experts, int tile, 
                     int32_t* counts, int32_t* rank, int32_t* hist, tf_stream_t stream);
 /* Decode form.  epi 0: fp32 out; 1: bf16 relu(bf16 a)^2; 2: bf16 SwiGLU(matrix 0, matrix 1) with clip `limit`.
  * Pair p reads x row p / slots when slots > 0, row p when slots == 0.  max_units = max items * nb bounds the grid;
- * the live item count is read on the device.  Replaces experts.cpp:43-48 `run`. */
+ * the live item count is read on the device.  xs (may be NULL): fp32 [x rows, kg] group sums of x, as
+ * tf_group_sums or a previous call's xs_out gives them; without it each workgroup sums its rows itself.
+ * xs_out (may be NULL; epi 1 and 2): receives fp32 [pairs, n / gs], the group sums of the activations written,
+ * which is the xs of the down projection over the same pairs.  Replaces experts.cpp:43-48 `run`. */
 int tf_experts_run(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg, int nb,
                    const int32_t* items, const int32_t* counts, const int32_t* members, void* out, int n, float limit,
-                   int64_t max_units, tf_stream_t stream);
+                   int64_t max_units, const float* xs, float* xs_out, tf_stream_t stream);
 /* Prefill form on bf16 MFMA, w = bf16(fma(q, s, b)); epi 3: bf16 out.  `tile` is the plan's item size (16, 64 or
  * 128).  Replaces experts.cpp:50-55 `prefill`. */
 int tf_experts_prefill(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg,

@@ -22,7 +22,7 @@ PROTOTYPES = {
     "tf_experts_pack": [P, P, P, I, I, I, I, P, P],
     "tf_experts_unpack": [P, L, I, I, I, I, P, P, P, P],
     "tf_experts_plan": [P, L, I, I, P, P, P, P, P, P],
-    "tf_experts_run": [I, I, P, L, I, P, I, I, P, P, P, P, I, F, L, P],
+    "tf_experts_run": [I, I, P, L, I, P, I, I, P, P, P, P, I, F, L, P, P, P],
     "tf_experts_prefill": [I, I, P, L, I, P, I, I, P, P, P, P, I, F, L, I, P],
     "tf_moe_router": [P, L, P, P, I, I, I, P],
     "tf_moe_topk": [P, L, I, I, I, I, P, P, P],
