@@ -20,7 +20,7 @@ import time
 import numpy as np
 import torch
 
-from tensorfold_amd import experts, moe, synthetic
+from tensorfold_amd import _lib, experts, moe, synthetic
 
 HBM_PEAK_GBS = 8000.0
 SHAPE = synthetic.C1
@@ -77,8 +77,8 @@ class Layer:
         """Route every pre-built plan on its own logits; returns the mean number of distinct experts a plan holds."""
 
         for j, b in enumerate(self.plans):
-            moe.select(self.logits[(7 * j + 3) % POOL], b, SHAPE.top_k, SHAPE.experts)
-            self.up(j, b)                     # fills the plan's activations for the down kernel
+            moe.decode(self.x[j % 4], self.logits[(7 * j + 3) % POOL], self.tables[j % len(self.tables)], b,
+                       SHAPE.top_k, SHAPE.experts)      # routes the plan and fills its descriptors and activations
         torch.cuda.synchronize()
         return float(np.mean([int(b.plan.counts[1]) for b in self.plans]))
 
@@ -86,10 +86,33 @@ class Layer:
         moe.combine(self.buf.y, self.buf.wts, self.out)
 
     def step(self, i: int) -> None:
+        """One layer pass the way ``moe.run`` issues it: routing, up, down, combine as separate launches, or (with
+        ``moe.FUSED_DECODE``) the routing launch and the fused experts launch."""
+
+        if moe.FUSED_DECODE:
+            return self.step_fused(i)
         self.route(i)
         self.up(i)
         self.down(i)
         self.combine()
+
+    def step_fused(self, i: int) -> None:
+        moe.decode(self.x[i % 4], self.logits[i % POOL], self.tables[i % len(self.tables)], self.buf, SHAPE.top_k,
+                   SHAPE.experts, self.out)
+
+    def fused_experts(self, i: int, buf) -> None:
+        """The fused experts launch alone, on a pre-routed buffer (its counters are cleared by a small fill)."""
+
+        ex, f = self.tables[i % len(self.tables)], buf.fused(SHAPE.gs)
+        f["counters"].zero_()
+        n = self.tokens
+        items = experts.max_items(n * buf.slots, SHAPE.experts, experts.TILE)
+        ctr = f["counters"]
+        _lib.call("tf_moe_decode_experts", ex.gs, int(ex.swiglu), _lib.ptr(self.x[i % 4]), self.x[i % 4].stride(0), n,
+                  buf.slots, _lib.ptr(ex.up), _lib.ptr(ex.down), ex.dims, ex.width, _lib.ptr(f["desc"]),
+                  _lib.ptr(buf.plan.counts), _lib.ptr(buf.wts), _lib.ptr(f["xs_x"]), _lib.ptr(buf.act),
+                  _lib.ptr(f["xs_act"]), _lib.ptr(buf.y), _lib.ptr(self.out), ctr.data_ptr() + 4,
+                  ctr.data_ptr() + 4 * (1 + f["items"]), _lib.ptr(ctr), ex.limit, items)
 
     def unique_experts(self, i: int) -> int:
         self.route(i)
@@ -108,20 +131,24 @@ def run_batch(tokens: int, tables, steps: int, warmup: int, dev: str) -> dict:
     s = SHAPE
     layer = Layer(tokens, tables, dev)
     uniq = [layer.unique_experts(i) for i in range(steps)]
-    for i in range(warmup):
-        layer.step(i)
-    torch.cuda.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        for i in range(steps):
-            layer.step(i)
-    graph.replay()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    graph.replay()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    layer_us = wall / steps * 1e6
+
+    def graph_us(step) -> float:
+        for i in range(warmup):
+            step(i)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(steps):
+                step(i)
+        graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        graph.replay()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e6
+
+    layer_us = graph_us(layer.step)
+    fused_layer_us = layer_us if moe.FUSED_DECODE else graph_us(layer.step_fused)
 
     # the two expert kernels by themselves: HIP events around back-to-back launches on the launch stream
     def kernel_us(fn) -> float:
@@ -144,6 +171,9 @@ def run_batch(tokens: int, tables, steps: int, warmup: int, dev: str) -> dict:
 
     u0 = layer.route_plans()
     up_us, down_us = kernel_us(layer.up), kernel_us(layer.down)
+    fill_us = kernel_us(lambda i, b: b.fused(SHAPE.gs)["counters"].zero_())
+    fused_us = kernel_us(layer.fused_experts) - fill_us
+    layer.buf.check()
     half = bytes_per_expert(s) // 2
     act_bytes = tokens * s.top_k * (s.hidden + s.width) * 2
     mean_u = float(np.mean(uniq))
@@ -151,7 +181,8 @@ def run_batch(tokens: int, tables, steps: int, warmup: int, dev: str) -> dict:
     return {
         "tokens": tokens, "layer_us": layer_us, "us_per_token": layer_us / tokens, "unique_experts": mean_u,
         "layer_bytes": algo, "layer_gbs": algo / layer_us * 1e-3, "layer_frac": algo / layer_us * 1e-3 / HBM_PEAK_GBS,
-        "up_kernel_us": up_us, "down_kernel_us": down_us,
+        "fused_layer_us": fused_layer_us, "up_kernel_us": up_us, "down_kernel_us": down_us, "fused_kernel_us": fused_us,
+        "fused_gbs": (u0 * 2 * half + act_bytes) / fused_us * 1e-3,
         "up_gbs": (u0 * half + act_bytes / 2) / up_us * 1e-3, "down_gbs": (u0 * half + act_bytes / 2) / down_us * 1e-3,
         "kernel_unique_experts": u0, "kernel_bytes": u0 * half,
     }
@@ -218,9 +249,14 @@ def main() -> int:
     tables, keep = device_tables(SHAPE, LAYERS, dev)
     results = {t: run_batch(t, tables, args.steps, args.warmup, dev) for t in sorted({1, 4, 8, args.tokens})}
     head = results[args.tokens]
-    dom = "up" if head["up_kernel_us"] >= head["down_kernel_us"] else "down"
-    dom_us = head[f"{dom}_kernel_us"]
-    achieved = head["kernel_bytes"] / dom_us * 1e-3
+    if moe.FUSED_DECODE:
+        dom_us, dom_bytes = head["fused_kernel_us"], 2 * head["kernel_bytes"]
+        dom = "moe_fused_kernel (up + down + combine"
+    else:
+        which = "up" if head["up_kernel_us"] >= head["down_kernel_us"] else "down"
+        dom_us, dom_bytes = head[f"{which}_kernel_us"], head["kernel_bytes"]
+        dom = f"expert_kernel ({which} projection"
+    achieved = dom_bytes / dom_us * 1e-3
     line = {
         "metric": "moe_decode_layer_us_per_token", "value": head["us_per_token"], "unit": "us/token", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["layer_us"] * 1e-3,
@@ -231,8 +267,8 @@ def main() -> int:
                    "intermediate": SHAPE.width, "top_k": SHAPE.top_k, "group_size": SHAPE.gs},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": f"expert_kernel ({dom} projection, {head['kernel_unique_experts']:.1f} experts a launch)",
-                     "kernel_us": dom_us, "bytes_per_launch": head["kernel_bytes"]},
+                     "kernel": f"{dom}, {head['kernel_unique_experts']:.1f} experts a launch)",
+                     "kernel_us": dom_us, "bytes_per_launch": dom_bytes},
         "layer_hbm": {"achieved": head["layer_gbs"], "frac": head["layer_frac"], "unit": "GB/s",
                       "bytes_per_step": head["layer_bytes"]},
         "batches": {str(t): {k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()}

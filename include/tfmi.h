@@ -58,8 +58,8 @@ int tf_group_sums(const uint16_t* x, int64_t ldx, int m, int k, int gs, float* x
 int tf_qmm(const uint16_t* x, int64_t ldx, const float* xs, const uint32_t* weight, const uint16_t* scales,
            const uint16_t* biases, int64_t sb_stride, void* out, float* part, int m, int n, int k, int sk, int gs,
            int bm, int f32, int reduce, tf_stream_t stream);
-/* Prefill-form matmul: w = bf16(fma(q, s, b)), one fp32 chain over K on bf16 MFMA.
- * Replaces kernels/qmm.cpp:83-102 `qmm_prefill`. */
+/* Prompt-form matmul on f16 MFMA: each weight rounded once (256 w to fp16; the reference rounds w to bf16), one
+ * fp32 chain over K.  Replaces kernels/qmm.cpp:83-102 `qmm_prefill`. */
 int tf_qmm_prefill(const uint16_t* x, int64_t ldx, const uint32_t* weight, const uint16_t* scales,
                    const uint16_t* biases, void* out, int m, int n, int k, int gs, int f32, int tile,
                    tf_stream_t stream);
@@ -88,8 +88,8 @@ int tf_experts_plan(const int32_t* picks, int64_t pairs, int experts, int tile, 
 int tf_experts_run(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg, int nb,
                    const int32_t* items, const int32_t* counts, const int32_t* members, void* out, int n, float limit,
                    int64_t max_units, const float* xs, float* xs_out, tf_stream_t stream);
-/* Prefill form on bf16 MFMA, w = bf16(fma(q, s, b)); epi 3: bf16 out.  `tile` is the plan's item size (16, 64 or
- * 128).  Replaces experts.cpp:50-55 `prefill`. */
+/* Prompt form on f16 MFMA, each weight rounded once as in tf_qmm_prefill; epi 3: bf16 out.  `tile` is the plan's
+ * item size (16, 64 or 128).  Replaces experts.cpp:50-55 `prefill`. */
 int tf_experts_prefill(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg,
                        int nb, const int32_t* items, const int32_t* counts, const int32_t* members, void* out, int n,
                        float limit, int64_t max_items, int tile, tf_stream_t stream);
@@ -108,6 +108,25 @@ int tf_moe_topk(const float* logits, int64_t ldl, int rows, int experts, int top
  * Replaces moe.py:131-151 `_combine` / `combine`. */
 int tf_moe_combine(const void* y, int y_bf16, const float* wts, uint16_t* out, int rows, int slots, int d,
                    tf_stream_t stream);
+
+/* The decode layer's routing in one launch, for rows * (top_k + shared) <= 1024: tf_moe_topk, tf_experts_plan (tile
+ * 16) and tf_group_sums of x, plus desc int32 [max items, 20] = {expert, count, first, 0, pairs[16]} an item and the
+ * zeroing of `zero` (n_zero ints: the counters of tf_moe_decode_experts).  No counterpart in the reference, which
+ * launches `_topk_rows`, `plan` and its group sums separately (moe.py:103-116, kernels/qmm.py:148-154). */
+int tf_moe_route_decode(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared,
+                        const uint16_t* x, int64_t ldx, int d, int gs, int32_t* pick, float* wts, int32_t* members,
+                        int32_t* items, int32_t* counts, int32_t* desc, float* xs_x, int32_t* zero, int n_zero,
+                        tf_stream_t stream);
+/* The decode layer's experts in one launch: up (+ relu^2 or SwiGLU), down and the weighted combine, with the bits
+ * of tf_experts_run, tf_experts_run and tf_moe_combine run in turn.  desc, counts, wts, xs_x as left by
+ * tf_moe_route_decode; scratch act bf16 [pairs, ni], xs_act fp32 [pairs, ni/gs], y fp32 [pairs, d]; counters done
+ * [max_items] and arrive [rows * d/64] zero on entry; status[0] is set to 1 if a bounded wait ran out (the output
+ * is then invalid).  d and ni multiples of 64.  Fuses experts.cpp:43-48 `run` (twice) and moe.py:131-151 `combine`. */
+int tf_moe_decode_experts(int gs, int swiglu, const uint16_t* x, int64_t x_stride, int rows, int slots,
+                          const uint32_t* up, const uint32_t* down, int d, int ni, const int32_t* desc,
+                          const int32_t* counts, const float* wts, const float* xs_x, uint16_t* act, float* xs_act,
+                          float* y, uint16_t* out, int32_t* done, int32_t* arrive, int32_t* status, float limit,
+                          int max_items, tf_stream_t stream);
 
 /* ---- EXL3 linear (exl3/linear.cpp:70-74, module tensorfold_exl3_linear_v3) ---------------------------------------- */
 

@@ -20,355 +20,26 @@
 
 #include <cstdlib>
 
-#include "tf_common.h"
+#include "gemv.h"
 
 namespace tf {
 namespace {
 
-typedef const __attribute__((address_space(4))) uint32_t* const_u32_ptr;   // constant address space: scalar loads
-
-__device__ __forceinline__ const_u32_ptr as_const(const void* p) {
-  return (const_u32_ptr)(reinterpret_cast<uintptr_t>(p));
-}
-
-__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
-  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c, false);
-}
-
-// weights are read once: nontemporal loads keep them from displacing the activations in the caches
-__device__ __forceinline__ uint4 ldg16(const uint32_t* p) {
-#ifdef TF_X_TEMPORAL
-  return *reinterpret_cast<const uint4*>(p);
-#else
-  const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
-  return make_uint4(v.x, v.y, v.z, v.w);
-#endif
-}
-
-// (x & mask) | magic in one VALU op; the mask rides in an SGPR and the magic in a VGPR (one constant-bus read)
-__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t magic) {
-  uint32_t r;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(mask), "v"(magic));
-  return r;
-}
-
-constexpr int SLICES = 16;      // K slices of the expert GEMV
-constexpr int DEPTH = 3;        // groups of weights a wave keeps in flight
-constexpr int RBMAX = 2;        // rows a pass
-
-// fp32 sums of each group of GS inputs of `rows` rows, for groups [0, KG), into xs[r * KG + g].
-// LPG lanes share a group (8 inputs each, in order), then a fixed xor tree over them.
-template <int GS>
-__device__ __forceinline__ void group_sums_block(const uint16_t* const* xrow, int rows, int KG, float* xs, int tid,
-                                                 int threads) {
-  constexpr int LPG = GS / 8;
-  const int part = tid % LPG;
-  for (int r = 0; r < rows; ++r) {
-    for (int g = tid / LPG; g < KG; g += threads / LPG) {
-      const uint4 v = *reinterpret_cast<const uint4*>(xrow[r] + (size_t)g * GS + part * 8);
-      float s = bf16_lo(v.x);
-      s += bf16_hi(v.x);
-      s += bf16_lo(v.y);
-      s += bf16_hi(v.y);
-      s += bf16_lo(v.z);
-      s += bf16_hi(v.z);
-      s += bf16_lo(v.w);
-      s += bf16_hi(v.w);
-#pragma unroll
-      for (int m = 1; m < LPG; m <<= 1) s += __shfl_xor(s, m);
-      if (part == 0) xs[r * KG + g] = s;
-    }
-  }
-}
-
-// dot2c with its first operand taken from lane J of the reader's row of 16 lanes
-template <int J>
-__device__ __forceinline__ float dot2_bcast(float acc, uint32_t x, uint32_t q) {
-  asm("v_dot2c_f32_bf16_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(x), "v"(q), "n"(J));
-  return acc;
-}
-
-// A group in registers: the weights of NM matrices (GS/32 16-byte chunks, scale and bias) and, of each of RB rows,
-// the lane's dword of each chunk of the group's inputs.
-template <int GS, int NM>
-struct Stage {
-  uint4 w[NM][GS / 32];
-  float s[NM], b[NM];
-  uint32_t x[RBMAX][GS / 32];
-};
-
-template <int GS, int NM, class WQ, class SB>
-__device__ __forceinline__ void load_weights(Stage<GS, NM>& st, const WQ& wq, const SB& sb, int g) {
-#pragma unroll
-  for (int m = 0; m < NM; ++m) {
-#pragma unroll
-    for (int i = 0; i < GS / 32; ++i) st.w[m][i] = wq(g, m, i);
-    sb(g, m, st.s[m], st.b[m]);
-  }
-}
-
-// xl[r]: row r's inputs as dwords, already offset by (lane % 16)
-template <int GS, int NM, int RB>
-__device__ __forceinline__ void load_inputs(Stage<GS, NM>& st, const uint32_t* const (&xl)[RB], int g) {
-#pragma unroll
-  for (int r = 0; r < RB; ++r)
-#pragma unroll
-    for (int i = 0; i < GS / 32; ++i) st.x[r][i] = xl[r][(g * (GS / 32) + i) * 16];
-}
-
-template <int J, int NM, int RB>
-__device__ __forceinline__ void word_dot(float (&p)[NM][RB], const uint32_t (&word)[NM], const uint32_t (&x)[RB],
-                                         uint32_t magic) {
-  if constexpr (J < 16) {
-#pragma unroll
-    for (int m = 0; m < NM; ++m) {
-      constexpr int q = J & 3;
-      const uint32_t b2 = and_or(q ? word[m] >> (4 * q) : word[m], NIB_MASK, magic);
-#pragma unroll
-      for (int r = 0; r < RB; ++r) p[m][r] = dot2_bcast<J>(p[m][r], x[r], b2);
-    }
-  }
-}
-
-// p += sum over chunk i of x * (128 + q)
-template <int GS, int NM, int RB>
-__device__ __forceinline__ void chunk_dot(float (&p)[NM][RB], const Stage<GS, NM>& st, int i) {
-  const uint32_t magic = BF16_128;
-  uint32_t x[RB];
-#pragma unroll
-  for (int r = 0; r < RB; ++r) x[r] = st.x[r][i];
-#define TF_WORD(J_, C_)                                                   \
-  {                                                                       \
-    uint32_t word[NM];                                                    \
-    _Pragma("unroll") for (int m = 0; m < NM; ++m) word[m] = st.w[m][i].C_; \
-    word_dot<J_, NM, RB>(p, word, x, magic);                              \
-    word_dot<J_ + 1, NM, RB>(p, word, x, magic);                          \
-    word_dot<J_ + 2, NM, RB>(p, word, x, magic);                          \
-    word_dot<J_ + 3, NM, RB>(p, word, x, magic);                          \
-  }
-  TF_WORD(0, x) TF_WORD(4, y) TF_WORD(8, z) TF_WORD(12, w)
-#undef TF_WORD
-}
-
-// One wave's share of a GEMV: groups [gA, gB) of NM matrices against RB rows.
-//   wq(g, m, i)     -> the lane's 16 bytes of chunk i of group g of matrix m
-//   sb(g, m, s, b)  -> the lane's column's scale and bias of that group
-//   xl[r]           -> row r's inputs as dwords, offset by lane % 16
-//   xsum(r, g)      -> row r's sum over group g (wave-uniform)
-//   flush(g, acc)   -> called after group g has been added (wave-uniform); may park and clear acc
-// `st` holds the weights of groups gA .. gA + DEPTH - 1 on entry when `loaded`.
-template <int GS, int NM, int RB, class WQ, class SB, class XS, class FLUSH>
-__device__ __forceinline__ void gemv_stream(float (&acc)[NM][RB], Stage<GS, NM> (&st)[DEPTH], bool loaded,
-                                            const WQ& wq, const SB& sb, const uint32_t* const (&xl)[RB],
-                                            const XS& xsum, int gA, int gB, FLUSH& flush) {
-  constexpr int CH = GS / 32;
-  if (gA >= gB) return;
-#pragma unroll
-  for (int d = 0; d < DEPTH; ++d)
-    if (gA + d < gB) {
-      if (!loaded) load_weights<GS, NM>(st[d], wq, sb, gA + d);
-      load_inputs<GS, NM, RB>(st[d], xl, gA + d);
-    }
-  for (int gb = gA; gb < gB; gb += DEPTH) {
-#pragma unroll
-    for (int d = 0; d < DEPTH; ++d) {
-      const int g = gb + d;
-      if (g < gB) {
-        float p[NM][RB];
-#pragma unroll
-        for (int m = 0; m < NM; ++m)
-#pragma unroll
-          for (int r = 0; r < RB; ++r) p[m][r] = 0.f;
-#pragma unroll
-        for (int i = 0; i < CH; ++i) chunk_dot<GS, NM, RB>(p, st[d], i);
-#pragma unroll
-        for (int r = 0; r < RB; ++r) {
-          const float sc = xsum(r, g);
-#pragma unroll
-          for (int m = 0; m < NM; ++m) {
-            const float pq = fmaf(-128.f, sc, p[m][r]);
-            acc[m][r] = fmaf(sc, st[d].b[m], fmaf(pq, st[d].s[m], acc[m][r]));
-          }
-        }
-        flush(g, acc);
-        if (g + DEPTH < gB) {
-          load_weights<GS, NM>(st[d], wq, sb, g + DEPTH);
-          load_inputs<GS, NM, RB>(st[d], xl, g + DEPTH);
-        }
-      }
-    }
-  }
-}
-
-// ---- routed experts -----------------------------------------------------------------------------------------------
-
-__device__ __forceinline__ int slice_begin(int s, int KG) { return (int)((long long)s * KG / SLICES); }
-
-// One pass of an item: RB of its rows (members[at0 ..]) against the workgroup's 64 columns.
-// XSG: the rows' group sums come from `xs_in` (fp32 [x rows, KG], scalar loads); otherwise they are summed here
-// into LDS first.  `xs_out` (may be null; epilogues 1 and 2) receives the group sums of the activations written,
-// fp32 [pairs, N / GS]: what the down projection of the same pairs reads as its `xs_in`.
-template <int GS, int NM, int EPI, int WAVES, int RB, bool XSG, class WQ, class SB>
-__device__ __forceinline__ void expert_pass(const uint16_t* __restrict__ X, int64_t x_stride, int slots, const WQ& wq,
-                                            const SB& sb, int KG, int NB, int cb2, const int* __restrict__ members,
-                                            int at0, void* __restrict__ out, int N, float limit, float* xs, float* part,
-                                            Stage<GS, NM> (&st)[DEPTH], bool loaded, bool first_pass,
-                                            const float* __restrict__ xs_in, float* __restrict__ xs_out) {
-  constexpr int SPW = SLICES / WAVES;               // slices a wave
-  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  int pr[RB];
-  const uint16_t* xrow[RB];
-  const uint32_t* xl[RB];
-  const float* xsr[RB];
-#pragma unroll
-  for (int r = 0; r < RB; ++r) {
-    pr[r] = members[at0 + r];
-    const int row = slots ? pr[r] / slots : pr[r];
-    xrow[r] = X + (size_t)row * x_stride;
-    xl[r] = reinterpret_cast<const uint32_t*>(xrow[r]) + (lane & 15);
-    xsr[r] = xs_in + (size_t)row * KG;
-  }
-  if (!first_pass || !XSG) __syncthreads();         // the previous pass is done with xs and part
-  if constexpr (!XSG) group_sums_block<GS>(xrow, RB, KG, xs, tid, WAVES * 64);
-  // slices with no group (K/gs < SLICES) still take part in the ordered sum: as zeros
-  if (KG < SLICES) {
-#pragma unroll
-    for (int q = 0; q < SPW; ++q)
-#pragma unroll
-      for (int m = 0; m < NM; ++m)
-#pragma unroll
-        for (int r = 0; r < RB; ++r) part[(((wave * SPW + q) * NM + m) * RB + r) * 64 + lane] = 0.f;
-  }
-  if (!XSG || KG < SLICES) __syncthreads();
-  float acc[NM][RB];
-#pragma unroll
-  for (int m = 0; m < NM; ++m)
-#pragma unroll
-    for (int r = 0; r < RB; ++r) acc[m][r] = 0.f;
-  int slice = wave * SPW;
-  while (slice < SLICES && slice_begin(slice + 1, KG) == slice_begin(slice, KG)) ++slice;   // skip empty slices
-  int slice_end = slice < SLICES ? slice_begin(slice + 1, KG) : -1;
-  auto flush = [&](int g, float (&a)[NM][RB]) {
-    if (g + 1 != slice_end) return;
-#pragma unroll
-    for (int m = 0; m < NM; ++m)
-#pragma unroll
-      for (int r = 0; r < RB; ++r) {
-        part[((slice * NM + m) * RB + r) * 64 + lane] = a[m][r];
-        a[m][r] = 0.f;
-      }
-    ++slice;
-    while (slice < SLICES && slice_begin(slice + 1, KG) == slice_begin(slice, KG)) ++slice;
-    slice_end = slice < SLICES ? slice_begin(slice + 1, KG) : -1;
-  };
-  const int gA = slice_begin(wave * SPW, KG), gB = slice_begin((wave + 1) * SPW, KG);
-  // with sums from memory, lane i keeps the sums of group gA + i (64 groups at a time) and readlane hands them out
-  float xsv[RB];
-  int xs_base = gA;
-  auto fetch_sums = [&](int base) {
-#pragma unroll
-    for (int r = 0; r < RB; ++r) xsv[r] = base + lane < gB ? xsr[r][base + lane] : 0.f;
-    xs_base = base;
-  };
-  if constexpr (XSG) fetch_sums(gA);
-  auto xsum = [&](int r, int g) {
-    if constexpr (XSG) {
-      if (g - xs_base >= 64) fetch_sums(g);
-      return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, xsv[r]), g - xs_base));
-    } else {
-      return xs[r * KG + g];
-    }
-  };
-  gemv_stream<GS, NM, RB>(acc, st, loaded, wq, sb, xl, xsum, gA, gB, flush);
-  __syncthreads();
-  // a wave a row, a lane a column: the slices' sums in slice order, then the epilogue
-  for (int r = wave; r < RB; r += WAVES) {
-    const int l = lane;
-    const int onb = 2 * cb2 + (l >> 5);
-    const bool ok = onb < NB;
-    float v[NM];
-#pragma unroll
-    for (int m = 0; m < NM; ++m) {
-      float s = part[(m * RB + r) * 64 + l];
-#pragma unroll
-      for (int q = 1; q < SLICES; ++q) s += part[((q * NM + m) * RB + r) * 64 + l];
-      v[m] = s;
-    }
-    int prow = pr[0];
-#pragma unroll
-    for (int q = 1; q < RB; ++q) prow = r == q ? pr[q] : prow;
-    const size_t at = (size_t)prow * N + onb * 32 + (l & 31);
-    if constexpr (EPI == 0) {
-      if (ok) reinterpret_cast<float*>(out)[at] = v[0];
-    } else {
-      const float o = round_bf16(EPI == 1 ? relu2(v[0]) : swiglu(v[0], v[NM - 1], limit));
-      if (ok) reinterpret_cast<uint16_t*>(out)[at] = (uint16_t)(__float_as_uint(o) >> 16);
-      if (xs_out) {
-        // group sums of the rounded activations: a fixed xor tree over the group's lanes
-        float t = ok ? o : 0.f;
-#pragma unroll
-        for (int m = 1; m < GS; m <<= 1) t += __shfl_xor(t, m);
-        if (ok && (l & (GS - 1)) == 0) xs_out[(size_t)prow * (N / GS) + (cb2 * 64 + l) / GS] = t;
-      }
-    }
-  }
-}
-
-// A workgroup takes (item, pair of 32-column blocks): lanes 0-31 the even block, lanes 32-63 the odd one.
-// Pair p reads X row p / slots when slots > 0, else row p (experts.cu:129).  The item's rows go through in passes
-// of 2 or 1; a row's arithmetic is the same in each, so its bits do not depend on the pass it lands in.
+// A workgroup takes (item, pair of 32-column blocks); see expert_unit.
 template <int GS, int NM, int EPI, int WAVES, bool XSG>
 __global__ void __launch_bounds__(WAVES * 64)
     expert_kernel(const uint16_t* __restrict__ X, int64_t x_stride, int slots, const uint32_t* __restrict__ W, int KG,
                   int NB, const int* __restrict__ items, const int* __restrict__ counts,
                   const int* __restrict__ members, void* __restrict__ out, int N, float limit,
                   const float* __restrict__ xs_in, float* __restrict__ xs_out) {
-  constexpr int BW = block_words(GS);
-  constexpr int SPW = SLICES / WAVES;
-  extern __shared__ float lds[];            // xs [RBMAX][KG], then the slices' sums [SLICES][NM][RBMAX][64]
+  extern __shared__ float lds[];
   const int NB2 = (NB + 1) >> 1;
   const int it = blockIdx.x / NB2, cb2 = blockIdx.x - it * NB2;
-#ifdef TF_X_FAKEITEM
-  if (it >= 41) return;
-  const int e = (it * 3) & 127, first = it, cnt = 1;
-#else
   if (it >= counts[0]) return;
   const int e = items[3 * it], first = items[3 * it + 1], cnt = items[3 * it + 2];
-#endif
-  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int nb = 2 * cb2 + (lane >> 5), c = lane & 31;
-  const bool col_ok = nb < NB;
-  const uint32_t* wbase =
-      W + (((size_t)e * NB + (col_ok ? nb : NB - 1)) * KG) * (size_t)(NM * BW) + c * 4;
-  const uint32_t* sbase = wbase - c * 4 + 32 * GS / 8 + c;
-  auto wq = [&](int g, int m, int i) { return ldg16(wbase + ((size_t)g * NM + m) * BW + i * 128); };
-  auto sb = [&](int g, int m, float& s, float& b) {
-    const uint32_t v = sbase[((size_t)g * NM + m) * BW];
-    s = bf16_lo(v);
-    b = bf16_hi(v);
-  };
-  const int gA = slice_begin(wave * SPW, KG), gB = slice_begin((wave + 1) * SPW, KG);
-  float* xs = lds;
-  float* part = lds + (XSG ? 0 : RBMAX * KG);
-  // the wave's first groups are on their way before anything else is read
-  Stage<GS, NM> st[DEPTH];
-#pragma unroll
-  for (int d = 0; d < DEPTH; ++d)
-    if (gA + d < gB) load_weights<GS, NM>(st[d], wq, sb, gA + d);
-  bool loaded = true, first_pass = true;
-  int r0 = 0;
-#define TF_PASS(RB_)                                                                                                 \
-  expert_pass<GS, NM, EPI, WAVES, RB_, XSG>(X, x_stride, slots, wq, sb, KG, NB, cb2, members, first + r0, out, N,    \
-                                            limit, xs, part, st, loaded, first_pass, xs_in, xs_out);                 \
-  first_pass = false;                                                                                                \
-  loaded = gB - gA <= DEPTH   /* a run that fits the stages stays in registers for the next pass */
-  for (; r0 + 2 <= cnt; r0 += 2) {
-    TF_PASS(2);
-  }
-  if (r0 < cnt) {
-    TF_PASS(1);
-  }
-#undef TF_PASS
+  NoHook none;
+  expert_unit<GS, NM, EPI, WAVES, XSG, 0>(X, x_stride, slots, W, KG, NB, e, cnt, members + first, cb2, out, N, limit, xs_in,
+                                       xs_out, lds, none);
 }
 
 // ---- dense lane matmul ---------------------------------------------------------------------------------------------
@@ -399,7 +70,7 @@ __device__ __forceinline__ void qmm_pass(const uint16_t* __restrict__ X, int64_t
   for (int r = 0; r < RB; ++r) acc[0][r] = 0.f;
   NoFlush none;
   auto xsum = [&](int r, int g) { return __uint_as_float(xsr[r][g]); };
-  gemv_stream<GS, 1, RB>(acc, st, loaded, wq, sb, xl, xsum, g0, g1, none);
+  gemv_stream<GS, 1, RB, 0>(acc, st, loaded, wq, sb, xl, xsum, g0, g1, none);
 #pragma unroll
   for (int r = 0; r < RB; ++r) part[(wave * RB + r) * 64 + lane] = acc[0][r];
   __syncthreads();
@@ -500,7 +171,7 @@ int launch_experts(const uint16_t* x, int64_t x_stride, int slots, const uint32_
   const int64_t grid = max_items * nb2;
   if (grid < 1) return 0;
   TF_REQUIRE(grid <= 0x7FFFFFFF, "experts: %lld workgroups exceed the grid limit", (long long)grid);
-  const size_t smem = sizeof(float) * ((XSG ? 0 : (size_t)RBMAX * kg) + (size_t)SLICES * NM * RBMAX * 64);
+  const size_t smem = sizeof(float) * expert_lds_floats(NM, kg, XSG);
   TF_REQUIRE(smem <= 64 * 1024, "experts: K/gs = %d groups need %zu bytes of LDS (limit 65536)", kg, smem);
   const dim3 g((unsigned)grid);
 #define TF_GO(W_)                                                                                                  \

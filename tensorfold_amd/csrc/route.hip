@@ -33,11 +33,9 @@ __global__ void __launch_bounds__(64)
 
 constexpr int TOPK_VPL = 16;     // values a lane: up to 1024 experts
 
-__global__ void __launch_bounds__(64)
-    topk_kernel(const float* __restrict__ L, int64_t ldl, int NE, int TOPK, int shared, int* __restrict__ pick,
-                float* __restrict__ wts) {
-  const int r = blockIdx.x, lane = threadIdx.x, slots = TOPK + (shared ? 1 : 0);
-  const float* row = L + (size_t)r * ldl;
+// one wave, one row: see tf_moe_topk
+__device__ __forceinline__ void topk_row(const float* __restrict__ row, int NE, int TOPK, int shared, int lane,
+                                         int* __restrict__ pick, float* __restrict__ wts) {
   const float NEG = -__builtin_inff();
   float v[TOPK_VPL];
 #pragma unroll
@@ -76,14 +74,21 @@ __global__ void __launch_bounds__(64)
     }
   }
   if (lane < TOPK) {
-    pick[(size_t)r * slots + lane] = mine_id;
-    wts[(size_t)r * slots + lane] = round_bf16(mine_ex / total);
+    pick[lane] = mine_id;
+    wts[lane] = round_bf16(mine_ex / total);
   }
   if (shared && lane == 0) {
     const float sg = round_bf16(row[NE]);
-    pick[(size_t)r * slots + TOPK] = NE;
-    wts[(size_t)r * slots + TOPK] = round_bf16(1.f / (1.f + expf(-sg)));
+    pick[TOPK] = NE;
+    wts[TOPK] = round_bf16(1.f / (1.f + expf(-sg)));
   }
+}
+
+__global__ void __launch_bounds__(64)
+    topk_kernel(const float* __restrict__ L, int64_t ldl, int NE, int TOPK, int shared, int* __restrict__ pick,
+                float* __restrict__ wts) {
+  const int r = blockIdx.x, slots = TOPK + (shared ? 1 : 0);
+  topk_row(L + (size_t)r * ldl, NE, TOPK, shared, threadIdx.x, pick + (size_t)r * slots, wts + (size_t)r * slots);
 }
 
 // ---- plan: stable counting sort of pairs by expert -------------------------------------------------------------------
@@ -167,6 +172,78 @@ __global__ void __launch_bounds__(PLAN_THREADS)
     int rank = 0;
     for (int q = 0; q < tid; ++q) rank += pk[q] == e;
     members[off[e] + rank] = tid;
+  }
+}
+
+// The decode layer's whole routing in one workgroup (rows * slots <= 1024): top-k of every row, the pair sort, one
+// descriptor an item for the fused expert kernel {expert, count, first, 0, pairs[16]}, the group sums of x, and the
+// zeroing of the fused kernel's counters.
+constexpr int DESC = 20;
+
+__global__ void __launch_bounds__(PLAN_THREADS)
+    route_decode_kernel(const float* __restrict__ L, int64_t ldl, int R, int NE, int TOPK, int shared,
+                        const uint16_t* __restrict__ X, int64_t ldx, int D, int gs, int* __restrict__ pick,
+                        float* __restrict__ wts, int* __restrict__ members, int* __restrict__ items,
+                        int* __restrict__ counts, int* __restrict__ desc, float* __restrict__ xs_x,
+                        int* __restrict__ zero, int n_zero) {
+  __shared__ int pk[PLAN_THREADS];
+  __shared__ int cnt[EMAX];
+  __shared__ int off[EMAX];
+  __shared__ int mem[PLAN_THREADS];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int slots = TOPK + (shared ? 1 : 0), P = R * slots, E = NE + (shared ? 1 : 0), T = 16;
+  cnt[tid] = 0;
+  for (int i = tid; i < n_zero; i += PLAN_THREADS) zero[i] = 0;
+  for (int r = wave; r < R; r += PLAN_THREADS / 64)
+    topk_row(L + (size_t)r * ldl, NE, TOPK, shared, lane, pick + (size_t)r * slots, wts + (size_t)r * slots);
+  // group sums of x: 8 (groups of 64) or 4 (groups of 32) lanes a group, as tf_group_sums
+  {
+    const int lpg = gs / 8, part = tid % lpg, KG = D / gs;
+    for (int o = tid / lpg; o < R * KG; o += PLAN_THREADS / lpg) {
+      const int r = o / KG, g = o - r * KG;
+      const uint4 v = *reinterpret_cast<const uint4*>(X + (size_t)r * ldx + (size_t)g * gs + part * 8);
+      float s = bf16_lo(v.x);
+      s += bf16_hi(v.x);
+      s += bf16_lo(v.y);
+      s += bf16_hi(v.y);
+      s += bf16_lo(v.z);
+      s += bf16_hi(v.z);
+      s += bf16_lo(v.w);
+      s += bf16_hi(v.w);
+      for (int m = 1; m < lpg; m <<= 1) s += __shfl_xor(s, m);
+      if (part == 0) xs_x[o] = s;
+    }
+  }
+  __threadfence_block();
+  __syncthreads();
+  int e = -1;
+  if (tid < P) {
+    e = pick[tid];
+    if ((unsigned)e >= (unsigned)E) e = -1;
+    pk[tid] = e;
+    if (e >= 0) atomicAdd(&cnt[e], 1);
+  }
+  __syncthreads();
+  const int o = place_items(tid < E ? cnt[tid] : 0, E, T, items, counts);
+  off[tid] = o;
+  __syncthreads();
+  if (tid < P && e >= 0) {
+    int rank = 0;
+    for (int q = 0; q < tid; ++q) rank += pk[q] == e;
+    members[off[e] + rank] = tid;
+    mem[off[e] + rank] = tid;
+  }
+  __threadfence_block();
+  __syncthreads();
+  const int n_items = counts[0];
+  for (int i = tid; i < n_items; i += PLAN_THREADS) {
+    const int ie = items[3 * i], first = items[3 * i + 1], c = items[3 * i + 2];
+    int* d = desc + (size_t)i * DESC;
+    d[0] = ie;
+    d[1] = c;
+    d[2] = first;
+    d[3] = 0;
+    for (int j = 0; j < 16; ++j) d[4 + j] = j < c ? mem[first + j] : 0;
   }
 }
 
@@ -272,6 +349,28 @@ extern "C" int tf_moe_topk(const float* logits, int64_t ldl, int rows, int exper
              experts + (shared ? 1 : 0));
   topk_kernel<<<rows, 64, 0, as_stream(stream)>>>(logits, ldl, experts, top_k, shared, pick, wts);
   TF_LAUNCH_OK("tf_moe_topk");
+  return 0;
+}
+
+extern "C" int tf_moe_route_decode(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared,
+                                   const uint16_t* x, int64_t ldx, int d, int gs, int32_t* pick, float* wts,
+                                   int32_t* members, int32_t* items, int32_t* counts, int32_t* desc, float* xs_x,
+                                   int32_t* zero, int n_zero, tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(logits && x && pick && wts && members && items && counts && desc && xs_x, "route: null pointer argument");
+  TF_REQUIRE(experts >= 1 && experts + (shared ? 1 : 0) <= EMAX && experts <= 64 * TOPK_VPL,
+             "route: at most %d experts", EMAX - 1);
+  TF_REQUIRE(top_k >= 1 && top_k <= 64 && top_k <= experts, "route: 1 to 64 experts a row, not %d", top_k);
+  TF_REQUIRE(rows >= 1 && (int64_t)rows * (top_k + (shared ? 1 : 0)) <= PLAN_THREADS,
+             "route: the fused decode routing takes at most %d pairs", PLAN_THREADS);
+  TF_REQUIRE(gs == 32 || gs == 64, "route: groups of 32 or 64 inputs");
+  TF_REQUIRE(d >= gs && d % gs == 0 && aligned16(x) && ldx % 8 == 0, "route: x rows of whole groups, 16-byte aligned");
+  TF_REQUIRE(ldl >= experts + (shared ? 1 : 0), "route: logits rows are too short");
+  TF_REQUIRE(n_zero >= 0 && (n_zero == 0 || zero), "route: bad counter range");
+  route_decode_kernel<<<1, PLAN_THREADS, 0, as_stream(stream)>>>(logits, ldl, rows, experts, top_k, shared, x, ldx, d,
+                                                                gs, pick, wts, members, items, counts, desc, xs_x, zero,
+                                                                n_zero);
+  TF_LAUNCH_OK("tf_moe_route_decode");
   return 0;
 }
 

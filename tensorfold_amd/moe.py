@@ -10,11 +10,16 @@ the optional shared expert rides in the last slot with a sigmoid gate.
 from __future__ import annotations
 
 import dataclasses
+import os
 
 import torch
 
 from . import _lib
 from . import experts as grouped
+
+# ``run`` issues a decode-sized layer as routing + up + down + combine launches; with this set it issues the routing
+# launch and the one fused experts launch (``decode``) instead.  Same bits either way.
+FUSED_DECODE = os.environ.get("TENSORFOLD_AMD_FUSED_DECODE", "0") == "1"
 
 
 def router(x: torch.Tensor, rows: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
@@ -55,6 +60,30 @@ class MoEBuffers:
         # rounding alone costs 1.1e-3 relative L2 at the combine, most of a 2e-3 budget.  ``experts.down`` still
         # writes bf16 into a bf16 ``out`` on a prompt plan for callers that want the smaller buffer.)
         self.y = torch.empty((rows, self.slots, cfg.hidden_size), device=device, dtype=torch.float32)
+        self.cfg, self.device, self._fused = cfg, device, None
+
+    def fused(self, gs: int) -> dict:
+        """Scratch of the fused decode layer (``decode``), made on first use: item descriptors, group sums, the
+        counters (status, then an arrival count an item, then one a (token, 64 columns) cell) and the output."""
+
+        if self._fused is None:
+            cfg, dev, pairs = self.cfg, self.device, self.rows * self.slots
+            items = grouped.max_items(pairs, cfg.num_experts + int(self.shared), grouped.TILE)
+            cells = self.rows * (cfg.hidden_size // 64)
+            self._fused = dict(
+                items=items,
+                desc=torch.zeros((items, 20), dtype=torch.int32, device=dev),
+                xs_x=torch.empty((self.rows, cfg.hidden_size // gs), dtype=torch.float32, device=dev),
+                xs_act=torch.empty((pairs, cfg.moe_intermediate_size // gs), dtype=torch.float32, device=dev),
+                counters=torch.zeros((1 + items + cells,), dtype=torch.int32, device=dev),
+                out=torch.empty((self.rows, cfg.hidden_size), dtype=torch.bfloat16, device=dev))
+        return self._fused
+
+    def check(self) -> None:
+        """Host-side look at the fused layer's status flag (synchronises): raises if a bounded wait ran out."""
+
+        if self._fused is not None and int(self._fused["counters"][0]):
+            raise RuntimeError("tensorfold-amd: the fused decode layer timed out waiting for its activations")
 
 
 def select_rows(logits: torch.Tensor, buf: MoEBuffers, top_k: int, experts: int) -> None:
@@ -87,6 +116,46 @@ def moe(x: torch.Tensor, router_rows: torch.Tensor, ex: grouped.Experts, buf: Mo
     grouped.gate_up(x, ex, buf.plan, act, n)
     grouped.down(act, ex, buf.plan, buf.y.view(-1, ex.dims), n)
     return buf
+
+
+def fusable(x: torch.Tensor, ex: grouped.Experts, buf: MoEBuffers) -> bool:
+    """Whether ``decode`` takes this call: decode arithmetic, at most 1,024 pairs, sizes in whole 64-column units."""
+
+    return (not buf.plan.prefill and x.shape[0] * buf.slots <= grouped.SMALL and ex.dims % 64 == 0
+            and ex.width % 64 == 0)
+
+
+def decode(x: torch.Tensor, logits: torch.Tensor, ex: grouped.Experts, buf: MoEBuffers, top_k: int, experts: int,
+           out: torch.Tensor | None = None) -> torch.Tensor:
+    """The decode layer in two launches: routing (top-k, pair sort, group sums), then every expert's up projection,
+    activation, down projection and the weighted combine in one kernel.  Same bits as ``select`` + ``gate_up`` +
+    ``down`` + ``combine``; bf16 [R, D] out.  ``buf.pick``, ``buf.wts`` and ``buf.plan`` are filled as by ``select``."""
+
+    _lib.on_gpu(x, logits)
+    n = int(x.shape[0])
+    if not fusable(x, ex, buf) or n > buf.rows:
+        raise ValueError("decode: this call does not fit the fused decode layer (see fusable)")
+    if x.dtype != torch.bfloat16 or x.stride(1) != 1 or x.stride(0) % 8 or x.shape[1] != ex.dims:
+        raise RuntimeError("x: rows of K = groups * group size inputs, 16-byte aligned")
+    if logits.dtype != torch.float32 or logits.stride(1) != 1:
+        raise ValueError("select: logits must be fp32 with unit-stride rows")
+    f = buf.fused(ex.gs)
+    if out is None:
+        out = f["out"][:n]
+    plan = buf.plan
+    plan.tile = grouped.TILE
+    items = grouped.max_items(n * buf.slots, experts + int(buf.shared), grouped.TILE)
+    cells = n * (ex.dims // 64)
+    ctr = f["counters"]
+    _lib.call("tf_moe_route_decode", _lib.ptr(logits), logits.stride(0), n, experts, top_k, int(buf.shared), _lib.ptr(x),
+              x.stride(0), ex.dims, ex.gs, _lib.ptr(buf.pick), _lib.ptr(buf.wts), _lib.ptr(plan.members),
+              _lib.ptr(plan.items), _lib.ptr(plan.counts), _lib.ptr(f["desc"]), _lib.ptr(f["xs_x"]), _lib.ptr(ctr),
+              1 + f["items"] + cells)
+    _lib.call("tf_moe_decode_experts", ex.gs, int(ex.swiglu), _lib.ptr(x), x.stride(0), n, buf.slots, _lib.ptr(ex.up),
+              _lib.ptr(ex.down), ex.dims, ex.width, _lib.ptr(f["desc"]), _lib.ptr(plan.counts), _lib.ptr(buf.wts),
+              _lib.ptr(f["xs_x"]), _lib.ptr(buf.act), _lib.ptr(f["xs_act"]), _lib.ptr(buf.y), _lib.ptr(out),
+              ctr.data_ptr() + 4, ctr.data_ptr() + 4 * (1 + f["items"]), _lib.ptr(ctr), ex.limit, items)
+    return out
 
 
 def combine(y: torch.Tensor, wts: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
@@ -136,5 +205,9 @@ def run(x: torch.Tensor, m: Routed, *, prefill: bool = False) -> torch.Tensor:
     key = (cap, m.count, m.top_k, m.experts.width, m.experts.dims, prefill, x.device)
     if key not in _pool:
         _pool[key] = MoEBuffers(cap, _Dims(m), x.device, prefill=prefill)
-    buf = moe(x.contiguous(), m.router, m.experts, _pool[key], m.top_k, m.count)
+    buf, x = _pool[key], x.contiguous()
+    if FUSED_DECODE and fusable(x, m.experts, buf):
+        router(x, m.router, buf.logits[:n])
+        return decode(x, buf.logits[:n], m.experts, buf, m.top_k, m.count).clone()
+    moe(x, m.router, m.experts, buf, m.top_k, m.count)
     return combine(buf.y[:n], buf.wts[:n])

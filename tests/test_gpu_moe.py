@@ -200,3 +200,34 @@ def test_moe_run_rows_do_not_depend_on_the_window():
     for r in (0, 7):
         assert torch.equal(moe.run(x[r:r + 1], layer, prefill=True)[0], whole_p[r]), r
     assert rel_l2(f32(whole_p), f32(whole)) < 1e-2
+
+
+@pytest.mark.parametrize("shape,ne,rows", [(synthetic.C1, 24, 1), (synthetic.C1, 24, 8), (synthetic.C2, 48, 32),
+                                           (synthetic.MoEShape("small", 512, 16, 128, 4, 32, True, True), 16, 5),
+                                           (synthetic.MoEShape("small64", 384, 12, 192, 3, 64, False, False), 12, 19)])
+def test_the_fused_decode_layer_equals_the_separate_kernels(shape, ne, rows):
+    """Routing in one launch and up + down + combine in one launch: ids, plan and output bits equal those of
+    select + gate_up + down + combine; twice in a row on different inputs (the counters are reset by the routing)."""
+
+    up, down = layer_tables(shape, 1500, ne)
+    ex = experts.make([tuple(t.to(DEV) for t in m) for m in up], tuple(t.to(DEV) for t in down), shape.gs)
+    cfg = type("c", (), dict(num_experts_per_tok=shape.top_k, num_experts=ne, moe_intermediate_size=shape.width,
+                             hidden_size=shape.hidden))
+    fused = moe.MoEBuffers(rows, cfg, DEV, shared=shape.shared)
+    for seed in (1, 2):
+        x = synthetic.activations(rows, shape.hidden, 1501 + seed).to(DEV)
+        l = synthetic.logits(rows, ne + int(shape.shared), 1510 + seed).to(DEV)
+        ref = moe.MoEBuffers(rows, cfg, DEV, shared=shape.shared)
+        moe.select(l, ref, shape.top_k, ne)
+        experts.gate_up(x, ex, ref.plan, ref.act.view(-1, ex.width), rows)
+        experts.down(ref.act.view(-1, ex.width), ex, ref.plan, ref.y.view(-1, ex.dims), rows)
+        want = moe.combine(ref.y, ref.wts)
+        got = moe.decode(x, l, ex, fused, shape.top_k, ne)
+        torch.cuda.synchronize()
+        fused.check()
+        assert torch.equal(fused.pick, ref.pick) and torch.equal(fused.wts, ref.wts)
+        n = int(ref.plan.counts[0])
+        assert torch.equal(fused.plan.counts, ref.plan.counts) and torch.equal(fused.plan.items[:n], ref.plan.items[:n])
+        assert torch.equal(fused.plan.members, ref.plan.members)
+        assert torch.equal(fused.act, ref.act) and torch.equal(fused.y, ref.y)
+        assert torch.equal(got, want), seed
