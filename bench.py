@@ -23,6 +23,12 @@ import torch
 from tensorfold_amd import _lib, experts, moe, synthetic
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes a launch of the expert kernels on this (seeded) workload, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
+# (KiB a dispatch; FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0, the factors a plain 256 MiB elementwise kernel gives).
+# Keyed by (projection, tokens); measured with --steps 20 --warmup 2 --copy-probe, independent of the step count.
+MEASURED_TRAFFIC = {("up", 8): (2 * 56634.0 + 215.6) * 1024, ("down", 8): (2 * 57177.0 + 504.0) * 1024,
+                    ("up", 4): (2 * 30367.4 + 107.8) * 1024, ("down", 4): (2 * 30637.7 + 252.0) * 1024,
+                    ("up", 1): (2 * 8308.9 + 27.0) * 1024, ("down", 1): (2 * 8365.3 + 63.0) * 1024}
 SHAPE = synthetic.C1
 LAYERS = 4          # 4 x 718 MB of expert tables
 POOL = 64           # distinct routing draws
@@ -239,6 +245,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--tokens", type=int, default=8, help="batch of the headline value (1, 4 and 8 are all reported)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain 256 MiB in / 256 MiB out elementwise kernel three times: the known-size "
+                         "dispatch that FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus above 1 is not supported (the path has no multi-GPU code)",
@@ -249,6 +258,7 @@ def main() -> int:
     tables, keep = device_tables(SHAPE, LAYERS, dev)
     results = {t: run_batch(t, tables, args.steps, args.warmup, dev) for t in sorted({1, 4, 8, args.tokens})}
     head = results[args.tokens]
+    traffic = None
     if moe.FUSED_DECODE:
         dom_us, dom_bytes = head["fused_kernel_us"], 2 * head["kernel_bytes"]
         dom = "moe_fused_kernel (up + down + combine"
@@ -256,6 +266,7 @@ def main() -> int:
         which = "up" if head["up_kernel_us"] >= head["down_kernel_us"] else "down"
         dom_us, dom_bytes = head[f"{which}_kernel_us"], head["kernel_bytes"]
         dom = f"expert_kernel ({which} projection"
+        traffic = MEASURED_TRAFFIC.get((which, args.tokens))
     achieved = dom_bytes / dom_us * 1e-3
     line = {
         "metric": "moe_decode_layer_us_per_token", "value": head["us_per_token"], "unit": "us/token", "n_gpus": 1,
@@ -266,7 +277,7 @@ def main() -> int:
                                f"cycled", "tokens": args.tokens, "hidden": SHAPE.hidden, "experts": SHAPE.experts,
                    "intermediate": SHAPE.width, "top_k": SHAPE.top_k, "group_size": SHAPE.gs},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "kernel": f"{dom}, {head['kernel_unique_experts']:.1f} experts a launch)",
                      "kernel_us": dom_us, "bytes_per_launch": dom_bytes},
         "layer_hbm": {"achieved": head["layer_gbs"], "frac": head["layer_frac"], "unit": "GB/s",
@@ -274,6 +285,13 @@ def main() -> int:
         "batches": {str(t): {k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()}
                     for t, r in results.items()},
     }
+    if args.copy_probe:
+        a = torch.ones(64 << 20, dtype=torch.float32, device=dev)
+        b = torch.empty_like(a)
+        for _ in range(3):
+            torch.mul(a, 2.0, out=b)
+        torch.cuda.synchronize()
+        del a, b
     if not args.no_cpu:
         del tables
         torch.cuda.empty_cache()
