@@ -1,0 +1,215 @@
+"""Kernel timings of the BASELINE configurations that are not bench.py's headline: 0 (dense 4-bit projection),
+2 (verify-window MoE layer), 3 (prompt chunk, grouped MFMA) and 4 (EXL3 projections).
+
+    python bench_configs.py [c0] [c2] [c3] [c4]
+
+One JSON line a configuration: time of one pass (hipGraph of back-to-back passes cycling over enough weight copies to
+miss the 256 MB Infinity Cache, HIP events around the replay), algorithmic bytes or flops, and the fraction of the
+MI355X peak (8 TB/s HBM, 2.5 PFLOP/s dense 16-bit MFMA).  Synthetic data drawn on the GPU; parity is the tests' job.
+"""
+
+from __future__ import annotations
+
+import json
+import sys
+
+import torch
+
+from tensorfold_amd import experts, moe, qmm, synthetic
+from tensorfold_amd.exl3 import linear as exl3
+
+DEV = "cuda:0"
+HBM, MFMA = 8000.0, 2500.0          # GB/s, TFLOP/s
+
+
+def graph_us(step, reps: int) -> float:
+    """Mean time of ``step(i)`` over a replayed graph of ``reps`` calls."""
+
+    for i in range(3):
+        step(i)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for i in range(reps):
+            step(i)
+    g.replay()
+    torch.cuda.synchronize()
+    best = []
+    for _ in range(5):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        g.replay()
+        b.record()
+        torch.cuda.synchronize()
+        best.append(a.elapsed_time(b) * 1e3 / reps)
+    return sorted(best)[len(best) // 2]
+
+
+def rand_affine(n: int, k: int, gs: int, gen, lead=()):
+    words = torch.randint(-(2 ** 31), 2 ** 31, (*lead, n, k // 8), generator=gen, device=DEV,
+                          dtype=torch.int64).to(torch.int32)
+    scales = (torch.rand((*lead, n, k // gs), generator=gen, device=DEV) * 0.018 + 0.002).bfloat16()
+    return words, scales, (scales.float() * -8).bfloat16()
+
+
+def c0() -> dict:
+    n = k = 4096
+    gen = torch.Generator(device=DEV).manual_seed(1)
+    copies = [qmm.pack(*rand_affine(n, k, 64, gen), 64) for _ in range(40)]       # 40 x 9.4 MB
+    out = {}
+    for m in (1, 8):
+        x = synthetic.activations(m, k, 7).to(DEV)
+        y = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+        xs = qmm.group_sums(x, 64)                  # the producer of x makes these in a model
+        part = torch.empty((qmm.split_k(n, k, 64), m, n), dtype=torch.float32, device=DEV)
+        us = graph_us(lambda i: qmm.matmul(x, copies[i % len(copies)], xs, out=y, part=part), 120)
+        nbytes = n * k // 2 + 2 * 2 * n * k // 64 + m * (k + n) * 2
+        out[m] = {"us": us, "bytes": nbytes, "gbs": nbytes / us * 1e-3, "frac": nbytes / us * 1e-3 / HBM}
+    return {"config": "c0: dense 4-bit/g64 projection, N = K = 4096 (qmm kernel + slice reduce; group sums given)",
+            "bound": "hbm", "rows": out}
+
+
+def moe_tables(shape, layers: int, gen):
+    e = shape.experts + int(shape.shared)
+    tabs = []
+    for _ in range(layers):
+        up = [rand_affine(shape.width, shape.hidden, shape.gs, gen, (e,)) for _ in range(2 if shape.swiglu else 1)]
+        down = rand_affine(shape.hidden, shape.width, shape.gs, gen, (e,))
+        tabs.append(experts.make(up, down, shape.gs))
+        del up, down
+    return tabs
+
+
+def cfg_of(shape):
+    return type("cfg", (), dict(num_experts_per_tok=shape.top_k, num_experts=shape.experts,
+                                moe_intermediate_size=shape.width, hidden_size=shape.hidden))
+
+
+def c2() -> dict:
+    s, rows = synthetic.C2, 32
+    gen = torch.Generator(device=DEV).manual_seed(2)
+    tabs = moe_tables(s, 2, gen)                                                  # 2 x 1.0 GB
+    x = synthetic.activations(rows, s.hidden, 1201).to(DEV)
+    logits = [synthetic.logits(rows, s.experts + 1, 3000 + i).to(DEV) for i in range(16)]
+    buf = moe.MoEBuffers(rows, cfg_of(s), DEV, shared=True)
+    out = torch.empty((rows, s.hidden), dtype=torch.bfloat16, device=DEV)
+    per_expert = 3 * (s.width * s.hidden // 2 + 2 * 2 * s.width * s.hidden // s.gs)
+    uniq = []
+    for l in logits:
+        moe.select(l, buf, s.top_k, s.experts)
+        torch.cuda.synchronize()
+        uniq.append(int(buf.plan.counts[1]))
+    mean_u = sum(uniq) / len(uniq)
+
+    def step(i):
+        ex = tabs[i % 2]
+        moe.select(logits[i % 16], buf, s.top_k, s.experts)
+        experts.gate_up(x, ex, buf.plan, buf.act.view(-1, ex.width), rows)
+        experts.down(buf.act.view(-1, ex.width), ex, buf.plan, buf.y.view(-1, ex.dims), rows)
+        moe.combine(buf.y, buf.wts, out)
+
+    def up_only(i):
+        ex = tabs[i % 2]
+        experts.gate_up(x, ex, buf.plan, buf.act.view(-1, ex.width), rows)
+
+    def down_only(i):
+        ex = tabs[i % 2]
+        experts.down(buf.act.view(-1, ex.width), ex, buf.plan, buf.y.view(-1, ex.dims), rows)
+
+    us = graph_us(step, 32)
+    moe.select(logits[0], buf, s.top_k, s.experts)
+    up_us, down_us = graph_us(up_only, 32), graph_us(down_only, 32)
+    nbytes = mean_u * per_expert + rows * s.hidden * 2 * 2
+    return {"config": "c2: verify-window MoE layer, 512 experts + shared, SwiGLU, top-10, g32, 32 rows",
+            "bound": "hbm", "layer_us": us, "us_per_token": us / rows, "distinct_experts": mean_u, "bytes": nbytes,
+            "gbs": nbytes / us * 1e-3, "frac": nbytes / us * 1e-3 / HBM, "up_kernel_us": up_us,
+            "down_kernel_us": down_us, "up_gbs": uniq[0] * per_expert * 2 / 3 / up_us * 1e-3,
+            "down_gbs": uniq[0] * per_expert / 3 / down_us * 1e-3}
+
+
+def c3() -> dict:
+    s, rows = synthetic.C2, 4096
+    gen = torch.Generator(device=DEV).manual_seed(3)
+    ex = moe_tables(s, 1, gen)[0]
+    x = synthetic.activations(rows, s.hidden, 1301).to(DEV)
+    ids = synthetic.zipf_picks(rows, s.experts, s.top_k, 1302)
+    picks = torch.cat([ids, torch.full((rows, 1), s.experts, dtype=torch.int32)], 1).contiguous().to(DEV)
+    sel = synthetic.logits(rows, s.top_k + 1, 1303)
+    wts = torch.cat([torch.softmax(sel[:, :-1], 1), torch.sigmoid(sel[:, -1:])], 1).bfloat16().float().contiguous().to(DEV)
+    slots = s.top_k + 1
+    out = {}
+    for tile in (64, 128):
+        plan = experts.Plan(rows, slots, s.experts + 1, DEV, prefill=True)
+        act = torch.empty((rows * slots, s.width), dtype=torch.bfloat16, device=DEV)
+        y = torch.empty((rows * slots, s.hidden), dtype=torch.float32, device=DEV)
+        res = torch.empty((rows, s.hidden), dtype=torch.bfloat16, device=DEV)
+
+        def step(i):
+            experts.route(picks, plan, tile)
+            experts.gate_up(x, ex, plan, act, rows)
+            experts.down(act, ex, plan, y, rows)
+            moe.combine(y.view(rows, slots, s.hidden), wts, res)
+
+        us = graph_us(step, 8)
+        experts.route(picks, plan, tile)
+        up_us = graph_us(lambda i: experts.gate_up(x, ex, plan, act, rows), 8)
+        down_us = graph_us(lambda i: experts.down(act, ex, plan, y, rows), 8)
+        route_us = graph_us(lambda i: experts.route(picks, plan, tile), 8)
+        flop = rows * slots * 3 * 2 * s.hidden * s.width
+        out[tile] = {"chunk_us": us, "tokens_per_s": rows / us * 1e6, "flop": flop, "tflops": flop / us * 1e-6,
+                     "frac": flop / us * 1e-6 / MFMA, "route_us": route_us, "up_us": up_us, "down_us": down_us,
+                     "up_tflops": flop * 2 / 3 / up_us * 1e-6, "down_tflops": flop / 3 / down_us * 1e-6,
+                     "items": int(plan.counts[0])}
+    return {"config": "c3: prompt chunk of 4,096 tokens, Zipf(1.1) over 512 experts + shared, SwiGLU, g32 "
+                      "(flops count the shared expert's 4,096 pairs)", "bound": "mfma", "tiles": out}
+
+
+def c4() -> dict:
+    gen = torch.Generator(device=DEV).manual_seed(4)
+
+    def layer(k, n):
+        trellis = torch.randint(-2 ** 15, 2 ** 15, (k // 16, n // 16, 48), generator=gen, device=DEV,
+                                dtype=torch.int32).to(torch.int16)
+        sc = lambda size: (torch.rand(size, generator=gen, device=DEV) * 1.5 + 0.5).half()
+        return exl3.Exl3Linear.from_tensors(trellis, sc(k), sc(n), "3inst", device=DEV)
+
+    mlps = [(layer(5120, 17408), layer(5120, 17408), layer(17408, 5120)) for _ in range(4)]     # 4 x 100 MB
+    out = {}
+    for m in (1, 8):
+        x = synthetic.activations(m, 5120, 4200 + m, dtype=torch.float16).to(DEV)
+        h = synthetic.activations(m, 17408, 4300 + m, dtype=torch.float16).to(DEV)
+        ys = [torch.empty((m, 17408), dtype=torch.float16, device=DEV) for _ in range(2)]
+        yd = torch.empty((m, 5120), dtype=torch.float16, device=DEV)
+        xh, hh = torch.empty_like(x), torch.empty_like(h)
+        z = torch.empty((16 * m * 17408,), dtype=torch.float32, device=DEV)
+
+        def step(i):
+            g, u, d = mlps[i % len(mlps)]
+            g(x, ys[0], xh=xh, z=z)
+            u(x, ys[1], xh=xh, z=z)
+            d(h, yd, xh=hh, z=z)
+
+        us = graph_us(step, 48)
+        gate_us = graph_us(lambda i: mlps[i % 4][0](x, ys[0], xh=xh, z=z), 48)
+        down_us = graph_us(lambda i: mlps[i % 4][2](h, yd, xh=hh, z=z), 48)
+        per = 5120 * 17408 * 3 // 8
+        nbytes = 3 * per + 3 * 2 * (5120 + 17408) + m * (2 * 5120 + 17408 + 17408 * 2 + 5120) * 2
+        out[m] = {"mlp_us": us, "bytes": nbytes, "gbs": nbytes / us * 1e-3, "frac": nbytes / us * 1e-3 / HBM,
+                  "gate_us": gate_us, "gate_gbs": per / gate_us * 1e-3, "down_us": down_us,
+                  "down_gbs": per / down_us * 1e-3}
+    return {"config": "c4: EXL3 3.0 bpw MLP, gate/up 5120 -> 17408, down 17408 -> 5120 (input rotation + linear kernel each)",
+            "bound": "hbm", "rows": out}
+
+
+def main() -> int:
+    torch.cuda.set_device(0)
+    which = sys.argv[1:] or ["c0", "c2", "c3", "c4"]
+    for name in which:
+        res = {"c0": c0, "c2": c2, "c3": c3, "c4": c4}[name]()
+        torch.cuda.empty_cache()
+        print(json.dumps(res, default=lambda v: round(v, 4)), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

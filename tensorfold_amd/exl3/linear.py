@@ -134,11 +134,20 @@ class Exl3Linear:
         m = int(x.shape[0])
         if out is None:
             out = x.new_empty((m, self.n), dtype=out_dtype or x.dtype)
+        elif tuple(out.shape) != (m, self.n) or out.dtype not in _DTYPES or not out.is_contiguous():
+            raise ValueError(f"out must be contiguous ({m}, {self.n}) fp16, bf16 or fp32")
+        else:
+            _lib.on_gpu(out)
         sk, wk = self.split
         if xh is None:
             xh = x.new_empty((m, self.k), dtype=torch.float16)
+        elif xh.dtype != torch.float16 or xh.numel() < m * self.k or not xh.is_contiguous() or xh.device != x.device:
+            raise ValueError(f"xh must hold {m} x {self.k} fp16 values on x's device")
         if sk > 1 and z is None:
             z = x.new_empty((sk * m * self.n,), dtype=torch.float32)
+        elif sk > 1 and (z.dtype != torch.float32 or z.numel() < sk * m * self.n or not z.is_contiguous()
+                         or z.device != x.device):
+            raise ValueError(f"z must hold {sk} x {m} x {self.n} fp32 values on x's device")
         stride_k, stride_nb = self.strides
         _lib.call("tf_exl3_rot_in", _lib.ptr(x), _DTYPES[x.dtype], _lib.ptr(self.suh), _lib.ptr(xh), m, self.k)
         _lib.call("tf_exl3_linear", _lib.ptr(xh), _lib.ptr(self.words), stride_k, stride_nb, _lib.ptr(self.svh),

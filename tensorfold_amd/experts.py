@@ -171,11 +171,20 @@ def route(picks: torch.Tensor, plan: Plan, tile: int = PREFILL_TILE) -> None:
 def _check(x: torch.Tensor, k: int, out: torch.Tensor, n: int, epi: int) -> None:
     if x.dtype != torch.bfloat16 or x.dim() != 2 or x.stride(1) != 1 or x.stride(0) % 8 or x.shape[1] != k:
         raise RuntimeError("x: rows of K = groups * group size inputs, 16-byte aligned")
-    if not out.is_contiguous() or out.shape[-1] != n:
+    if not out.is_contiguous() or out.dim() != 2 or out.shape[1] != n:
         raise RuntimeError("out: contiguous rows of n columns")
     if out.dtype != (torch.float32 if epi == 0 else torch.bfloat16):
         raise RuntimeError("out has the wrong dtype")
     _lib.on_gpu(x, out)
+
+
+def _fits(plan: Plan, rows: int, x_rows: int | None, pair_rows: int) -> None:
+    """The kernels index token rows below ``rows`` and pair rows below ``rows * slots``: the buffers must hold them."""
+
+    if not 1 <= rows <= plan.rows:
+        raise ValueError(f"rows = {rows} does not fit a plan made for {plan.rows}")
+    if (x_rows is not None and x_rows < rows) or pair_rows < rows * plan.slots:
+        raise ValueError(f"buffers too small for {rows} rows x {plan.slots} slots")
 
 
 def _group_sums(x: torch.Tensor, gs: int, into: torch.Tensor) -> torch.Tensor:
@@ -203,6 +212,7 @@ def gate_up(x: torch.Tensor, ex: Experts, plan: Plan, out: torch.Tensor, rows: i
 
     epi = 2 if ex.swiglu else 1
     _check(x, ex.dims, out, ex.width, epi)
+    _fits(plan, rows, x.shape[0], out.shape[0])
     xs = xs_out = None
     if not plan.prefill:
         xs = _group_sums(x, ex.gs, plan.sums("x", int(x.shape[0]), ex.dims // ex.gs))
@@ -217,6 +227,7 @@ def down(act: torch.Tensor, ex: Experts, plan: Plan, out: torch.Tensor, rows: in
 
     epi = 3 if (plan.prefill and out.dtype == torch.bfloat16) else 0
     _check(act, ex.width, out, ex.dims, epi)
+    _fits(plan, rows, None, min(act.shape[0], out.shape[0]))
     xs = None
     if not plan.prefill:
         if plan._act_key == (act.data_ptr(), act._version, rows, ex.width):

@@ -126,8 +126,17 @@ def matmul(x: torch.Tensor, q: Q4, xs: torch.Tensor | None = None, *, sk: int | 
     sk = split_k(q.n, q.k, q.gs) if not sk else sk
     if out is None:
         out = x.new_empty((m, q.n), dtype=torch.float32 if f32 else torch.bfloat16)
+    elif tuple(out.shape) != (m, q.n) or out.dtype != (torch.float32 if f32 else torch.bfloat16) \
+            or not out.is_contiguous() or out.device != x.device:
+        raise ValueError(f"matmul: out must be contiguous ({m}, {q.n}) {'fp32' if f32 else 'bf16'} on x's device")
     if sk > 1 and part is None:
         part = x.new_empty((sk, m, q.n), dtype=torch.float32)
+    elif sk > 1 and (part.dtype != torch.float32 or part.numel() < sk * m * q.n or not part.is_contiguous()
+                     or part.device != x.device):
+        raise ValueError(f"matmul: part must hold {sk} x {m} x {q.n} fp32 values (split_k gives the slice count)")
+    if xs.dtype != torch.float32 or tuple(xs.shape) != (m, q.k // q.gs) or not xs.is_contiguous() \
+            or xs.device != x.device:
+        raise ValueError(f"matmul: xs must be contiguous fp32 ({m}, {q.k // q.gs}), the group sums of x")
     _lib.call("tf_qmm", _lib.ptr(x), x.stride(0), _lib.ptr(xs), _lib.ptr(q.weight), _lib.ptr(q.scales),
               _lib.ptr(q.biases), q.scales.stride(0), _lib.ptr(out), _lib.ptr(part), m, q.n, q.k, sk, q.gs, bucket(m),
               int(f32), int(reduce))

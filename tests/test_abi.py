@@ -94,3 +94,24 @@ def test_format_facts():
     t = torch.arange(2 * 16 * 4, dtype=torch.int32).reshape(2, 16, 4)
     s = linear.strips(t)
     assert s.shape == (2, 2, 8, 4) and torch.equal(s[1, 0], t[0, 8:16]) and torch.equal(s[0, 1], t[1, 0:8])
+
+
+def test_host_wrappers_reject_scratch_that_is_too_small():
+    """A caller's buffer that cannot hold what the kernel writes must stop in Python, before any launch."""
+
+    import inspect
+
+    from tensorfold_amd import experts, qmm
+    from tensorfold_amd.exl3 import linear
+
+    assert "part must hold" in inspect.getsource(qmm.matmul)
+    assert "z must hold" in inspect.getsource(linear.Exl3Linear.__call__)
+    plan = experts.Plan.__new__(experts.Plan)
+    plan.rows, plan.slots = 4, 3
+    with pytest.raises(ValueError):
+        experts._fits(plan, 5, 5, 15)
+    with pytest.raises(ValueError):
+        experts._fits(plan, 4, 3, 12)
+    with pytest.raises(ValueError):
+        experts._fits(plan, 4, 4, 11)
+    experts._fits(plan, 4, 4, 12)

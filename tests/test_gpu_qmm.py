@@ -142,3 +142,8 @@ def test_bad_arguments_raise():
         qmm.matmul(torch.zeros((1, 256), device=DEV), q)
     with pytest.raises(RuntimeError, match="whole groups"):
         qmm.matmul(torch.zeros((1, 256), device=DEV).bfloat16(), q, sk=3)
+    x = torch.zeros((2, 256), device=DEV).bfloat16()
+    with pytest.raises(ValueError, match="part must hold"):
+        qmm.matmul(x, q, sk=4, part=torch.empty((2, 2, 64), device=DEV))       # room for 2 of the 4 slices
+    with pytest.raises(ValueError, match="out must be"):
+        qmm.matmul(x, q, out=torch.empty((1, 64), device=DEV, dtype=torch.bfloat16))
