@@ -29,40 +29,45 @@ constexpr float WSCALE = 256.f, WUNSCALE = 1.f / 256.f;     // weights ride the 
 
 typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
 
-// one packed word -> the B operand, inputs in the order (0, 4, 1, 5, 2, 6, 3, 7), each fp16(fma(q, s2, b2))
-__device__ __forceinline__ f16x8_t dequant8(uint32_t w, f16x2_t s2, f16x2_t b2) {
-  // slot p holds input 2 (p % 4) + p / 4: lo bytes are inputs 0, 4, 1, 5; hi bytes are inputs 2, 6, 3, 7
-  const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
-  const f16x2_t q0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 512.f, false);
-  const f16x2_t q1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 512.f, true);
-  const f16x2_t q2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 512.f, false);
-  const f16x2_t q3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 512.f, true);
-  const f16x2_t w0 = __builtin_elementwise_fma(q0, s2, b2), w1 = __builtin_elementwise_fma(q1, s2, b2);
-  const f16x2_t w2 = __builtin_elementwise_fma(q2, s2, b2), w3 = __builtin_elementwise_fma(q3, s2, b2);
-  f16x8_t r;
-  r[0] = w0[0]; r[1] = w0[1]; r[2] = w1[0]; r[3] = w1[1];
-  r[4] = w2[0]; r[5] = w2[1]; r[6] = w3[0]; r[7] = w3[1];
-  return r;
-}
-
-// (256 s, 256 b) of a column as fp16 pairs
-__device__ __forceinline__ void sb_pairs(float s, float b, f16x2_t& s2, f16x2_t& b2) {
-  const _Float16 sh = (_Float16)(s * WSCALE), bh = (_Float16)(b * WSCALE);
-  s2 = (f16x2_t){sh, sh};
-  b2 = (f16x2_t){bh, bh};
-}
-
-// eight consecutive bf16 inputs -> fp16 in the operand order (0, 4, 1, 5, 2, 6, 3, 7), clamped to the fp16 range
+// eight consecutive bf16 inputs -> fp16 in the operand order (0, 4, 1, 5, 2, 6, 3, 7).  The conversion rounds toward
+// zero, which is exact for every bf16 value in fp16's normal range and saturates a finite one beyond it at 65504.
 __device__ __forceinline__ uint4 stage8(uint4 v) {
   const uint32_t d[4] = {v.x, v.y, v.z, v.w};
   float f[8];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    f[2 * i] = fminf(fmaxf(bf16_lo(d[i]), -65504.f), 65504.f);
-    f[2 * i + 1] = fminf(fmaxf(bf16_hi(d[i]), -65504.f), 65504.f);
+    f[2 * i] = bf16_lo(d[i]);
+    f[2 * i + 1] = bf16_hi(d[i]);
   }
   auto pk = [](float a, float b) { return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a, b)); };
   return make_uint4(pk(f[0], f[4]), pk(f[1], f[5]), pk(f[2], f[6]), pk(f[3], f[7]));
+}
+
+// A column's stored (scale | bias << 16) bf16 pair -> (fp16(256 s) | fp16(256 b) << 16).  Adding 8 to both exponents
+// is the multiplication; bf16 -> fp16 is exact in fp16's normal range.
+__device__ __forceinline__ uint32_t sb_half2(uint32_t v) {
+  const uint32_t u = v + 0x04000400u;
+  return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(__uint_as_float(u << 16), __uint_as_float(u & 0xFFFF0000u)));
+}
+
+// q * s + b on two fp16 lanes, s and b being the low and high half of one register
+__device__ __forceinline__ f16x2_t fma_sb(f16x2_t q, uint32_t sb) {
+  f16x2_t r;
+  asm("v_pk_fma_f16 %0, %1, %2, %2 op_sel:[0,0,1] op_sel_hi:[1,0,1]" : "=v"(r) : "v"(q), "v"(sb));
+  return r;
+}
+
+// one packed word -> the B operand, inputs in the order (0, 4, 1, 5, 2, 6, 3, 7), each fp16(fma(q, 256 s, 256 b))
+__device__ __forceinline__ f16x8_t dequant8h(uint32_t w, uint32_t sb) {
+  const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
+  const f16x2_t w0 = fma_sb(__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 512.f, false), sb);
+  const f16x2_t w1 = fma_sb(__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(lo, 512.f, true), sb);
+  const f16x2_t w2 = fma_sb(__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 512.f, false), sb);
+  const f16x2_t w3 = fma_sb(__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(hi, 512.f, true), sb);
+  f16x8_t r;
+  r[0] = w0[0]; r[1] = w0[1]; r[2] = w1[0]; r[3] = w1[1];
+  r[4] = w2[0]; r[5] = w2[1]; r[6] = w3[0]; r[7] = w3[1];
+  return r;
 }
 
 // EPI 0: fp32; 1: bf16 relu(bf16 a)^2; 2: bf16 SwiGLU(matrix 0, matrix 1); 3: bf16
@@ -77,7 +82,7 @@ __device__ __forceinline__ void store_out(void* out, size_t at, float a, float u
 // The shared body.  SRC gives, for the workgroup's item: rows(), src_row(r), dst_row(r); WSRC gives the lane's
 // packed word and its column's scale and bias.
 //   word(g, m, i, t): group g, matrix m, chunk i (32 inputs) of the group, column tile t (16 columns) of the wave
-//   sb(g, m, t, s, b)
+//   sb(g, m, t): that column's stored (scale | bias << 16) pair of group g
 template <int GS, int NM, int EPI, int RT, class WSRC>
 __device__ __forceinline__ void mfma_body(const uint16_t* __restrict__ X, int64_t x_stride, int K, const WSRC& ws,
                                           const int* src_rows, int cnt, void* out, int N, int col0, int wave_cols_ok,
@@ -118,8 +123,8 @@ __device__ __forceinline__ void mfma_body(const uint16_t* __restrict__ X, int64_
   };
 
   uint32_t wcur[NM][CPS][2], wnxt[NM][CPS][2];
-  f16x2_t scur[NM][GPS][2], bcur[NM][GPS][2], snxt[NM][GPS][2], bnxt[NM][GPS][2];
-  auto load_w = [&](int step, uint32_t (&w)[NM][CPS][2], f16x2_t (&s)[NM][GPS][2], f16x2_t (&b)[NM][GPS][2]) {
+  uint32_t scur[NM][GPS][2], snxt[NM][GPS][2];
+  auto load_w = [&](int step, uint32_t (&w)[NM][CPS][2], uint32_t (&s)[NM][GPS][2]) {
 #pragma unroll
     for (int m = 0; m < NM; ++m)
 #pragma unroll
@@ -132,9 +137,7 @@ __device__ __forceinline__ void mfma_body(const uint16_t* __restrict__ X, int64_
 #pragma unroll
         for (int gi = 0; gi < GPS; ++gi) {
           const int k0 = step * KSTEP + GS * gi;
-          float sf = 0.f, bf = 0.f;
-          if (k0 < K) ws.sb(k0 / GS, m, t, sf, bf);
-          sb_pairs(sf, bf, s[m][gi][t], b[m][gi][t]);
+          s[m][gi][t] = k0 < K ? ws.sb(k0 / GS, m, t) : 0u;
         }
       }
   };
@@ -150,14 +153,14 @@ __device__ __forceinline__ void mfma_body(const uint16_t* __restrict__ X, int64_
   const int nt = (cnt + 15) >> 4;              // row tiles in use
   uint4 areg[PPT];
   load_a(0, areg);
-  load_w(0, wcur, scur, bcur);
+  load_w(0, wcur, scur);
   store_a(0, areg);
   __syncthreads();
   for (int step = 0; step < steps; ++step) {
     const bool more = step + 1 < steps;
     if (more) {
       load_a(step + 1, areg);
-      load_w(step + 1, wnxt, snxt, bnxt);
+      load_w(step + 1, wnxt, snxt);
     }
     const unsigned char* abuf = smem + (step & 1) * (ROWS * AROW);
 #pragma unroll
@@ -169,7 +172,7 @@ __device__ __forceinline__ void mfma_body(const uint16_t* __restrict__ X, int64_
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
           const int gi = (32 * i) / GS;
-          bfrag[m][t] = dequant8(wcur[m][i][t], scur[m][gi][t], bcur[m][gi][t]);
+          bfrag[m][t] = dequant8h(wcur[m][i][t], sb_half2(scur[m][gi][t]));
         }
 #pragma unroll
       for (int r = 0; r < RT; ++r) {
@@ -193,10 +196,7 @@ __device__ __forceinline__ void mfma_body(const uint16_t* __restrict__ X, int64_
 #pragma unroll
         for (int gi = 0; gi < GPS; ++gi)
 #pragma unroll
-          for (int t = 0; t < 2; ++t) {
-            scur[m][gi][t] = snxt[m][gi][t];
-            bcur[m][gi][t] = bnxt[m][gi][t];
-          }
+          for (int t = 0; t < 2; ++t) scur[m][gi][t] = snxt[m][gi][t];
       }
     }
     __syncthreads();
@@ -230,10 +230,8 @@ struct ExpertWords {
   __device__ __forceinline__ uint32_t word(int g, int m, int i, int t) const {
     return base[((size_t)g * NM + m) * block_words(GS) + i * 128 + t * 64];
   }
-  __device__ __forceinline__ void sb(int g, int m, int t, float& s, float& b) const {
-    const uint32_t v = sbase[((size_t)g * NM + m) * block_words(GS) + t * 16];
-    s = bf16_lo(v);
-    b = bf16_hi(v);
+  __device__ __forceinline__ uint32_t sb(int g, int m, int t) const {
+    return sbase[((size_t)g * NM + m) * block_words(GS) + t * 16];
   }
 };
 
@@ -264,6 +262,182 @@ __global__ void __launch_bounds__(256)
   mfma_body<GS, NM, EPI, RT>(X, x_stride, KG * GS, ws, src_rows, cnt, out, N, nb * 32, ok, dst_rows, limit, smem);
 }
 
+// ---- routed experts, big items ---------------------------------------------------------------------------------------
+//
+// An item of up to 128 pairs against 256 weight columns (NM = 1: 256 output columns; NM = 2: 128 output columns of
+// gate and of up).  Each of the four waves owns 64 weight columns = four B operands and all eight 16-row tiles, so
+// one dequantized operand feeds eight MFMAs and one LDS read of the activations feeds four: per 32 inputs a wave
+// issues 32 MFMAs against 8 LDS reads and 4 dequantizations.  Weights are requested two steps (128 inputs) ahead
+// into registers, activations one step ahead through registers into LDS (two stages), one barrier a step.  The arithmetic of a row (operand values, MFMA, K order) is the small kernel's, so the bits are too.
+
+constexpr int BIG_ROWS = 128;
+
+// The pipeline for an item of at most 16 * RT rows (RT = 2, 4 or 8): no branch inside a step, so that the LDS reads of
+// the next row tile are in flight under the MFMAs of this one.
+template <int GS, int NM, int EPI, int RT>
+__device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t x_stride,
+                                         const uint32_t* __restrict__ We, const uint32_t (&wp)[4],
+                                         const uint32_t (&sp)[4], const int (&ocol)[4], const bool (&jok)[4],
+                                         int K, const int* src_rows, const int* dst_rows, int cnt,
+                                         void* __restrict__ out, int N, float limit, unsigned char* smem) {
+  constexpr int TJ = 4, CPS = KSTEP / 32, GPS = KSTEP / GS, BW = block_words(GS);
+  constexpr int ROWS = 16 * RT;
+  constexpr int PPT = ROWS * 8 / 256;             // 16-byte pieces of a staged tile a thread (1, 2 or 4)
+  constexpr int STAGE = BIG_ROWS * AROW;
+  constexpr size_t GSTRIDE = (size_t)NM * BW;     // words from one group to the next
+  const int tid = threadIdx.x, lane = tid & 63, c = lane & 15, kq = lane >> 4;
+  const int steps = (K + KSTEP - 1) / KSTEP;
+  auto load_w = [&](int step, uint32_t (&w)[TJ][CPS], uint32_t (&sb)[TJ][GPS]) {
+#pragma unroll
+    for (int j = 0; j < TJ; ++j) {
+#pragma unroll
+      for (int i = 0; i < CPS; ++i) {
+        const int k0 = step * KSTEP + 32 * i;
+        w[j][i] = k0 < K ? We[wp[j] + (uint32_t)((k0 / GS) * GSTRIDE + ((k0 % GS) / 32) * 128)] : 0u;
+      }
+#pragma unroll
+      for (int gi = 0; gi < GPS; ++gi) {
+        const int k0 = step * KSTEP + GS * gi;
+        sb[j][gi] = k0 < K ? We[sp[j] + (uint32_t)((k0 / GS) * GSTRIDE)] : 0u;
+      }
+    }
+  };
+  // this thread's pieces of the activation tile: piece q = (row q / 8, 16 bytes q % 8)
+  const uint16_t* asrc[PPT];
+  bool aok[PPT];
+#pragma unroll
+  for (int j = 0; j < PPT; ++j) {
+    const int q = tid + j * 256, r = q >> 3, ch = q & 7;
+    aok[j] = r < cnt;
+    asrc[j] = X + (size_t)src_rows[aok[j] ? r : 0] * x_stride + ch * 8;
+  }
+  auto load_a = [&](int step, uint4 (&v)[PPT]) {
+#pragma unroll
+    for (int j = 0; j < PPT; ++j) {
+      const int ch = (tid + j * 256) & 7;
+      v[j] = make_uint4(0u, 0u, 0u, 0u);
+      if (aok[j] && step * KSTEP + ch * 8 < K) v[j] = *reinterpret_cast<const uint4*>(asrc[j] + (size_t)step * KSTEP);
+    }
+  };
+  auto store_a = [&](int buf, const uint4 (&v)[PPT]) {
+#pragma unroll
+    for (int j = 0; j < PPT; ++j) {
+      const int q = tid + j * 256;
+      *reinterpret_cast<uint4*>(smem + buf * STAGE + (q >> 3) * AROW + (q & 7) * 16) = stage8(v[j]);
+    }
+  };
+
+  f32x4_t acc[TJ][RT];
+#pragma unroll
+  for (int j = 0; j < TJ; ++j)
+#pragma unroll
+    for (int r = 0; r < RT; ++r) acc[j][r] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+
+  uint32_t wr[2][TJ][CPS], sr[2][TJ][GPS];
+  uint4 ar[PPT];
+  load_w(0, wr[0], sr[0]);
+  load_a(0, ar);
+  if (steps > 1) load_w(1, wr[1], sr[1]);
+  store_a(0, ar);
+  __syncthreads();
+  for (int step0 = 0; step0 < steps; step0 += 2) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int step = step0 + u;
+      if (step < steps) {
+        // stage `u` of LDS holds this step's activations, wr[u] its weights; the next step's activations are
+        // requested now and staged at the end of the step
+        if (step + 1 < steps) load_a(step + 1, ar);
+        const unsigned char* abuf = smem + u * STAGE + c * AROW + kq * 16;
+        f16x8_t a = *reinterpret_cast<const f16x8_t*>(abuf);
+#pragma unroll
+        for (int i = 0; i < CPS; ++i) {
+          f16x8_t bfrag[TJ];
+#pragma unroll
+          for (int j = 0; j < TJ; ++j) bfrag[j] = dequant8h(wr[u][j][i], sb_half2(sr[u][j][(32 * i) / GS]));
+          if (i == CPS - 1 && step + 2 < steps) load_w(step + 2, wr[u], sr[u]);
+#pragma unroll
+          for (int r = 0; r < RT; ++r) {
+            // the next operand (next row tile, or the next chunk's first) is requested before this one is used
+            const int rn = r + 1 < RT ? r + 1 : 0, in = r + 1 < RT ? i : i + 1;
+            f16x8_t an = a;
+            if (in < CPS) an = *reinterpret_cast<const f16x8_t*>(abuf + 16 * rn * AROW + in * 64);
+#pragma unroll
+            for (int j = 0; j < TJ; ++j)
+              acc[j][r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bfrag[j], acc[j][r], 0, 0, 0);
+            a = an;
+          }
+        }
+        if (step + 1 < steps) store_a(1 - u, ar);
+        __syncthreads();
+      }
+    }
+  }
+  // D[row 4 kq + i][column c] of each 16 x 16 tile
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 16 * r + 4 * kq + i;
+      if (row >= cnt) continue;
+      const size_t base = (size_t)dst_rows[row] * N;
+      if constexpr (NM == 2) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          if (jok[j])
+            store_out<EPI>(out, base + ocol[j], acc[j][r][i] * WUNSCALE, acc[j + 2][r][i] * WUNSCALE, limit);
+      } else {
+#pragma unroll
+        for (int j = 0; j < TJ; ++j)
+          if (jok[j]) store_out<EPI>(out, base + ocol[j], acc[j][r][i] * WUNSCALE, 0.f, limit);
+      }
+    }
+  }
+}
+
+template <int GS, int NM, int EPI>
+__global__ void __launch_bounds__(256, 2)
+    experts_prefill_big_kernel(const uint16_t* __restrict__ X, int64_t x_stride, int slots,
+                               const uint32_t* __restrict__ W, int KG, int NB, const int* __restrict__ items,
+                               const int* __restrict__ counts, const int* __restrict__ members,
+                               void* __restrict__ out, int N, float limit) {
+  constexpr int BW = block_words(GS);
+  constexpr int NBW = NM == 2 ? 4 : 8;            // 32-column blocks a workgroup
+  extern __shared__ __align__(16) unsigned char smem[];
+  __shared__ int src_rows[BIG_ROWS], dst_rows[BIG_ROWS];
+  const int nbt = (NB + NBW - 1) / NBW;
+  const int it = blockIdx.x / nbt, cbt = blockIdx.x - it * nbt;
+  if (it >= counts[0]) return;
+  const int e = items[3 * it], first = items[3 * it + 1], cnt = min(items[3 * it + 2], BIG_ROWS);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, kq = lane >> 4;
+  if (tid < BIG_ROWS) {
+    const int p = members[first + (tid < cnt ? tid : 0)];
+    dst_rows[tid] = p;
+    src_rows[tid] = slots ? p / slots : p;
+  }
+  __syncthreads();
+  // the wave's four B operands: (matrix, 32-column block, 16-column half)
+  const uint32_t* We = W + (size_t)e * NB * KG * (size_t)(NM * BW);      // the expert's matrices (wave-uniform)
+  uint32_t wp[4], sp[4];              // word offsets inside the expert: always below 2^32
+  int ocol[4];
+  bool jok[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int m = NM == 2 ? j >> 1 : 0;
+    const int nb = NM == 2 ? cbt * 4 + wave : cbt * 8 + wave * 2 + (j >> 1);
+    const int toff = (j & 1) * 16;
+    jok[j] = nb < NB;
+    const uint32_t blk = (uint32_t)((jok[j] ? nb : NB - 1) * KG) * (uint32_t)(NM * BW) + m * BW;
+    wp[j] = blk + (toff + c) * 4 + kq;
+    sp[j] = blk + 32 * GS / 8 + toff + c;
+    ocol[j] = nb * 32 + toff + c;
+  }
+  const int K = KG * GS;
+  if (cnt <= 32) big_body<GS, NM, EPI, 2>(X, x_stride, We, wp, sp, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
+  else if (cnt <= 64) big_body<GS, NM, EPI, 4>(X, x_stride, We, wp, sp, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
+  else big_body<GS, NM, EPI, 8>(X, x_stride, We, wp, sp, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
+}
+
 // ---- dense prompt matmul --------------------------------------------------------------------------------------------
 
 template <int GS>
@@ -276,9 +450,8 @@ struct LaneWords {
   __device__ __forceinline__ uint32_t word(int g, int, int i, int t) const {
     return base[((size_t)g * (GS / 32) + i) * 256 + t * 64];
   }
-  __device__ __forceinline__ void sb(int g, int, int t, float& s, float& b) const {
-    s = bf16_f32(S[(size_t)g * stride + t * 16]);
-    b = bf16_f32(B[(size_t)g * stride + t * 16]);
+  __device__ __forceinline__ uint32_t sb(int g, int, int t) const {
+    return (uint32_t)S[(size_t)g * stride + t * 16] | ((uint32_t)B[(size_t)g * stride + t * 16] << 16);
   }
 };
 
@@ -320,15 +493,16 @@ int launch_experts_prefill(int tile, const uint16_t* x, int64_t x_stride, int sl
   if (grid < 1) return 0;
   TF_REQUIRE(grid <= 0x7FFFFFFF, "experts: %lld workgroups exceed the grid limit", (long long)grid);
   const dim3 g((unsigned)grid), b(256);
-  if (tile == 16)
+  if (tile == 16) {
     experts_prefill_kernel<GS, NM, EPI, 1><<<g, b, stage_bytes<1>(), s>>>(x, x_stride, slots, w, kg, nb, items, counts,
                                                                          members, out, n, limit);
-  else if (tile == 64)
-    experts_prefill_kernel<GS, NM, EPI, 4><<<g, b, stage_bytes<4>(), s>>>(x, x_stride, slots, w, kg, nb, items, counts,
-                                                                         members, out, n, limit);
-  else
-    experts_prefill_kernel<GS, NM, EPI, 8><<<g, b, stage_bytes<8>(), s>>>(x, x_stride, slots, w, kg, nb, items, counts,
-                                                                         members, out, n, limit);
+  } else {
+    constexpr int NBW = NM == 2 ? 4 : 8;
+    const int64_t big = max_items * ((nb + NBW - 1) / NBW);
+    TF_REQUIRE(big <= 0x7FFFFFFF, "experts: %lld workgroups exceed the grid limit", (long long)big);
+    experts_prefill_big_kernel<GS, NM, EPI><<<dim3((unsigned)big), b, 2 * BIG_ROWS * AROW, s>>>(
+        x, x_stride, slots, w, kg, nb, items, counts, members, out, n, limit);
+  }
   TF_LAUNCH_OK("tf_experts_prefill");
   return 0;
 }
