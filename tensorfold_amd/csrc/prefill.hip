@@ -50,11 +50,11 @@ __device__ __forceinline__ uint32_t sb_half2(uint32_t v) {
   return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(__uint_as_float(u << 16), __uint_as_float(u & 0xFFFF0000u)));
 }
 
-// q * s + b on two fp16 lanes, s and b being the low and high half of one register
+// q * s + b on two fp16 lanes, s and b being the low and high half of one register (the splats fold into the
+// packed instruction's operand selects)
 __device__ __forceinline__ f16x2_t fma_sb(f16x2_t q, uint32_t sb) {
-  f16x2_t r;
-  asm("v_pk_fma_f16 %0, %1, %2, %2 op_sel:[0,0,1] op_sel_hi:[1,0,1]" : "=v"(r) : "v"(q), "v"(sb));
-  return r;
+  const f16x2_t v = __builtin_bit_cast(f16x2_t, sb);
+  return __builtin_elementwise_fma(q, __builtin_shufflevector(v, v, 0, 0), __builtin_shufflevector(v, v, 1, 1));
 }
 
 // one packed word -> the B operand, inputs in the order (0, 4, 1, 5, 2, 6, 3, 7), each fp16(fma(q, 256 s, 256 b))
@@ -264,16 +264,19 @@ __global__ void __launch_bounds__(256)
 
 // ---- routed experts, big items ---------------------------------------------------------------------------------------
 //
-// An item of up to 128 pairs against 256 weight columns (NM = 1: 256 output columns; NM = 2: 128 output columns of
-// gate and of up).  Each of the four waves owns 64 weight columns = four B operands and all eight 16-row tiles, so
+// An item of up to 128 pairs against 512 weight columns (NM = 1: 512 output columns; NM = 2: 256 output columns of
+// gate and of up).  Each of the eight waves owns 64 weight columns = four B operands and all eight 16-row tiles, so
 // one dequantized operand feeds eight MFMAs and one LDS read of the activations feeds four: per 32 inputs a wave
 // issues 32 MFMAs against 8 LDS reads and 4 dequantizations.  Weights are requested two steps (128 inputs) ahead
 // into registers, activations one step ahead through registers into LDS (two stages), one barrier a step.  The arithmetic of a row (operand values, MFMA, K order) is the small kernel's, so the bits are too.
 
 constexpr int BIG_ROWS = 128;
+constexpr int BIG_WAVES = 8;
+constexpr int BIG_THREADS = BIG_WAVES * 64;
 
-// The pipeline for an item of at most 16 * RT rows (RT = 2, 4 or 8): no branch inside a step, so that the LDS reads of
-// the next row tile are in flight under the MFMAs of this one.
+// The pipeline for an item of at most 16 * RT rows (RT = 2, 4 or 8).  K is a multiple of KSTEP and nothing inside a
+// step is conditional (prefetches past the end re-read the last step, rows past the item read its first row), so the
+// compiler is free to keep the LDS reads of the next row tile in flight under the MFMAs of this one.
 template <int GS, int NM, int EPI, int RT>
 __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t x_stride,
                                          const uint32_t* __restrict__ We, const uint32_t (&wp)[4],
@@ -282,48 +285,42 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
                                          void* __restrict__ out, int N, float limit, unsigned char* smem) {
   constexpr int TJ = 4, CPS = KSTEP / 32, GPS = KSTEP / GS, BW = block_words(GS);
   constexpr int ROWS = 16 * RT;
-  constexpr int PPT = ROWS * 8 / 256;             // 16-byte pieces of a staged tile a thread (1, 2 or 4)
+  constexpr int PIECES = ROWS * 8;                // 16-byte pieces of a staged tile
+  constexpr int PPT = (PIECES + BIG_THREADS - 1) / BIG_THREADS;
   constexpr int STAGE = BIG_ROWS * AROW;
-  constexpr size_t GSTRIDE = (size_t)NM * BW;     // words from one group to the next
+  constexpr uint32_t GSTRIDE = NM * BW;           // words from one group to the next
+  constexpr uint32_t SSTRIDE = GPS * GSTRIDE;     // words from one step to the next
   const int tid = threadIdx.x, lane = tid & 63, c = lane & 15, kq = lane >> 4;
-  const int steps = (K + KSTEP - 1) / KSTEP;
+  const int steps = K / KSTEP;
   auto load_w = [&](int step, uint32_t (&w)[TJ][CPS], uint32_t (&sb)[TJ][GPS]) {
+    const uint32_t* base = We + (size_t)step * SSTRIDE;           // wave-uniform
 #pragma unroll
     for (int j = 0; j < TJ; ++j) {
 #pragma unroll
-      for (int i = 0; i < CPS; ++i) {
-        const int k0 = step * KSTEP + 32 * i;
-        w[j][i] = k0 < K ? We[wp[j] + (uint32_t)((k0 / GS) * GSTRIDE + ((k0 % GS) / 32) * 128)] : 0u;
-      }
+      for (int i = 0; i < CPS; ++i) w[j][i] = base[wp[j] + ((32 * i) / GS) * GSTRIDE + (((32 * i) % GS) / 32) * 128];
 #pragma unroll
-      for (int gi = 0; gi < GPS; ++gi) {
-        const int k0 = step * KSTEP + GS * gi;
-        sb[j][gi] = k0 < K ? We[sp[j] + (uint32_t)((k0 / GS) * GSTRIDE)] : 0u;
-      }
+      for (int gi = 0; gi < GPS; ++gi) sb[j][gi] = base[sp[j] + gi * GSTRIDE];
     }
   };
   // this thread's pieces of the activation tile: piece q = (row q / 8, 16 bytes q % 8)
   const uint16_t* asrc[PPT];
-  bool aok[PPT];
 #pragma unroll
   for (int j = 0; j < PPT; ++j) {
-    const int q = tid + j * 256, r = q >> 3, ch = q & 7;
-    aok[j] = r < cnt;
-    asrc[j] = X + (size_t)src_rows[aok[j] ? r : 0] * x_stride + ch * 8;
+    const int q = tid + j * BIG_THREADS, r = q >> 3, ch = q & 7;
+    asrc[j] = X + (size_t)src_rows[r < cnt ? r : 0] * x_stride + ch * 8;
   }
   auto load_a = [&](int step, uint4 (&v)[PPT]) {
 #pragma unroll
-    for (int j = 0; j < PPT; ++j) {
-      const int ch = (tid + j * 256) & 7;
-      v[j] = make_uint4(0u, 0u, 0u, 0u);
-      if (aok[j] && step * KSTEP + ch * 8 < K) v[j] = *reinterpret_cast<const uint4*>(asrc[j] + (size_t)step * KSTEP);
-    }
+    for (int j = 0; j < PPT; ++j)
+      if (PIECES % BIG_THREADS == 0 || tid + j * BIG_THREADS < PIECES)
+        v[j] = *reinterpret_cast<const uint4*>(asrc[j] + (size_t)step * KSTEP);
   };
   auto store_a = [&](int buf, const uint4 (&v)[PPT]) {
 #pragma unroll
     for (int j = 0; j < PPT; ++j) {
-      const int q = tid + j * 256;
-      *reinterpret_cast<uint4*>(smem + buf * STAGE + (q >> 3) * AROW + (q & 7) * 16) = stage8(v[j]);
+      const int q = tid + j * BIG_THREADS;
+      if (PIECES % BIG_THREADS == 0 || q < PIECES)
+        *reinterpret_cast<uint4*>(smem + buf * STAGE + (q >> 3) * AROW + (q & 7) * 16) = stage8(v[j]);
     }
   };
 
@@ -335,27 +332,29 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
 
   uint32_t wr[2][TJ][CPS], sr[2][TJ][GPS];
   uint4 ar[PPT];
+  const int last = steps - 1;
   load_w(0, wr[0], sr[0]);
   load_a(0, ar);
-  if (steps > 1) load_w(1, wr[1], sr[1]);
+  load_w(min(1, last), wr[1], sr[1]);
   store_a(0, ar);
+  // Software pipeline: the operands of the NEXT 32 inputs are dequantized under the MFMAs of these 32.
+  f16x8_t bcur[TJ];
+#pragma unroll
+  for (int j = 0; j < TJ; ++j) bcur[j] = dequant8h(wr[0][j][0], sb_half2(sr[0][j][0]));
   __syncthreads();
   for (int step0 = 0; step0 < steps; step0 += 2) {
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int step = step0 + u;
       if (step < steps) {
-        // stage `u` of LDS holds this step's activations, wr[u] its weights; the next step's activations are
-        // requested now and staged at the end of the step
-        if (step + 1 < steps) load_a(step + 1, ar);
+        // stage `u` of LDS holds this step's activations, wr[u] its weights (wr[1 - u] the next step's); the next
+        // step's activations are requested now and staged at the end of the step
+        load_a(min(step + 1, last), ar);
         const unsigned char* abuf = smem + u * STAGE + c * AROW + kq * 16;
         f16x8_t a = *reinterpret_cast<const f16x8_t*>(abuf);
 #pragma unroll
         for (int i = 0; i < CPS; ++i) {
-          f16x8_t bfrag[TJ];
-#pragma unroll
-          for (int j = 0; j < TJ; ++j) bfrag[j] = dequant8h(wr[u][j][i], sb_half2(sr[u][j][(32 * i) / GS]));
-          if (i == CPS - 1 && step + 2 < steps) load_w(step + 2, wr[u], sr[u]);
+          f16x8_t bnext[TJ];
 #pragma unroll
           for (int r = 0; r < RT; ++r) {
             // the next operand (next row tile, or the next chunk's first) is requested before this one is used
@@ -364,11 +363,26 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
             if (in < CPS) an = *reinterpret_cast<const f16x8_t*>(abuf + 16 * rn * AROW + in * 64);
 #pragma unroll
             for (int j = 0; j < TJ; ++j)
-              acc[j][r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bfrag[j], acc[j][r], 0, 0, 0);
+              acc[j][r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bcur[j], acc[j][r], 0, 0, 0);
             a = an;
+            // a share of the next chunk's dequantization rides along with each row tile
+            constexpr int JPR = (TJ + RT - 1) / RT;          // operands a row tile (2, 1, 1 for RT = 2, 4, 8)
+#pragma unroll
+            for (int jj = 0; jj < JPR; ++jj) {
+              const int j = r * JPR + jj;
+              if (j < TJ) {
+                if (i + 1 < CPS) bnext[j] = dequant8h(wr[u][j][i + 1], sb_half2(sr[u][j][(32 * (i + 1)) / GS]));
+                else bnext[j] = dequant8h(wr[1 - u][j][0], sb_half2(sr[1 - u][j][0]));
+              }
+            }
+            if (i + 2 == CPS && r * JPR + JPR >= TJ && (r - 1) * JPR + JPR < TJ)
+              load_w(min(step + 2, last), wr[u], sr[u]);     // wr[u] has just been used for the last time
           }
+          if (CPS == 1) load_w(min(step + 2, last), wr[u], sr[u]);
+#pragma unroll
+          for (int j = 0; j < TJ; ++j) bcur[j] = bnext[j];
         }
-        if (step + 1 < steps) store_a(1 - u, ar);
+        store_a(1 - u, ar);
         __syncthreads();
       }
     }
@@ -395,14 +409,17 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
   }
 }
 
+// 32-column blocks a workgroup of the big kernel covers
+constexpr int big_blocks(int nm) { return nm == 2 ? BIG_WAVES : 2 * BIG_WAVES; }
+
 template <int GS, int NM, int EPI>
-__global__ void __launch_bounds__(256, 2)
+__global__ void __launch_bounds__(BIG_THREADS, 1)
     experts_prefill_big_kernel(const uint16_t* __restrict__ X, int64_t x_stride, int slots,
                                const uint32_t* __restrict__ W, int KG, int NB, const int* __restrict__ items,
                                const int* __restrict__ counts, const int* __restrict__ members,
                                void* __restrict__ out, int N, float limit) {
   constexpr int BW = block_words(GS);
-  constexpr int NBW = NM == 2 ? 4 : 8;            // 32-column blocks a workgroup
+  constexpr int NBW = big_blocks(NM);
   extern __shared__ __align__(16) unsigned char smem[];
   __shared__ int src_rows[BIG_ROWS], dst_rows[BIG_ROWS];
   const int nbt = (NB + NBW - 1) / NBW;
@@ -424,7 +441,7 @@ __global__ void __launch_bounds__(256, 2)
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int m = NM == 2 ? j >> 1 : 0;
-    const int nb = NM == 2 ? cbt * 4 + wave : cbt * 8 + wave * 2 + (j >> 1);
+    const int nb = NM == 2 ? cbt * NBW + wave : cbt * NBW + wave * 2 + (j >> 1);
     const int toff = (j & 1) * 16;
     jok[j] = nb < NB;
     const uint32_t blk = (uint32_t)((jok[j] ? nb : NB - 1) * KG) * (uint32_t)(NM * BW) + m * BW;
@@ -496,11 +513,19 @@ int launch_experts_prefill(int tile, const uint16_t* x, int64_t x_stride, int sl
   if (tile == 16) {
     experts_prefill_kernel<GS, NM, EPI, 1><<<g, b, stage_bytes<1>(), s>>>(x, x_stride, slots, w, kg, nb, items, counts,
                                                                          members, out, n, limit);
+  } else if ((kg * GS) % KSTEP) {
+    // a K that is not whole steps of 64 (odd group counts at g32): the small kernel's tail handling
+    if (tile == 64)
+      experts_prefill_kernel<GS, NM, EPI, 4><<<g, b, stage_bytes<4>(), s>>>(x, x_stride, slots, w, kg, nb, items,
+                                                                           counts, members, out, n, limit);
+    else
+      experts_prefill_kernel<GS, NM, EPI, 8><<<g, b, stage_bytes<8>(), s>>>(x, x_stride, slots, w, kg, nb, items,
+                                                                           counts, members, out, n, limit);
   } else {
-    constexpr int NBW = NM == 2 ? 4 : 8;
+    constexpr int NBW = big_blocks(NM);
     const int64_t big = max_items * ((nb + NBW - 1) / NBW);
     TF_REQUIRE(big <= 0x7FFFFFFF, "experts: %lld workgroups exceed the grid limit", (long long)big);
-    experts_prefill_big_kernel<GS, NM, EPI><<<dim3((unsigned)big), b, 2 * BIG_ROWS * AROW, s>>>(
+    experts_prefill_big_kernel<GS, NM, EPI><<<dim3((unsigned)big), BIG_THREADS, 2 * BIG_ROWS * AROW, s>>>(
         x, x_stride, slots, w, kg, nb, items, counts, members, out, n, limit);
   }
   TF_LAUNCH_OK("tf_experts_prefill");

@@ -18,7 +18,7 @@ from . import _lib
 
 COLS = 32             # columns of one weight block
 TILE = 16             # largest decode item, in pairs
-PREFILL_TILE = 64     # default prompt item; the MFMA kernel also takes 16 and 128
+PREFILL_TILE = 128    # default prompt item; the MFMA kernels also take 16 and 64
 SMALL = 1024          # a plan up to this many pairs is sorted by one workgroup
 _GROUPS = (32, 64)
 
