@@ -72,18 +72,30 @@ class Layer:
         moe.select(self.logits[i % POOL], self.buf, SHAPE.top_k, SHAPE.experts)
 
     def up(self, i: int, buf=None) -> None:
+        """The routing + up projection launch alone."""
+
         ex, buf = self.tables[i % len(self.tables)], buf or self.buf
-        experts.gate_up(self.x[i % 4], ex, buf.plan, buf.act.view(-1, ex.width), self.tokens)
+        f, x, l = buf.fused(SHAPE.gs), self.x[i % 4], self.logits[getattr(buf, "draw", i % POOL)]
+        items = experts.max_items(self.tokens * buf.slots, SHAPE.experts, experts.TILE)
+        _lib.call("tf_moe_route_up", _lib.ptr(l), l.stride(0), self.tokens, SHAPE.experts, SHAPE.top_k, 0, ex.gs,
+                  int(ex.swiglu), _lib.ptr(x), x.stride(0), _lib.ptr(ex.up), ex.dims, ex.width, _lib.ptr(buf.pick),
+                  _lib.ptr(buf.wts), _lib.ptr(buf.plan.members), _lib.ptr(buf.plan.items), _lib.ptr(buf.plan.counts),
+                  _lib.ptr(f["desc"]), _lib.ptr(buf.act), _lib.ptr(f["xs_act"]), ex.limit, items)
 
     def down(self, i: int, buf=None) -> None:
         ex, buf = self.tables[i % len(self.tables)], buf or self.buf
-        experts.down(buf.act.view(-1, ex.width), ex, buf.plan, buf.y.view(-1, ex.dims), self.tokens)
+        f = buf.fused(SHAPE.gs)
+        items = experts.max_items(self.tokens * buf.slots, SHAPE.experts, experts.TILE)
+        _lib.call("tf_experts_run_desc", ex.gs, 0, _lib.ptr(buf.act), ex.width, 0, _lib.ptr(ex.down),
+                  ex.width // ex.gs, ex.dims // experts.COLS, _lib.ptr(f["desc"]), _lib.ptr(buf.plan.counts),
+                  _lib.ptr(buf.y), ex.dims, 0.0, items, _lib.ptr(f["xs_act"]), None)
 
     def route_plans(self) -> float:
         """Route every pre-built plan on its own logits; returns the mean number of distinct experts a plan holds."""
 
         for j, b in enumerate(self.plans):
-            moe.decode(self.x[j % 4], self.logits[(7 * j + 3) % POOL], self.tables[j % len(self.tables)], b,
+            b.draw = (7 * j + 3) % POOL          # the routing draw this buffer keeps for the kernel timings
+            moe.decode(self.x[j % 4], self.logits[b.draw], self.tables[j % len(self.tables)], b,
                        SHAPE.top_k, SHAPE.experts)      # routes the plan and fills its descriptors and activations
         torch.cuda.synchronize()
         return float(np.mean([int(b.plan.counts[1]) for b in self.plans]))
@@ -92,17 +104,9 @@ class Layer:
         moe.combine(self.buf.y, self.buf.wts, self.out)
 
     def step(self, i: int) -> None:
-        """One layer pass the way ``moe.run`` issues it: routing, up, down, combine as separate launches, or (with
-        ``moe.FUSED_DECODE``) the routing launch and the fused experts launch."""
+        """One layer pass the way ``moe.run`` issues it: the routing launch, then up, down and combine launches, or
+        (with ``moe.FUSED_DECODE``) the one fused experts launch."""
 
-        if moe.FUSED_DECODE:
-            return self.step_fused(i)
-        self.route(i)
-        self.up(i)
-        self.down(i)
-        self.combine()
-
-    def step_fused(self, i: int) -> None:
         moe.decode(self.x[i % 4], self.logits[i % POOL], self.tables[i % len(self.tables)], self.buf, SHAPE.top_k,
                    SHAPE.experts, self.out)
 
@@ -154,7 +158,16 @@ def run_batch(tokens: int, tables, steps: int, warmup: int, dev: str) -> dict:
         return (time.perf_counter() - t0) / steps * 1e6
 
     layer_us = graph_us(layer.step)
-    fused_layer_us = layer_us if moe.FUSED_DECODE else graph_us(layer.step_fused)
+
+    def other_path(i: int) -> None:
+        moe.FUSED_DECODE = not moe.FUSED_DECODE
+        try:
+            layer.step(i)
+        finally:
+            moe.FUSED_DECODE = not moe.FUSED_DECODE
+
+    other_us = graph_us(other_path)
+    fused_layer_us, split_layer_us = (layer_us, other_us) if moe.FUSED_DECODE else (other_us, layer_us)
 
     # the two expert kernels by themselves: HIP events around back-to-back launches on the launch stream
     def kernel_us(fn) -> float:
@@ -187,7 +200,7 @@ def run_batch(tokens: int, tables, steps: int, warmup: int, dev: str) -> dict:
     return {
         "tokens": tokens, "layer_us": layer_us, "us_per_token": layer_us / tokens, "unique_experts": mean_u,
         "layer_bytes": algo, "layer_gbs": algo / layer_us * 1e-3, "layer_frac": algo / layer_us * 1e-3 / HBM_PEAK_GBS,
-        "fused_layer_us": fused_layer_us, "up_kernel_us": up_us, "down_kernel_us": down_us, "fused_kernel_us": fused_us,
+        "fused_layer_us": fused_layer_us, "split_layer_us": split_layer_us, "up_kernel_us": up_us, "down_kernel_us": down_us, "fused_kernel_us": fused_us,
         "fused_gbs": (u0 * 2 * half + act_bytes) / fused_us * 1e-3,
         "up_gbs": (u0 * half + act_bytes / 2) / up_us * 1e-3, "down_gbs": (u0 * half + act_bytes / 2) / down_us * 1e-3,
         "kernel_unique_experts": u0, "kernel_bytes": u0 * half,
@@ -265,7 +278,7 @@ def main() -> int:
     else:
         which = "up" if head["up_kernel_us"] >= head["down_kernel_us"] else "down"
         dom_us, dom_bytes = head[f"{which}_kernel_us"], head["kernel_bytes"]
-        dom = f"expert_kernel ({which} projection"
+        dom = ("route_up_kernel (routing + up projection" if which == "up" else "expert_desc_kernel (down projection")
         traffic = MEASURED_TRAFFIC.get((which, args.tokens))
     achieved = dom_bytes / dom_us * 1e-3
     line = {

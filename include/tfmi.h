@@ -88,6 +88,12 @@ int tf_experts_plan(const int32_t* picks, int64_t pairs, int experts, int tile, 
 int tf_experts_run(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg, int nb,
                    const int32_t* items, const int32_t* counts, const int32_t* members, void* out, int n, float limit,
                    int64_t max_units, const float* xs, float* xs_out, tf_stream_t stream);
+/* tf_experts_run with the items given as descriptors (int32 [max_items, 20]: expert, count, first member, 0, the
+ * item's pairs[16]) as tf_moe_route_decode writes them; xs is required.  Same bits as tf_experts_run on the same
+ * plan.  Same reference counterpart (experts.cpp:43-48 `run`); the descriptor form has none. */
+int tf_experts_run_desc(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg,
+                        int nb, const int32_t* desc, const int32_t* counts, void* out, int n, float limit,
+                        int64_t max_items, const float* xs, float* xs_out, tf_stream_t stream);
 /* Prompt form on f16 MFMA, each weight rounded once as in tf_qmm_prefill; epi 3: bf16 out.  `tile` is the plan's
  * item size (16, 64 or 128).  Replaces experts.cpp:50-55 `prefill`. */
 int tf_experts_prefill(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg,
@@ -109,6 +115,16 @@ int tf_moe_topk(const float* logits, int64_t ldl, int rows, int experts, int top
 int tf_moe_combine(const void* y, int y_bf16, const float* wts, uint16_t* out, int rows, int slots, int d,
                    tf_stream_t stream);
 
+/* Routing and the up projection of the decode layer in ONE launch, for rows * (top_k + shared) <= 1024: workgroup 0
+ * writes what tf_moe_topk and tf_experts_plan (tile 16) would (pick, wts, members, items, counts) plus the item
+ * descriptors int32 [max_items, 20] that tf_experts_run_desc reads; every other workgroup finds its own item from the
+ * logits and runs the up unit of tf_experts_run (epilogue relu^2, or SwiGLU when swiglu != 0): act bf16 [pairs, ni] and
+ * its group sums xs_act fp32 [pairs, ni / gs].  Same bits as the separate calls.  No counterpart in the reference
+ * (moe.py:88-128 issues them one by one). */
+int tf_moe_route_up(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared, int gs, int swiglu,
+                    const uint16_t* x, int64_t x_stride, const uint32_t* up, int d, int ni, int32_t* pick, float* wts,
+                    int32_t* members, int32_t* items, int32_t* counts, int32_t* desc, uint16_t* act, float* xs_act,
+                    float limit, int max_items, tf_stream_t stream);
 /* The decode layer's routing in one launch, for rows * (top_k + shared) <= 1024: tf_moe_topk, tf_experts_plan (tile
  * 16) and tf_group_sums of x, plus desc int32 [max items, 20] = {expert, count, first, 0, pairs[16]} an item and the
  * zeroing of `zero` (n_zero ints: the counters of tf_moe_decode_experts).  No counterpart in the reference, which

@@ -42,6 +42,30 @@ __global__ void __launch_bounds__(WAVES * 64)
                                        xs_out, lds, none);
 }
 
+// The same unit taken from an item descriptor (int32 [20]: expert, count, first member, 0, pairs[16]) as
+// tf_moe_route_decode writes them: one read instead of the items -> members chain.
+constexpr int DESC = 20;
+
+template <int GS, int NM, int EPI, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64)
+    expert_desc_kernel(const uint16_t* __restrict__ X, int64_t x_stride, int slots, const uint32_t* __restrict__ W,
+                       int KG, int NB, const int* __restrict__ desc, const int* __restrict__ counts,
+                       void* __restrict__ out, int N, float limit, const float* __restrict__ xs_in,
+                       float* __restrict__ xs_out) {
+  extern __shared__ float lds[];
+  __shared__ int pairs[16];
+  const int NB2 = (NB + 1) >> 1;
+  const int it = blockIdx.x / NB2, cb2 = blockIdx.x - it * NB2;
+  if (it >= counts[0]) return;
+  const int* d = desc + (size_t)it * DESC;
+  const int e = d[0], cnt = d[1];
+  if (threadIdx.x < 16) pairs[threadIdx.x] = d[4 + threadIdx.x];
+  __syncthreads();
+  NoHook none;
+  expert_unit<GS, NM, EPI, WAVES, true, 0>(X, x_stride, slots, W, KG, NB, e, cnt, pairs, cb2, out, N, limit, xs_in,
+                                           xs_out, lds, none);
+}
+
 // ---- dense lane matmul ---------------------------------------------------------------------------------------------
 
 struct NoFlush {
@@ -187,10 +211,56 @@ int launch_experts(const uint16_t* x, int64_t x_stride, int slots, const uint32_
   return 0;
 }
 
+template <int GS, int NM, int EPI>
+int launch_experts_desc(const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg, int nb,
+                        const int* desc, const int* counts, void* out, int n, float limit, int64_t max_items,
+                        const float* xs_in, float* xs_out, hipStream_t stream) {
+  const int nb2 = (nb + 1) / 2;
+  const int64_t grid = max_items * nb2;
+  if (grid < 1) return 0;
+  TF_REQUIRE(grid <= 0x7FFFFFFF, "experts: %lld workgroups exceed the grid limit", (long long)grid);
+  const size_t smem = sizeof(float) * expert_lds_floats(NM, kg, true);
+  const dim3 g((unsigned)grid);
+#define TF_GO(W_)                                                                                                 \
+  expert_desc_kernel<GS, NM, EPI, W_><<<g, W_ * 64, smem, stream>>>(x, x_stride, slots, w, kg, nb, desc, counts, out, n, \
+                                                                    limit, xs_in, xs_out)
+  switch (expert_waves(grid)) {
+    case 16: TF_GO(16); break;
+    case 8: TF_GO(8); break;
+    default: TF_GO(4);
+  }
+#undef TF_GO
+  TF_LAUNCH_OK("tf_experts_run_desc");
+  return 0;
+}
+
 }  // namespace
 }  // namespace tf
 
 using namespace tf;
+
+extern "C" int tf_experts_run_desc(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w,
+                                   int kg, int nb, const int32_t* desc, const int32_t* counts, void* out, int n,
+                                   float limit, int64_t max_items, const float* xs, float* xs_out,
+                                   tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(gs == 32 || gs == 64, "experts: groups of 32 or 64 inputs, not %d", gs);
+  TF_REQUIRE(x && w && desc && counts && out && xs, "experts: null pointer argument");
+  TF_REQUIRE(!xs_out || (epi != 0 && n % gs == 0), "experts: xs_out goes with an activation epilogue and whole groups");
+  TF_REQUIRE(kg >= 1 && nb >= 1 && n == nb * 32, "experts: n (%d) must be the column blocks (%d) times 32", n, nb);
+  TF_REQUIRE(aligned16(x) && x_stride % 8 == 0, "x: rows of K = groups * group size inputs, 16-byte aligned");
+  TF_REQUIRE(aligned16(w), "w must be 16-byte aligned");
+  TF_REQUIRE(slots >= 0 && max_items >= 0, "experts: negative slots or max_items");
+  hipStream_t s = as_stream(stream);
+#define TF_RUN(GS_, NM_, EPI_)            \
+  if (gs == GS_ && epi == EPI_)           \
+    return launch_experts_desc<GS_, NM_, EPI_>(x, x_stride, slots, w, kg, nb, desc, counts, out, n, limit, max_items, \
+                                               xs, xs_out, s);
+  TF_RUN(32, 1, 0) TF_RUN(32, 1, 1) TF_RUN(32, 2, 2) TF_RUN(64, 1, 0) TF_RUN(64, 1, 1) TF_RUN(64, 2, 2)
+#undef TF_RUN
+  set_error("experts: no kernel for group %d and epilogue %d", gs, epi);
+  return 1;
+}
 
 extern "C" int tf_experts_run(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w,
                               int kg, int nb, const int32_t* items, const int32_t* counts, const int32_t* members,

@@ -16,11 +16,14 @@
 // one after the other.
 
 #include "gemv.h"
+#include "routing.h"
 
 namespace tf {
 namespace {
 
 constexpr int DESC = 20;      // int32 an item descriptor: expert, count, first, 0, pairs[16]
+
+int fused_waves(int64_t grid) { return grid < 768 ? 16 : grid < 1536 ? 8 : 4; }
 
 struct WaitItem {
   const int* flag;
@@ -100,7 +103,133 @@ __global__ void __launch_bounds__(WAVES * 64)
   }
 }
 
-int fused_waves(int64_t grid) { return grid < 768 ? 16 : grid < 1536 ? 8 : 4; }
+
+// ---- routing and the up projection in one launch -------------------------------------------------------------------
+//
+// Workgroup 0 writes the routing's outputs (picks, weights, members, items, counts, item descriptors) for the kernels
+// that follow; every other workgroup repeats the cheap part for itself (top-k of every row, a histogram, one scan)
+// to learn which expert and which pairs its item holds, then runs the up unit.  The routing's launch and its trip
+// through memory are gone; the price is about a microsecond of arithmetic at the head of each workgroup.
+
+template <int GS, int NM, int EPI, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64)
+    route_up_kernel(const float* __restrict__ L, int64_t ldl, int R, int NE, int TOPK, int shared,
+                    const uint16_t* __restrict__ X, int64_t x_stride, const uint32_t* __restrict__ Wup, int D, int NI,
+                    int* __restrict__ pick, float* __restrict__ wts, int* __restrict__ members,
+                    int* __restrict__ items, int* __restrict__ counts, int* __restrict__ desc,
+                    uint16_t* __restrict__ act, float* __restrict__ xs_act, float limit) {
+  extern __shared__ float lds[];
+  __shared__ int pk[PLAN_THREADS];
+  __shared__ ItemLds item;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, threads = WAVES * 64;
+  const int slots = TOPK + (shared ? 1 : 0), P = R * slots, E = NE + (shared ? 1 : 0);
+  const bool writer = blockIdx.x == 0;
+  for (int r = wave; r < R; r += WAVES) {
+    int id;
+    float w;
+    topk_lane(L + (size_t)r * ldl, NE, TOPK, shared, lane, id, w);
+    if (lane < slots) {
+      pk[r * slots + lane] = (unsigned)id < (unsigned)E ? id : -1;
+      if (writer) {
+        pick[r * slots + lane] = id;
+        wts[r * slots + lane] = w;
+      }
+    }
+  }
+  __syncthreads();
+  if (writer) {
+    // the whole plan: first member and first item of every expert (wave 0 scans), then items, members, descriptors
+    int* off = reinterpret_cast<int*>(lds);
+    int* itoff = off + EMAX;
+    for (int e = tid; e < E; e += threads) item.cnt[e] = 0;
+    __syncthreads();
+    for (int p = tid; p < P; p += threads)
+      if (pk[p] >= 0) atomicAdd(&item.cnt[pk[p]], 1);
+    __syncthreads();
+    if (tid < 64) {
+      int items_before = 0, pairs_before = 0, used = 0;
+      for (int e0 = 0; e0 < E; e0 += 64) {
+        const int e = e0 + lane, c = e < E ? item.cnt[e] : 0, t = (c + 15) >> 4;
+        int ti = t, ci = c;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+          const int ut = __shfl_up(ti, o), uc = __shfl_up(ci, o);
+          if (lane >= o) {
+            ti += ut;
+            ci += uc;
+          }
+        }
+        if (e < E) {
+          off[e] = pairs_before + ci - c;
+          itoff[e] = items_before + ti - t;
+        }
+        items_before += __shfl(ti, 63);
+        pairs_before += __shfl(ci, 63);
+        used += __popcll(__ballot(c > 0));
+      }
+      if (lane == 0) {
+        counts[0] = items_before;
+        counts[1] = used;
+      }
+    }
+    __syncthreads();
+    for (int e = tid; e < E; e += threads) {
+      const int c = item.cnt[e];
+      for (int j = 0; 16 * j < c; ++j) {
+        const int i = itoff[e] + j, first = off[e] + 16 * j, n = min(16, c - 16 * j);
+        items[3 * i] = e;
+        items[3 * i + 1] = first;
+        items[3 * i + 2] = n;
+        int* d = desc + (size_t)i * DESC;
+        d[0] = e;
+        d[1] = n;
+        d[2] = first;
+        d[3] = 0;
+      }
+    }
+    for (int p = tid; p < P; p += threads) {
+      const int e = pk[p];
+      if (e < 0) continue;
+      int rank = 0;
+      for (int q = 0; q < p; ++q) rank += pk[q] == e;
+      members[off[e] + rank] = p;
+      desc[(size_t)(itoff[e] + (rank >> 4)) * DESC + 4 + (rank & 15)] = p;
+    }
+    return;
+  }
+  const int NB2 = (NI / 32 + 1) >> 1;
+  const int u = blockIdx.x - 1, it = u / NB2, cb2 = u - it * NB2;
+  if (!find_item(item, pk, P, E, it)) return;
+  NoHook none;
+  expert_unit<GS, NM, EPI, WAVES, false, 0>(X, x_stride, slots, Wup, D / GS, NI / 32, item.sel[0], item.sel[2],
+                                            item.pairs, cb2, act, NI, limit, nullptr, xs_act, lds, none);
+}
+
+template <int GS, int NM, int EPI>
+int launch_route_up(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared, const uint16_t* x,
+                    int64_t x_stride, const uint32_t* wup, int d, int ni, int* pick, float* wts, int* members,
+                    int* items, int* counts, int* desc, uint16_t* act, float* xs_act, float limit, int max_items,
+                    hipStream_t stream) {
+  const int nb2 = (ni / 32 + 1) / 2;
+  const int64_t grid = 1 + (int64_t)max_items * nb2;
+  TF_REQUIRE(grid <= 0x7FFFFFFF, "moe: %lld workgroups exceed the grid limit", (long long)grid);
+  const size_t floats = expert_lds_floats(NM, d / GS, false);
+  const size_t smem = sizeof(float) * (floats > 2 * EMAX ? floats : 2 * EMAX);
+  TF_REQUIRE(smem <= 48 * 1024, "moe: %d input groups need %zu bytes of LDS", d / GS, smem);
+  const dim3 g((unsigned)grid);
+#define TF_GO(W_)                                                                                                  \
+  route_up_kernel<GS, NM, EPI, W_><<<g, W_ * 64, smem, stream>>>(logits, ldl, rows, experts, top_k, shared, x, x_stride, \
+                                                                 wup, d, ni, pick, wts, members, items, counts, desc,  \
+                                                                 act, xs_act, limit)
+  switch (fused_waves(2 * grid)) {
+    case 16: TF_GO(16); break;
+    case 8: TF_GO(8); break;
+    default: TF_GO(4);
+  }
+#undef TF_GO
+  TF_LAUNCH_OK("tf_moe_route_up");
+  return 0;
+}
 
 template <int GS, int NM, int EPI_UP>
 int launch_fused(const uint16_t* x, int64_t x_stride, int slots, const uint32_t* wup, const uint32_t* wdown, int d,
@@ -157,4 +286,36 @@ extern "C" int tf_moe_decode_experts(int gs, int swiglu, const uint16_t* x, int6
                                          out, done, arrive, status, limit, max_items, s)
                 : launch_fused<32, 1, 1>(x, x_stride, slots, up, down, d, ni, desc, counts, wts, xs_x, act, xs_act, y,
                                          out, done, arrive, status, limit, max_items, s);
+}
+
+extern "C" int tf_moe_route_up(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared, int gs,
+                               int swiglu, const uint16_t* x, int64_t x_stride, const uint32_t* up, int d, int ni,
+                               int32_t* pick, float* wts, int32_t* members, int32_t* items, int32_t* counts,
+                               int32_t* desc, uint16_t* act, float* xs_act, float limit, int max_items,
+                               tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(gs == 32 || gs == 64, "moe: groups of 32 or 64 inputs, not %d", gs);
+  TF_REQUIRE(logits && x && up && pick && wts && members && items && counts && desc && act && xs_act,
+             "moe: null pointer argument");
+  TF_REQUIRE(experts >= 1 && experts + (shared ? 1 : 0) <= EMAX && experts <= 64 * TOPK_VPL,
+             "route: at most %d experts", EMAX - 1);
+  TF_REQUIRE(top_k >= 1 && top_k + (shared ? 1 : 0) <= 64 && top_k <= experts, "route: 1 to 64 slots a row, not %d",
+             top_k);
+  TF_REQUIRE(rows >= 1 && (int64_t)rows * (top_k + (shared ? 1 : 0)) <= PLAN_THREADS,
+             "route: the decode routing takes at most %d pairs", PLAN_THREADS);
+  TF_REQUIRE(ldl >= experts + (shared ? 1 : 0), "route: logits rows are too short");
+  TF_REQUIRE(d % gs == 0 && ni % 32 == 0 && ni % gs == 0 && d >= gs && max_items >= 1,
+             "moe: hidden and intermediate sizes in whole groups and 32-column blocks");
+  TF_REQUIRE(aligned16(x) && x_stride % 8 == 0 && aligned16(up) && aligned16(act),
+             "x: rows of K = groups * group size inputs, 16-byte aligned");
+  hipStream_t s = as_stream(stream);
+  if (gs == 64)
+    return swiglu ? launch_route_up<64, 2, 2>(logits, ldl, rows, experts, top_k, shared, x, x_stride, up, d, ni, pick,
+                                              wts, members, items, counts, desc, act, xs_act, limit, max_items, s)
+                  : launch_route_up<64, 1, 1>(logits, ldl, rows, experts, top_k, shared, x, x_stride, up, d, ni, pick,
+                                              wts, members, items, counts, desc, act, xs_act, limit, max_items, s);
+  return swiglu ? launch_route_up<32, 2, 2>(logits, ldl, rows, experts, top_k, shared, x, x_stride, up, d, ni, pick, wts,
+                                            members, items, counts, desc, act, xs_act, limit, max_items, s)
+                : launch_route_up<32, 1, 1>(logits, ldl, rows, experts, top_k, shared, x, x_stride, up, d, ni, pick, wts,
+                                            members, items, counts, desc, act, xs_act, limit, max_items, s);
 }

@@ -174,6 +174,12 @@ __device__ __forceinline__ void gemv_stream(float (&acc)[NM][RB], Stage<GS, NM> 
           for (int r = 0; r < RB; ++r) p[m][r] = 0.f;
 #pragma unroll
         for (int i = 0; i < CH; ++i) chunk_dot<GS, NM, RB>(p, st[d], i);
+        // A dot instruction's result may be read by a different VALU instruction only three wait states later;
+        // the compiler inserts them for instructions it emits itself, not after inline assembly.
+#pragma unroll
+        for (int m = 0; m < NM; ++m)
+#pragma unroll
+          for (int r = 0; r < RB; ++r) asm volatile("s_nop 2" : "+v"(p[m][r]));
 #pragma unroll
         for (int r = 0; r < RB; ++r) {
           const float sc = xsum(r, g);

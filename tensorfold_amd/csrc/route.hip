@@ -1,7 +1,7 @@
 // MoE glue around the expert kernels: router logits, per-row top-k, the stable grouping of pairs by expert, and the
 // weighted combine.  All integer results (ids, members, items) are deterministic and independent of the row count.
 
-#include "tf_common.h"
+#include "routing.h"
 
 namespace tf {
 namespace {
@@ -29,61 +29,6 @@ __global__ void __launch_bounds__(64)
   }
 }
 
-// ---- top-k: one wave a row ------------------------------------------------------------------------------------------
-
-constexpr int TOPK_VPL = 16;     // values a lane: up to 1024 experts
-
-// one wave, one row: see tf_moe_topk
-__device__ __forceinline__ void topk_row(const float* __restrict__ row, int NE, int TOPK, int shared, int lane,
-                                         int* __restrict__ pick, float* __restrict__ wts) {
-  const float NEG = -__builtin_inff();
-  float v[TOPK_VPL];
-#pragma unroll
-  for (int i = 0; i < TOPK_VPL; ++i) {
-    const int e = lane + 64 * i;
-    v[i] = e < NE ? row[e] : NEG;
-  }
-  float top = 0.f, total = 0.f, mine_ex = 0.f;
-  int mine_id = 0;
-  for (int k = 0; k < TOPK; ++k) {
-    float bv = v[0];
-    int bi = lane;
-#pragma unroll
-    for (int i = 1; i < TOPK_VPL; ++i)
-      if (v[i] > bv) {
-        bv = v[i];
-        bi = lane + 64 * i;
-      }
-    float m = bv;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
-    int idx = bv == m ? bi : 0x7FFFFFFF;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) idx = min(idx, __shfl_xor(idx, o));
-    if (k == 0) top = m;
-    const float ex = expf(m - top);
-    total += ex;
-    if (lane == k) {
-      mine_ex = ex;
-      mine_id = idx;
-    }
-    if ((idx & 63) == lane) {
-#pragma unroll
-      for (int i = 0; i < TOPK_VPL; ++i)
-        if (i == (idx >> 6)) v[i] = NEG;
-    }
-  }
-  if (lane < TOPK) {
-    pick[lane] = mine_id;
-    wts[lane] = round_bf16(mine_ex / total);
-  }
-  if (shared && lane == 0) {
-    const float sg = round_bf16(row[NE]);
-    pick[TOPK] = NE;
-    wts[TOPK] = round_bf16(1.f / (1.f + expf(-sg)));
-  }
-}
-
 __global__ void __launch_bounds__(64)
     topk_kernel(const float* __restrict__ L, int64_t ldl, int NE, int TOPK, int shared, int* __restrict__ pick,
                 float* __restrict__ wts) {
@@ -92,60 +37,6 @@ __global__ void __launch_bounds__(64)
 }
 
 // ---- plan: stable counting sort of pairs by expert -------------------------------------------------------------------
-
-constexpr int PLAN_THREADS = 1024;
-constexpr int EMAX = 1024;
-
-// Block-wide exclusive prefix sums of three per-thread values (1024 threads = 16 waves of 64); totals in tot[3].
-__device__ void scan3(int (&val)[3], int (&excl)[3], int (&tot)[3]) {
-  __shared__ int wsum[3][16];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  int inc[3];
-#pragma unroll
-  for (int s = 0; s < 3; ++s) {
-    int a = val[s];
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-      const int u = __shfl_up(a, o);
-      if (lane >= o) a += u;
-    }
-    inc[s] = a;
-    if (lane == 63) wsum[s][wave] = a;
-  }
-  __syncthreads();
-#pragma unroll
-  for (int s = 0; s < 3; ++s) {
-    int base = 0, all = 0;
-    for (int w = 0; w < 16; ++w) {
-      const int t = wsum[s][w];
-      if (w < wave) base += t;
-      all += t;
-    }
-    excl[s] = base + inc[s] - val[s];
-    tot[s] = all;
-  }
-  __syncthreads();
-}
-
-// thread e: expert e's pair count c -> its first member; writes the items (expert order) and counts
-__device__ int place_items(int c, int E, int T, int* __restrict__ items, int* __restrict__ counts) {
-  const int tid = threadIdx.x;
-  const int tiles = (c + T - 1) / T;
-  int val[3] = {c, tiles, c > 0 ? 1 : 0}, excl[3], tot[3];
-  scan3(val, excl, tot);
-  if (tid == 0) {
-    counts[0] = tot[1];
-    counts[1] = tot[2];
-  }
-  if (tid < E)
-    for (int j = 0; j < tiles; ++j) {
-      int* it = items + 3 * (excl[1] + j);
-      it[0] = tid;
-      it[1] = excl[0] + T * j;
-      it[2] = min(T, c - T * j);
-    }
-  return excl[0];
-}
 
 // up to 1024 pairs: one block does everything
 __global__ void __launch_bounds__(PLAN_THREADS)
@@ -344,7 +235,7 @@ extern "C" int tf_moe_topk(const float* logits, int64_t ldl, int rows, int exper
   clear_error();
   TF_REQUIRE(logits && pick && wts && rows >= 1, "topk: null pointer or empty shape");
   TF_REQUIRE(experts >= 1 && experts <= 64 * TOPK_VPL, "topk: 1 to %d experts, not %d", 64 * TOPK_VPL, experts);
-  TF_REQUIRE(top_k >= 1 && top_k <= 64 && top_k <= experts, "topk: 1 to 64 experts a row, not %d", top_k);
+  TF_REQUIRE(top_k >= 1 && top_k + (shared ? 1 : 0) <= 64 && top_k <= experts, "topk: 1 to 64 slots a row, not %d", top_k);
   TF_REQUIRE(ldl >= experts + (shared ? 1 : 0), "topk: logits rows hold %lld values, %d are read", (long long)ldl,
              experts + (shared ? 1 : 0));
   topk_kernel<<<rows, 64, 0, as_stream(stream)>>>(logits, ldl, experts, top_k, shared, pick, wts);
@@ -360,7 +251,7 @@ extern "C" int tf_moe_route_decode(const float* logits, int64_t ldl, int rows, i
   TF_REQUIRE(logits && x && pick && wts && members && items && counts && desc && xs_x, "route: null pointer argument");
   TF_REQUIRE(experts >= 1 && experts + (shared ? 1 : 0) <= EMAX && experts <= 64 * TOPK_VPL,
              "route: at most %d experts", EMAX - 1);
-  TF_REQUIRE(top_k >= 1 && top_k <= 64 && top_k <= experts, "route: 1 to 64 experts a row, not %d", top_k);
+  TF_REQUIRE(top_k >= 1 && top_k + (shared ? 1 : 0) <= 64 && top_k <= experts, "route: 1 to 64 slots a row, not %d", top_k);
   TF_REQUIRE(rows >= 1 && (int64_t)rows * (top_k + (shared ? 1 : 0)) <= PLAN_THREADS,
              "route: the fused decode routing takes at most %d pairs", PLAN_THREADS);
   TF_REQUIRE(gs == 32 || gs == 64, "route: groups of 32 or 64 inputs");

@@ -127,9 +127,10 @@ def fusable(x: torch.Tensor, ex: grouped.Experts, buf: MoEBuffers) -> bool:
 
 def decode(x: torch.Tensor, logits: torch.Tensor, ex: grouped.Experts, buf: MoEBuffers, top_k: int, experts: int,
            out: torch.Tensor | None = None) -> torch.Tensor:
-    """The decode layer in two launches: routing (top-k, pair sort, group sums), then every expert's up projection,
-    activation, down projection and the weighted combine in one kernel.  Same bits as ``select`` + ``gate_up`` +
-    ``down`` + ``combine``; bf16 [R, D] out.  ``buf.pick``, ``buf.wts`` and ``buf.plan`` are filled as by ``select``."""
+    """The decode layer in three launches (routing + up projection, down projection, combine) or, with
+    ``FUSED_DECODE``, in two (routing; up + down + combine).  Same bits as
+    ``select`` + ``gate_up`` + ``down`` + ``combine``; bf16 [R, D] out.  ``buf.pick``, ``buf.wts`` and ``buf.plan``
+    are filled as by ``select``."""
 
     _lib.on_gpu(x, logits)
     n = int(x.shape[0])
@@ -147,14 +148,27 @@ def decode(x: torch.Tensor, logits: torch.Tensor, ex: grouped.Experts, buf: MoEB
     items = grouped.max_items(n * buf.slots, experts + int(buf.shared), grouped.TILE)
     cells = n * (ex.dims // 64)
     ctr = f["counters"]
-    _lib.call("tf_moe_route_decode", _lib.ptr(logits), logits.stride(0), n, experts, top_k, int(buf.shared), _lib.ptr(x),
-              x.stride(0), ex.dims, ex.gs, _lib.ptr(buf.pick), _lib.ptr(buf.wts), _lib.ptr(plan.members),
-              _lib.ptr(plan.items), _lib.ptr(plan.counts), _lib.ptr(f["desc"]), _lib.ptr(f["xs_x"]), _lib.ptr(ctr),
-              1 + f["items"] + cells)
-    _lib.call("tf_moe_decode_experts", ex.gs, int(ex.swiglu), _lib.ptr(x), x.stride(0), n, buf.slots, _lib.ptr(ex.up),
-              _lib.ptr(ex.down), ex.dims, ex.width, _lib.ptr(f["desc"]), _lib.ptr(plan.counts), _lib.ptr(buf.wts),
-              _lib.ptr(f["xs_x"]), _lib.ptr(buf.act), _lib.ptr(f["xs_act"]), _lib.ptr(buf.y), _lib.ptr(out),
-              ctr.data_ptr() + 4, ctr.data_ptr() + 4 * (1 + f["items"]), _lib.ptr(ctr), ex.limit, items)
+    if FUSED_DECODE:
+        _lib.call("tf_moe_route_decode", _lib.ptr(logits), logits.stride(0), n, experts, top_k, int(buf.shared),
+                  _lib.ptr(x), x.stride(0), ex.dims, ex.gs, _lib.ptr(buf.pick), _lib.ptr(buf.wts), _lib.ptr(plan.members),
+                  _lib.ptr(plan.items), _lib.ptr(plan.counts), _lib.ptr(f["desc"]), _lib.ptr(f["xs_x"]), _lib.ptr(ctr),
+                  1 + f["items"] + cells)
+        _lib.call("tf_moe_decode_experts", ex.gs, int(ex.swiglu), _lib.ptr(x), x.stride(0), n, buf.slots,
+                  _lib.ptr(ex.up), _lib.ptr(ex.down), ex.dims, ex.width, _lib.ptr(f["desc"]), _lib.ptr(plan.counts),
+                  _lib.ptr(buf.wts), _lib.ptr(f["xs_x"]), _lib.ptr(buf.act), _lib.ptr(f["xs_act"]), _lib.ptr(buf.y),
+                  _lib.ptr(out), ctr.data_ptr() + 4, ctr.data_ptr() + 4 * (1 + f["items"]), _lib.ptr(ctr), ex.limit,
+                  items)
+        return out
+    # three launches: routing + up, down, combine; the down kernel takes the routing's item descriptors
+    act = buf.act.view(-1, ex.width)
+    _lib.call("tf_moe_route_up", _lib.ptr(logits), logits.stride(0), n, experts, top_k, int(buf.shared), ex.gs,
+              int(ex.swiglu), _lib.ptr(x), x.stride(0), _lib.ptr(ex.up), ex.dims, ex.width, _lib.ptr(buf.pick),
+              _lib.ptr(buf.wts), _lib.ptr(plan.members), _lib.ptr(plan.items), _lib.ptr(plan.counts),
+              _lib.ptr(f["desc"]), _lib.ptr(act), _lib.ptr(f["xs_act"]), ex.limit, items)
+    _lib.call("tf_experts_run_desc", ex.gs, 0, _lib.ptr(act), ex.width, 0, _lib.ptr(ex.down), ex.width // ex.gs,
+              ex.dims // grouped.COLS, _lib.ptr(f["desc"]), _lib.ptr(plan.counts), _lib.ptr(buf.y), ex.dims, 0.0, items,
+              _lib.ptr(f["xs_act"]), None)
+    _lib.call("tf_moe_combine", _lib.ptr(buf.y), 0, _lib.ptr(buf.wts), _lib.ptr(out), n, buf.slots, ex.dims)
     return out
 
 
@@ -206,7 +220,7 @@ def run(x: torch.Tensor, m: Routed, *, prefill: bool = False) -> torch.Tensor:
     if key not in _pool:
         _pool[key] = MoEBuffers(cap, _Dims(m), x.device, prefill=prefill)
     buf, x = _pool[key], x.contiguous()
-    if FUSED_DECODE and fusable(x, m.experts, buf):
+    if fusable(x, m.experts, buf):
         router(x, m.router, buf.logits[:n])
         return decode(x, buf.logits[:n], m.experts, buf, m.top_k, m.count).clone()
     moe(x, m.router, m.experts, buf, m.top_k, m.count)

@@ -86,6 +86,28 @@ def test_plan_groups_pairs_by_expert(rows, prefill, tile):
     assert np.array_equal(plan.members.cpu().numpy(), members)
 
 
+@pytest.mark.parametrize("case", CASES)
+def test_group_sums_made_by_the_kernel_equal_those_passed_in(case):
+    """tf_experts_run without ``xs`` sums each group of its rows itself: same bits as with tf_group_sums' sums."""
+
+    from tensorfold_amd import _lib, qmm
+    ex, _, _ = build(case, 44)
+    for rows in (1, 9):
+        x = synthetic.activations(rows, ex.dims, 45, 0.5).to(DEV)
+        picks = picks_for(rows, case, 46, hot=True if rows > 1 else None)
+        act, y, plan = run(ex, x, picks)
+        slots = picks.shape[1]
+        bound = experts.max_items(rows * slots, ex.count, experts.TILE)
+        act2, y2 = torch.empty_like(act), torch.empty_like(y)
+        _lib.call("tf_experts_run", ex.gs, 2 if ex.swiglu else 1, _lib.ptr(x), x.stride(0), slots, _lib.ptr(ex.up),
+                  ex.dims // ex.gs, ex.width // 32, _lib.ptr(plan.items), _lib.ptr(plan.counts), _lib.ptr(plan.members),
+                  _lib.ptr(act2), ex.width, ex.limit, bound * (ex.width // 32), None, None)
+        _lib.call("tf_experts_run", ex.gs, 0, _lib.ptr(act2), ex.width, 0, _lib.ptr(ex.down), ex.width // ex.gs,
+                  ex.dims // 32, _lib.ptr(plan.items), _lib.ptr(plan.counts), _lib.ptr(plan.members), _lib.ptr(y2),
+                  ex.dims, 0.0, bound * (ex.dims // 32), None, None)
+        assert torch.equal(act2, act) and torch.equal(y2, y), rows
+
+
 def test_an_expert_shared_by_many_rows_makes_items_of_16():
     picks = torch.full((37, 1), 5, dtype=torch.int32)
     plan = experts.Plan(37, 1, 8, DEV)
