@@ -150,21 +150,13 @@ __global__ void __launch_bounds__(WAVES * 64)
       int items_before = 0, pairs_before = 0, used = 0;
       for (int e0 = 0; e0 < E; e0 += 64) {
         const int e = e0 + lane, c = e < E ? item.cnt[e] : 0, t = (c + 15) >> 4;
-        int ti = t, ci = c;
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-          const int ut = __shfl_up(ti, o), uc = __shfl_up(ci, o);
-          if (lane >= o) {
-            ti += ut;
-            ci += uc;
-          }
-        }
+        const int ti = wave_scan(t), ci = wave_scan(c);
         if (e < E) {
           off[e] = pairs_before + ci - c;
           itoff[e] = items_before + ti - t;
         }
-        items_before += __shfl(ti, 63);
-        pairs_before += __shfl(ci, 63);
+        items_before += __builtin_amdgcn_readlane(ti, 63);
+        pairs_before += __builtin_amdgcn_readlane(ci, 63);
         used += __popcll(__ballot(c > 0));
       }
       if (lane == 0) {
@@ -201,6 +193,7 @@ __global__ void __launch_bounds__(WAVES * 64)
   const int u = blockIdx.x - 1, it = u / NB2, cb2 = u - it * NB2;
   if (!find_item(item, pk, P, E, it)) return;
   NoHook none;
+  // the item's rows are summed group by group inside the unit (a pass at a time), under its first weight loads
   expert_unit<GS, NM, EPI, WAVES, false, 0>(X, x_stride, slots, Wup, D / GS, NI / 32, item.sel[0], item.sel[2],
                                             item.pairs, cb2, act, NI, limit, nullptr, xs_act, lds, none);
 }

@@ -87,24 +87,9 @@ __global__ void __launch_bounds__(PLAN_THREADS)
   for (int i = tid; i < n_zero; i += PLAN_THREADS) zero[i] = 0;
   for (int r = wave; r < R; r += PLAN_THREADS / 64)
     topk_row(L + (size_t)r * ldl, NE, TOPK, shared, lane, pick + (size_t)r * slots, wts + (size_t)r * slots);
-  // group sums of x: 8 (groups of 64) or 4 (groups of 32) lanes a group, as tf_group_sums
-  {
-    const int lpg = gs / 8, part = tid % lpg, KG = D / gs;
-    for (int o = tid / lpg; o < R * KG; o += PLAN_THREADS / lpg) {
-      const int r = o / KG, g = o - r * KG;
-      const uint4 v = *reinterpret_cast<const uint4*>(X + (size_t)r * ldx + (size_t)g * gs + part * 8);
-      float s = bf16_lo(v.x);
-      s += bf16_hi(v.x);
-      s += bf16_lo(v.y);
-      s += bf16_hi(v.y);
-      s += bf16_lo(v.z);
-      s += bf16_hi(v.z);
-      s += bf16_lo(v.w);
-      s += bf16_hi(v.w);
-      for (int m = 1; m < lpg; m <<= 1) s += __shfl_xor(s, m);
-      if (part == 0) xs_x[o] = s;
-    }
-  }
+  // group sums of x, as tf_group_sums
+  if (gs == 64) group_sums_rows<64>(X, ldx, R, D / 64, xs_x, tid, PLAN_THREADS);
+  else group_sums_rows<32>(X, ldx, R, D / 32, xs_x, tid, PLAN_THREADS);
   __threadfence_block();
   __syncthreads();
   int e = -1;

@@ -11,34 +11,55 @@ namespace {
 
 constexpr int TOPK_VPL = 16;     // values a lane: up to 1024 experts
 
+// Maximum over the 64 lanes, the same value in every lane: a butterfly inside each row of 16 lanes through DPP
+// (no LDS round trips), then the four rows' maxima through readlane.
+__device__ __forceinline__ float wave_max(float x) {
+#define TF_DPP(V_, CTRL_) \
+  __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, V_), CTRL_, 0xf, 0xf, false))
+  x = fmaxf(x, TF_DPP(x, 0xB1));        // quad_perm [1, 0, 3, 2]
+  x = fmaxf(x, TF_DPP(x, 0x4E));        // quad_perm [2, 3, 0, 1]
+  x = fmaxf(x, TF_DPP(x, 0x141));       // row_half_mirror
+  x = fmaxf(x, TF_DPP(x, 0x140));       // row_mirror
+#undef TF_DPP
+  auto row = [&](int l) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), l)); };
+  return fmaxf(fmaxf(row(0), row(16)), fmaxf(row(32), row(48)));
+}
+
 // one wave, one row (see tf_moe_topk): lane k < TOPK leaves with the k-th pick and its weight, lane TOPK with the
-// shared expert's when there is one
-__device__ __forceinline__ void topk_lane(const float* __restrict__ row, int NE, int TOPK, int shared, int lane,
-                                          int& id, float& w) {
-  const float NEG = -__builtin_inff();
-  float v[TOPK_VPL];
+// shared expert's when there is one.  VPL values a lane cover 64 * VPL experts.
+template <int VPL>
+__device__ __forceinline__ void topk_load(const float* __restrict__ row, int NE, int lane, float (&v)[VPL]) {
 #pragma unroll
-  for (int i = 0; i < TOPK_VPL; ++i) {
+  for (int i = 0; i < VPL; ++i) {
     const int e = lane + 64 * i;
-    v[i] = e < NE ? row[e] : NEG;
+    v[i] = e < NE ? row[e] : -__builtin_inff();
   }
+}
+
+template <int VPL>
+__device__ __forceinline__ void topk_pick(float (&v)[VPL], const float* __restrict__ row, int NE, int TOPK, int shared,
+                                          int lane, int& id, float& w) {
+  const float NEG = -__builtin_inff();
   float top = 0.f, total = 0.f, mine_ex = 0.f;
   int mine_id = 0;
   for (int k = 0; k < TOPK; ++k) {
     float bv = v[0];
     int bi = lane;
 #pragma unroll
-    for (int i = 1; i < TOPK_VPL; ++i)
+    for (int i = 1; i < VPL; ++i)
       if (v[i] > bv) {
         bv = v[i];
         bi = lane + 64 * i;
       }
-    float m = bv;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
-    int idx = bv == m ? bi : 0x7FFFFFFF;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) idx = min(idx, __shfl_xor(idx, o));
+    const float m = wave_max(bv);
+    // the lowest expert id among the lanes that hold the maximum (nearly always one lane)
+    unsigned long long cand = __ballot(bv == m);
+    int idx = 0x7FFFFFFF;
+    while (cand) {
+      const int l = __builtin_ctzll(cand);
+      idx = min(idx, __builtin_amdgcn_readlane(bi, l));
+      cand &= cand - 1;
+    }
     if (k == 0) top = m;
     const float ex = expf(m - top);
     total += ex;
@@ -48,7 +69,7 @@ __device__ __forceinline__ void topk_lane(const float* __restrict__ row, int NE,
     }
     if ((idx & 63) == lane) {
 #pragma unroll
-      for (int i = 0; i < TOPK_VPL; ++i)
+      for (int i = 0; i < VPL; ++i)
         if (i == (idx >> 6)) v[i] = NEG;
     }
   }
@@ -58,6 +79,45 @@ __device__ __forceinline__ void topk_lane(const float* __restrict__ row, int NE,
     const float sg = round_bf16(row[NE]);
     id = NE;
     w = round_bf16(1.f / (1.f + expf(-sg)));
+  }
+}
+
+template <int VPL>
+__device__ __forceinline__ void topk_lane_n(const float* __restrict__ row, int NE, int TOPK, int shared, int lane,
+                                            int& id, float& w) {
+  float v[VPL];
+  topk_load<VPL>(row, NE, lane, v);
+  topk_pick<VPL>(v, row, NE, TOPK, shared, lane, id, w);
+}
+
+__device__ __forceinline__ void topk_lane(const float* __restrict__ row, int NE, int TOPK, int shared, int lane,
+                                          int& id, float& w) {
+  if (NE <= 128) topk_lane_n<2>(row, NE, TOPK, shared, lane, id, w);
+  else if (NE <= 512) topk_lane_n<8>(row, NE, TOPK, shared, lane, id, w);
+  else topk_lane_n<TOPK_VPL>(row, NE, TOPK, shared, lane, id, w);
+}
+
+// fp32 sums of every group of GS inputs of R rows into xs[r * KG + g]: the arithmetic of tf_group_sums (eight
+// inputs a lane in order, then a fixed xor tree over the group's lanes)
+template <int GS>
+__device__ __forceinline__ void group_sums_rows(const uint16_t* __restrict__ X, int64_t ldx, int R, int KG, float* xs,
+                                                int tid, int threads) {
+  constexpr int LPG = GS / 8;
+  const int part = tid % LPG;
+  for (int o = tid / LPG; o < R * KG; o += threads / LPG) {
+    const int r = o / KG, g = o - r * KG;
+    const uint4 v = *reinterpret_cast<const uint4*>(X + (size_t)r * ldx + (size_t)g * GS + part * 8);
+    float s = bf16_lo(v.x);
+    s += bf16_hi(v.x);
+    s += bf16_lo(v.y);
+    s += bf16_hi(v.y);
+    s += bf16_lo(v.z);
+    s += bf16_hi(v.z);
+    s += bf16_lo(v.w);
+    s += bf16_hi(v.w);
+#pragma unroll
+    for (int m = 1; m < LPG; m <<= 1) s += __shfl_xor(s, m);
+    if (part == 0) xs[o] = s;
   }
 }
 
@@ -128,6 +188,21 @@ __device__ int place_items(int c, int E, int T, int* __restrict__ items, int* __
   return excl[0];
 }
 
+// Inclusive prefix sums over the 64 lanes: shifts inside each row of 16 lanes through DPP, then the rows' totals
+// through readlane.
+__device__ __forceinline__ int wave_scan(int x) {
+#define TF_SHR(V_, N_) __builtin_amdgcn_update_dpp(0, V_, 0x110 + N_, 0xf, 0xf, false)
+  x += TF_SHR(x, 1);
+  x += TF_SHR(x, 2);
+  x += TF_SHR(x, 4);
+  x += TF_SHR(x, 8);
+#undef TF_SHR
+  const int t0 = __builtin_amdgcn_readlane(x, 15), t1 = __builtin_amdgcn_readlane(x, 31),
+            t2 = __builtin_amdgcn_readlane(x, 47);
+  const int row = (threadIdx.x & 63) >> 4;
+  return x + (row > 0 ? t0 : 0) + (row > 1 ? t1 : 0) + (row > 2 ? t2 : 0);
+}
+
 // ---- one item of the plan, found by every workgroup for itself -----------------------------------------------------
 //
 // The plan orders experts ascending, an expert's pairs in pair order, in items of at most 16.  A workgroup that knows
@@ -154,15 +229,7 @@ __device__ __forceinline__ bool find_item(ItemLds& L, const int* pk, int P, int 
     int items_before = 0, pairs_before = 0;
     for (int e0 = 0; e0 < E; e0 += 64) {
       const int e = e0 + lane, c = e < E ? L.cnt[e] : 0, t = (c + 15) >> 4;
-      int ti = t, ci = c;                        // inclusive scans over the 64 experts of this step
-#pragma unroll
-      for (int o = 1; o < 64; o <<= 1) {
-        const int ut = __shfl_up(ti, o), uc = __shfl_up(ci, o);
-        if (lane >= o) {
-          ti += ut;
-          ci += uc;
-        }
-      }
+      const int ti = wave_scan(t), ci = wave_scan(c);      // inclusive, over the 64 experts of this step
       const int first_item = items_before + ti - t;
       if (it >= first_item && it < first_item + t) {
         const int j = it - first_item;
@@ -171,8 +238,8 @@ __device__ __forceinline__ bool find_item(ItemLds& L, const int* pk, int P, int 
         L.sel[2] = min(16, c - 16 * j);
         L.sel[4] = 16 * j;
       }
-      items_before += __shfl(ti, 63);
-      pairs_before += __shfl(ci, 63);
+      items_before += __builtin_amdgcn_readlane(ti, 63);
+      pairs_before += __builtin_amdgcn_readlane(ci, 63);
     }
     if (lane == 0) L.sel[3] = items_before;
   }

@@ -20,6 +20,9 @@ from . import experts as grouped
 # ``run`` issues a decode-sized layer as routing + up + down + combine launches; with this set it issues the routing
 # launch and the one fused experts launch (``decode``) instead.  Same bits either way.
 FUSED_DECODE = os.environ.get("TENSORFOLD_AMD_FUSED_DECODE", "0") == "1"
+# Up to this many router logits (rows x experts) a call, the up projection's workgroups each repeat the routing
+# instead of waiting for a routing launch; past it the repeated top-k would cost more than the launch it saves.
+ROUTE_UP_LOGITS = 2048
 
 
 def router(x: torch.Tensor, rows: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
@@ -159,12 +162,23 @@ def decode(x: torch.Tensor, logits: torch.Tensor, ex: grouped.Experts, buf: MoEB
                   _lib.ptr(out), ctr.data_ptr() + 4, ctr.data_ptr() + 4 * (1 + f["items"]), _lib.ptr(ctr), ex.limit,
                   items)
         return out
-    # three launches: routing + up, down, combine; the down kernel takes the routing's item descriptors
     act = buf.act.view(-1, ex.width)
-    _lib.call("tf_moe_route_up", _lib.ptr(logits), logits.stride(0), n, experts, top_k, int(buf.shared), ex.gs,
-              int(ex.swiglu), _lib.ptr(x), x.stride(0), _lib.ptr(ex.up), ex.dims, ex.width, _lib.ptr(buf.pick),
-              _lib.ptr(buf.wts), _lib.ptr(plan.members), _lib.ptr(plan.items), _lib.ptr(plan.counts),
-              _lib.ptr(f["desc"]), _lib.ptr(act), _lib.ptr(f["xs_act"]), ex.limit, items)
+    if n * (experts + int(buf.shared)) > ROUTE_UP_LOGITS:
+        # many logits: one routing launch, then up, down and combine from its item descriptors
+        _lib.call("tf_moe_route_decode", _lib.ptr(logits), logits.stride(0), n, experts, top_k, int(buf.shared),
+                  _lib.ptr(x), x.stride(0), ex.dims, ex.gs, _lib.ptr(buf.pick), _lib.ptr(buf.wts), _lib.ptr(plan.members),
+                  _lib.ptr(plan.items), _lib.ptr(plan.counts), _lib.ptr(f["desc"]), _lib.ptr(f["xs_x"]), None, 0)
+        _lib.call("tf_experts_run_desc", ex.gs, 2 if ex.swiglu else 1, _lib.ptr(x), x.stride(0), buf.slots,
+                  _lib.ptr(ex.up), ex.dims // ex.gs, ex.width // grouped.COLS, _lib.ptr(f["desc"]),
+                  _lib.ptr(plan.counts), _lib.ptr(act), ex.width, ex.limit, items, _lib.ptr(f["xs_x"]),
+                  _lib.ptr(f["xs_act"]))
+    else:
+        # few logits: every workgroup of the up projection routes for itself (three launches: routing + up, down,
+        # combine)
+        _lib.call("tf_moe_route_up", _lib.ptr(logits), logits.stride(0), n, experts, top_k, int(buf.shared), ex.gs,
+                  int(ex.swiglu), _lib.ptr(x), x.stride(0), _lib.ptr(ex.up), ex.dims, ex.width, _lib.ptr(buf.pick),
+                  _lib.ptr(buf.wts), _lib.ptr(plan.members), _lib.ptr(plan.items), _lib.ptr(plan.counts),
+                  _lib.ptr(f["desc"]), _lib.ptr(act), _lib.ptr(f["xs_act"]), ex.limit, items)
     _lib.call("tf_experts_run_desc", ex.gs, 0, _lib.ptr(act), ex.width, 0, _lib.ptr(ex.down), ex.width // ex.gs,
               ex.dims // grouped.COLS, _lib.ptr(f["desc"]), _lib.ptr(plan.counts), _lib.ptr(buf.y), ex.dims, 0.0, items,
               _lib.ptr(f["xs_act"]), None)

@@ -205,13 +205,14 @@ def test_moe_run_rows_do_not_depend_on_the_window():
 @pytest.mark.parametrize("shape,ne,rows", [(synthetic.C1, 24, 1), (synthetic.C1, 24, 8), (synthetic.C2, 48, 32),
                                            (synthetic.MoEShape("small", 512, 16, 128, 4, 32, True, True), 16, 5),
                                            (synthetic.MoEShape("small64", 384, 12, 192, 3, 64, False, False), 12, 19)])
-@pytest.mark.parametrize("one_launch", [False, True])
-def test_the_fused_decode_layer_equals_the_separate_kernels(shape, ne, rows, one_launch, monkeypatch):
-    """Routing in one launch, then up + down + combine from its item descriptors (three launches, or one with
-    FUSED_DECODE): ids, plan and output bits equal those of select + gate_up + down + combine; twice in a row on
-    different inputs (the counters are reset by the routing)."""
+@pytest.mark.parametrize("path", ["route_up", "route_then_up", "one_launch"])
+def test_the_fused_decode_layer_equals_the_separate_kernels(shape, ne, rows, path, monkeypatch):
+    """The three forms of ``decode`` (routing inside the up launch; a routing launch, then up, down, combine from its
+    item descriptors; a routing launch and one launch for up + down + combine): ids, plan and output bits equal those
+    of select + gate_up + down + combine; twice in a row on different inputs."""
 
-    monkeypatch.setattr(moe, "FUSED_DECODE", one_launch)
+    monkeypatch.setattr(moe, "FUSED_DECODE", path == "one_launch")
+    monkeypatch.setattr(moe, "ROUTE_UP_LOGITS", 0 if path == "route_then_up" else 1 << 30)
 
     up, down = layer_tables(shape, 1500, ne)
     ex = experts.make([tuple(t.to(DEV) for t in m) for m in up], tuple(t.to(DEV) for t in down), shape.gs)
