@@ -76,7 +76,7 @@ class Layer:
 
         ex, buf = self.tables[i % len(self.tables)], buf or self.buf
         f, x, l = buf.fused(SHAPE.gs), self.x[i % 4], self.logits[getattr(buf, "draw", i % POOL)]
-        items = experts.max_items(self.tokens * buf.slots, SHAPE.experts, experts.TILE)
+        items = experts.max_items(self.tokens * buf.slots, SHAPE.experts, moe.DESC_TILE)
         _lib.call("tf_moe_route_up", _lib.ptr(l), l.stride(0), self.tokens, SHAPE.experts, SHAPE.top_k, 0, ex.gs,
                   int(ex.swiglu), _lib.ptr(x), x.stride(0), _lib.ptr(ex.up), ex.dims, ex.width, _lib.ptr(buf.pick),
                   _lib.ptr(buf.wts), _lib.ptr(buf.plan.members), _lib.ptr(buf.plan.items), _lib.ptr(buf.plan.counts),
@@ -85,7 +85,7 @@ class Layer:
     def down(self, i: int, buf=None) -> None:
         ex, buf = self.tables[i % len(self.tables)], buf or self.buf
         f = buf.fused(SHAPE.gs)
-        items = experts.max_items(self.tokens * buf.slots, SHAPE.experts, experts.TILE)
+        items = experts.max_items(self.tokens * buf.slots, SHAPE.experts, moe.DESC_TILE)
         _lib.call("tf_experts_run_desc", ex.gs, 0, _lib.ptr(buf.act), ex.width, 0, _lib.ptr(ex.down),
                   ex.width // ex.gs, ex.dims // experts.COLS, _lib.ptr(f["desc"]), _lib.ptr(buf.plan.counts),
                   _lib.ptr(buf.y), ex.dims, 0.0, items, _lib.ptr(f["xs_act"]), None)
@@ -116,7 +116,7 @@ class Layer:
         ex, f = self.tables[i % len(self.tables)], buf.fused(SHAPE.gs)
         f["counters"].zero_()
         n = self.tokens
-        items = experts.max_items(n * buf.slots, SHAPE.experts, experts.TILE)
+        items = experts.max_items(n * buf.slots, SHAPE.experts, moe.DESC_TILE)
         ctr = f["counters"]
         _lib.call("tf_moe_decode_experts", ex.gs, int(ex.swiglu), _lib.ptr(self.x[i % 4]), self.x[i % 4].stride(0), n,
                   buf.slots, _lib.ptr(ex.up), _lib.ptr(ex.down), ex.dims, ex.width, _lib.ptr(f["desc"]),

@@ -88,9 +88,16 @@ int tf_experts_plan(const int32_t* picks, int64_t pairs, int experts, int tile, 
 int tf_experts_run(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg, int nb,
                    const int32_t* items, const int32_t* counts, const int32_t* members, void* out, int n, float limit,
                    int64_t max_units, const float* xs, float* xs_out, tf_stream_t stream);
-/* tf_experts_run with the items given as descriptors (int32 [max_items, 20]: expert, count, first member, 0, the
- * item's pairs[16]) as tf_moe_route_decode writes them; xs is required.  Same bits as tf_experts_run on the same
- * plan.  Same reference counterpart (experts.cpp:43-48 `run`); the descriptor form has none. */
+/* Item descriptors, written by tf_moe_route_decode and tf_moe_route_up for the decode expert kernels: int32 rows of
+ * TF_DESC_INTS; row 0 holds the number of descriptors, row 1 + i = {expert, count, first member, 0, pairs[4]}: the plan
+ * cut into items of at most TF_DESC_TILE pairs.  A buffer for P pairs over E experts needs
+ * 1 + min(P, E) + P / TF_DESC_TILE rows; that bound is the max_items of the calls that read descriptors. */
+#define TF_DESC_INTS 8
+#define TF_DESC_TILE 4
+
+/* tf_experts_run with the items given as descriptors; xs is required; counts is not read (kept for symmetry).
+ * Same bits as tf_experts_run on the same plan.  Same reference counterpart (experts.cpp:43-48 `run`); the
+ * descriptor form has none. */
 int tf_experts_run_desc(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg,
                         int nb, const int32_t* desc, const int32_t* counts, void* out, int n, float limit,
                         int64_t max_items, const float* xs, float* xs_out, tf_stream_t stream);
@@ -117,7 +124,7 @@ int tf_moe_combine(const void* y, int y_bf16, const float* wts, uint16_t* out, i
 
 /* Routing and the up projection of the decode layer in ONE launch, for rows * (top_k + shared) <= 1024: workgroup 0
  * writes what tf_moe_topk and tf_experts_plan (tile 16) would (pick, wts, members, items, counts) plus the item
- * descriptors int32 [max_items, 20] that tf_experts_run_desc reads; every other workgroup finds its own item from the
+ * descriptors that tf_experts_run_desc reads; every other workgroup finds its own item from the
  * logits and runs the up unit of tf_experts_run (epilogue relu^2, or SwiGLU when swiglu != 0): act bf16 [pairs, ni] and
  * its group sums xs_act fp32 [pairs, ni / gs].  Same bits as the separate calls.  No counterpart in the reference
  * (moe.py:88-128 issues them one by one). */
@@ -126,7 +133,7 @@ int tf_moe_route_up(const float* logits, int64_t ldl, int rows, int experts, int
                     int32_t* members, int32_t* items, int32_t* counts, int32_t* desc, uint16_t* act, float* xs_act,
                     float limit, int max_items, tf_stream_t stream);
 /* The decode layer's routing in one launch, for rows * (top_k + shared) <= 1024: tf_moe_topk, tf_experts_plan (tile
- * 16) and tf_group_sums of x, plus desc int32 [max items, 20] = {expert, count, first, 0, pairs[16]} an item and the
+ * 16) and tf_group_sums of x, plus the item descriptors and the
  * zeroing of `zero` (n_zero ints: the counters of tf_moe_decode_experts).  No counterpart in the reference, which
  * launches `_topk_rows`, `plan` and its group sums separately (moe.py:103-116, kernels/qmm.py:148-154). */
 int tf_moe_route_decode(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared,
@@ -136,7 +143,7 @@ int tf_moe_route_decode(const float* logits, int64_t ldl, int rows, int experts,
 /* The decode layer's experts in one launch: up (+ relu^2 or SwiGLU), down and the weighted combine, with the bits
  * of tf_experts_run, tf_experts_run and tf_moe_combine run in turn.  desc, counts, wts, xs_x as left by
  * tf_moe_route_decode; scratch act bf16 [pairs, ni], xs_act fp32 [pairs, ni/gs], y fp32 [pairs, d]; counters done
- * [max_items] and arrive [rows * d/64] zero on entry; status[0] is set to 1 if a bounded wait ran out (the output
+ * [max_items] (one a descriptor) and arrive [rows * d/64] zero on entry; status[0] is set to 1 if a bounded wait ran out (the output
  * is then invalid).  d and ni multiples of 64.  Fuses experts.cpp:43-48 `run` (twice) and moe.py:131-151 `combine`. */
 int tf_moe_decode_experts(int gs, int swiglu, const uint16_t* x, int64_t x_stride, int rows, int slots,
                           const uint32_t* up, const uint32_t* down, int d, int ni, const int32_t* desc,

@@ -21,6 +21,7 @@
 #include <cstdlib>
 
 #include "gemv.h"
+#include "routing.h"
 
 namespace tf {
 namespace {
@@ -42,10 +43,8 @@ __global__ void __launch_bounds__(WAVES * 64)
                                        xs_out, lds, none);
 }
 
-// The same unit taken from an item descriptor (int32 [20]: expert, count, first member, 0, pairs[16]) as
-// tf_moe_route_decode writes them: one read instead of the items -> members chain.
-constexpr int DESC = 20;
-
+// The same unit taken from an item descriptor as tf_moe_route_decode and tf_moe_route_up write them: one read
+// instead of the items -> members chain, and items of at most DTILE pairs.
 template <int GS, int NM, int EPI, int WAVES>
 __global__ void __launch_bounds__(WAVES * 64)
     expert_desc_kernel(const uint16_t* __restrict__ X, int64_t x_stride, int slots, const uint32_t* __restrict__ W,
@@ -56,10 +55,10 @@ __global__ void __launch_bounds__(WAVES * 64)
   __shared__ int pairs[16];
   const int NB2 = (NB + 1) >> 1;
   const int it = blockIdx.x / NB2, cb2 = blockIdx.x - it * NB2;
-  if (it >= counts[0]) return;
-  const int* d = desc + (size_t)it * DESC;
+  if (it >= desc[0]) return;
+  const int* d = desc + (size_t)(1 + it) * DESC;
   const int e = d[0], cnt = d[1];
-  if (threadIdx.x < 16) pairs[threadIdx.x] = d[4 + threadIdx.x];
+  if (threadIdx.x < DTILE) pairs[threadIdx.x] = d[4 + threadIdx.x];
   __syncthreads();
   NoHook none;
   expert_unit<GS, NM, EPI, WAVES, true, 0>(X, x_stride, slots, W, KG, NB, e, cnt, pairs, cb2, out, N, limit, xs_in,

@@ -21,8 +21,6 @@
 namespace tf {
 namespace {
 
-constexpr int DESC = 20;      // int32 an item descriptor: expert, count, first, 0, pairs[16]
-
 int fused_waves(int64_t grid) { return grid < 768 ? 16 : grid < 1536 ? 8 : 4; }
 
 struct WaitItem {
@@ -61,10 +59,10 @@ __global__ void __launch_bounds__(WAVES * 64)
   const bool up = b < U;
   const int it = up ? b / NB2u : (b - U) / NB2d;
   const int cb2 = up ? b - it * NB2u : (b - U) - it * NB2d;
-  if (it >= counts[0]) return;
-  const int* d = desc + (size_t)it * DESC;
+  if (it >= desc[0]) return;
+  const int* d = desc + (size_t)(1 + it) * DESC;
   const int e = d[0], cnt = d[1];
-  if (tid < 16) pairs[tid] = d[4 + tid];
+  if (tid < DTILE) pairs[tid] = d[4 + tid];
   __syncthreads();
   if (up) {
     NoHook none;
@@ -141,27 +139,31 @@ __global__ void __launch_bounds__(WAVES * 64)
     // the whole plan: first member and first item of every expert (wave 0 scans), then items, members, descriptors
     int* off = reinterpret_cast<int*>(lds);
     int* itoff = off + EMAX;
+    int* dtoff = itoff + EMAX;
     for (int e = tid; e < E; e += threads) item.cnt[e] = 0;
     __syncthreads();
     for (int p = tid; p < P; p += threads)
       if (pk[p] >= 0) atomicAdd(&item.cnt[pk[p]], 1);
     __syncthreads();
     if (tid < 64) {
-      int items_before = 0, pairs_before = 0, used = 0;
+      int items_before = 0, pairs_before = 0, descs_before = 0, used = 0;
       for (int e0 = 0; e0 < E; e0 += 64) {
-        const int e = e0 + lane, c = e < E ? item.cnt[e] : 0, t = (c + 15) >> 4;
-        const int ti = wave_scan(t), ci = wave_scan(c);
+        const int e = e0 + lane, c = e < E ? item.cnt[e] : 0, t = (c + 15) >> 4, t4 = (c + DTILE - 1) / DTILE;
+        const int ti = wave_scan(t), ci = wave_scan(c), di = wave_scan(t4);
         if (e < E) {
           off[e] = pairs_before + ci - c;
           itoff[e] = items_before + ti - t;
+          dtoff[e] = descs_before + di - t4;
         }
         items_before += __builtin_amdgcn_readlane(ti, 63);
         pairs_before += __builtin_amdgcn_readlane(ci, 63);
+        descs_before += __builtin_amdgcn_readlane(di, 63);
         used += __popcll(__ballot(c > 0));
       }
       if (lane == 0) {
         counts[0] = items_before;
         counts[1] = used;
+        desc[0] = descs_before;
       }
     }
     __syncthreads();
@@ -172,10 +174,12 @@ __global__ void __launch_bounds__(WAVES * 64)
         items[3 * i] = e;
         items[3 * i + 1] = first;
         items[3 * i + 2] = n;
-        int* d = desc + (size_t)i * DESC;
+      }
+      for (int j = 0; DTILE * j < c; ++j) {
+        int* d = desc + (size_t)(1 + dtoff[e] + j) * DESC;
         d[0] = e;
-        d[1] = n;
-        d[2] = first;
+        d[1] = min(DTILE, c - DTILE * j);
+        d[2] = off[e] + DTILE * j;
         d[3] = 0;
       }
     }
@@ -185,13 +189,13 @@ __global__ void __launch_bounds__(WAVES * 64)
       int rank = 0;
       for (int q = 0; q < p; ++q) rank += pk[q] == e;
       members[off[e] + rank] = p;
-      desc[(size_t)(itoff[e] + (rank >> 4)) * DESC + 4 + (rank & 15)] = p;
+      desc[(size_t)(1 + dtoff[e] + rank / DTILE) * DESC + 4 + rank % DTILE] = p;
     }
     return;
   }
   const int NB2 = (NI / 32 + 1) >> 1;
   const int u = blockIdx.x - 1, it = u / NB2, cb2 = u - it * NB2;
-  if (!find_item(item, pk, P, E, it)) return;
+  if (!find_item<DTILE>(item, pk, P, E, it)) return;
   NoHook none;
   // the item's rows are summed group by group inside the unit (a pass at a time), under its first weight loads
   expert_unit<GS, NM, EPI, WAVES, false, 0>(X, x_stride, slots, Wup, D / GS, NI / 32, item.sel[0], item.sel[2],
@@ -207,7 +211,7 @@ int launch_route_up(const float* logits, int64_t ldl, int rows, int experts, int
   const int64_t grid = 1 + (int64_t)max_items * nb2;
   TF_REQUIRE(grid <= 0x7FFFFFFF, "moe: %lld workgroups exceed the grid limit", (long long)grid);
   const size_t floats = expert_lds_floats(NM, d / GS, false);
-  const size_t smem = sizeof(float) * (floats > 2 * EMAX ? floats : 2 * EMAX);
+  const size_t smem = sizeof(float) * (floats > 3 * EMAX ? floats : 3 * EMAX);
   TF_REQUIRE(smem <= 48 * 1024, "moe: %d input groups need %zu bytes of LDS", d / GS, smem);
   const dim3 g((unsigned)grid);
 #define TF_GO(W_)                                                                                                  \

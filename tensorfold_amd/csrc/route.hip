@@ -69,7 +69,6 @@ __global__ void __launch_bounds__(PLAN_THREADS)
 // The decode layer's whole routing in one workgroup (rows * slots <= 1024): top-k of every row, the pair sort, one
 // descriptor an item for the fused expert kernel {expert, count, first, 0, pairs[16]}, the group sums of x, and the
 // zeroing of the fused kernel's counters.
-constexpr int DESC = 20;
 
 __global__ void __launch_bounds__(PLAN_THREADS)
     route_decode_kernel(const float* __restrict__ L, int64_t ldl, int R, int NE, int TOPK, int shared,
@@ -111,15 +110,19 @@ __global__ void __launch_bounds__(PLAN_THREADS)
   }
   __threadfence_block();
   __syncthreads();
-  const int n_items = counts[0];
-  for (int i = tid; i < n_items; i += PLAN_THREADS) {
-    const int ie = items[3 * i], first = items[3 * i + 1], c = items[3 * i + 2];
-    int* d = desc + (size_t)i * DESC;
-    d[0] = ie;
-    d[1] = c;
+  // the descriptors: the same order cut into items of DTILE
+  const int c = tid < E ? cnt[tid] : 0, t4 = (c + DTILE - 1) / DTILE;
+  int val[3] = {t4, 0, 0}, excl[3], tot[3];
+  scan3(val, excl, tot);
+  if (tid == 0) desc[0] = tot[0];
+  for (int j = 0; j < t4; ++j) {
+    int* d = desc + (size_t)(1 + excl[0] + j) * DESC;
+    const int first = off[tid] + DTILE * j, n = min(DTILE, c - DTILE * j);
+    d[0] = tid;
+    d[1] = n;
     d[2] = first;
     d[3] = 0;
-    for (int j = 0; j < 16; ++j) d[4 + j] = j < c ? mem[first + j] : 0;
+    for (int k = 0; k < DTILE; ++k) d[4 + k] = k < n ? mem[first + k] : 0;
   }
 }
 

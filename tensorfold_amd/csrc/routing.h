@@ -203,9 +203,18 @@ __device__ __forceinline__ int wave_scan(int x) {
   return x + (row > 0 ? t0 : 0) + (row > 1 ? t1 : 0) + (row > 2 ? t2 : 0);
 }
 
+// ---- item descriptors ---------------------------------------------------------------------------------------------------
+//
+// What the routing kernels leave for the decode expert kernels: the plan cut again into items of at most DTILE pairs
+// (a workgroup walks its rows two at a time, so short items keep every workgroup to two passes over its weights and
+// spread an expert that many rows share over more workgroups).  int32 rows of DESC: row 0 holds the number of
+// descriptors, row 1 + i = {expert, count, first member, 0, pairs[DTILE]}.
+constexpr int DESC = 8;
+constexpr int DTILE = 4;
+
 // ---- one item of the plan, found by every workgroup for itself -----------------------------------------------------
 //
-// The plan orders experts ascending, an expert's pairs in pair order, in items of at most 16.  A workgroup that knows
+// The plan orders experts ascending, an expert's pairs in pair order, in items of at most TILE.  A workgroup that knows
 // every pair's expert (pk[0 .. P), in LDS) finds item `it` with a histogram, a scan over the experts by wave 0 and a
 // ballot walk over the pairs: no global memory, no quadratic rank loop.
 
@@ -217,6 +226,7 @@ struct ItemLds {
 
 // Every thread of the workgroup calls this (it has barriers); pk holds P expert ids (negative = none).
 // Returns false when there is no item `it`.  On return L.sel and L.pairs describe the item.
+template <int TILE>
 __device__ __forceinline__ bool find_item(ItemLds& L, const int* pk, int P, int E, int it) {
   const int tid = threadIdx.x, threads = blockDim.x, lane = tid & 63;
   for (int e = tid; e < E; e += threads) L.cnt[e] = 0;
@@ -228,15 +238,15 @@ __device__ __forceinline__ bool find_item(ItemLds& L, const int* pk, int P, int 
   if (tid < 64) {
     int items_before = 0, pairs_before = 0;
     for (int e0 = 0; e0 < E; e0 += 64) {
-      const int e = e0 + lane, c = e < E ? L.cnt[e] : 0, t = (c + 15) >> 4;
+      const int e = e0 + lane, c = e < E ? L.cnt[e] : 0, t = (c + TILE - 1) / TILE;
       const int ti = wave_scan(t), ci = wave_scan(c);      // inclusive, over the 64 experts of this step
       const int first_item = items_before + ti - t;
       if (it >= first_item && it < first_item + t) {
         const int j = it - first_item;
         L.sel[0] = e;
-        L.sel[1] = pairs_before + ci - c + 16 * j;
-        L.sel[2] = min(16, c - 16 * j);
-        L.sel[4] = 16 * j;
+        L.sel[1] = pairs_before + ci - c + TILE * j;
+        L.sel[2] = min(TILE, c - TILE * j);
+        L.sel[4] = TILE * j;
       }
       items_before += __builtin_amdgcn_readlane(ti, 63);
       pairs_before += __builtin_amdgcn_readlane(ci, 63);
@@ -247,7 +257,7 @@ __device__ __forceinline__ bool find_item(ItemLds& L, const int* pk, int P, int 
   const int e = L.sel[0];
   if (e < 0) return false;
   if (tid < 64) {
-    // the expert's pairs in pair order; the item takes ranks [16 j, 16 j + count)
+    // the expert's pairs in pair order; the item takes ranks [TILE j, TILE j + count)
     int before = 0;
     const int skip = L.sel[4], cnt = L.sel[2];
     for (int p0 = 0; p0 < P && before < skip + cnt; p0 += 64) {

@@ -23,6 +23,9 @@ FUSED_DECODE = os.environ.get("TENSORFOLD_AMD_FUSED_DECODE", "0") == "1"
 # Up to this many router logits (rows x experts) a call, the up projection's workgroups each repeat the routing
 # instead of waiting for a routing launch; past it the repeated top-k would cost more than the launch it saves.
 ROUTE_UP_LOGITS = 2048
+# Item descriptors the routing launches leave for the decode expert kernels: rows of DESC_INTS int32, row 0 the
+# count; items of at most DESC_TILE pairs (TF_DESC_INTS / TF_DESC_TILE of the C header).
+DESC_INTS, DESC_TILE = 8, 4
 
 
 def router(x: torch.Tensor, rows: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
@@ -66,16 +69,16 @@ class MoEBuffers:
         self.cfg, self.device, self._fused = cfg, device, None
 
     def fused(self, gs: int) -> dict:
-        """Scratch of the fused decode layer (``decode``), made on first use: item descriptors, group sums, the
-        counters (status, then an arrival count an item, then one a (token, 64 columns) cell) and the output."""
+        """Scratch of ``decode``, made on first use: item descriptors, group sums, the counters of the one-launch
+        form (status, then an arrival count a descriptor, then one a (token, 64 columns) cell) and the output."""
 
         if self._fused is None:
             cfg, dev, pairs = self.cfg, self.device, self.rows * self.slots
-            items = grouped.max_items(pairs, cfg.num_experts + int(self.shared), grouped.TILE)
+            items = grouped.max_items(pairs, cfg.num_experts + int(self.shared), DESC_TILE)
             cells = self.rows * (cfg.hidden_size // 64)
             self._fused = dict(
                 items=items,
-                desc=torch.zeros((items, 20), dtype=torch.int32, device=dev),
+                desc=torch.zeros((1 + items, DESC_INTS), dtype=torch.int32, device=dev),
                 xs_x=torch.empty((self.rows, cfg.hidden_size // gs), dtype=torch.float32, device=dev),
                 xs_act=torch.empty((pairs, cfg.moe_intermediate_size // gs), dtype=torch.float32, device=dev),
                 counters=torch.zeros((1 + items + cells,), dtype=torch.int32, device=dev),
@@ -148,7 +151,7 @@ def decode(x: torch.Tensor, logits: torch.Tensor, ex: grouped.Experts, buf: MoEB
         out = f["out"][:n]
     plan = buf.plan
     plan.tile = grouped.TILE
-    items = grouped.max_items(n * buf.slots, experts + int(buf.shared), grouped.TILE)
+    items = grouped.max_items(n * buf.slots, experts + int(buf.shared), DESC_TILE)
     cells = n * (ex.dims // 64)
     ctr = f["counters"]
     if FUSED_DECODE:
