@@ -38,30 +38,42 @@ __host__ __device__ constexpr int delta(int j) {
   return stream_end<K2>(j) - stream_end<K2>(0);
 }
 
-// The 16-bit states of values p0 .. p0 + 3 (p0 = 8 L + 4 h) of the tile at `tile` (global or LDS words).
+// The stored words lane (L, h) needs of a tile for its four values p0 .. p0 + 3 (p0 = 8 L + 4 h): two, or three when
+// a window can reach past the second.
 template <int K2>
-__device__ __forceinline__ void states4(const uint32_t* tile, int L, int h, uint32_t (&s)[4]) {
-  constexpr int TW = tile_words<K2>(), R = 32 * TW;
-  constexpr bool NEED_LO = delta<K2>(3) + 16 > 32;      // a window reaches past the first aligned word
-  constexpr bool NEED_W2 = 31 + delta<K2>(3) + 16 > 64; // ... and past the second stored word
-  const int p0 = 8 * L + 4 * h;
-  const int first = (stream_end<K2>(0) + p0 * K2 / 2 - 16 + R) % R;   // E(p0) - 16, p0 even so p0 * K2 / 2 is whole
-  const int wi = first >> 5, o = first & 31;
-  const uint32_t w0 = tile[wi], w1 = tile[(wi + 1) % TW];
-  const uint32_t hi = __funnelshift_l(w1, w0, o);       // the stream from the first window on, 32 bits
-  uint32_t lo = 0;
-  if constexpr (NEED_LO) {
-    const uint32_t w2 = NEED_W2 ? tile[(wi + 2) % TW] : 0u;
-    lo = __funnelshift_l(w2, w1, o);
+struct Windows {
+  static constexpr int TW = tile_words<K2>(), R = 32 * TW;
+  static constexpr bool NEED_LO = delta<K2>(3) + 16 > 32;      // a window reaches past the first aligned word
+  static constexpr bool NEED_W2 = 31 + delta<K2>(3) + 16 > 64; // ... and past the second stored word
+  static constexpr int NW = NEED_LO && NEED_W2 ? 3 : 2;
+  int wi, wi1, wi2, o;                                         // the words and the bit offset: the same for every tile
+  __device__ __forceinline__ Windows(int L, int h) {
+    const int p0 = 8 * L + 4 * h;
+    const int first = (stream_end<K2>(0) + p0 * K2 / 2 - 16 + R) % R;   // E(p0) - 16; p0 is even, p0 * K2 / 2 whole
+    wi = first >> 5;
+    wi1 = (wi + 1) % TW;
+    wi2 = (wi + 2) % TW;
+    o = first & 31;
   }
+  __device__ __forceinline__ void load(const uint32_t* tile, uint32_t (&w)[NW]) const {
+    w[0] = tile[wi];
+    w[1] = tile[wi1];
+    if constexpr (NW == 3) w[2] = tile[wi2];
+  }
+  // the 16-bit states of the four values
+  __device__ __forceinline__ void states(const uint32_t (&w)[NW], uint32_t (&s)[4]) const {
+    const uint32_t hi = __funnelshift_l(w[1], w[0], o);        // the stream from the first window on, 32 bits
+    uint32_t lo = 0;
+    if constexpr (NEED_LO) lo = __funnelshift_l(NW == 3 ? w[NW - 1] : 0u, w[1], o);
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int d = delta<K2>(j);
-    if (d + 16 <= 32) s[j] = (hi >> (16 - d)) & 0xFFFFu;
-    else if (d < 32) s[j] = __funnelshift_l(lo, hi, d) >> 16;
-    else s[j] = (lo >> (48 - d)) & 0xFFFFu;
+    for (int j = 0; j < 4; ++j) {
+      const int d = delta<K2>(j);
+      if (d + 16 <= 32) s[j] = (hi >> (16 - d)) & 0xFFFFu;
+      else if (d < 32) s[j] = __funnelshift_l(lo, hi, d) >> 16;
+      else s[j] = (lo >> (48 - d)) & 0xFFFFu;
+    }
   }
-}
+};
 
 // fp16 bits of the codebook value of state s
 template <int CB>
@@ -80,12 +92,26 @@ __device__ __forceinline__ uint16_t code_value(uint32_t s) {
   }
 }
 
+// the fp16 bits of the lane's four values of one tile, as two packed words
+template <int K2, int CB>
+__device__ __forceinline__ void decode4(const Windows<K2>& win, const uint32_t (&w)[Windows<K2>::NW], uint32_t& lo,
+                                        uint32_t& hi) {
+  uint32_t s[4];
+  win.states(w, s);
+  lo = (uint32_t)code_value<CB>(s[0]) | ((uint32_t)code_value<CB>(s[1]) << 16);
+  hi = (uint32_t)code_value<CB>(s[2]) | ((uint32_t)code_value<CB>(s[3]) << 16);
+}
+
 template <int K2, int CB>
 __device__ __forceinline__ void values4(const uint32_t* tile, int L, int h, uint16_t (&v)[4]) {
-  uint32_t s[4];
-  states4<K2>(tile, L, h, s);
-#pragma unroll
-  for (int j = 0; j < 4; ++j) v[j] = code_value<CB>(s[j]);
+  const Windows<K2> win(L, h);
+  uint32_t w[Windows<K2>::NW], lo, hi;
+  win.load(tile, w);
+  decode4<K2, CB>(win, w, lo, hi);
+  v[0] = (uint16_t)lo;
+  v[1] = (uint16_t)(lo >> 16);
+  v[2] = (uint16_t)hi;
+  v[3] = (uint16_t)(hi >> 16);
 }
 
 // Unscaled Walsh-Hadamard transform of 128 values, two a lane (elements 2 lane, 2 lane + 1), fixed butterfly order.
@@ -184,22 +210,39 @@ __global__ void __launch_bounds__(WK * 64)
     for (int j = 0; j < 8; ++j) acc[j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
     // the A operand's row: lane (row c, quarter kq); rows past the pass read a valid row and are dropped later
     const uint16_t* xr = xh + (size_t)(m0 + (c < R ? c : R - 1)) * K + 2 * kq;
-    for (int pr = pr0; pr < pr1; ++pr) {
+    // the stored words of the 16 tiles of a k-tile pair and the pair's activations are requested one pair ahead
+    constexpr int NW = Windows<K2>::NW;
+    const Windows<K2> win(L, h);
+    uint32_t wc[16][NW], wn[16][NW];
+    u32x4_t av, an;
+    auto fetch = [&](int pr, uint32_t (&w)[16][NW], u32x4_t& a) {
       const uint32_t* xk = reinterpret_cast<const uint32_t*>(xr + 32 * pr);
-      const u32x4_t av = {xk[0], xk[4], xk[8], xk[12]};
-      const f16x8_t a = __builtin_bit_cast(f16x8_t, av);
+      a = (u32x4_t){xk[0], xk[4], xk[8], xk[12]};
       const uint32_t* t0 = tiles + (size_t)(2 * pr) * stride_k;
-      const uint32_t* t1 = t0 + stride_k;
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        uint16_t v0[4], v1[4];
-        values4<K2, CB>(t0 + j * TW, L, h, v0);
-        values4<K2, CB>(t1 + j * TW, L, h, v1);
-        const u32x4_t bw = {(uint32_t)v0[0] | ((uint32_t)v0[1] << 16), (uint32_t)v0[2] | ((uint32_t)v0[3] << 16),
-                            (uint32_t)v1[0] | ((uint32_t)v1[1] << 16), (uint32_t)v1[2] | ((uint32_t)v1[3] << 16)};
+        win.load(t0 + j * TW, w[2 * j]);
+        win.load(t0 + stride_k + j * TW, w[2 * j + 1]);
+      }
+    };
+    if (pr0 < pr1) fetch(pr0, wc, av);
+    for (int pr = pr0; pr < pr1; ++pr) {
+      fetch(pr + 1 < pr1 ? pr + 1 : pr, wn, an);
+      const f16x8_t a = __builtin_bit_cast(f16x8_t, av);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        uint32_t b0, b1, b2, b3;
+        decode4<K2, CB>(win, wc[2 * j], b0, b1);
+        decode4<K2, CB>(win, wc[2 * j + 1], b2, b3);
+        const u32x4_t bw = {b0, b1, b2, b3};
         const f16x8_t b = __builtin_bit_cast(f16x8_t, bw);
         acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[j], 0, 0, 0);
       }
+#pragma unroll
+      for (int t = 0; t < 16; ++t)
+#pragma unroll
+        for (int q = 0; q < NW; ++q) wc[t][q] = wn[t][q];
+      av = an;
     }
     // D[row 4 kq + i][column c] of column tile j -> red[wave][row][16 j + c]
     __syncthreads();
@@ -218,15 +261,21 @@ __global__ void __launch_bounds__(WK * 64)
       }
       const size_t at = (size_t)(m0 + r) * N + col0 + 2 * lane;
       if (SK == 1) finish_row(s.x, s.y, lane, svh, bias, col0 + 2 * lane, y, y_dtype, at);
-      else *reinterpret_cast<float2*>(Z + (size_t)split * M * N + at) = s;
+      else {
+        // partial sums cross to another XCD's workgroup: agent-scope stores and loads are coherent by themselves
+        // (a cache-wide write-back or invalidate, which __threadfence would issue, costs far more than the sums)
+        float* zp = Z + (size_t)split * M * N + at;
+        __hip_atomic_store(zp, s.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(zp + 1, s.y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
     }
     if (SK > 1) {
-      __threadfence();
-      __syncthreads();
-      if (threadIdx.x == 0) last = atomicAdd(counters + pass * NB + nb, 1) == SK - 1;
+      __builtin_amdgcn_s_waitcnt(0);        // this wave's stores are acknowledged ...
+      __syncthreads();                      // ... every wave's are ...
+      if (threadIdx.x == 0)                 // ... then the block counts itself in
+        last = __hip_atomic_fetch_add(counters + pass * NB + nb, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == SK - 1;
       __syncthreads();
       if (last) {
-        __threadfence();
         for (int r = wave; r < R; r += WK) {
           const size_t at = (size_t)(m0 + r) * N + col0 + 2 * lane;
           float sx = __hip_atomic_load(Z + at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -25,17 +25,18 @@ def k2_of(bits: float) -> int:
     return int(2 * fmt.check_bits(bits))
 
 
-def plan(k: int, n: int, blocks: int = 512, min_pairs: int = 4) -> tuple[int, int]:
+def plan(k: int, n: int, waves: int = 4608, min_pairs: int = 4) -> tuple[int, int]:
     """(K splits, waves a workgroup) of a K x N layer, from the shape alone so that a layer keeps one reduction
-    order at every row count.  An MI355X wants about two workgroups on each of its 256 CUs: K is split until
-    N/128 * splits reaches ``blocks`` while every wave keeps ``min_pairs`` pairs of k tiles."""
+    order at every row count.  The decode is arithmetic-bound and wants about four waves on each of an MI355X's
+    1,024 SIMDs: K is split while N/128 * splits * 4 stays within ``waves`` and every wave keeps ``min_pairs`` pairs
+    of k tiles."""
 
     pairs, nb = k // 32, n // 128
     wk = 4
     while wk > 2 and pairs // wk < min_pairs:
         wk //= 2
     sk = 1
-    while sk < 64 and nb * sk < blocks and pairs // (2 * sk * wk) >= min_pairs:
+    while sk < 64 and nb * 2 * sk * wk <= waves and pairs // (2 * sk * wk) >= min_pairs:
         sk *= 2
     return sk, wk
 
