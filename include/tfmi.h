@@ -58,6 +58,14 @@ int tf_group_sums(const uint16_t* x, int64_t ldx, int m, int k, int gs, float* x
 int tf_qmm(const uint16_t* x, int64_t ldx, const float* xs, const uint32_t* weight, const uint16_t* scales,
            const uint16_t* biases, int64_t sb_stride, void* out, float* part, int m, int n, int k, int sk, int gs,
            int bm, int f32, int reduce, tf_stream_t stream);
+/* `count` (1 to 4) weights against one x in one launch (plus one reduce launch when any K is split): the bits of
+ * tf_qmm on each.  The arrays are host arrays of `count` entries, read during the call: packed weights, transposed
+ * scales and biases with their row strides, outputs, parts (fp32 [sks[i], m, ns[i]], may be NULL where sks[i] == 1),
+ * column counts and slice counts.  Replaces kernels/qmm.cpp:51-80 `qmm_group`. */
+int tf_qmm_group(const uint16_t* x, int64_t ldx, const float* xs, int count, const uint32_t* const* weights,
+                 const uint16_t* const* scales, const uint16_t* const* biases, const int64_t* sb_strides,
+                 void* const* outs, float* const* parts, const int* ns, const int* sks, int m, int k, int gs, int bm,
+                 int f32, tf_stream_t stream);
 /* Prompt-form matmul on f16 MFMA: each weight rounded once (256 w to fp16; the reference rounds w to bf16), one
  * fp32 chain over K.  Replaces kernels/qmm.cpp:83-102 `qmm_prefill`. */
 int tf_qmm_prefill(const uint16_t* x, int64_t ldx, const uint32_t* weight, const uint16_t* scales,

@@ -112,14 +112,13 @@ __device__ __forceinline__ void qmm_pass(const uint16_t* __restrict__ X, int64_t
 // grid (column tiles of 64 x row tiles of BM, 1, SK).  Slice z takes groups [z * per, (z + 1) * per), its waves
 // split them again (added in wave order); SK > 1 leaves the slice's fp32 sums in part[z].  Rows go in passes of 2 or 1.
 template <int GS, int WAVES>
-__global__ void __launch_bounds__(WAVES * 64)
-    qmm_kernel(const uint16_t* __restrict__ X, int64_t ldx, const float* __restrict__ XS,
-               const uint32_t* __restrict__ W, const uint16_t* __restrict__ S, const uint16_t* __restrict__ B,
-               int64_t sb_stride, void* __restrict__ out, float* __restrict__ part_out, int M, int N, int KG, int SK,
-               int BM, int f32) {
-  extern __shared__ float lds[];            // partials [WAVES][RBMAX][64]
+__device__ __forceinline__ void qmm_block(const uint16_t* __restrict__ X, int64_t ldx, const float* __restrict__ XS,
+                                          const uint32_t* __restrict__ W, const uint16_t* __restrict__ S,
+                                          const uint16_t* __restrict__ B, int64_t sb_stride, void* __restrict__ out,
+                                          float* __restrict__ part_out, int M, int N, int KG, int SK, int BM, int f32,
+                                          int block, int slice, float* lds) {
   const int tiles = (N + 63) >> 6;
-  const int tile = blockIdx.x % tiles, rt = blockIdx.x / tiles, slice = blockIdx.z;
+  const int tile = block % tiles, rt = block / tiles;
   const int per = KG / SK, gs0 = slice * per;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   constexpr int CH = GS / 32;
@@ -151,6 +150,61 @@ __global__ void __launch_bounds__(WAVES * 64)
     TF_QMM_PASS(1);
   }
 #undef TF_QMM_PASS
+}
+
+template <int GS, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64)
+    qmm_kernel(const uint16_t* __restrict__ X, int64_t ldx, const float* __restrict__ XS,
+               const uint32_t* __restrict__ W, const uint16_t* __restrict__ S, const uint16_t* __restrict__ B,
+               int64_t sb_stride, void* __restrict__ out, float* __restrict__ part_out, int M, int N, int KG, int SK,
+               int BM, int f32) {
+  extern __shared__ float lds[];            // partials [WAVES][RBMAX][64]
+  qmm_block<GS, WAVES>(X, ldx, XS, W, S, B, sb_stride, out, part_out, M, N, KG, SK, BM, f32, blockIdx.x, blockIdx.z, lds);
+}
+
+// Up to four weights against one x in one launch (and one reduce launch): workgroups [first[w], first[w + 1]) take
+// weight w's (column tile, row tile) pairs; grid.z is the largest slice count and a weight's surplus slices leave.
+constexpr int GROUP_MAX = 4;
+struct GroupArgs {
+  const uint32_t* w[GROUP_MAX];
+  const uint16_t* s[GROUP_MAX];
+  const uint16_t* b[GROUP_MAX];
+  void* out[GROUP_MAX];
+  float* part[GROUP_MAX];
+  int64_t sb_stride[GROUP_MAX];
+  int n[GROUP_MAX], sk[GROUP_MAX];
+  int first[GROUP_MAX + 1];      // workgroups (matmul) or 256-element chunks (reduce) before weight w
+  int count;
+};
+
+template <int GS, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64)
+    qmm_group_kernel(const uint16_t* __restrict__ X, int64_t ldx, const float* __restrict__ XS, GroupArgs a, int M,
+                     int KG, int BM, int f32) {
+  extern __shared__ float lds[];
+  int w = 0;
+#pragma unroll
+  for (int i = 1; i < GROUP_MAX; ++i)
+    if (i < a.count && (int)blockIdx.x >= a.first[i]) w = i;
+  if ((int)blockIdx.z >= a.sk[w]) return;
+  qmm_block<GS, WAVES>(X, ldx, XS, a.w[w], a.s[w], a.b[w], a.sb_stride[w], a.out[w], a.part[w], M, a.n[w], KG, a.sk[w],
+                       BM, f32, blockIdx.x - a.first[w], blockIdx.z, lds);
+}
+
+__global__ void qmm_group_reduce_kernel(GroupArgs a, int M, int f32) {
+  int w = 0;
+#pragma unroll
+  for (int i = 1; i < GROUP_MAX; ++i)
+    if (i < a.count && (int)blockIdx.x >= a.first[i]) w = i;
+  if (a.sk[w] == 1) return;
+  const long long total = (long long)M * a.n[w];
+  const long long i = (long long)(blockIdx.x - a.first[w]) * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const float* part = a.part[w];
+  float acc = part[i];
+  for (int s = 1; s < a.sk[w]; ++s) acc = acc + part[s * total + i];
+  if (f32) reinterpret_cast<float*>(a.out[w])[i] = acc;
+  else reinterpret_cast<uint16_t*>(a.out[w])[i] = (uint16_t)f32_bf16_bits(acc);
 }
 
 // the K slices' partial sums added in slice order, then rounded once (qmm.cu:222-230)
@@ -327,6 +381,67 @@ extern "C" int tf_qmm(const uint16_t* x, int64_t ldx, const float* xs, const uin
     const long long total = (long long)m * n;
     qmm_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(part, out, total, sk, f32);
     TF_LAUNCH_OK("tf_qmm reduce");
+  }
+  return 0;
+}
+
+extern "C" int tf_qmm_group(const uint16_t* x, int64_t ldx, const float* xs, int count, const uint32_t* const* weights,
+                            const uint16_t* const* scales, const uint16_t* const* biases, const int64_t* sb_strides,
+                            void* const* outs, float* const* parts, const int* ns, const int* sks, int m, int k, int gs,
+                            int bm, int f32, tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(gs == 32 || gs == 64, "groups of 32 or 64");
+  TF_REQUIRE(bm == 16 || bm == 32 || bm == 64, "row tile 16, 32 or 64");
+  TF_REQUIRE(count >= 1 && count <= GROUP_MAX, "qmm_group: 1 to %d weights, not %d", GROUP_MAX, count);
+  TF_REQUIRE(x && xs && weights && scales && biases && sb_strides && outs && parts && ns && sks && m >= 1,
+             "qmm_group: null pointer or empty shape");
+  TF_REQUIRE(aligned16(x) && (m == 1 || ldx % 8 == 0), "x rows must start on 16-byte boundaries");
+  TF_REQUIRE(ldx >= k || m == 1, "x: (M, K) bf16 with contiguous rows");
+  TF_REQUIRE(k % gs == 0, "K splits into whole groups a slice");
+  const int kg = k / gs, rts = (m + bm - 1) / bm;
+  GroupArgs a{}, r{};
+  int max_sk = 1;
+  int64_t blocks = 0, chunks = 0;
+  bool any_split = false;
+  for (int i = 0; i < count; ++i) {
+    const int n = ns[i], sk = sks[i], npad = (n + 127) / 128 * 128;
+    TF_REQUIRE(weights[i] && scales[i] && biases[i] && outs[i] && n >= 1, "qmm_group: null pointer or empty shape");
+    TF_REQUIRE(sk >= 1 && sk <= 65535 && kg % sk == 0, "K splits into whole groups a slice");
+    TF_REQUIRE(sb_strides[i] >= npad, "scales and biases: (K / gs, n padded to 128) bf16, rows may be strided");
+    TF_REQUIRE(aligned16(weights[i]), "packed weight must be 16-byte aligned");
+    TF_REQUIRE(sk == 1 || parts[i], "part: at least (SK, M, n) fp32 is needed when K is split");
+    a.w[i] = weights[i];
+    a.s[i] = scales[i];
+    a.b[i] = biases[i];
+    a.out[i] = outs[i];
+    a.part[i] = parts[i];
+    a.sb_stride[i] = sb_strides[i];
+    a.n[i] = n;
+    a.sk[i] = sk;
+    a.first[i] = (int)blocks;
+    r.first[i] = (int)chunks;
+    blocks += (int64_t)((n + 63) / 64) * rts;
+    chunks += ((int64_t)m * n + 255) / 256;
+    TF_REQUIRE(blocks <= 0x7FFFFFFF && chunks <= 0x7FFFFFFF, "qmm_group: grid too large");
+    max_sk = sk > max_sk ? sk : max_sk;
+    any_split = any_split || sk > 1;
+  }
+  a.count = count;
+  a.first[count] = (int)blocks;
+  hipStream_t s = as_stream(stream);
+  const size_t smem = sizeof(float) * ((size_t)QMM_WAVES * RBMAX * 64);
+  const dim3 grid((unsigned)blocks, 1, (unsigned)max_sk);
+  if (gs == 64) qmm_group_kernel<64, QMM_WAVES><<<grid, QMM_WAVES * 64, smem, s>>>(x, ldx, xs, a, m, kg, bm, f32);
+  else qmm_group_kernel<32, QMM_WAVES><<<grid, QMM_WAVES * 64, smem, s>>>(x, ldx, xs, a, m, kg, bm, f32);
+  TF_LAUNCH_OK("tf_qmm_group");
+  if (any_split) {
+    int first[GROUP_MAX + 1];
+    for (int i = 0; i < count; ++i) first[i] = r.first[i];
+    r = a;
+    for (int i = 0; i < count; ++i) r.first[i] = first[i];
+    r.first[count] = (int)chunks;
+    qmm_group_reduce_kernel<<<(unsigned)chunks, 256, 0, s>>>(r, m, f32);
+    TF_LAUNCH_OK("tf_qmm_group reduce");
   }
   return 0;
 }

@@ -145,6 +145,49 @@ def matmul(x: torch.Tensor, q: Q4, xs: torch.Tensor | None = None, *, sk: int | 
     return part.reshape(-1)[:sk * m * q.n].view(sk, m, q.n)
 
 
+def matmul_group(x: torch.Tensor, qs: list[Q4], xs: torch.Tensor | None = None, *, f32: bool = False,
+                 sks: list[int] | None = None, outs: list[torch.Tensor] | None = None,
+                 parts: list[torch.Tensor | None] | None = None) -> list[torch.Tensor]:
+    """``[matmul(x, q) for q in qs]`` for one to four weights of the same K and group size in one launch (plus one
+    reduce launch), same bits.  ``outs`` and ``parts`` may bring preallocated buffers (a part where sks[i] > 1)."""
+
+    import ctypes
+
+    if not 1 <= len(qs) <= 4:
+        raise ValueError("matmul_group: one to four weights")
+    if x.dtype != torch.bfloat16 or x.dim() != 2 or any(x.shape[1] != q.k for q in qs):
+        raise ValueError("matmul_group: x must be (M, K) bf16 with every weight's K")
+    if any(q.gs != qs[0].gs for q in qs):
+        raise ValueError("matmul_group: the weights must share a group size")
+    x = _check_x(x, qs[0], "matmul_group")
+    m, gs, k = int(x.shape[0]), qs[0].gs, qs[0].k
+    xs = group_sums(x, gs) if xs is None else xs
+    if xs.dtype != torch.float32 or tuple(xs.shape) != (m, k // gs) or not xs.is_contiguous() or xs.device != x.device:
+        raise ValueError(f"matmul_group: xs must be contiguous fp32 ({m}, {k // gs}), the group sums of x")
+    sks = list(sks) if sks else [split_k(q.n, q.k, q.gs) for q in qs]
+    dtype = torch.float32 if f32 else torch.bfloat16
+    if outs is None:
+        outs = [x.new_empty((m, q.n), dtype=dtype) for q in qs]
+    parts = list(parts) if parts else [None] * len(qs)
+    if len(sks) != len(qs) or len(outs) != len(qs) or len(parts) != len(qs):
+        raise ValueError("matmul_group: one slice count, output and part a weight")
+    for i, (q, sk, out) in enumerate(zip(qs, sks, outs)):
+        if tuple(out.shape) != (m, q.n) or out.dtype != dtype or not out.is_contiguous() or out.device != x.device:
+            raise ValueError(f"matmul_group: outs[{i}] must be contiguous ({m}, {q.n}) {'fp32' if f32 else 'bf16'}")
+        if sk > 1 and parts[i] is None:
+            parts[i] = x.new_empty((sk, m, q.n), dtype=torch.float32)
+        elif sk > 1 and (parts[i].dtype != torch.float32 or parts[i].numel() < sk * m * q.n
+                         or not parts[i].is_contiguous() or parts[i].device != x.device):
+            raise ValueError(f"matmul_group: parts[{i}] must hold {sk} x {m} x {q.n} fp32 values")
+    n = len(qs)
+    ptrs = lambda ts: (ctypes.c_void_p * n)(*[None if t is None else t.data_ptr() for t in ts])
+    _lib.call("tf_qmm_group", _lib.ptr(x), x.stride(0), _lib.ptr(xs), n, ptrs([q.weight for q in qs]),
+              ptrs([q.scales for q in qs]), ptrs([q.biases for q in qs]),
+              (ctypes.c_int64 * n)(*[q.scales.stride(0) for q in qs]), ptrs(outs), ptrs(parts),
+              (ctypes.c_int * n)(*[q.n for q in qs]), (ctypes.c_int * n)(*sks), m, k, gs, bucket(m), int(f32))
+    return outs
+
+
 def prefill_matmul(x: torch.Tensor, q: Q4, *, f32: bool = False, tile: int = 0,
                    out: torch.Tensor | None = None) -> torch.Tensor:
     """Prompt-form x @ W.T on bf16 MFMA: every weight is rounded to bf16 once and K is one fp32 chain, so chunking a

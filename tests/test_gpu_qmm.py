@@ -123,6 +123,29 @@ def test_strided_rows_buffers_and_unreduced_slices():
     assert torch.equal(total, qmm.matmul(x, q, f32=True))
 
 
+@pytest.mark.parametrize("m", [1, 3, 17])
+def test_grouped_launch_has_the_bits_of_single_calls(m):
+    """Up to four weights against one x in one launch (after tests/cuda/test_qmm_group.py): each output equals
+    matmul's bit for bit, for mixed widths and slice counts, bf16 and fp32."""
+
+    k = 2048
+    x = gpu(synthetic.activations(m, k, 50 + m))[0]
+    for gs, ns in ((64, (256, 1024, 96, 4096)), (32, (128, 640)), (64, (512,))):
+        qs = [qmm.pack(*gpu(*synthetic.affine_general(n, k, gs, 60 + n)), gs) for n in ns]
+        for f32 in (False, True):
+            got = qmm.matmul_group(x, qs, f32=f32)
+            for q, y in zip(qs, got):
+                assert torch.equal(y, qmm.matmul(x, q, f32=f32)), (gs, q.n, f32)
+        sks = [1] + [2] * (len(qs) - 1)
+        got = qmm.matmul_group(x, qs, sks=sks)
+        for q, sk, y in zip(qs, sks, got):
+            assert torch.equal(y, qmm.matmul(x, q, sk=sk))
+    with pytest.raises(ValueError):
+        qmm.matmul_group(x, [])
+    with pytest.raises(ValueError):
+        qmm.matmul_group(x, [qs[0]] * 5)
+
+
 def test_group_sums():
     x = synthetic.activations(5, 2048, 3).to(DEV)
     for gs in (32, 64):
