@@ -43,7 +43,7 @@ __device__ __forceinline__ void st_agent(T* p, T v) {
 constexpr int COH_IN = 1, COH_OUT = 2;     // which side of a unit goes through agent-scope accesses
 
 constexpr int SLICES = 16;      // K slices of the expert GEMV
-constexpr int DEPTH = 3;        // groups of weights a wave keeps in flight
+constexpr int DEPTH = 2;        // groups of weights a wave keeps in flight
 constexpr int RBMAX = 2;        // rows a pass
 
 // fp32 sums of each group of GS inputs of `rows` rows, for groups [0, KG), into xs[r * KG + g].

@@ -210,7 +210,7 @@ __device__ __forceinline__ int wave_scan(int x) {
 // spread an expert that many rows share over more workgroups).  int32 rows of DESC: row 0 holds the number of
 // descriptors, row 1 + i = {expert, count, first member, 0, pairs[DTILE]}.
 constexpr int DESC = 8;
-constexpr int DTILE = 4;
+constexpr int DTILE = 2;
 
 // ---- one item of the plan, found by every workgroup for itself -----------------------------------------------------
 //

@@ -25,7 +25,7 @@ FUSED_DECODE = os.environ.get("TENSORFOLD_AMD_FUSED_DECODE", "0") == "1"
 ROUTE_UP_LOGITS = 2048
 # Item descriptors the routing launches leave for the decode expert kernels: rows of DESC_INTS int32, row 0 the
 # count; items of at most DESC_TILE pairs (TF_DESC_INTS / TF_DESC_TILE of the C header).
-DESC_INTS, DESC_TILE = 8, 4
+DESC_INTS, DESC_TILE = 8, 2
 
 
 def router(x: torch.Tensor, rows: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
