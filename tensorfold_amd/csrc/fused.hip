@@ -122,16 +122,39 @@ __global__ void __launch_bounds__(WAVES * 64)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, threads = WAVES * 64;
   const int slots = TOPK + (shared ? 1 : 0), P = R * slots, E = NE + (shared ? 1 : 0);
   const bool writer = blockIdx.x == 0;
-  for (int r = wave; r < R; r += WAVES) {
-    int id;
-    float w;
-    topk_lane(L + (size_t)r * ldl, NE, TOPK, shared, lane, id, w);
+  auto keep = [&](int r, int id, float w) {
     if (lane < slots) {
       pk[r * slots + lane] = (unsigned)id < (unsigned)E ? id : -1;
       if (writer) {
         pick[r * slots + lane] = id;
         wts[r * slots + lane] = w;
       }
+    }
+  };
+  if (NE <= 128) {
+    // a wave's rows two at a time: both requested, then ranked together
+    for (int r = wave; r < R; r += 2 * WAVES) {
+      const int r2 = r + WAVES;
+      float v[2], v2[2];
+      topk_load<2>(L + (size_t)r * ldl, NE, lane, v);
+      if (r2 < R) topk_load<2>(L + (size_t)r2 * ldl, NE, lane, v2);
+      int id, id2;
+      float w, w2;
+      if (r2 < R) {
+        topk_pick2<2>(v, v2, L + (size_t)r * ldl, L + (size_t)r2 * ldl, NE, TOPK, shared, lane, id, w, id2, w2);
+        keep(r, id, w);
+        keep(r2, id2, w2);
+      } else {
+        topk_pick<2>(v, L + (size_t)r * ldl, NE, TOPK, shared, lane, id, w);
+        keep(r, id, w);
+      }
+    }
+  } else {
+    for (int r = wave; r < R; r += WAVES) {
+      int id;
+      float w;
+      topk_lane(L + (size_t)r * ldl, NE, TOPK, shared, lane, id, w);
+      keep(r, id, w);
     }
   }
   __syncthreads();

@@ -40,7 +40,7 @@ template <int VPL>
 __device__ __forceinline__ void topk_pick(float (&v)[VPL], const float* __restrict__ row, int NE, int TOPK, int shared,
                                           int lane, int& id, float& w) {
   const float NEG = -__builtin_inff();
-  float top = 0.f, total = 0.f, mine_ex = 0.f;
+  float mine_m = 0.f;
   int mine_id = 0;
   for (int k = 0; k < TOPK; ++k) {
     float bv = v[0];
@@ -60,11 +60,8 @@ __device__ __forceinline__ void topk_pick(float (&v)[VPL], const float* __restri
       idx = min(idx, __builtin_amdgcn_readlane(bi, l));
       cand &= cand - 1;
     }
-    if (k == 0) top = m;
-    const float ex = expf(m - top);
-    total += ex;
     if (lane == k) {
-      mine_ex = ex;
+      mine_m = m;
       mine_id = idx;
     }
     if ((idx & 63) == lane) {
@@ -73,13 +70,88 @@ __device__ __forceinline__ void topk_pick(float (&v)[VPL], const float* __restri
         if (i == (idx >> 6)) v[i] = NEG;
     }
   }
+  // weights: exp(l_k - l_0) over their sum, added in pick order (lane k holds pick k)
+  const float top = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine_m), 0));
+  const float ex = expf(mine_m - top);
+  float total = 0.f;
+  for (int k = 0; k < TOPK; ++k)
+    total += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ex), k));
   id = mine_id;
-  w = round_bf16(mine_ex / total);
+  w = round_bf16(ex / total);
   if (shared && lane == TOPK) {
     const float sg = round_bf16(row[NE]);
     id = NE;
     w = round_bf16(1.f / (1.f + expf(-sg)));
   }
+}
+
+// Two rows at once on one wave: the same arithmetic as topk_pick on each, with the two dependent chains interleaved
+template <int VPL>
+__device__ __forceinline__ void topk_pick2(float (&va)[VPL], float (&vb)[VPL], const float* __restrict__ rowa,
+                                           const float* __restrict__ rowb, int NE, int TOPK, int shared, int lane,
+                                           int& ida, float& wa, int& idb, float& wb) {
+  const float NEG = -__builtin_inff();
+  float mma = 0.f, mmb = 0.f;
+  int mia = 0, mib = 0;
+  auto best = [&](const float (&v)[VPL], float& bv, int& bi) {
+    bv = v[0];
+    bi = lane;
+#pragma unroll
+    for (int i = 1; i < VPL; ++i)
+      if (v[i] > bv) {
+        bv = v[i];
+        bi = lane + 64 * i;
+      }
+  };
+  auto lowest = [&](unsigned long long cand, int bi) {
+    int idx = 0x7FFFFFFF;
+    while (cand) {
+      const int l = __builtin_ctzll(cand);
+      idx = min(idx, __builtin_amdgcn_readlane(bi, l));
+      cand &= cand - 1;
+    }
+    return idx;
+  };
+  auto drop = [&](float (&v)[VPL], int idx) {
+    if ((idx & 63) == lane) {
+#pragma unroll
+      for (int i = 0; i < VPL; ++i)
+        if (i == (idx >> 6)) v[i] = NEG;
+    }
+  };
+  for (int k = 0; k < TOPK; ++k) {
+    float bva, bvb;
+    int bia, bib;
+    best(va, bva, bia);
+    best(vb, bvb, bib);
+    const float ma = wave_max(bva), mb = wave_max(bvb);
+    const int xa = lowest(__ballot(bva == ma), bia), xb = lowest(__ballot(bvb == mb), bib);
+    if (lane == k) {
+      mma = ma;
+      mia = xa;
+      mmb = mb;
+      mib = xb;
+    }
+    drop(va, xa);
+    drop(vb, xb);
+  }
+  auto weight = [&](float mine_m, const float* row, int& id, float& w) {
+    const float top = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine_m), 0));
+    const float ex = expf(mine_m - top);
+    float total = 0.f;
+    for (int k = 0; k < TOPK; ++k)
+      total += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ex), k));
+    w = round_bf16(ex / total);
+    if (shared && lane == TOPK) {
+      const float sg = round_bf16(row[NE]);
+      id = NE;
+      w = round_bf16(1.f / (1.f + expf(-sg)));
+    }
+  };
+  ida = mia;
+  idb = mib;
+  weight(mma, rowa, ida, wa);
+  weight(mmb, rowb, idb, wb);
 }
 
 template <int VPL>
