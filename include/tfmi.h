@@ -134,12 +134,21 @@ int tf_moe_combine(const void* y, int y_bf16, const float* wts, uint16_t* out, i
  * writes what tf_moe_topk and tf_experts_plan (tile 16) would (pick, wts, members, items, counts) plus the item
  * descriptors that tf_experts_run_desc reads; every other workgroup finds its own item from the
  * logits and runs the up unit of tf_experts_run (epilogue relu^2, or SwiGLU when swiglu != 0): act bf16 [pairs, ni] and
- * its group sums xs_act fp32 [pairs, ni / gs].  Same bits as the separate calls.  No counterpart in the reference
+ * its group sums xs_act fp32 [pairs, ni / gs]; it also zeroes `zero` (n_zero ints: the next launch's counters).  Same
+ * bits as the separate calls.  No counterpart in the reference
  * (moe.py:88-128 issues them one by one). */
 int tf_moe_route_up(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared, int gs, int swiglu,
                     const uint16_t* x, int64_t x_stride, const uint32_t* up, int d, int ni, int32_t* pick, float* wts,
                     int32_t* members, int32_t* items, int32_t* counts, int32_t* desc, uint16_t* act, float* xs_act,
-                    float limit, int max_items, tf_stream_t stream);
+                    float limit, int max_items, int32_t* zero, int n_zero, tf_stream_t stream);
+/* The down projection from item descriptors with the weighted combine folded in: y fp32 [pairs, d] as
+ * tf_experts_run_desc (epilogue 0) writes it, and out bf16 [rows, d] with the bits of tf_moe_combine, written by
+ * whichever workgroup completes a (token, 64 columns) cell.  `arrive` int32 [rows * ceil(d / 64)] must be zero on
+ * entry (tf_moe_route_up and tf_moe_route_decode clear a `zero` range for this) and is left non-zero.  Fuses
+ * experts.cpp:43-48 `run` and moe.py:131-151 `combine`. */
+int tf_moe_down_combine(int gs, const uint16_t* act, int rows, int slots, const uint32_t* down, int d, int ni,
+                        const int32_t* desc, const float* wts, const float* xs_act, float* y, uint16_t* out,
+                        int32_t* arrive, int max_items, tf_stream_t stream);
 /* The decode layer's routing in one launch, for rows * (top_k + shared) <= 1024: tf_moe_topk, tf_experts_plan (tile
  * 16) and tf_group_sums of x, plus the item descriptors and the
  * zeroing of `zero` (n_zero ints: the counters of tf_moe_decode_experts).  No counterpart in the reference, which

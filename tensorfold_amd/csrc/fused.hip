@@ -42,6 +42,58 @@ struct WaitItem {
   }
 };
 
+// A down unit has written its 64 columns of y (agent-scope stores) for its rows: count it in each row's token; the
+// unit that completes a (token, 64 columns) cell adds the token's slots in slot order (fp32 fma, as tf_moe_combine)
+// and writes bf16.  `arrive` [tokens * NB2d] starts at zero.
+template <int WAVES>
+__device__ __forceinline__ void combine_cells(const int* pairs, int* last, int cnt, int slots, int cb2, int NB2d, int D,
+                                              const float* __restrict__ wts, const float* __restrict__ y,
+                                              uint16_t* __restrict__ out, int* __restrict__ arrive) {
+  const int tid = threadIdx.x;
+  __builtin_amdgcn_s_waitcnt(0);      // every store of this wave is acknowledged ...
+  __syncthreads();                    // ... of every wave ...
+  if (tid < cnt) {                    // ... then the unit counts itself in
+    const int token = pairs[tid] / slots;
+    last[tid] = __hip_atomic_fetch_add(arrive + (size_t)token * NB2d + cb2, 1, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT) == slots - 1;
+  }
+  __syncthreads();
+  const int lane = tid & 63, wave = tid >> 6;
+  const int col = cb2 * 64 + lane;
+  for (int r = wave; r < cnt; r += WAVES) {
+    if (!last[r] || col >= D) continue;
+    const int token = pairs[r] / slots;
+    float a = 0.f;
+    for (int k = 0; k < slots; ++k) {
+      const float w = wts[(size_t)token * slots + k];
+      a = fmaf(w, ld_agent(y + ((size_t)token * slots + k) * D + col), a);
+    }
+    out[(size_t)token * D + col] = (uint16_t)f32_bf16_bits(a);
+  }
+}
+
+// The down projection from item descriptors with the combine folded in (see combine_cells).
+template <int GS, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64)
+    down_combine_kernel(const uint16_t* __restrict__ act, int slots, const uint32_t* __restrict__ Wdown, int D, int NI,
+                        const int* __restrict__ desc, const float* __restrict__ wts, const float* __restrict__ xs_act,
+                        float* __restrict__ y, uint16_t* __restrict__ out, int* __restrict__ arrive) {
+  extern __shared__ float lds[];
+  __shared__ int pairs[16];
+  __shared__ int last[16];
+  const int NB = D / 32, NB2d = (NB + 1) >> 1;
+  const int it = blockIdx.x / NB2d, cb2 = blockIdx.x - it * NB2d;
+  if (it >= desc[0]) return;
+  const int* d = desc + (size_t)(1 + it) * DESC;
+  const int e = d[0], cnt = d[1];
+  if (threadIdx.x < DTILE) pairs[threadIdx.x] = d[4 + threadIdx.x];
+  __syncthreads();
+  NoHook none;
+  expert_unit<GS, 1, 0, WAVES, true, COH_OUT>(act, NI, 0, Wdown, NI / GS, NB, e, cnt, pairs, cb2, y, D, 0.f, xs_act,
+                                              nullptr, lds, none);
+  combine_cells<WAVES>(pairs, last, cnt, slots, cb2, NB2d, D, wts, y, out, arrive);
+}
+
 template <int GS, int NM, int EPI_UP, int WAVES>
 __global__ void __launch_bounds__(WAVES * 64)
     moe_fused_kernel(const uint16_t* __restrict__ X, int64_t x_stride, int slots, const uint32_t* __restrict__ Wup,
@@ -78,27 +130,7 @@ __global__ void __launch_bounds__(WAVES * 64)
   if (!expert_unit<GS, 1, 0, WAVES, true, DCOH>(act, NI, 0, Wdown, NI / GS, D / 32, e, cnt, pairs, cb2, y, D,
                                                             0.f, xs_act, nullptr, lds, wait))
     return;                     // the wait ran out: status is set, nothing is published
-  // this unit's 64 columns of y are written for its rows: count it in each row's token; the last one combines
-  __builtin_amdgcn_s_waitcnt(0);
-  __syncthreads();
-  if (tid < cnt) {
-    const int token = pairs[tid] / slots;
-    last[tid] = __hip_atomic_fetch_add(arrive + (size_t)token * NB2d + cb2, 1, __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT) == slots - 1;
-  }
-  __syncthreads();
-  const int lane = tid & 63, wave = tid >> 6;
-  const int col = cb2 * 64 + lane;
-  for (int r = wave; r < cnt; r += WAVES) {
-    if (!last[r] || col >= D) continue;
-    const int token = pairs[r] / slots;
-    float a = 0.f;
-    for (int k = 0; k < slots; ++k) {
-      const float w = wts[(size_t)token * slots + k];
-      a = fmaf(w, ld_agent(y + ((size_t)token * slots + k) * D + col), a);
-    }
-    out[(size_t)token * D + col] = (uint16_t)f32_bf16_bits(a);
-  }
+  combine_cells<WAVES>(pairs, last, cnt, slots, cb2, NB2d, D, wts, y, out, arrive);
 }
 
 
@@ -115,7 +147,8 @@ __global__ void __launch_bounds__(WAVES * 64)
                     const uint16_t* __restrict__ X, int64_t x_stride, const uint32_t* __restrict__ Wup, int D, int NI,
                     int* __restrict__ pick, float* __restrict__ wts, int* __restrict__ members,
                     int* __restrict__ items, int* __restrict__ counts, int* __restrict__ desc,
-                    uint16_t* __restrict__ act, float* __restrict__ xs_act, float limit) {
+                    uint16_t* __restrict__ act, float* __restrict__ xs_act, float limit, int* __restrict__ zero,
+                    int n_zero) {
   extern __shared__ float lds[];
   __shared__ int pk[PLAN_THREADS];
   __shared__ ItemLds item;
@@ -131,22 +164,19 @@ __global__ void __launch_bounds__(WAVES * 64)
       }
     }
   };
-  if (NE <= 128) {
-    // a wave's rows two at a time: both requested, then ranked together
-    for (int r = wave; r < R; r += 2 * WAVES) {
-      const int r2 = r + WAVES;
-      float v[2], v2[2];
-      topk_load<2>(L + (size_t)r * ldl, NE, lane, v);
-      if (r2 < R) topk_load<2>(L + (size_t)r2 * ldl, NE, lane, v2);
-      int id, id2;
-      float w, w2;
-      if (r2 < R) {
-        topk_pick2<2>(v, v2, L + (size_t)r * ldl, L + (size_t)r2 * ldl, NE, TOPK, shared, lane, id, w, id2, w2);
-        keep(r, id, w);
-        keep(r2, id2, w2);
-      } else {
-        topk_pick<2>(v, L + (size_t)r * ldl, NE, TOPK, shared, lane, id, w);
-        keep(r, id, w);
+  if (NE <= 128 && slots <= 16 && R > WAVES) {
+    // more rows than waves: four logits rows a wave, each on a row of 16 lanes
+    for (int r0 = 4 * wave; r0 < R; r0 += 4 * WAVES) {
+      const int r = r0 + (lane >> 4);
+      int id;
+      float w;
+      topk_row16(r < R ? L + (size_t)r * ldl : nullptr, NE, TOPK, shared, lane, id, w);
+      if (r < R && (lane & 15) < slots) {
+        pk[r * slots + (lane & 15)] = (unsigned)id < (unsigned)E ? id : -1;
+        if (writer) {
+          pick[r * slots + (lane & 15)] = id;
+          wts[r * slots + (lane & 15)] = w;
+        }
       }
     }
   } else {
@@ -159,6 +189,7 @@ __global__ void __launch_bounds__(WAVES * 64)
   }
   __syncthreads();
   if (writer) {
+    for (int i = tid; i < n_zero; i += threads) zero[i] = 0;      // the next launch's arrival counters
     // the whole plan: first member and first item of every expert (wave 0 scans), then items, members, descriptors
     int* off = reinterpret_cast<int*>(lds);
     int* itoff = off + EMAX;
@@ -229,7 +260,7 @@ template <int GS, int NM, int EPI>
 int launch_route_up(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared, const uint16_t* x,
                     int64_t x_stride, const uint32_t* wup, int d, int ni, int* pick, float* wts, int* members,
                     int* items, int* counts, int* desc, uint16_t* act, float* xs_act, float limit, int max_items,
-                    hipStream_t stream) {
+                    int* zero, int n_zero, hipStream_t stream) {
   const int nb2 = (ni / 32 + 1) / 2;
   const int64_t grid = 1 + (int64_t)max_items * nb2;
   TF_REQUIRE(grid <= 0x7FFFFFFF, "moe: %lld workgroups exceed the grid limit", (long long)grid);
@@ -240,7 +271,7 @@ int launch_route_up(const float* logits, int64_t ldl, int rows, int experts, int
 #define TF_GO(W_)                                                                                                  \
   route_up_kernel<GS, NM, EPI, W_><<<g, W_ * 64, smem, stream>>>(logits, ldl, rows, experts, top_k, shared, x, x_stride, \
                                                                  wup, d, ni, pick, wts, members, items, counts, desc,  \
-                                                                 act, xs_act, limit)
+                                                                 act, xs_act, limit, zero, n_zero)
   switch (fused_waves(2 * grid)) {
     case 16: TF_GO(16); break;
     case 8: TF_GO(8); break;
@@ -312,7 +343,7 @@ extern "C" int tf_moe_route_up(const float* logits, int64_t ldl, int rows, int e
                                int swiglu, const uint16_t* x, int64_t x_stride, const uint32_t* up, int d, int ni,
                                int32_t* pick, float* wts, int32_t* members, int32_t* items, int32_t* counts,
                                int32_t* desc, uint16_t* act, float* xs_act, float limit, int max_items,
-                               tf_stream_t stream) {
+                               int32_t* zero, int n_zero, tf_stream_t stream) {
   clear_error();
   TF_REQUIRE(gs == 32 || gs == 64, "moe: groups of 32 or 64 inputs, not %d", gs);
   TF_REQUIRE(logits && x && up && pick && wts && members && items && counts && desc && act && xs_act,
@@ -328,14 +359,45 @@ extern "C" int tf_moe_route_up(const float* logits, int64_t ldl, int rows, int e
              "moe: hidden and intermediate sizes in whole groups and 32-column blocks");
   TF_REQUIRE(aligned16(x) && x_stride % 8 == 0 && aligned16(up) && aligned16(act),
              "x: rows of K = groups * group size inputs, 16-byte aligned");
+  TF_REQUIRE(n_zero >= 0 && (n_zero == 0 || zero), "route: bad counter range");
   hipStream_t s = as_stream(stream);
   if (gs == 64)
     return swiglu ? launch_route_up<64, 2, 2>(logits, ldl, rows, experts, top_k, shared, x, x_stride, up, d, ni, pick,
-                                              wts, members, items, counts, desc, act, xs_act, limit, max_items, s)
+                                              wts, members, items, counts, desc, act, xs_act, limit, max_items, zero, n_zero, s)
                   : launch_route_up<64, 1, 1>(logits, ldl, rows, experts, top_k, shared, x, x_stride, up, d, ni, pick,
-                                              wts, members, items, counts, desc, act, xs_act, limit, max_items, s);
+                                              wts, members, items, counts, desc, act, xs_act, limit, max_items, zero, n_zero, s);
   return swiglu ? launch_route_up<32, 2, 2>(logits, ldl, rows, experts, top_k, shared, x, x_stride, up, d, ni, pick, wts,
-                                            members, items, counts, desc, act, xs_act, limit, max_items, s)
+                                            members, items, counts, desc, act, xs_act, limit, max_items, zero, n_zero, s)
                 : launch_route_up<32, 1, 1>(logits, ldl, rows, experts, top_k, shared, x, x_stride, up, d, ni, pick, wts,
-                                            members, items, counts, desc, act, xs_act, limit, max_items, s);
+                                            members, items, counts, desc, act, xs_act, limit, max_items, zero, n_zero, s);
+}
+
+extern "C" int tf_moe_down_combine(int gs, const uint16_t* act, int rows, int slots, const uint32_t* down, int d, int ni,
+                                   const int32_t* desc, const float* wts, const float* xs_act, float* y, uint16_t* out,
+                                   int32_t* arrive, int max_items, tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(gs == 32 || gs == 64, "moe: groups of 32 or 64 inputs, not %d", gs);
+  TF_REQUIRE(act && down && desc && wts && xs_act && y && out && arrive, "moe: null pointer argument");
+  TF_REQUIRE(d % 32 == 0 && ni % gs == 0 && ni >= gs && rows >= 1 && slots >= 1 && max_items >= 1,
+             "moe: hidden size in 32-column blocks, intermediate size in whole groups");
+  TF_REQUIRE(aligned16(act) && ni % 8 == 0 && aligned16(down), "act: rows of whole groups, 16-byte aligned");
+  const int nb2 = (d / 32 + 1) / 2;
+  const int64_t grid = (int64_t)max_items * nb2;
+  TF_REQUIRE(grid <= 0x7FFFFFFF, "moe: %lld workgroups exceed the grid limit", (long long)grid);
+  const size_t smem = sizeof(float) * expert_lds_floats(1, 0, true);
+  hipStream_t s = as_stream(stream);
+  const dim3 g((unsigned)grid);
+#define TF_GO(GS_, W_)                                                                                             \
+  down_combine_kernel<GS_, W_><<<g, W_ * 64, smem, s>>>(act, slots, down, d, ni, desc, wts, xs_act, y, out, arrive)
+#define TF_GS(GS_)                      \
+  switch (fused_waves(2 * grid)) {      \
+    case 16: TF_GO(GS_, 16); break;     \
+    case 8: TF_GO(GS_, 8); break;       \
+    default: TF_GO(GS_, 4);             \
+  }
+  if (gs == 64) { TF_GS(64) } else { TF_GS(32) }
+#undef TF_GS
+#undef TF_GO
+  TF_LAUNCH_OK("tf_moe_down_combine");
+  return 0;
 }

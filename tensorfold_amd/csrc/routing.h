@@ -85,73 +85,68 @@ __device__ __forceinline__ void topk_pick(float (&v)[VPL], const float* __restri
   }
 }
 
-// Two rows at once on one wave: the same arithmetic as topk_pick on each, with the two dependent chains interleaved
-template <int VPL>
-__device__ __forceinline__ void topk_pick2(float (&va)[VPL], float (&vb)[VPL], const float* __restrict__ rowa,
-                                           const float* __restrict__ rowb, int NE, int TOPK, int shared, int lane,
-                                           int& ida, float& wa, int& idb, float& wb) {
+// Up to 128 experts and 16 slots: a logits row on a ROW of 16 lanes (eight values a lane), four logits rows a wave.
+// Every reduction stays inside the 16 lanes (DPP), so the four rows cost one row's instructions.  `row` is this
+// lane group's logits row, or null when it has none.  Lane k of the group (k < TOPK) leaves with pick k and its
+// weight, lane TOPK with the shared expert's.  The arithmetic, and so every bit, is topk_pick's.
+__device__ __forceinline__ void topk_row16(const float* __restrict__ row, int NE, int TOPK, int shared, int lane,
+                                           int& id, float& w) {
+#define TF_ROW_F(V_, CTRL_) \
+  __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, V_), CTRL_, 0xf, 0xf, false))
+#define TF_ROW_I(V_, CTRL_) __builtin_amdgcn_update_dpp(0, V_, CTRL_, 0xf, 0xf, false)
   const float NEG = -__builtin_inff();
-  float mma = 0.f, mmb = 0.f;
-  int mia = 0, mib = 0;
-  auto best = [&](const float (&v)[VPL], float& bv, int& bi) {
-    bv = v[0];
-    bi = lane;
+  const int l = lane & 15;
+  float v[8];
 #pragma unroll
-    for (int i = 1; i < VPL; ++i)
+  for (int i = 0; i < 8; ++i) {
+    const int e = l + 16 * i;
+    v[i] = row && e < NE ? row[e] : NEG;
+  }
+  float mine_m = 0.f;
+  int mine_id = 0;
+  for (int k = 0; k < TOPK; ++k) {
+    float bv = v[0];
+    int bi = l;
+#pragma unroll
+    for (int i = 1; i < 8; ++i)
       if (v[i] > bv) {
         bv = v[i];
-        bi = lane + 64 * i;
+        bi = l + 16 * i;
       }
-  };
-  auto lowest = [&](unsigned long long cand, int bi) {
-    int idx = 0x7FFFFFFF;
-    while (cand) {
-      const int l = __builtin_ctzll(cand);
-      idx = min(idx, __builtin_amdgcn_readlane(bi, l));
-      cand &= cand - 1;
+    float m = bv;
+    m = fmaxf(m, TF_ROW_F(m, 0xB1));         // quad_perm [1, 0, 3, 2]
+    m = fmaxf(m, TF_ROW_F(m, 0x4E));         // quad_perm [2, 3, 0, 1]
+    m = fmaxf(m, TF_ROW_F(m, 0x141));        // row_half_mirror
+    m = fmaxf(m, TF_ROW_F(m, 0x140));        // row_mirror
+    int idx = bv == m ? bi : 0x7FFFFFFF;     // the lowest id among the lanes that hold the maximum
+    idx = min(idx, TF_ROW_I(idx, 0xB1));
+    idx = min(idx, TF_ROW_I(idx, 0x4E));
+    idx = min(idx, TF_ROW_I(idx, 0x141));
+    idx = min(idx, TF_ROW_I(idx, 0x140));
+    if (l == k) {
+      mine_m = m;
+      mine_id = idx;
     }
-    return idx;
-  };
-  auto drop = [&](float (&v)[VPL], int idx) {
-    if ((idx & 63) == lane) {
+    if ((idx & 15) == l) {
 #pragma unroll
-      for (int i = 0; i < VPL; ++i)
-        if (i == (idx >> 6)) v[i] = NEG;
+      for (int i = 0; i < 8; ++i)
+        if (i == (idx >> 4)) v[i] = NEG;
     }
-  };
-  for (int k = 0; k < TOPK; ++k) {
-    float bva, bvb;
-    int bia, bib;
-    best(va, bva, bia);
-    best(vb, bvb, bib);
-    const float ma = wave_max(bva), mb = wave_max(bvb);
-    const int xa = lowest(__ballot(bva == ma), bia), xb = lowest(__ballot(bvb == mb), bib);
-    if (lane == k) {
-      mma = ma;
-      mia = xa;
-      mmb = mb;
-      mib = xb;
-    }
-    drop(va, xa);
-    drop(vb, xb);
   }
-  auto weight = [&](float mine_m, const float* row, int& id, float& w) {
-    const float top = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine_m), 0));
-    const float ex = expf(mine_m - top);
-    float total = 0.f;
-    for (int k = 0; k < TOPK; ++k)
-      total += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ex), k));
-    w = round_bf16(ex / total);
-    if (shared && lane == TOPK) {
-      const float sg = round_bf16(row[NE]);
-      id = NE;
-      w = round_bf16(1.f / (1.f + expf(-sg)));
-    }
-  };
-  ida = mia;
-  idb = mib;
-  weight(mma, rowa, ida, wa);
-  weight(mmb, rowb, idb, wb);
+  const float top = TF_ROW_F(mine_m, 0x150);                // row_newbcast:0
+  const float ex = l < TOPK ? expf(mine_m - top) : 0.f;
+  float sum = ex;                                           // lane j ends with ((e0 + e1) + ...) + ej
+  for (int k = 1; k < TOPK; ++k) sum = TF_ROW_F(sum, 0x111) + ex;     // row_shr:1, zero shifted in
+  const float total = __shfl(sum, (lane & 48) + TOPK - 1);
+  id = mine_id;
+  w = round_bf16(ex / total);
+  if (shared && l == TOPK && row) {
+    const float sg = round_bf16(row[NE]);
+    id = NE;
+    w = round_bf16(1.f / (1.f + expf(-sg)));
+  }
+#undef TF_ROW_F
+#undef TF_ROW_I
 }
 
 template <int VPL>

@@ -133,8 +133,8 @@ def fusable(x: torch.Tensor, ex: grouped.Experts, buf: MoEBuffers) -> bool:
 
 def decode(x: torch.Tensor, logits: torch.Tensor, ex: grouped.Experts, buf: MoEBuffers, top_k: int, experts: int,
            out: torch.Tensor | None = None) -> torch.Tensor:
-    """The decode layer in three launches (routing + up projection, down projection, combine) or, with
-    ``FUSED_DECODE``, in two (routing; up + down + combine).  Same bits as
+    """The decode layer in two launches (routing + up projection; down projection + combine), three when there are
+    many router logits (routing; up; down + combine), or, with ``FUSED_DECODE``, routing and one launch for the rest.  Same bits as
     ``select`` + ``gate_up`` + ``down`` + ``combine``; bf16 [R, D] out.  ``buf.pick``, ``buf.wts`` and ``buf.plan``
     are filled as by ``select``."""
 
@@ -166,26 +166,25 @@ def decode(x: torch.Tensor, logits: torch.Tensor, ex: grouped.Experts, buf: MoEB
                   items)
         return out
     act = buf.act.view(-1, ex.width)
+    arrive = ctr.data_ptr() + 4 * (1 + f["items"])        # one arrival counter a (token, 64 columns) cell
     if n * (experts + int(buf.shared)) > ROUTE_UP_LOGITS:
         # many logits: one routing launch, then up, down and combine from its item descriptors
         _lib.call("tf_moe_route_decode", _lib.ptr(logits), logits.stride(0), n, experts, top_k, int(buf.shared),
                   _lib.ptr(x), x.stride(0), ex.dims, ex.gs, _lib.ptr(buf.pick), _lib.ptr(buf.wts), _lib.ptr(plan.members),
-                  _lib.ptr(plan.items), _lib.ptr(plan.counts), _lib.ptr(f["desc"]), _lib.ptr(f["xs_x"]), None, 0)
+                  _lib.ptr(plan.items), _lib.ptr(plan.counts), _lib.ptr(f["desc"]), _lib.ptr(f["xs_x"]), arrive, cells)
         _lib.call("tf_experts_run_desc", ex.gs, 2 if ex.swiglu else 1, _lib.ptr(x), x.stride(0), buf.slots,
                   _lib.ptr(ex.up), ex.dims // ex.gs, ex.width // grouped.COLS, _lib.ptr(f["desc"]),
                   _lib.ptr(plan.counts), _lib.ptr(act), ex.width, ex.limit, items, _lib.ptr(f["xs_x"]),
                   _lib.ptr(f["xs_act"]))
     else:
-        # few logits: every workgroup of the up projection routes for itself (three launches: routing + up, down,
-        # combine)
+        # few logits: every workgroup of the up projection routes for itself
         _lib.call("tf_moe_route_up", _lib.ptr(logits), logits.stride(0), n, experts, top_k, int(buf.shared), ex.gs,
                   int(ex.swiglu), _lib.ptr(x), x.stride(0), _lib.ptr(ex.up), ex.dims, ex.width, _lib.ptr(buf.pick),
                   _lib.ptr(buf.wts), _lib.ptr(plan.members), _lib.ptr(plan.items), _lib.ptr(plan.counts),
-                  _lib.ptr(f["desc"]), _lib.ptr(act), _lib.ptr(f["xs_act"]), ex.limit, items)
-    _lib.call("tf_experts_run_desc", ex.gs, 0, _lib.ptr(act), ex.width, 0, _lib.ptr(ex.down), ex.width // ex.gs,
-              ex.dims // grouped.COLS, _lib.ptr(f["desc"]), _lib.ptr(plan.counts), _lib.ptr(buf.y), ex.dims, 0.0, items,
-              _lib.ptr(f["xs_act"]), None)
-    _lib.call("tf_moe_combine", _lib.ptr(buf.y), 0, _lib.ptr(buf.wts), _lib.ptr(out), n, buf.slots, ex.dims)
+                  _lib.ptr(f["desc"]), _lib.ptr(act), _lib.ptr(f["xs_act"]), ex.limit, items, arrive, cells)
+    # the down projection; the workgroup that completes a (token, 64 columns) cell writes the combined output
+    _lib.call("tf_moe_down_combine", ex.gs, _lib.ptr(act), n, buf.slots, _lib.ptr(ex.down), ex.dims, ex.width,
+              _lib.ptr(f["desc"]), _lib.ptr(buf.wts), _lib.ptr(f["xs_act"]), _lib.ptr(buf.y), _lib.ptr(out), arrive, items)
     return out
 
 
