@@ -279,8 +279,9 @@ constexpr int BIG_THREADS = BIG_WAVES * 64;
 // compiler is free to keep the LDS reads of the next row tile in flight under the MFMAs of this one.
 template <int GS, int NM, int EPI, int RT>
 __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t x_stride,
-                                         const uint32_t* __restrict__ We, const uint32_t (&wp)[4],
-                                         const uint32_t (&sp)[4], const int (&ocol)[4], const bool (&jok)[4],
+                                         const uint32_t* __restrict__ We, uint32_t we_bytes,
+                                         const uint32_t (&wp)[4], const uint32_t (&sp)[4], const int (&ocol)[4],
+                                         const bool (&jok)[4],
                                          int K, const int* src_rows, const int* dst_rows, int cnt,
                                          void* __restrict__ out, int N, float limit, unsigned char* smem) {
   constexpr int TJ = 4, CPS = KSTEP / 32, GPS = KSTEP / GS, BW = block_words(GS);
@@ -292,14 +293,20 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
   constexpr uint32_t SSTRIDE = GPS * GSTRIDE;     // words from one step to the next
   const int tid = threadIdx.x, lane = tid & 63, c = lane & 15, kq = lane >> 4;
   const int steps = K / KSTEP;
+  // buffer loads: the expert's base in scalar registers, the step as the scalar offset, the lane's part as the vector
+  // offset and the chunk or group as the immediate, so no address arithmetic is left on the vector unit
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(We), 0, we_bytes, 0x00020000);
   auto load_w = [&](int step, uint32_t (&w)[TJ][CPS], uint32_t (&sb)[TJ][GPS]) {
-    const uint32_t* base = We + (size_t)step * SSTRIDE;           // wave-uniform
+    const int soff = step * (int)(SSTRIDE * 4);                   // wave-uniform
 #pragma unroll
     for (int j = 0; j < TJ; ++j) {
 #pragma unroll
-      for (int i = 0; i < CPS; ++i) w[j][i] = base[wp[j] + ((32 * i) / GS) * GSTRIDE + (((32 * i) % GS) / 32) * 128];
+      for (int i = 0; i < CPS; ++i)
+        w[j][i] = __builtin_amdgcn_raw_buffer_load_b32(
+            rsrc, (wp[j] + ((32 * i) / GS) * GSTRIDE + (((32 * i) % GS) / 32) * 128) * 4, soff, 0);
 #pragma unroll
-      for (int gi = 0; gi < GPS; ++gi) sb[j][gi] = base[sp[j] + gi * GSTRIDE];
+      for (int gi = 0; gi < GPS; ++gi)
+        sb[j][gi] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (sp[j] + gi * GSTRIDE) * 4, soff, 0);
     }
   };
   // this thread's pieces of the activation tile: piece q = (row q / 8, 16 bytes q % 8)
@@ -435,6 +442,7 @@ __global__ void __launch_bounds__(BIG_THREADS, 1)
   __syncthreads();
   // the wave's four B operands: (matrix, 32-column block, 16-column half)
   const uint32_t* We = W + (size_t)e * NB * KG * (size_t)(NM * BW);      // the expert's matrices (wave-uniform)
+  const uint32_t we_bytes = (uint32_t)NB * KG * (NM * BW) * 4u;
   uint32_t wp[4], sp[4];              // word offsets inside the expert: always below 2^32
   int ocol[4];
   bool jok[4];
@@ -450,9 +458,9 @@ __global__ void __launch_bounds__(BIG_THREADS, 1)
     ocol[j] = nb * 32 + toff + c;
   }
   const int K = KG * GS;
-  if (cnt <= 32) big_body<GS, NM, EPI, 2>(X, x_stride, We, wp, sp, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
-  else if (cnt <= 64) big_body<GS, NM, EPI, 4>(X, x_stride, We, wp, sp, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
-  else big_body<GS, NM, EPI, 8>(X, x_stride, We, wp, sp, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
+  if (cnt <= 32) big_body<GS, NM, EPI, 2>(X, x_stride, We, we_bytes, wp, sp, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
+  else if (cnt <= 64) big_body<GS, NM, EPI, 4>(X, x_stride, We, we_bytes, wp, sp, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
+  else big_body<GS, NM, EPI, 8>(X, x_stride, We, we_bytes, wp, sp, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
 }
 
 // ---- dense prompt matmul --------------------------------------------------------------------------------------------
