@@ -1,4 +1,4 @@
-"""Benchmark of the hot path on one MI355X: the 4-bit decode MoE layer of BASELINE config 1.
+"""Benchmark of the hot path on one MI355X: the 4-bit decode MoE layer of benchmark configuration 1.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--tokens T]
 
@@ -291,7 +291,7 @@ def main() -> int:
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["layer_us"] * 1e-3,
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 x int4 -> fp32",
         "data": "synthetic",
-        "config": {"workload": f"BASELINE config 1: {SHAPE.name}; {args.tokens} tokens a step; {LAYERS} layers' tables "
+        "config": {"workload": f"benchmark configuration 1: {SHAPE.name}; {args.tokens} tokens a step; {LAYERS} layers' tables "
                                f"cycled", "tokens": args.tokens, "hidden": SHAPE.hidden, "experts": SHAPE.experts,
                    "intermediate": SHAPE.width, "top_k": SHAPE.top_k, "group_size": SHAPE.gs},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",

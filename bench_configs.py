@@ -1,4 +1,4 @@
-"""Kernel timings of the BASELINE configurations that are not bench.py's headline: 0 (dense 4-bit projection),
+"""Kernel timings of the benchmark configurations that are not bench.py's headline: 0 (dense 4-bit projection),
 2 (verify-window MoE layer), 3 (prompt chunk, grouped MFMA) and 4 (EXL3 projections).
 
     python bench_configs.py [c0] [c2] [c3] [c4]

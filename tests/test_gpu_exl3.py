@@ -36,7 +36,7 @@ def test_decode_is_bit_exact(codebook, bits):
 
 
 def test_config4_decode_is_bit_exact_at_full_size():
-    """BASELINE config 4's gate/up trellis [320, 1088, 48] at 3 bits, all three codebooks, against the C decoder."""
+    """benchmark configuration 4's gate/up trellis [320, 1088, 48] at 3 bits, all three codebooks, against the C decoder."""
 
     trellis, suh, svh = synthetic.exl3_layer(5120, 17408, 3, 4000)
     for cb in ("3inst", "mcg", "mul1"):
@@ -49,7 +49,7 @@ def test_config4_decode_is_bit_exact_at_full_size():
 @pytest.mark.parametrize("m", [1, 8])
 @pytest.mark.parametrize("k,n", [(5120, 17408), (17408, 5120)])
 def test_config4_projections(k, n, m):
-    """BASELINE config 4: 3.0 bpw, default codebook, fp16 in and out, tokens 1 and 8; rel-L2 <= 2e-3 against the
+    """benchmark configuration 4: 3.0 bpw, default codebook, fp16 in and out, tokens 1 and 8; rel-L2 <= 2e-3 against the
     float64 forward with the fp16-rounded rotated input (a 1,024-column slice of N for the CPU's sake)."""
 
     trellis, suh, svh = synthetic.exl3_layer(k, n, 3, 4100 + k // 1000)

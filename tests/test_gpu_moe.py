@@ -1,4 +1,4 @@
-"""The MoE layer on the GPU (router, top-k, plan, experts, combine) against the CPU oracle, at the BASELINE shapes
+"""The MoE layer on the GPU (router, top-k, plan, experts, combine) against the CPU oracle, at the benchmark shapes
 (configs 1 and 2) and in small; ids are checked bit for bit."""
 
 import numpy as np
@@ -98,7 +98,7 @@ def run_layer(shape, up, down, x, l, ne, prefill=False):
 
 @pytest.mark.parametrize("tokens", [1, 4, 8])
 def test_config1_decode_layer(tokens):
-    """BASELINE config 1: D 2688, NI 1856, relu^2, top-6, g64, tokens 1 / 4 / 8 (ids drawn over the first 24 of the
+    """benchmark configuration 1: D 2688, NI 1856, relu^2, top-6, g64, tokens 1 / 4 / 8 (ids drawn over the first 24 of the
     128 experts so the CPU oracle's table stays small; every other shape is the config's)."""
 
     shape, ne = synthetic.C1, 24
@@ -121,7 +121,7 @@ def test_config1_decode_layer(tokens):
 
 @pytest.mark.parametrize("prefill", [False, True])
 def test_config2_verify_layer(prefill):
-    """BASELINE config 2: D 2048, NI 512, SwiGLU, top-10 + shared, g32, 32 rows (8 lanes x 4 draft tokens); ids over
+    """benchmark configuration 2: D 2048, NI 512, SwiGLU, top-10 + shared, g32, 32 rows (8 lanes x 4 draft tokens); ids over
     the first 48 experts.  Both arithmetic forms: decode, and the prefill form the reference runs this window in."""
 
     shape, ne = synthetic.C2, 48
@@ -146,7 +146,7 @@ def test_config2_verify_layer(prefill):
 
 
 def test_config3_prefill_chunk_small():
-    """BASELINE config 3 in small: Zipf(1.1) picks over 64 experts, 512 tokens, SwiGLU g32, bf16 MFMA path, items of
+    """benchmark configuration 3 in small: Zipf(1.1) picks over 64 experts, 512 tokens, SwiGLU g32, bf16 MFMA path, items of
     64 and 128; weighted scatter-add back to token order.  Sort permutation bit-exact, output within 2e-3."""
 
     shape, ne, rows = synthetic.C2, 64, 512

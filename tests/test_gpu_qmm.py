@@ -11,7 +11,7 @@ from tests.helpers import bits16, f32, max_abs, rel_l2, u32
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
-TOL = 2e-3          # relative L2 bound on bf16 outputs (fp32 accumulation), as BASELINE states
+TOL = 2e-3          # relative L2 bound on bf16 outputs (fp32 accumulation), as the benchmark states
 
 
 def gpu(*ts):
@@ -43,7 +43,7 @@ def test_every_nibble_decodes_exactly(n, k, gs):
 
 
 def test_config0_single_linear_matches_the_oracle():
-    """BASELINE config 0: N = K = 4096, g64, one row; bf16 out against dequant-then-matmul."""
+    """benchmark configuration 0: N = K = 4096, g64, one row; bf16 out against dequant-then-matmul."""
 
     n = k = 4096
     w = synthetic.affine(n, k, 64, 1000)
