@@ -65,8 +65,15 @@ def c0() -> dict:
         us = graph_us(lambda i: qmm.matmul(x, copies[i % len(copies)], xs, out=y, part=part), 120)
         nbytes = n * k // 2 + 2 * 2 * n * k // 64 + m * (k + n) * 2
         out[m] = {"us": us, "bytes": nbytes, "gbs": nbytes / us * 1e-3, "frac": nbytes / us * 1e-3 / HBM}
+    # the prompt form of the same weight: 4,096 rows on the matrix cores
+    m = 4096
+    x = synthetic.activations(m, k, 8).to(DEV)
+    y = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+    us = graph_us(lambda i: qmm.prefill_matmul(x, copies[i % len(copies)], out=y), 12)
+    flop = 2.0 * m * n * k
+    prompt = {"rows": m, "us": us, "tflops": flop / us * 1e-6, "frac_mfma": flop / us * 1e-6 / MFMA}
     return {"config": "c0: dense 4-bit/g64 projection, N = K = 4096 (qmm kernel + slice reduce; group sums given)",
-            "bound": "hbm", "rows": out}
+            "bound": "hbm", "rows": out, "prompt_form": prompt}
 
 
 def moe_tables(shape, layers: int, gen):

@@ -277,29 +277,20 @@ constexpr int BIG_THREADS = BIG_WAVES * 64;
 // The pipeline for an item of at most 16 * RT rows (RT = 2, 4 or 8).  K is a multiple of KSTEP and nothing inside a
 // step is conditional (prefetches past the end re-read the last step, rows past the item read its first row), so the
 // compiler is free to keep the LDS reads of the next row tile in flight under the MFMAs of this one.
-template <int GS, int NM, int EPI, int RT>
-__device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t x_stride,
-                                         const uint32_t* __restrict__ We, uint32_t we_bytes,
-                                         const uint32_t (&wp)[4], const uint32_t (&sp)[4], const int (&ocol)[4],
-                                         const bool (&jok)[4],
-                                         int K, const int* src_rows, const int* dst_rows, int cnt,
-                                         void* __restrict__ out, int N, float limit, unsigned char* smem) {
-  constexpr int TJ = 4, CPS = KSTEP / 32, GPS = KSTEP / GS, BW = block_words(GS);
-  constexpr int ROWS = 16 * RT;
-  constexpr int PIECES = ROWS * 8;                // 16-byte pieces of a staged tile
-  constexpr int PPT = (PIECES + BIG_THREADS - 1) / BIG_THREADS;
-  constexpr int STAGE = BIG_ROWS * AROW;
-  constexpr uint32_t GSTRIDE = NM * BW;           // words from one group to the next
-  constexpr uint32_t SSTRIDE = GPS * GSTRIDE;     // words from one step to the next
-  const int tid = threadIdx.x, lane = tid & 63, c = lane & 15, kq = lane >> 4;
-  const int steps = K / KSTEP;
-  // buffer loads: the expert's base in scalar registers, the step as the scalar offset, the lane's part as the vector
-  // offset and the chunk or group as the immediate, so no address arithmetic is left on the vector unit
-  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(We), 0, we_bytes, 0x00020000);
-  auto load_w = [&](int step, uint32_t (&w)[TJ][CPS], uint32_t (&sb)[TJ][GPS]) {
-    const int soff = step * (int)(SSTRIDE * 4);                   // wave-uniform
+// Where a wave's weights come from.  load(step, w, sb): the lane's packed word of each of the four operands and two
+// chunks of the step, and the stored (scale | bias << 16) pair of each operand and group of the step.  Buffer loads:
+// the base in scalar registers, the step as the scalar offset, the lane's part as the vector offset and the chunk or
+// group as the immediate, so no address arithmetic is left on the vector unit.
+template <int GS, int NM>
+struct ExpertSource {
+  static constexpr int CPS = KSTEP / 32, GPS = KSTEP / GS;
+  static constexpr uint32_t GSTRIDE = NM * block_words(GS);      // words from one group to the next
+  __amdgpu_buffer_rsrc_t rsrc;                                    // one expert's matrices
+  uint32_t wp[4], sp[4];                                          // word offsets inside the expert: below 2^32
+  __device__ __forceinline__ void load(int step, uint32_t (&w)[4][CPS], uint32_t (&sb)[4][GPS]) const {
+    const int soff = step * (int)(GPS * GSTRIDE * 4);
 #pragma unroll
-    for (int j = 0; j < TJ; ++j) {
+    for (int j = 0; j < 4; ++j) {
 #pragma unroll
       for (int i = 0; i < CPS; ++i)
         w[j][i] = __builtin_amdgcn_raw_buffer_load_b32(
@@ -308,7 +299,46 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
       for (int gi = 0; gi < GPS; ++gi)
         sb[j][gi] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (sp[j] + gi * GSTRIDE) * 4, soff, 0);
     }
-  };
+  }
+};
+
+// The dense layout: codes [n / 64][K / gs][gs / 32][64][4] words, scales and biases bf16 [K / gs][npad].
+template <int GS>
+struct DenseSource {
+  static constexpr int CPS = KSTEP / 32, GPS = KSTEP / GS;
+  __amdgpu_buffer_rsrc_t codes, scales, biases;
+  uint32_t wp[4], cp[4];                                          // byte offsets: the lane's word; its column's bf16
+  int row_bytes;                                                  // bytes from one group's scales to the next
+  __device__ __forceinline__ void load(int step, uint32_t (&w)[4][CPS], uint32_t (&sb)[4][GPS]) const {
+    const int soff = step * (KSTEP / 32) * 1024;                  // 32 inputs of a 64-column tile are 1 KB of codes
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int i = 0; i < CPS; ++i) w[j][i] = __builtin_amdgcn_raw_buffer_load_b32(codes, wp[j] + i * 1024, soff, 0);
+#pragma unroll
+      for (int gi = 0; gi < GPS; ++gi) {
+        const int goff = (step * GPS + gi) * row_bytes;
+        const uint32_t sv = __builtin_amdgcn_raw_buffer_load_b16(scales, cp[j], goff, 0);
+        const uint32_t bv = __builtin_amdgcn_raw_buffer_load_b16(biases, cp[j], goff, 0);
+        sb[j][gi] = sv | (bv << 16);
+      }
+    }
+  }
+};
+
+template <int GS, int NM, int EPI, int RT, class WS>
+__device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t x_stride, const WS& ws,
+                                         const int (&ocol)[4], const bool (&jok)[4],
+                                         int K, const int* src_rows, const int* dst_rows, int cnt,
+                                         void* __restrict__ out, int N, float limit, unsigned char* smem) {
+  constexpr int TJ = 4, CPS = KSTEP / 32, GPS = KSTEP / GS;
+  constexpr int ROWS = 16 * RT;
+  constexpr int PIECES = ROWS * 8;                // 16-byte pieces of a staged tile
+  constexpr int PPT = (PIECES + BIG_THREADS - 1) / BIG_THREADS;
+  constexpr int STAGE = BIG_ROWS * AROW;
+  const int tid = threadIdx.x, lane = tid & 63, c = lane & 15, kq = lane >> 4;
+  const int steps = K / KSTEP;
+  auto load_w = [&](int step, uint32_t (&w)[TJ][CPS], uint32_t (&sb)[TJ][GPS]) { ws.load(step, w, sb); };
   // this thread's pieces of the activation tile: piece q = (row q / 8, 16 bytes q % 8)
   const uint16_t* asrc[PPT];
 #pragma unroll
@@ -442,8 +472,8 @@ __global__ void __launch_bounds__(BIG_THREADS, 1)
   __syncthreads();
   // the wave's four B operands: (matrix, 32-column block, 16-column half)
   const uint32_t* We = W + (size_t)e * NB * KG * (size_t)(NM * BW);      // the expert's matrices (wave-uniform)
-  const uint32_t we_bytes = (uint32_t)NB * KG * (NM * BW) * 4u;
-  uint32_t wp[4], sp[4];              // word offsets inside the expert: always below 2^32
+  ExpertSource<GS, NM> ws;
+  ws.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(We), 0, (uint32_t)NB * KG * (NM * BW) * 4u, 0x00020000);
   int ocol[4];
   bool jok[4];
 #pragma unroll
@@ -453,14 +483,51 @@ __global__ void __launch_bounds__(BIG_THREADS, 1)
     const int toff = (j & 1) * 16;
     jok[j] = nb < NB;
     const uint32_t blk = (uint32_t)((jok[j] ? nb : NB - 1) * KG) * (uint32_t)(NM * BW) + m * BW;
-    wp[j] = blk + (toff + c) * 4 + kq;
-    sp[j] = blk + 32 * GS / 8 + toff + c;
+    ws.wp[j] = blk + (toff + c) * 4 + kq;
+    ws.sp[j] = blk + 32 * GS / 8 + toff + c;
     ocol[j] = nb * 32 + toff + c;
   }
   const int K = KG * GS;
-  if (cnt <= 32) big_body<GS, NM, EPI, 2>(X, x_stride, We, we_bytes, wp, sp, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
-  else if (cnt <= 64) big_body<GS, NM, EPI, 4>(X, x_stride, We, we_bytes, wp, sp, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
-  else big_body<GS, NM, EPI, 8>(X, x_stride, We, we_bytes, wp, sp, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
+  if (cnt <= 32) big_body<GS, NM, EPI, 2>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
+  else if (cnt <= 64) big_body<GS, NM, EPI, 4>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
+  else big_body<GS, NM, EPI, 8>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
+}
+
+// The dense prompt matmul on the same pipeline: 128 rows x 512 columns a workgroup, a wave a 64-column tile.
+template <int GS, int EPI>
+__global__ void __launch_bounds__(BIG_THREADS, 1)
+    qmm_prefill_big_kernel(const uint16_t* __restrict__ X, int64_t ldx, const uint32_t* __restrict__ W,
+                           const uint16_t* __restrict__ S, const uint16_t* __restrict__ B, void* __restrict__ out,
+                           int M, int N, int KG, int npad) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  __shared__ int rows[BIG_ROWS];
+  const int ct = (N + 511) >> 9;
+  const int rt = blockIdx.x / ct, cbt = blockIdx.x - rt * ct;
+  const int m0 = rt * BIG_ROWS, cnt = min(BIG_ROWS, M - m0);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, kq = lane >> 4;
+  if (tid < BIG_ROWS) rows[tid] = m0 + (tid < cnt ? tid : 0);
+  __syncthreads();
+  const int tiles = npad >> 6, tile = cbt * 8 + wave;
+  const bool ok = tile < tiles;
+  DenseSource<GS> ws;
+  ws.codes = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(W), 0, (uint32_t)tiles * KG * (GS / 32) * 1024u, 0x00020000);
+  ws.scales = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(S), 0, (uint32_t)KG * npad * 2u, 0x00020000);
+  ws.biases = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(B), 0, (uint32_t)KG * npad * 2u, 0x00020000);
+  ws.row_bytes = npad * 2;
+  int ocol[4];
+  bool jok[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int col = (ok ? tile : 0) * 64 + 32 * (j >> 1) + 16 * (j & 1) + c;      // columns up to npad are stored zeros
+    ws.wp[j] = ((uint32_t)(ok ? tile : 0) * KG * (GS / 32) * 256u + (32 * (j >> 1) + 16 * (j & 1) + c) * 4 + kq) * 4u;
+    ws.cp[j] = col * 2;
+    ocol[j] = col;
+    jok[j] = ok && col < N;
+  }
+  const int K = KG * GS;
+  if (cnt <= 32) big_body<GS, 1, EPI, 2>(X, ldx, ws, ocol, jok, K, rows, rows, cnt, out, N, 0.f, smem);
+  else if (cnt <= 64) big_body<GS, 1, EPI, 4>(X, ldx, ws, ocol, jok, K, rows, rows, cnt, out, N, 0.f, smem);
+  else big_body<GS, 1, EPI, 8>(X, ldx, ws, ocol, jok, K, rows, rows, cnt, out, N, 0.f, smem);
 }
 
 // ---- dense prompt matmul --------------------------------------------------------------------------------------------
@@ -551,6 +618,11 @@ int launch_qmm_prefill(const uint16_t* x, int64_t ldx, const uint32_t* w, const 
   } else if (m <= 64) {
     qmm_prefill_kernel<GS, EPI, 4><<<(unsigned)(((m + 63) / 64) * ct), 256, stage_bytes<4>(), st>>>(x, ldx, w, s, b, out,
                                                                                                    m, n, kg, npad);
+  } else if ((kg * GS) % KSTEP == 0 && (int64_t)npad * kg * GS / 2 < (1ll << 32)) {
+    const int64_t grid = (int64_t)((m + BIG_ROWS - 1) / BIG_ROWS) * ((n + 511) / 512);
+    TF_REQUIRE(grid <= 0x7FFFFFFF, "qmm_prefill: grid too large");
+    qmm_prefill_big_kernel<GS, EPI><<<(unsigned)grid, BIG_THREADS, 2 * BIG_ROWS * AROW, st>>>(x, ldx, w, s, b, out, m, n,
+                                                                                            kg, npad);
   } else {
     const int64_t grid = (int64_t)((m + 127) / 128) * ct;
     TF_REQUIRE(grid <= 0x7FFFFFFF, "qmm_prefill: grid too large");

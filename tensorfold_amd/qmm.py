@@ -190,13 +190,16 @@ def matmul_group(x: torch.Tensor, qs: list[Q4], xs: torch.Tensor | None = None, 
 
 def prefill_matmul(x: torch.Tensor, q: Q4, *, f32: bool = False, tile: int = 0,
                    out: torch.Tensor | None = None) -> torch.Tensor:
-    """Prompt-form x @ W.T on bf16 MFMA: every weight is rounded to bf16 once and K is one fp32 chain, so chunking a
-    prompt never changes a row's bits (they differ from ``matmul``'s)."""
+    """Prompt-form x @ W.T on f16 MFMA: every weight is rounded once (256 w to fp16) and K is one fp32 chain, so
+    chunking a prompt never changes a row's bits (they differ from ``matmul``'s)."""
 
     x = _check_x(x, q, "prefill_matmul")
     m = int(x.shape[0])
     if out is None:
         out = x.new_empty((m, q.n), dtype=torch.float32 if f32 else torch.bfloat16)
+    elif tuple(out.shape) != (m, q.n) or out.dtype != (torch.float32 if f32 else torch.bfloat16) \
+            or not out.is_contiguous() or out.device != x.device:
+        raise ValueError(f"prefill_matmul: out must be contiguous ({m}, {q.n}) {'fp32' if f32 else 'bf16'}")
     _lib.call("tf_qmm_prefill", _lib.ptr(x), x.stride(0), _lib.ptr(q.weight), _lib.ptr(q.scales.contiguous()),
               _lib.ptr(q.biases.contiguous()), _lib.ptr(out), m, q.n, q.k, q.gs, int(f32), tile)
     return out
