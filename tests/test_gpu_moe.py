@@ -70,6 +70,12 @@ def test_combine_is_the_slot_ordered_sum():
     got16 = f32(moe.combine(y.bfloat16().to(DEV), w.to(DEV)))
     want16 = ora.combine(f32(y.bfloat16()), w.numpy())
     assert rel_l2(got16, want16) < 1e-3
+    # many rows take the kernel with 16-byte loads: the same bits a row as the narrow one
+    y2 = torch.randn((80, 7, 2688), generator=g).to(DEV)
+    w2 = torch.rand((80, 7), generator=g).to(DEV)
+    wide = moe.combine(y2, w2)
+    for r in (0, 41, 79):
+        assert torch.equal(moe.combine(y2[r:r + 1].contiguous(), w2[r:r + 1].contiguous())[0], wide[r]), r
 
 
 def layer_tables(shape, seed, experts_built):
