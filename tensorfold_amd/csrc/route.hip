@@ -126,28 +126,42 @@ __global__ void __launch_bounds__(PLAN_THREADS)
   }
 }
 
-// wide plans, pass 1: block b ranks its 1024 pairs within each expert (pair order) and leaves its counts in hist[b]
+// wide plans, pass 1: block b ranks its 1024 pairs within each expert (pair order) and leaves its counts in hist[b].
+// A pair's rank = the pairs of its expert in earlier waves of the block + those in earlier lanes of its wave: the
+// lanes are compared through 64 readlanes, the waves' counts (one writer each: the expert's last lane in the wave)
+// are prefixed by a thread an expert.
 __global__ void __launch_bounds__(PLAN_THREADS)
     plan_rank_kernel(const int* __restrict__ picks, int P, int E, int* __restrict__ rank, int* __restrict__ hist) {
-  __shared__ int pk[PLAN_THREADS];
-  __shared__ int cnt[EMAX];
-  const int tid = threadIdx.x, p = blockIdx.x * PLAN_THREADS + tid;
-  cnt[tid] = 0;
-  __syncthreads();
+  constexpr int NW = PLAN_THREADS / 64;
+  __shared__ unsigned short wcnt[NW][EMAX];      // pairs of expert e in wave w; then: in the waves before w
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, p = blockIdx.x * PLAN_THREADS + tid;
+  for (int i = tid; i < NW * EMAX; i += PLAN_THREADS) (&wcnt[0][0])[i] = 0;
   int e = -1;
   if (p < P) {
     e = picks[p];
     if ((unsigned)e >= (unsigned)E) e = -1;
-    if (e >= 0) atomicAdd(&cnt[e], 1);
   }
-  pk[tid] = e;
+  int before = 0, later = 0;
+  for (int l = 0; l < 64; ++l) {
+    const int el = __builtin_amdgcn_readlane(e, l);
+    before += (l < lane) & (el == e);
+    later |= (l > lane) & (el == e);
+  }
   __syncthreads();
-  if (p < P && e >= 0) {
-    int rk = 0;
-    for (int q = 0; q < tid; ++q) rk += pk[q] == e;
-    rank[p] = rk;
+  if (e >= 0 && !later) wcnt[wave][e] = (unsigned short)(before + 1);
+  __syncthreads();
+  if (tid < E) {
+    int acc = 0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      const int c = wcnt[w][tid];
+      wcnt[w][tid] = (unsigned short)acc;
+      acc += c;
+    }
+    hist[(size_t)blockIdx.x * E + tid] = acc;
   }
-  if (tid < E) hist[(size_t)blockIdx.x * E + tid] = cnt[tid];
+  __syncthreads();
+  if (e >= 0) rank[p] = wcnt[wave][e] + before;
 }
 
 // pass 2, one block: hist[b][e] becomes block b's first member of expert e; items and counts are written
@@ -155,17 +169,29 @@ __global__ void __launch_bounds__(PLAN_THREADS)
     plan_offsets_kernel(int nblk, int E, int T, int* __restrict__ hist, int* __restrict__ items,
                         int* __restrict__ counts) {
   const int tid = threadIdx.x;
+  constexpr int CH = 16;             // blocks read together: independent loads, one trip through memory a chunk
   int c = 0;
   if (tid < E)
-    for (int b = 0; b < nblk; ++b) {
-      int* h = hist + (size_t)b * E + tid;
-      const int v = *h;
-      *h = c;
-      c += v;
+    for (int b0 = 0; b0 < nblk; b0 += CH) {
+      int v[CH];
+#pragma unroll
+      for (int i = 0; i < CH; ++i) v[i] = b0 + i < nblk ? hist[(size_t)(b0 + i) * E + tid] : 0;
+#pragma unroll
+      for (int i = 0; i < CH; ++i) c += v[i];
     }
-  const int off = place_items(c, E, T, items, counts);
+  int run = place_items(c, E, T, items, counts);
   if (tid < E)
-    for (int b = 0; b < nblk; ++b) hist[(size_t)b * E + tid] += off;
+    for (int b0 = 0; b0 < nblk; b0 += CH) {
+      int v[CH];
+#pragma unroll
+      for (int i = 0; i < CH; ++i) v[i] = b0 + i < nblk ? hist[(size_t)(b0 + i) * E + tid] : 0;
+#pragma unroll
+      for (int i = 0; i < CH; ++i)
+        if (b0 + i < nblk) {
+          hist[(size_t)(b0 + i) * E + tid] = run;
+          run += v[i];
+        }
+    }
 }
 
 // pass 3: every pair to its place
