@@ -242,3 +242,35 @@ def test_the_fused_decode_layer_equals_the_separate_kernels(shape, ne, rows, pat
         assert torch.equal(fused.plan.members, ref.plan.members)
         assert torch.equal(fused.act, ref.act) and torch.equal(fused.y, ref.y)
         assert torch.equal(got, want), seed
+
+
+def test_decode_replays_in_a_graph_with_new_logits_and_inputs():
+    """``decode`` captured once and replayed on changed logits and activations (in place): every replay equals the
+    eager result, so the arrival counters the routing launch clears are right on every pass, not only the first."""
+
+    shape, ne, rows = synthetic.C1, 24, 8
+    up, down = layer_tables(shape, 1600, ne)
+    ex = experts.make([tuple(t.to(DEV) for t in m) for m in up], tuple(t.to(DEV) for t in down), shape.gs)
+    cfg = type("c", (), dict(num_experts_per_tok=shape.top_k, num_experts=ne, moe_intermediate_size=shape.width,
+                             hidden_size=shape.hidden))
+    buf, ref = moe.MoEBuffers(rows, cfg, DEV, shared=False), moe.MoEBuffers(rows, cfg, DEV, shared=False)
+    x = synthetic.activations(rows, shape.hidden, 1601).to(DEV)
+    l = synthetic.logits(rows, ne, 1602).to(DEV)
+    out = torch.empty((rows, shape.hidden), dtype=torch.bfloat16, device=DEV)
+    moe.decode(x, l, ex, buf, shape.top_k, ne, out)              # warm-up: scratch is allocated outside the capture
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        moe.decode(x, l, ex, buf, shape.top_k, ne, out)
+    for seed in (1, 2, 3):
+        x.copy_(synthetic.activations(rows, shape.hidden, 1610 + seed).to(DEV))
+        l.copy_(synthetic.logits(rows, ne, 1620 + seed).to(DEV))
+        g.replay()
+        torch.cuda.synchronize()
+        want = moe.decode(x, l, ex, ref, shape.top_k, ne).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), seed
+    with pytest.raises(RuntimeError):
+        moe.decode(x[:, :64], l, ex, buf, shape.top_k, ne)           # not the table's K
+    with pytest.raises(ValueError):
+        moe.decode(torch.cat([x, x]), torch.cat([l, l]), ex, buf, shape.top_k, ne)      # more rows than the buffers hold
