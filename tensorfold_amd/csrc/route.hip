@@ -75,7 +75,7 @@ __global__ void __launch_bounds__(PLAN_THREADS)
                         const uint16_t* __restrict__ X, int64_t ldx, int D, int gs, int* __restrict__ pick,
                         float* __restrict__ wts, int* __restrict__ members, int* __restrict__ items,
                         int* __restrict__ counts, int* __restrict__ desc, float* __restrict__ xs_x,
-                        int* __restrict__ zero, int n_zero) {
+                        int* __restrict__ zero, int n_zero, int have_picks) {
   __shared__ int pk[PLAN_THREADS];
   __shared__ int cnt[EMAX];
   __shared__ int off[EMAX];
@@ -84,8 +84,9 @@ __global__ void __launch_bounds__(PLAN_THREADS)
   const int slots = TOPK + (shared ? 1 : 0), P = R * slots, E = NE + (shared ? 1 : 0), T = 16;
   cnt[tid] = 0;
   for (int i = tid; i < n_zero; i += PLAN_THREADS) zero[i] = 0;
-  for (int r = wave; r < R; r += PLAN_THREADS / 64)
-    topk_row(L + (size_t)r * ldl, NE, TOPK, shared, lane, pick + (size_t)r * slots, wts + (size_t)r * slots);
+  if (!have_picks)
+    for (int r = wave; r < R; r += PLAN_THREADS / 64)
+      topk_row(L + (size_t)r * ldl, NE, TOPK, shared, lane, pick + (size_t)r * slots, wts + (size_t)r * slots);
   // group sums of x, as tf_group_sums
   if (gs == 64) group_sums_rows<64>(X, ldx, R, D / 64, xs_x, tid, PLAN_THREADS);
   else group_sums_rows<32>(X, ldx, R, D / 32, xs_x, tid, PLAN_THREADS);
@@ -292,9 +293,12 @@ extern "C" int tf_moe_route_decode(const float* logits, int64_t ldl, int rows, i
   TF_REQUIRE(d >= gs && d % gs == 0 && aligned16(x) && ldx % 8 == 0, "route: x rows of whole groups, 16-byte aligned");
   TF_REQUIRE(ldl >= experts + (shared ? 1 : 0), "route: logits rows are too short");
   TF_REQUIRE(n_zero >= 0 && (n_zero == 0 || zero), "route: bad counter range");
+  // more rows than the one workgroup has waves: the top-k runs first on a workgroup a row, spread over the chip
+  const int spread = rows > PLAN_THREADS / 64;
+  if (spread) topk_kernel<<<rows, 64, 0, as_stream(stream)>>>(logits, ldl, experts, top_k, shared, pick, wts);
   route_decode_kernel<<<1, PLAN_THREADS, 0, as_stream(stream)>>>(logits, ldl, rows, experts, top_k, shared, x, ldx, d,
                                                                 gs, pick, wts, members, items, counts, desc, xs_x, zero,
-                                                                n_zero);
+                                                                n_zero, spread);
   TF_LAUNCH_OK("tf_moe_route_decode");
   return 0;
 }
