@@ -149,9 +149,9 @@ int tf_moe_route_up(const float* logits, int64_t ldl, int rows, int experts, int
 int tf_moe_down_combine(int gs, const uint16_t* act, int rows, int slots, const uint32_t* down, int d, int ni,
                         const int32_t* desc, const float* wts, const float* xs_act, float* y, uint16_t* out,
                         int32_t* arrive, int max_items, tf_stream_t stream);
-/* The decode layer's routing in one launch, for rows * (top_k + shared) <= 1024: tf_moe_topk, tf_experts_plan (tile
- * 16) and tf_group_sums of x, plus the item descriptors and the
- * zeroing of `zero` (n_zero ints: the counters of tf_moe_decode_experts).  No counterpart in the reference, which
+/* The decode layer's routing in one launch (two past 16 rows: the top-k then runs a workgroup a row first), for
+ * rows * (top_k + shared) <= 1024: tf_moe_topk, tf_experts_plan (tile 16) and tf_group_sums of x, plus the item
+ * descriptors and the zeroing of `zero` (n_zero ints: the counters of tf_moe_down_combine or tf_moe_decode_experts).  No counterpart in the reference, which
  * launches `_topk_rows`, `plan` and its group sums separately (moe.py:103-116, kernels/qmm.py:148-154). */
 int tf_moe_route_decode(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared,
                         const uint16_t* x, int64_t ldx, int d, int gs, int32_t* pick, float* wts, int32_t* members,
