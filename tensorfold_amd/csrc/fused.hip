@@ -193,34 +193,40 @@ __global__ void __launch_bounds__(WAVES * 64)
     // the whole plan: first member and first item of every expert (wave 0 scans), then items, members, descriptors
     int* off = reinterpret_cast<int*>(lds);
     int* itoff = off + EMAX;
-    int* dtoff = itoff + EMAX;
+    int* dtoff = itoff + EMAX;                 // descriptors: an expert's first full item; full items come first
+    int* shoff = dtoff + EMAX;                 // and its short last item among the short ones, which follow
     for (int e = tid; e < E; e += threads) item.cnt[e] = 0;
     __syncthreads();
     for (int p = tid; p < P; p += threads)
       if (pk[p] >= 0) atomicAdd(&item.cnt[pk[p]], 1);
     __syncthreads();
     if (tid < 64) {
-      int items_before = 0, pairs_before = 0, descs_before = 0, used = 0;
+      int items_before = 0, pairs_before = 0, full_before = 0, short_before = 0, used = 0;
       for (int e0 = 0; e0 < E; e0 += 64) {
-        const int e = e0 + lane, c = e < E ? item.cnt[e] : 0, t = (c + 15) >> 4, t4 = (c + DTILE - 1) / DTILE;
-        const int ti = wave_scan(t), ci = wave_scan(c), di = wave_scan(t4);
+        const int e = e0 + lane, c = e < E ? item.cnt[e] : 0, t = (c + 15) >> 4, f = c / DTILE,
+                  r = c - DTILE * f > 0 ? 1 : 0;
+        const int ti = wave_scan(t), ci = wave_scan(c), fi = wave_scan(f), ri = wave_scan(r);
         if (e < E) {
           off[e] = pairs_before + ci - c;
           itoff[e] = items_before + ti - t;
-          dtoff[e] = descs_before + di - t4;
+          dtoff[e] = full_before + fi - f;
+          shoff[e] = short_before + ri - r;
         }
         items_before += __builtin_amdgcn_readlane(ti, 63);
         pairs_before += __builtin_amdgcn_readlane(ci, 63);
-        descs_before += __builtin_amdgcn_readlane(di, 63);
+        full_before += __builtin_amdgcn_readlane(fi, 63);
+        short_before += __builtin_amdgcn_readlane(ri, 63);
         used += __popcll(__ballot(c > 0));
       }
       if (lane == 0) {
         counts[0] = items_before;
         counts[1] = used;
-        desc[0] = descs_before;
+        desc[0] = full_before + short_before;
+        item.sel[5] = full_before;
       }
     }
     __syncthreads();
+    const int F = item.sel[5];
     for (int e = tid; e < E; e += threads) {
       const int c = item.cnt[e];
       for (int j = 0; 16 * j < c; ++j) {
@@ -230,9 +236,10 @@ __global__ void __launch_bounds__(WAVES * 64)
         items[3 * i + 2] = n;
       }
       for (int j = 0; DTILE * j < c; ++j) {
-        int* d = desc + (size_t)(1 + dtoff[e] + j) * DESC;
+        const int n = min(DTILE, c - DTILE * j);
+        int* d = desc + (size_t)(1 + (n == DTILE ? dtoff[e] + j : F + shoff[e])) * DESC;
         d[0] = e;
-        d[1] = min(DTILE, c - DTILE * j);
+        d[1] = n;
         d[2] = off[e] + DTILE * j;
         d[3] = 0;
       }
@@ -243,7 +250,8 @@ __global__ void __launch_bounds__(WAVES * 64)
       int rank = 0;
       for (int q = 0; q < p; ++q) rank += pk[q] == e;
       members[off[e] + rank] = p;
-      desc[(size_t)(1 + dtoff[e] + rank / DTILE) * DESC + 4 + rank % DTILE] = p;
+      const int j = rank / DTILE, row = DTILE * (j + 1) <= item.cnt[e] ? dtoff[e] + j : F + shoff[e];
+      desc[(size_t)(1 + row) * DESC + 4 + rank % DTILE] = p;
     }
     return;
   }
@@ -265,7 +273,7 @@ int launch_route_up(const float* logits, int64_t ldl, int rows, int experts, int
   const int64_t grid = 1 + (int64_t)max_items * nb2;
   TF_REQUIRE(grid <= 0x7FFFFFFF, "moe: %lld workgroups exceed the grid limit", (long long)grid);
   const size_t floats = expert_lds_floats(NM, d / GS, false);
-  const size_t smem = sizeof(float) * (floats > 3 * EMAX ? floats : 3 * EMAX);
+  const size_t smem = sizeof(float) * (floats > 4 * EMAX ? floats : 4 * EMAX);
   TF_REQUIRE(smem <= 48 * 1024, "moe: %d input groups need %zu bytes of LDS", d / GS, smem);
   const dim3 g((unsigned)grid);
 #define TF_GO(W_)                                                                                                  \

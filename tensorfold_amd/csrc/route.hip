@@ -111,13 +111,14 @@ __global__ void __launch_bounds__(PLAN_THREADS)
   }
   __threadfence_block();
   __syncthreads();
-  // the descriptors: the same order cut into items of DTILE
-  const int c = tid < E ? cnt[tid] : 0, t4 = (c + DTILE - 1) / DTILE;
-  int val[3] = {t4, 0, 0}, excl[3], tot[3];
+  // the descriptors: the same members cut into items of DTILE, every full item first (they take longest), then the
+  // experts' short last items
+  const int c = tid < E ? cnt[tid] : 0, f = c / DTILE, r = c - DTILE * f > 0 ? 1 : 0;
+  int val[3] = {f, r, 0}, excl[3], tot[3];
   scan3(val, excl, tot);
-  if (tid == 0) desc[0] = tot[0];
-  for (int j = 0; j < t4; ++j) {
-    int* d = desc + (size_t)(1 + excl[0] + j) * DESC;
+  if (tid == 0) desc[0] = tot[0] + tot[1];
+  for (int j = 0; j < f + r; ++j) {
+    int* d = desc + (size_t)(1 + (j < f ? excl[0] + j : tot[0] + excl[1])) * DESC;
     const int first = off[tid] + DTILE * j, n = min(DTILE, c - DTILE * j);
     d[0] = tid;
     d[1] = n;

@@ -287,38 +287,49 @@ constexpr int DTILE = 2;
 
 struct ItemLds {
   int cnt[EMAX];       // pairs an expert
-  int sel[5];          // expert, first member, count, items in all, rank of the item's first pair in its expert
+  int sel[6];          // expert, first member, count, items in all, rank of the item's first pair in its expert, full items
   int pairs[16];
 };
 
+// Item order: every full item (TILE pairs) first, in expert order, then the experts' short last items, in expert
+// order — the items that take longest start first.  Item `it` of expert e's j-th tile sits at
+// it < F: (full tiles before e) + j, else F + (experts with a short tile before e), F = full items in all.
+//
 // Every thread of the workgroup calls this (it has barriers); pk holds P expert ids (negative = none).
 // Returns false when there is no item `it`.  On return L.sel and L.pairs describe the item.
 template <int TILE>
 __device__ __forceinline__ bool find_item(ItemLds& L, const int* pk, int P, int E, int it) {
   const int tid = threadIdx.x, threads = blockDim.x, lane = tid & 63;
   for (int e = tid; e < E; e += threads) L.cnt[e] = 0;
-  if (tid < 5) L.sel[tid] = tid == 0 ? -1 : 0;
+  if (tid < 6) L.sel[tid] = tid == 0 ? -1 : 0;
   __syncthreads();
   for (int p = tid; p < P; p += threads)
-    if (pk[p] >= 0) atomicAdd(&L.cnt[pk[p]], 1);
+    if (pk[p] >= 0) {
+      const int old = atomicAdd(&L.cnt[pk[p]], 1);
+      if (old % TILE == TILE - 1) atomicAdd(&L.sel[5], 1);     // this pair completes a tile
+    }
   __syncthreads();
   if (tid < 64) {
-    int items_before = 0, pairs_before = 0;
+    const int F = L.sel[5];
+    int full_before = 0, short_before = 0, pairs_before = 0;
     for (int e0 = 0; e0 < E; e0 += 64) {
-      const int e = e0 + lane, c = e < E ? L.cnt[e] : 0, t = (c + TILE - 1) / TILE;
-      const int ti = wave_scan(t), ci = wave_scan(c);      // inclusive, over the 64 experts of this step
-      const int first_item = items_before + ti - t;
-      if (it >= first_item && it < first_item + t) {
-        const int j = it - first_item;
+      const int e = e0 + lane, c = e < E ? L.cnt[e] : 0, f = c / TILE, r = c - TILE * f > 0 ? 1 : 0;
+      const int cf = wave_scan(c | (f << 16)), ri = wave_scan(r);      // inclusive, over the 64 experts of this step
+      const int ci = cf & 0xFFFF, fi = cf >> 16;
+      const int first_full = full_before + fi - f;
+      if (it < F ? (it >= first_full && it < first_full + f) : (r && it - F == short_before + ri - 1)) {
+        const int j = it < F ? it - first_full : f;
         L.sel[0] = e;
         L.sel[1] = pairs_before + ci - c + TILE * j;
         L.sel[2] = min(TILE, c - TILE * j);
         L.sel[4] = TILE * j;
       }
-      items_before += __builtin_amdgcn_readlane(ti, 63);
-      pairs_before += __builtin_amdgcn_readlane(ci, 63);
+      const int last = __builtin_amdgcn_readlane(cf, 63);
+      full_before += last >> 16;
+      pairs_before += last & 0xFFFF;
+      short_before += __builtin_amdgcn_readlane(ri, 63);
     }
-    if (lane == 0) L.sel[3] = items_before;
+    if (lane == 0) L.sel[3] = full_before + short_before;
   }
   __syncthreads();
   const int e = L.sel[0];
