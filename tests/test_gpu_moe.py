@@ -274,3 +274,54 @@ def test_decode_replays_in_a_graph_with_new_logits_and_inputs():
         moe.decode(x[:, :64], l, ex, buf, shape.top_k, ne)           # not the table's K
     with pytest.raises(ValueError):
         moe.decode(torch.cat([x, x]), torch.cat([l, l]), ex, buf, shape.top_k, ne)      # more rows than the buffers hold
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_shapes_of_the_decode_layer(seed):
+    """Drawn shapes (hidden, width, experts, slots, group size, activation, rows): every form of ``decode`` gives the
+    bits of the separate kernels, ids equal the oracle's, and the output is within 2e-3 of the CPU oracle's layer."""
+
+    import random
+
+    rnd = random.Random(seed)
+    gs = rnd.choice([32, 64])
+    hidden, width = 64 * rnd.randint(1, 12), 64 * rnd.randint(1, 10)
+    ne = rnd.choice([2, 3, 5, 8, 17, 33, 64, 100, 128, 130, 200])
+    shared = rnd.random() < 0.4
+    top_k = rnd.randint(1, min(8, ne))
+    swiglu = rnd.random() < 0.5
+    rows = rnd.choice([1, 2, 3, 5, 8, 13, 16, 17, 24, 33, 40])
+    shape = synthetic.MoEShape(f"drawn{seed}", hidden, ne, width, top_k, gs, swiglu, shared)
+    up, down = layer_tables(shape, 3000 + seed, ne)
+    ex = experts.make([tuple(t.to(DEV) for t in m) for m in up], tuple(t.to(DEV) for t in down), gs)
+    cfg = type("c", (), dict(num_experts_per_tok=top_k, num_experts=ne, moe_intermediate_size=width,
+                             hidden_size=hidden))
+    x = synthetic.activations(rows, hidden, 4000 + seed).to(DEV)
+    l = synthetic.logits(rows, ne + int(shared), 5000 + seed).to(DEV)
+    ref = moe.MoEBuffers(rows, cfg, DEV, shared=shared)
+    moe.select(l, ref, top_k, ne)
+    experts.gate_up(x, ex, ref.plan, ref.act.view(-1, ex.width), rows)
+    experts.down(ref.act.view(-1, ex.width), ex, ref.plan, ref.y.view(-1, ex.dims), rows)
+    want = moe.combine(ref.y, ref.wts)
+    saved = moe.FUSED_DECODE, moe.ROUTE_UP_LOGITS
+    try:
+        for path in ("route_up", "route_then_up", "one_launch"):
+            moe.FUSED_DECODE = path == "one_launch"
+            moe.ROUTE_UP_LOGITS = 0 if path == "route_then_up" else 1 << 30
+            buf = moe.MoEBuffers(rows, cfg, DEV, shared=shared)
+            for _ in range(2):
+                got = moe.decode(x, l, ex, buf, top_k, ne)
+                torch.cuda.synchronize()
+                buf.check()
+                assert torch.equal(buf.pick, ref.pick) and torch.equal(buf.wts, ref.wts), path
+                assert torch.equal(buf.plan.members, ref.plan.members), path
+                assert torch.equal(buf.act, ref.act) and torch.equal(buf.y, ref.y), path
+                assert torch.equal(got, want), path
+    finally:
+        moe.FUSED_DECODE, moe.ROUTE_UP_LOGITS = saved
+    picks, _ = orr.topk_rows(l.cpu().numpy(), ne, top_k, shared=shared)
+    assert np.array_equal(ref.pick.cpu().numpy(), picks)
+    t = lambda m: (u32(m[0]), bits16(m[1]), bits16(m[2]))
+    want_bits = native.moe_layer(bits16(x.cpu()), picks, ref.wts.cpu().numpy(), t(up[0]) if swiglu else None,
+                                 t(up[1]) if swiglu else t(up[0]), t(down), gs)
+    assert rel_l2(f32(want), ora.bf16_from_bits(want_bits)) <= TOL
