@@ -164,6 +164,38 @@ __global__ void __launch_bounds__(WAVES * 64)
       }
     }
   };
+  const int NB2 = (NI / 32 + 1) >> 1;
+  const int u = blockIdx.x - 1, it = u / NB2, cb2 = u - it * NB2;
+  if (R == 1 && !writer) {
+    // one row: every pick is its own item and the items go in expert order, so the item is the pick whose id
+    // ranks `it` among the picks; wave 0 finds it in registers
+    if (it >= slots) return;
+    if (wave == 0) {
+      int id;
+      float w;
+      topk_lane(L, NE, TOPK, shared, lane, id, w);
+      const int mine = lane < slots && (unsigned)id < (unsigned)E ? id : 0x7FFFFFFF;
+      int rank = 0;
+      for (int i = 0; i < slots; ++i) {
+        const int other = __builtin_amdgcn_readlane(mine, i);
+        rank += other < mine || (other == mine && i < lane);
+      }
+      const bool found = mine != 0x7FFFFFFF && rank == it;
+      if (found) {
+        item.sel[0] = mine;
+        item.sel[2] = 1;
+        item.pairs[0] = lane;
+      }
+      const unsigned long long any = __ballot(found);
+      if (lane == 0 && !any) item.sel[0] = -1;
+    }
+    __syncthreads();
+    if (item.sel[0] < 0) return;
+    NoHook none;
+    expert_unit<GS, NM, EPI, WAVES, false, 0>(X, x_stride, slots, Wup, D / GS, NI / 32, item.sel[0], 1, item.pairs, cb2,
+                                              act, NI, limit, nullptr, xs_act, lds, none);
+    return;
+  }
   if (NE <= 128 && slots <= 16 && R > WAVES) {
     // more rows than waves: four logits rows a wave, each on a row of 16 lanes
     for (int r0 = 4 * wave; r0 < R; r0 += 4 * WAVES) {
@@ -255,8 +287,6 @@ __global__ void __launch_bounds__(WAVES * 64)
     }
     return;
   }
-  const int NB2 = (NI / 32 + 1) >> 1;
-  const int u = blockIdx.x - 1, it = u / NB2, cb2 = u - it * NB2;
   if (!find_item<DTILE>(item, pk, P, E, it)) return;
   NoHook none;
   // the item's rows are summed group by group inside the unit (a pass at a time), under its first weight loads
