@@ -173,7 +173,8 @@ __global__ void __launch_bounds__(WAVES * 64)
     if (wave == 0) {
       int id;
       float w;
-      topk_lane(L, NE, TOPK, shared, lane, id, w);
+      if (L) topk_lane(L, NE, TOPK, shared, lane, id, w);
+      else id = lane < slots ? pick[lane] : -1;
       const int mine = lane < slots && (unsigned)id < (unsigned)E ? id : 0x7FFFFFFF;
       int rank = 0;
       for (int i = 0; i < slots; ++i) {
@@ -196,7 +197,10 @@ __global__ void __launch_bounds__(WAVES * 64)
                                               act, NI, limit, nullptr, xs_act, lds, none);
     return;
   }
-  if (NE <= 128 && slots <= 16 && R > WAVES) {
+  if (!L) {
+    // the picks are given (a top-k launch ran before): only the plan is made here
+    for (int p = tid; p < P; p += threads) pk[p] = (unsigned)pick[p] < (unsigned)E ? pick[p] : -1;
+  } else if (NE <= 128 && slots <= 16 && R > WAVES) {
     // more rows than waves: four logits rows a wave, each on a row of 16 lanes
     for (int r0 = 4 * wave; r0 < R; r0 += 4 * WAVES) {
       const int r = r0 + (lane >> 4);
@@ -384,7 +388,7 @@ extern "C" int tf_moe_route_up(const float* logits, int64_t ldl, int rows, int e
                                int32_t* zero, int n_zero, tf_stream_t stream) {
   clear_error();
   TF_REQUIRE(gs == 32 || gs == 64, "moe: groups of 32 or 64 inputs, not %d", gs);
-  TF_REQUIRE(logits && x && up && pick && wts && members && items && counts && desc && act && xs_act,
+  TF_REQUIRE(x && up && pick && wts && members && items && counts && desc && act && xs_act,
              "moe: null pointer argument");
   TF_REQUIRE(experts >= 1 && experts + (shared ? 1 : 0) <= EMAX && experts <= 64 * TOPK_VPL,
              "route: at most %d experts", EMAX - 1);
@@ -392,7 +396,7 @@ extern "C" int tf_moe_route_up(const float* logits, int64_t ldl, int rows, int e
              top_k);
   TF_REQUIRE(rows >= 1 && (int64_t)rows * (top_k + (shared ? 1 : 0)) <= PLAN_THREADS,
              "route: the decode routing takes at most %d pairs", PLAN_THREADS);
-  TF_REQUIRE(ldl >= experts + (shared ? 1 : 0), "route: logits rows are too short");
+  TF_REQUIRE(!logits || ldl >= experts + (shared ? 1 : 0), "route: logits rows are too short");
   TF_REQUIRE(d % gs == 0 && ni % 32 == 0 && ni % gs == 0 && d >= gs && max_items >= 1,
              "moe: hidden and intermediate sizes in whole groups and 32-column blocks");
   TF_REQUIRE(aligned16(x) && x_stride % 8 == 0 && aligned16(up) && aligned16(act),

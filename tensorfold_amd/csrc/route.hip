@@ -36,6 +36,18 @@ __global__ void __launch_bounds__(64)
   topk_row(L + (size_t)r * ldl, NE, TOPK, shared, threadIdx.x, pick + (size_t)r * slots, wts + (size_t)r * slots);
 }
 
+// A row's top-k and the group sums of its inputs: what the decode routing needs a row, spread a wave a row over the
+// chip when one workgroup would take too long over many rows.
+__global__ void __launch_bounds__(64)
+    topk_sums_kernel(const float* __restrict__ L, int64_t ldl, int NE, int TOPK, int shared, int* __restrict__ pick,
+                     float* __restrict__ wts, const uint16_t* __restrict__ X, int64_t ldx, int D, int gs,
+                     float* __restrict__ xs_x) {
+  const int r = blockIdx.x, slots = TOPK + (shared ? 1 : 0);
+  if (gs == 64) group_sums_rows<64>(X + (size_t)r * ldx, ldx, 1, D / 64, xs_x + (size_t)r * (D / 64), threadIdx.x, 64);
+  else group_sums_rows<32>(X + (size_t)r * ldx, ldx, 1, D / 32, xs_x + (size_t)r * (D / 32), threadIdx.x, 64);
+  topk_row(L + (size_t)r * ldl, NE, TOPK, shared, threadIdx.x, pick + (size_t)r * slots, wts + (size_t)r * slots);
+}
+
 // ---- plan: stable counting sort of pairs by expert -------------------------------------------------------------------
 
 // up to 1024 pairs: one block does everything
@@ -84,12 +96,13 @@ __global__ void __launch_bounds__(PLAN_THREADS)
   const int slots = TOPK + (shared ? 1 : 0), P = R * slots, E = NE + (shared ? 1 : 0), T = 16;
   cnt[tid] = 0;
   for (int i = tid; i < n_zero; i += PLAN_THREADS) zero[i] = 0;
-  if (!have_picks)
+  if (!have_picks) {      // else a launch before this one has left the picks, the weights and the group sums
     for (int r = wave; r < R; r += PLAN_THREADS / 64)
       topk_row(L + (size_t)r * ldl, NE, TOPK, shared, lane, pick + (size_t)r * slots, wts + (size_t)r * slots);
-  // group sums of x, as tf_group_sums
-  if (gs == 64) group_sums_rows<64>(X, ldx, R, D / 64, xs_x, tid, PLAN_THREADS);
-  else group_sums_rows<32>(X, ldx, R, D / 32, xs_x, tid, PLAN_THREADS);
+    // group sums of x, as tf_group_sums
+    if (gs == 64) group_sums_rows<64>(X, ldx, R, D / 64, xs_x, tid, PLAN_THREADS);
+    else group_sums_rows<32>(X, ldx, R, D / 32, xs_x, tid, PLAN_THREADS);
+  }
   __threadfence_block();
   __syncthreads();
   int e = -1;
@@ -294,9 +307,11 @@ extern "C" int tf_moe_route_decode(const float* logits, int64_t ldl, int rows, i
   TF_REQUIRE(d >= gs && d % gs == 0 && aligned16(x) && ldx % 8 == 0, "route: x rows of whole groups, 16-byte aligned");
   TF_REQUIRE(ldl >= experts + (shared ? 1 : 0), "route: logits rows are too short");
   TF_REQUIRE(n_zero >= 0 && (n_zero == 0 || zero), "route: bad counter range");
-  // more rows than the one workgroup has waves: the top-k runs first on a workgroup a row, spread over the chip
+  // more rows than the one workgroup has waves: top-k and group sums run first, a workgroup a row, spread over the chip
   const int spread = rows > PLAN_THREADS / 64;
-  if (spread) topk_kernel<<<rows, 64, 0, as_stream(stream)>>>(logits, ldl, experts, top_k, shared, pick, wts);
+  if (spread)
+    topk_sums_kernel<<<rows, 64, 0, as_stream(stream)>>>(logits, ldl, experts, top_k, shared, pick, wts, x, ldx, d, gs,
+                                                         xs_x);
   route_decode_kernel<<<1, PLAN_THREADS, 0, as_stream(stream)>>>(logits, ldl, rows, experts, top_k, shared, x, ldx, d,
                                                                 gs, pick, wts, members, items, counts, desc, xs_x, zero,
                                                                 n_zero, spread);

@@ -20,9 +20,12 @@ from . import experts as grouped
 # ``run`` issues a decode-sized layer as routing + up + down + combine launches; with this set it issues the routing
 # launch and the one fused experts launch (``decode``) instead.  Same bits either way.
 FUSED_DECODE = os.environ.get("TENSORFOLD_AMD_FUSED_DECODE", "0") == "1"
-# Up to this many router logits (rows x experts) a call, the up projection's workgroups each repeat the routing
-# instead of waiting for a routing launch; past it the repeated top-k would cost more than the launch it saves.
+# Up to this many router logits (rows x experts) a call, the up projection's workgroups each repeat the top-k
+# instead of waiting for a launch; past it the top-k runs once, a launch before, and they rebuild only the plan.
 ROUTE_UP_LOGITS = 2048
+# With this set ``decode`` makes the whole routing (top-k, plan, group sums, descriptors) in launches of its own and
+# runs the up projection from its descriptors: one launch more, for callers that want the plan before the experts.
+ROUTING_LAUNCH = os.environ.get("TENSORFOLD_AMD_ROUTING_LAUNCH", "0") == "1"
 # Item descriptors the routing launches leave for the decode expert kernels: rows of DESC_INTS int32, row 0 the
 # count; items of at most DESC_TILE pairs (TF_DESC_INTS / TF_DESC_TILE of the C header).
 DESC_INTS, DESC_TILE = 8, 2
@@ -134,7 +137,8 @@ def fusable(x: torch.Tensor, ex: grouped.Experts, buf: MoEBuffers) -> bool:
 def decode(x: torch.Tensor, logits: torch.Tensor, ex: grouped.Experts, buf: MoEBuffers, top_k: int, experts: int,
            out: torch.Tensor | None = None) -> torch.Tensor:
     """The decode layer in two launches (routing + up projection; down projection + combine), three when there are
-    many router logits (routing; up; down + combine), or, with ``FUSED_DECODE``, routing and one launch for the rest.  Same bits as
+    many router logits (top-k; plan + up; down + combine) or with ``ROUTING_LAUNCH``, or, with ``FUSED_DECODE``, routing
+    and one launch for the rest.  Same bits as
     ``select`` + ``gate_up`` + ``down`` + ``combine``; bf16 [R, D] out.  ``buf.pick``, ``buf.wts`` and ``buf.plan``
     are filled as by ``select``."""
 
@@ -167,8 +171,8 @@ def decode(x: torch.Tensor, logits: torch.Tensor, ex: grouped.Experts, buf: MoEB
         return out
     act = buf.act.view(-1, ex.width)
     arrive = ctr.data_ptr() + 4 * (1 + f["items"])        # one arrival counter a (token, 64 columns) cell
-    if n * (experts + int(buf.shared)) > ROUTE_UP_LOGITS:
-        # many logits: one routing launch, then up, down and combine from its item descriptors
+    if ROUTING_LAUNCH:
+        # the routing in a launch of its own, then up, down and combine from its item descriptors
         _lib.call("tf_moe_route_decode", _lib.ptr(logits), logits.stride(0), n, experts, top_k, int(buf.shared),
                   _lib.ptr(x), x.stride(0), ex.dims, ex.gs, _lib.ptr(buf.pick), _lib.ptr(buf.wts), _lib.ptr(plan.members),
                   _lib.ptr(plan.items), _lib.ptr(plan.counts), _lib.ptr(f["desc"]), _lib.ptr(f["xs_x"]), arrive, cells)
@@ -177,8 +181,13 @@ def decode(x: torch.Tensor, logits: torch.Tensor, ex: grouped.Experts, buf: MoEB
                   _lib.ptr(plan.counts), _lib.ptr(act), ex.width, ex.limit, items, _lib.ptr(f["xs_x"]),
                   _lib.ptr(f["xs_act"]))
     else:
-        # few logits: every workgroup of the up projection routes for itself
-        _lib.call("tf_moe_route_up", _lib.ptr(logits), logits.stride(0), n, experts, top_k, int(buf.shared), ex.gs,
+        # few logits: every workgroup of the up projection routes for itself; many: the top-k runs once, in a launch
+        # before, and the workgroups only rebuild the plan from its picks
+        given = n * (experts + int(buf.shared)) > ROUTE_UP_LOGITS
+        if given:
+            select_rows(logits, buf, top_k, experts)
+        _lib.call("tf_moe_route_up", None if given else _lib.ptr(logits), logits.stride(0), n, experts, top_k,
+                  int(buf.shared), ex.gs,
                   int(ex.swiglu), _lib.ptr(x), x.stride(0), _lib.ptr(ex.up), ex.dims, ex.width, _lib.ptr(buf.pick),
                   _lib.ptr(buf.wts), _lib.ptr(plan.members), _lib.ptr(plan.items), _lib.ptr(plan.counts),
                   _lib.ptr(f["desc"]), _lib.ptr(act), _lib.ptr(f["xs_act"]), ex.limit, items, arrive, cells)

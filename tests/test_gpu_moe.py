@@ -211,14 +211,16 @@ def test_moe_run_rows_do_not_depend_on_the_window():
 @pytest.mark.parametrize("shape,ne,rows", [(synthetic.C1, 24, 1), (synthetic.C1, 24, 8), (synthetic.C2, 48, 32),
                                            (synthetic.MoEShape("small", 512, 16, 128, 4, 32, True, True), 16, 5),
                                            (synthetic.MoEShape("small64", 384, 12, 192, 3, 64, False, False), 12, 19)])
-@pytest.mark.parametrize("path", ["route_up", "route_then_up", "one_launch"])
+@pytest.mark.parametrize("path", ["route_up", "topk_then_up", "route_then_up", "one_launch"])
 def test_the_fused_decode_layer_equals_the_separate_kernels(shape, ne, rows, path, monkeypatch):
-    """The three forms of ``decode`` (routing inside the up launch; a routing launch, then up, down, combine from its
-    item descriptors; a routing launch and one launch for up + down + combine): ids, plan and output bits equal those
-    of select + gate_up + down + combine; twice in a row on different inputs."""
+    """The forms of ``decode`` (routing inside the up launch; a top-k launch, then the plan inside the up launch; a
+    routing launch, then up, down, combine from its item descriptors; a routing launch and one launch for up + down +
+    combine): ids, plan and output bits equal those of select + gate_up + down + combine; twice in a row on
+    different inputs."""
 
     monkeypatch.setattr(moe, "FUSED_DECODE", path == "one_launch")
-    monkeypatch.setattr(moe, "ROUTE_UP_LOGITS", 0 if path == "route_then_up" else 1 << 30)
+    monkeypatch.setattr(moe, "ROUTING_LAUNCH", path == "route_then_up")
+    monkeypatch.setattr(moe, "ROUTE_UP_LOGITS", 0 if path == "topk_then_up" else 1 << 30)
 
     up, down = layer_tables(shape, 1500, ne)
     ex = experts.make([tuple(t.to(DEV) for t in m) for m in up], tuple(t.to(DEV) for t in down), shape.gs)
@@ -303,11 +305,12 @@ def test_random_shapes_of_the_decode_layer(seed):
     experts.gate_up(x, ex, ref.plan, ref.act.view(-1, ex.width), rows)
     experts.down(ref.act.view(-1, ex.width), ex, ref.plan, ref.y.view(-1, ex.dims), rows)
     want = moe.combine(ref.y, ref.wts)
-    saved = moe.FUSED_DECODE, moe.ROUTE_UP_LOGITS
+    saved = moe.FUSED_DECODE, moe.ROUTE_UP_LOGITS, moe.ROUTING_LAUNCH
     try:
-        for path in ("route_up", "route_then_up", "one_launch"):
+        for path in ("route_up", "topk_then_up", "route_then_up", "one_launch"):
             moe.FUSED_DECODE = path == "one_launch"
-            moe.ROUTE_UP_LOGITS = 0 if path == "route_then_up" else 1 << 30
+            moe.ROUTING_LAUNCH = path == "route_then_up"
+            moe.ROUTE_UP_LOGITS = 0 if path == "topk_then_up" else 1 << 30
             buf = moe.MoEBuffers(rows, cfg, DEV, shared=shared)
             for _ in range(2):
                 got = moe.decode(x, l, ex, buf, top_k, ne)
@@ -318,7 +321,7 @@ def test_random_shapes_of_the_decode_layer(seed):
                 assert torch.equal(buf.act, ref.act) and torch.equal(buf.y, ref.y), path
                 assert torch.equal(got, want), path
     finally:
-        moe.FUSED_DECODE, moe.ROUTE_UP_LOGITS = saved
+        moe.FUSED_DECODE, moe.ROUTE_UP_LOGITS, moe.ROUTING_LAUNCH = saved
     picks, _ = orr.topk_rows(l.cpu().numpy(), ne, top_k, shared=shared)
     assert np.array_equal(ref.pick.cpu().numpy(), picks)
     t = lambda m: (u32(m[0]), bits16(m[1]), bits16(m[2]))
