@@ -162,6 +162,103 @@ __global__ void __launch_bounds__(WAVES * 64)
   qmm_block<GS, WAVES>(X, ldx, XS, W, S, B, sb_stride, out, part_out, M, N, KG, SK, BM, f32, blockIdx.x, blockIdx.z, lds);
 }
 
+// The split matmul and its reduce in ONE launch, with no traffic between workgroups: a workgroup of FW waves takes a
+// (column tile, row tile) with ALL of K.  The 4 * SK sub-slices (SK slices x the 4 waves qmm_kernel runs a slice on)
+// keep their boundaries; wave w streams 4 * SK / FW consecutive ones, parking each sum in LDS, and the end adds a
+// slice's four in wave order, then the slices in slice order: the arithmetic, and so the bits, of qmm_kernel followed
+// by qmm_reduce_kernel.  The same waves are in flight as in the split launch; only the grouping differs.
+template <int GS, int FW, int RB, class WQ, class SB>
+__device__ __forceinline__ void qmm_fat_pass(const uint16_t* __restrict__ X, int64_t ldx, const float* __restrict__ XS,
+                                             const WQ& wq, const SB& sb, int r0, int tile, int per, int SK, int gA,
+                                             int gB, void* __restrict__ out, int N, int KG, int f32, float* part,
+                                             Stage<GS, 1> (&st)[DEPTH], bool loaded) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int U = 4 * SK, SPW = U / FW;
+  auto sub_begin = [&](int u) { return (u >> 2) * per + (int)((long long)(u & 3) * per / 4); };
+  const uint32_t* xl[RB];
+  const_u32_ptr xsr[RB];
+#pragma unroll
+  for (int r = 0; r < RB; ++r) {
+    xl[r] = reinterpret_cast<const uint32_t*>(X + (size_t)(r0 + r) * ldx) + (lane & 15);
+    xsr[r] = as_const(XS + (size_t)(r0 + r) * KG);
+  }
+  __syncthreads();                                  // the previous pass is done with part
+  if (per < 4) {                                    // sub-slices with no group still take part in the sums: as zeros
+    for (int q = 0; q < SPW; ++q)
+#pragma unroll
+      for (int r = 0; r < RB; ++r) part[((wave * SPW + q) * RB + r) * 64 + lane] = 0.f;
+  }
+  float acc[1][RB];
+#pragma unroll
+  for (int r = 0; r < RB; ++r) acc[0][r] = 0.f;
+  int sub = wave * SPW;
+  const int sub_last = (wave + 1) * SPW;
+  while (sub < sub_last && sub_begin(sub + 1) == sub_begin(sub)) ++sub;
+  int sub_end = sub < sub_last ? sub_begin(sub + 1) : -1;
+  auto flush = [&](int g, float (&a)[1][RB]) {
+    if (g + 1 != sub_end) return;
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+      part[(sub * RB + r) * 64 + lane] = a[0][r];
+      a[0][r] = 0.f;
+    }
+    ++sub;
+    while (sub < sub_last && sub_begin(sub + 1) == sub_begin(sub)) ++sub;
+    sub_end = sub < sub_last ? sub_begin(sub + 1) : -1;
+  };
+  auto xsum = [&](int r, int g) { return __uint_as_float(xsr[r][g]); };
+  gemv_stream<GS, 1, RB, 0>(acc, st, loaded, wq, sb, xl, xsum, gA, gB, flush);
+  __syncthreads();
+  for (int o = tid; o < RB * 64; o += FW * 64) {
+    const int r = o >> 6, l = o & 63, cc = tile * 64 + l;
+    if (cc >= N) continue;
+    float total = 0.f;
+    for (int z = 0; z < SK; ++z) {
+      float t = part[((4 * z) * RB + r) * 64 + l];
+      for (int j = 1; j < 4; ++j) t += part[((4 * z + j) * RB + r) * 64 + l];
+      total = z ? total + t : t;
+    }
+    const size_t at = (size_t)(r0 + r) * N + cc;
+    if (f32) reinterpret_cast<float*>(out)[at] = total;
+    else reinterpret_cast<uint16_t*>(out)[at] = (uint16_t)f32_bf16_bits(total);
+  }
+}
+
+template <int GS, int FW>
+__global__ void __launch_bounds__(FW * 64)
+    qmm_fat_kernel(const uint16_t* __restrict__ X, int64_t ldx, const float* __restrict__ XS,
+                   const uint32_t* __restrict__ W, const uint16_t* __restrict__ S, const uint16_t* __restrict__ B,
+                   int64_t sb_stride, void* __restrict__ out, int M, int N, int KG, int SK, int BM, int f32) {
+  extern __shared__ float lds[];            // sub-slice sums [4 * SK][RBMAX][64]
+  const int tiles = (N + 63) >> 6;
+  const int tile = blockIdx.x % tiles, rt = blockIdx.x / tiles;
+  const int per = KG / SK;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  constexpr int CH = GS / 32;
+  const uint32_t* wbase = W + ((size_t)tile * KG) * (size_t)(CH * 256) + lane * 4;
+  const int col = tile * 64 + lane;
+  auto wq = [&](int g, int m, int i) { return ldg16(wbase + ((size_t)g * CH + i) * 256); };
+  auto sb = [&](int g, int m, float& s, float& b) {
+    s = bf16_f32(S[(size_t)g * sb_stride + col]);
+    b = bf16_f32(B[(size_t)g * sb_stride + col]);
+  };
+  auto sub_begin = [&](int u) { return (u >> 2) * per + (int)((long long)(u & 3) * per / 4); };
+  const int SPW = 4 * SK / FW;
+  const int gA = sub_begin(wave * SPW), gB = sub_begin((wave + 1) * SPW);
+  const int m_end = min(M, (rt + 1) * BM);
+  int r0 = rt * BM;
+  Stage<GS, 1> st[DEPTH];
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d)
+    if (gA + d < gB) load_weights<GS, 1>(st[d], wq, sb, gA + d);
+  bool loaded = true;
+  for (; r0 + 2 <= m_end; r0 += 2) {
+    qmm_fat_pass<GS, FW, 2>(X, ldx, XS, wq, sb, r0, tile, per, SK, gA, gB, out, N, KG, f32, lds, st, loaded);
+    loaded = gB - gA <= DEPTH;
+  }
+  if (r0 < m_end) qmm_fat_pass<GS, FW, 1>(X, ldx, XS, wq, sb, r0, tile, per, SK, gA, gB, out, N, KG, f32, lds, st, loaded);
+}
+
 // Up to four weights against one x in one launch (and one reduce launch): workgroups [first[w], first[w + 1]) take
 // weight w's (column tile, row tile) pairs; grid.z is the largest slice count and a weight's surplus slices leave.
 constexpr int GROUP_MAX = 4;
@@ -369,6 +466,25 @@ extern "C" int tf_qmm(const uint16_t* x, int64_t ldx, const float* xs, const uin
   const int tiles = (n + 63) / 64, rts = (m + bm - 1) / bm, per = kg / sk;
   const size_t smem = sizeof(float) * ((size_t)QMM_WAVES * RBMAX * 64);
   TF_REQUIRE((int64_t)tiles * rts <= 0x7FFFFFFF && sk <= 65535, "qmm: grid too large");
+  if (reduce && m <= RBMAX && (sk == 2 || sk == 4 || sk == 8 || sk == 16)) {
+    // one pass of rows: split and reduce in one launch, a workgroup of 8 or 16 waves a tile taking every slice (same
+    // bits).  With more passes the split launch is better: its waves keep their one or two groups in registers from
+    // pass to pass, these would stream theirs again.
+    const dim3 fat((unsigned)(tiles * rts));
+    const size_t fat_smem = sizeof(float) * ((size_t)4 * sk * RBMAX * 64);
+#define TF_FAT(GS_, FW_) \
+  qmm_fat_kernel<GS_, FW_><<<fat, FW_ * 64, fat_smem, s>>>(x, ldx, xs, weight, scales, biases, sb_stride, out, m, n, kg, sk, bm, f32)
+    if (gs == 64) {
+      if (sk == 2) TF_FAT(64, 8);
+      else TF_FAT(64, 16);
+    } else {
+      if (sk == 2) TF_FAT(32, 8);
+      else TF_FAT(32, 16);
+    }
+#undef TF_FAT
+    TF_LAUNCH_OK("tf_qmm");
+    return 0;
+  }
   const dim3 grid((unsigned)(tiles * rts), 1, (unsigned)sk);
   if (gs == 64)
     qmm_kernel<64, QMM_WAVES><<<grid, QMM_WAVES * 64, smem, s>>>(x, ldx, xs, weight, scales, biases, sb_stride, out,
