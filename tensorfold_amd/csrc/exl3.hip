@@ -75,17 +75,33 @@ struct Windows {
   }
 };
 
+// s * C + A modulo 2^32 for a 16-bit s: the full 32-bit multiply runs at a quarter of the rate of the 24-bit ones,
+// so the constant goes in as two 16-bit halves (s * lo + A, then s * hi shifted in): three full-rate instructions.
+// (Written as instructions: the compiler folds the C expression back into the one 32-bit multiply.)
+template <uint32_t C, uint32_t A>
+__device__ __forceinline__ uint32_t mul16(uint32_t s) {
+  uint32_t lo, hi;
+  if constexpr (A != 0) {
+    const uint32_t add = A;
+    asm("v_mad_u32_u24 %0, %1, %2, %3" : "=v"(lo) : "v"(s), "s"(C & 0xFFFFu), "v"(add));
+  } else {
+    asm("v_mul_u32_u24 %0, %2, %1" : "=v"(lo) : "v"(s), "s"(C & 0xFFFFu));
+  }
+  asm("v_mul_u32_u24 %0, %2, %1" : "=v"(hi) : "v"(s), "s"(C >> 16));
+  return (hi << 16) + lo;
+}
+
 // fp16 bits of the codebook value of state s
 template <int CB>
 __device__ __forceinline__ uint16_t code_value(uint32_t s) {
   if constexpr (CB == 2) {
-    const uint32_t x = s * 0x83DCD12Du;
+    const uint32_t x = mul16<0x83DCD12Du, 0u>(s);
     const uint32_t hs = 1024u + (x & 255u) + ((x >> 8) & 255u) + ((x >> 16) & 255u) + (x >> 24);
     const __half hv = __ushort_as_half((unsigned short)(0x6400u + (hs - 1024u)));   // fp16 of 1024 + byte sum (< 2048)
     const __half r = __hfma(hv, __ushort_as_half((unsigned short)0x1EEE), __ushort_as_half((unsigned short)0xC931));
     return __half_as_ushort(r);
   } else {
-    uint32_t x = CB == 1 ? s * 0xCBAC1FEDu : s * 89226354u + 64248484u;
+    uint32_t x = CB == 1 ? mul16<0xCBAC1FEDu, 0u>(s) : mul16<89226354u, 64248484u>(s);
     x = (x & 0x8FFF8FFFu) ^ 0x3B603B60u;
     const __half r = __hadd(__ushort_as_half((unsigned short)(x & 0xFFFFu)), __ushort_as_half((unsigned short)(x >> 16)));
     return __half_as_ushort(r);
@@ -210,38 +226,61 @@ __global__ void __launch_bounds__(WK * 64)
     for (int j = 0; j < 8; ++j) acc[j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
     // the A operand's row: lane (row c, quarter kq); rows past the pass read a valid row and are dropped later
     const uint16_t* xr = xh + (size_t)(m0 + (c < R ? c : R - 1)) * K + 2 * kq;
-    // the stored words of the 16 tiles of a k-tile pair and the pair's activations are requested one pair ahead
+    // The stored words of a k-tile pair (two runs of 8 tiles) come in with coalesced loads, a dword a lane, one pair
+    // ahead, and go through the wave's own part of LDS: each lane then reads the two or three words its windows
+    // start in.  (A lane loading its words itself costs sixteen times the load instructions, and the kernel was
+    // bound by their issue.)  A staged tile repeats its first two words at its end, so a window never wraps.
     constexpr int NW = Windows<K2>::NW;
+    constexpr int TWP = TW + 2, RUN = 8 * TW, GL = (RUN + 63) / 64;
     const Windows<K2> win(L, h);
-    uint32_t wc[16][NW], wn[16][NW];
+    uint32_t* stage = reinterpret_cast<uint32_t*>(red) + wave * (16 * 128);       // 16 tiles of TWP words
+    if (pass) __syncthreads();                 // the previous pass is done with red
+    uint32_t g[2][GL];
     u32x4_t av, an;
-    auto fetch = [&](int pr, uint32_t (&w)[16][NW], u32x4_t& a) {
+    auto fetch = [&](int pr, uint32_t (&w)[2][GL], u32x4_t& a) {
       const uint32_t* xk = reinterpret_cast<const uint32_t*>(xr + 32 * pr);
       a = (u32x4_t){xk[0], xk[4], xk[8], xk[12]};
-      const uint32_t* t0 = tiles + (size_t)(2 * pr) * stride_k;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        win.load(t0 + j * TW, w[2 * j]);
-        win.load(t0 + stride_k + j * TW, w[2 * j + 1]);
+      for (int r = 0; r < 2; ++r) {
+        const uint32_t* run = tiles + (size_t)(2 * pr + r) * stride_k;
+#pragma unroll
+        for (int i = 0; i < GL; ++i) w[r][i] = lane + 64 * i < RUN ? run[lane + 64 * i] : 0u;
       }
     };
-    if (pr0 < pr1) fetch(pr0, wc, av);
+    auto put = [&](const uint32_t (&w)[2][GL]) {
+#pragma unroll
+      for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int i = 0; i < GL; ++i) {
+          const int idx = lane + 64 * i, j = idx / TW, q = idx - j * TW;
+          if (idx < RUN) {
+            stage[(8 * r + j) * TWP + q] = w[r][i];
+            if (q < 2) stage[(8 * r + j) * TWP + TW + q] = w[r][i];
+          }
+        }
+    };
+    if (pr0 < pr1) fetch(pr0, g, av);
     for (int pr = pr0; pr < pr1; ++pr) {
-      fetch(pr + 1 < pr1 ? pr + 1 : pr, wn, an);
+      put(g);
+      __builtin_amdgcn_wave_barrier();         // the wave's LDS accesses run in program order: no wait beyond the data's
+      fetch(pr + 1 < pr1 ? pr + 1 : pr, g, an);
       const f16x8_t a = __builtin_bit_cast(f16x8_t, av);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
+        uint32_t w0[NW], w1[NW];
+#pragma unroll
+        for (int q = 0; q < NW; ++q) {
+          w0[q] = stage[j * TWP + win.wi + q];
+          w1[q] = stage[(8 + j) * TWP + win.wi + q];
+        }
         uint32_t b0, b1, b2, b3;
-        decode4<K2, CB>(win, wc[2 * j], b0, b1);
-        decode4<K2, CB>(win, wc[2 * j + 1], b2, b3);
+        decode4<K2, CB>(win, w0, b0, b1);
+        decode4<K2, CB>(win, w1, b2, b3);
         const u32x4_t bw = {b0, b1, b2, b3};
         const f16x8_t b = __builtin_bit_cast(f16x8_t, bw);
         acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[j], 0, 0, 0);
       }
-#pragma unroll
-      for (int t = 0; t < 16; ++t)
-#pragma unroll
-        for (int q = 0; q < NW; ++q) wc[t][q] = wn[t][q];
+      __builtin_amdgcn_wave_barrier();
       av = an;
     }
     // D[row 4 kq + i][column c] of column tile j -> red[wave][row][16 j + c]
