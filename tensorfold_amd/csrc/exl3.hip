@@ -75,33 +75,17 @@ struct Windows {
   }
 };
 
-// s * C + A modulo 2^32 for a 16-bit s: the full 32-bit multiply runs at a quarter of the rate of the 24-bit ones,
-// so the constant goes in as two 16-bit halves (s * lo + A, then s * hi shifted in): three full-rate instructions.
-// (Written as instructions: the compiler folds the C expression back into the one 32-bit multiply.)
-template <uint32_t C, uint32_t A>
-__device__ __forceinline__ uint32_t mul16(uint32_t s) {
-  uint32_t lo, hi;
-  if constexpr (A != 0) {
-    const uint32_t add = A;
-    asm("v_mad_u32_u24 %0, %1, %2, %3" : "=v"(lo) : "v"(s), "s"(C & 0xFFFFu), "v"(add));
-  } else {
-    asm("v_mul_u32_u24 %0, %2, %1" : "=v"(lo) : "v"(s), "s"(C & 0xFFFFu));
-  }
-  asm("v_mul_u32_u24 %0, %2, %1" : "=v"(hi) : "v"(s), "s"(C >> 16));
-  return (hi << 16) + lo;
-}
-
 // fp16 bits of the codebook value of state s
 template <int CB>
 __device__ __forceinline__ uint16_t code_value(uint32_t s) {
   if constexpr (CB == 2) {
-    const uint32_t x = mul16<0x83DCD12Du, 0u>(s);
+    const uint32_t x = s * 0x83DCD12Du;
     const uint32_t hs = 1024u + (x & 255u) + ((x >> 8) & 255u) + ((x >> 16) & 255u) + (x >> 24);
     const __half hv = __ushort_as_half((unsigned short)(0x6400u + (hs - 1024u)));   // fp16 of 1024 + byte sum (< 2048)
     const __half r = __hfma(hv, __ushort_as_half((unsigned short)0x1EEE), __ushort_as_half((unsigned short)0xC931));
     return __half_as_ushort(r);
   } else {
-    uint32_t x = CB == 1 ? mul16<0xCBAC1FEDu, 0u>(s) : mul16<89226354u, 64248484u>(s);
+    uint32_t x = CB == 1 ? s * 0xCBAC1FEDu : s * 89226354u + 64248484u;
     x = (x & 0x8FFF8FFFu) ^ 0x3B603B60u;
     const __half r = __hadd(__ushort_as_half((unsigned short)(x & 0xFFFFu)), __ushort_as_half((unsigned short)(x >> 16)));
     return __half_as_ushort(r);
