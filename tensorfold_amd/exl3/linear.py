@@ -38,6 +38,8 @@ def plan(k: int, n: int, waves: int = 4608, min_pairs: int = 4) -> tuple[int, in
     sk = 1
     while sk < 64 and nb * 2 * sk * wk <= waves and pairs // (2 * sk * wk) >= min_pairs:
         sk *= 2
+    if wk == 4 and nb * sk * 8 <= 5120 and pairs // (sk * 8) >= min_pairs:
+        wk = 8              # few column blocks: five waves a SIMD (the kernel's register budget) still fit
     return sk, wk
 
 
