@@ -278,22 +278,11 @@ def test_decode_replays_in_a_graph_with_new_logits_and_inputs():
         moe.decode(torch.cat([x, x]), torch.cat([l, l]), ex, buf, shape.top_k, ne)      # more rows than the buffers hold
 
 
-@pytest.mark.parametrize("seed", range(12))
-def test_random_shapes_of_the_decode_layer(seed):
-    """Drawn shapes (hidden, width, experts, slots, group size, activation, rows): every form of ``decode`` gives the
-    bits of the separate kernels, ids equal the oracle's, and the output is within 2e-3 of the CPU oracle's layer."""
+def check_decode_forms(shape, ne, rows, seed, oracle=True):
+    """Every form of ``decode`` gives the bits of the separate kernels (twice in a row), ids equal the oracle's, and
+    the output is within 2e-3 of the CPU oracle's layer."""
 
-    import random
-
-    rnd = random.Random(seed)
-    gs = rnd.choice([32, 64])
-    hidden, width = 64 * rnd.randint(1, 12), 64 * rnd.randint(1, 10)
-    ne = rnd.choice([2, 3, 5, 8, 17, 33, 64, 100, 128, 130, 200])
-    shared = rnd.random() < 0.4
-    top_k = rnd.randint(1, min(8, ne))
-    swiglu = rnd.random() < 0.5
-    rows = rnd.choice([1, 2, 3, 5, 8, 13, 16, 17, 24, 33, 40])
-    shape = synthetic.MoEShape(f"drawn{seed}", hidden, ne, width, top_k, gs, swiglu, shared)
+    gs, top_k, shared, swiglu, hidden, width = shape.gs, shape.top_k, shape.shared, shape.swiglu, shape.hidden, shape.width
     up, down = layer_tables(shape, 3000 + seed, ne)
     ex = experts.make([tuple(t.to(DEV) for t in m) for m in up], tuple(t.to(DEV) for t in down), gs)
     cfg = type("c", (), dict(num_experts_per_tok=top_k, num_experts=ne, moe_intermediate_size=width,
@@ -324,7 +313,35 @@ def test_random_shapes_of_the_decode_layer(seed):
         moe.FUSED_DECODE, moe.ROUTE_UP_LOGITS, moe.ROUTING_LAUNCH = saved
     picks, _ = orr.topk_rows(l.cpu().numpy(), ne, top_k, shared=shared)
     assert np.array_equal(ref.pick.cpu().numpy(), picks)
-    t = lambda m: (u32(m[0]), bits16(m[1]), bits16(m[2]))
-    want_bits = native.moe_layer(bits16(x.cpu()), picks, ref.wts.cpu().numpy(), t(up[0]) if swiglu else None,
-                                 t(up[1]) if swiglu else t(up[0]), t(down), gs)
-    assert rel_l2(f32(want), ora.bf16_from_bits(want_bits)) <= TOL
+    if oracle:
+        t = lambda m: (u32(m[0]), bits16(m[1]), bits16(m[2]))
+        want_bits = native.moe_layer(bits16(x.cpu()), picks, ref.wts.cpu().numpy(), t(up[0]) if swiglu else None,
+                                     t(up[1]) if swiglu else t(up[0]), t(down), gs)
+        assert rel_l2(f32(want), ora.bf16_from_bits(want_bits)) <= TOL
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_shapes_of_the_decode_layer(seed):
+    """Drawn shapes (hidden, width, experts, slots, group size, activation, rows) through ``check_decode_forms``."""
+
+    import random
+
+    rnd = random.Random(seed)
+    gs = rnd.choice([32, 64])
+    hidden, width = 64 * rnd.randint(1, 12), 64 * rnd.randint(1, 10)
+    ne = rnd.choice([2, 3, 5, 8, 17, 33, 64, 100, 128, 130, 200])
+    shared = rnd.random() < 0.4
+    top_k = rnd.randint(1, min(8, ne))
+    swiglu = rnd.random() < 0.5
+    rows = rnd.choice([1, 2, 3, 5, 8, 13, 16, 17, 24, 33, 40])
+    check_decode_forms(synthetic.MoEShape(f"drawn{seed}", hidden, ne, width, top_k, gs, swiglu, shared), ne, rows, seed)
+
+
+@pytest.mark.parametrize("hidden,width,ne,top_k,gs,swiglu,shared,rows", [
+    (64, 64, 256, 8, 64, False, False, 128),          # 1,024 pairs
+    (128, 64, 64, 63, 32, True, True, 16),            # 64 slots a row
+    (64, 128, 1023, 4, 64, False, True, 2),           # the most experts
+    (64, 64, 1, 1, 32, False, False, 1024),           # one expert takes every pair
+])
+def test_the_decode_layer_at_its_limits(hidden, width, ne, top_k, gs, swiglu, shared, rows):
+    check_decode_forms(synthetic.MoEShape("limit", hidden, ne, width, top_k, gs, swiglu, shared), ne, rows, 99)
