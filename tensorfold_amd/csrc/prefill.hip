@@ -388,20 +388,25 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
         // step's activations are requested now and staged at the end of the step
         load_a(min(step + 1, last), ar);
         const unsigned char* abuf = smem + u * STAGE + c * AROW + kq * 16;
-        f16x8_t a = *reinterpret_cast<const f16x8_t*>(abuf);
+        // activation operands are requested two row tiles before their MFMAs (an LDS read takes about as long as
+        // one row tile's four MFMAs): operand t of the step is (chunk t / RT, row tile t % RT)
+        auto read_a = [&](int t) {
+          return *reinterpret_cast<const f16x8_t*>(abuf + 16 * (t % RT) * AROW + (t / RT) * 64);
+        };
+        f16x8_t a = read_a(0), a1 = read_a(1);
 #pragma unroll
         for (int i = 0; i < CPS; ++i) {
           f16x8_t bnext[TJ];
 #pragma unroll
           for (int r = 0; r < RT; ++r) {
-            // the next operand (next row tile, or the next chunk's first) is requested before this one is used
-            const int rn = r + 1 < RT ? r + 1 : 0, in = r + 1 < RT ? i : i + 1;
-            f16x8_t an = a;
-            if (in < CPS) an = *reinterpret_cast<const f16x8_t*>(abuf + 16 * rn * AROW + in * 64);
+            const int t = i * RT + r;
+            f16x8_t a2 = a1;
+            if (t + 2 < CPS * RT) a2 = read_a(t + 2);
 #pragma unroll
             for (int j = 0; j < TJ; ++j)
               acc[j][r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bcur[j], acc[j][r], 0, 0, 0);
-            a = an;
+            a = a1;
+            a1 = a2;
             // a share of the next chunk's dequantization rides along with each row tile
             constexpr int JPR = (TJ + RT - 1) / RT;          // operands a row tile (2, 1, 1 for RT = 2, 4, 8)
 #pragma unroll
