@@ -26,7 +26,9 @@
 namespace tf {
 namespace {
 
-// A workgroup takes (item, pair of 32-column blocks); see expert_unit.
+// A workgroup takes (item, pair of 32-column blocks, RBMAX of the item's rows): one pass over its weights, as with
+// item descriptors.  (Taking all of an item's up to 16 rows made it stream the same weights up to eight times, and
+// a compute unit's workgroups together overflow the L2 between passes.)  blockIdx.y picks the rows; see expert_unit.
 template <int GS, int NM, int EPI, int WAVES, bool XSG>
 __global__ void __launch_bounds__(WAVES * 64)
     expert_kernel(const uint16_t* __restrict__ X, int64_t x_stride, int slots, const uint32_t* __restrict__ W, int KG,
@@ -37,10 +39,14 @@ __global__ void __launch_bounds__(WAVES * 64)
   const int NB2 = (NB + 1) >> 1;
   const int it = blockIdx.x / NB2, cb2 = blockIdx.x - it * NB2;
   if (it >= counts[0]) return;
-  const int e = items[3 * it], first = items[3 * it + 1], cnt = items[3 * it + 2];
+  const int e = items[3 * it], first = items[3 * it + 1], total = items[3 * it + 2];
   NoHook none;
-  expert_unit<GS, NM, EPI, WAVES, XSG, 0>(X, x_stride, slots, W, KG, NB, e, cnt, members + first, cb2, out, N, limit, xs_in,
-                                       xs_out, lds, none);
+  // rows RBMAX y .. of every 16 (a decode item holds at most 16, so this runs once)
+  for (int skip = RBMAX * blockIdx.y; skip < total; skip += RBMAX * gridDim.y) {
+    if (skip != RBMAX * (int)blockIdx.y) __syncthreads();
+    expert_unit<GS, NM, EPI, WAVES, XSG, 0>(X, x_stride, slots, W, KG, NB, e, min(RBMAX, total - skip),
+                                            members + first + skip, cb2, out, N, limit, xs_in, xs_out, lds, none);
+  }
 }
 
 // The same unit taken from an item descriptor as tf_moe_route_decode and tf_moe_route_up write them: one read
@@ -347,7 +353,7 @@ int launch_experts(const uint16_t* x, int64_t x_stride, int slots, const uint32_
   TF_REQUIRE(grid <= 0x7FFFFFFF, "experts: %lld workgroups exceed the grid limit", (long long)grid);
   const size_t smem = sizeof(float) * expert_lds_floats(NM, kg, XSG);
   TF_REQUIRE(smem <= 64 * 1024, "experts: K/gs = %d groups need %zu bytes of LDS (limit 65536)", kg, smem);
-  const dim3 g((unsigned)grid);
+  const dim3 g((unsigned)grid, 16 / RBMAX);          // decode items hold at most 16 pairs
 #define TF_GO(W_)                                                                                                  \
   expert_kernel<GS, NM, EPI, W_, XSG><<<g, W_ * 64, smem, stream>>>(x, x_stride, slots, w, kg, nb, items, counts, \
                                                                     members, out, n, limit, xs_in, xs_out)
