@@ -330,6 +330,7 @@ __global__ void __launch_bounds__(256)
 }
 
 constexpr int QMM_WAVES = 4;
+constexpr int FAT_ROWS = 8;          // rows up to which tf_qmm runs the one-launch form
 
 // Waves a workgroup of the expert GEMV: few workgroups (a small batch) spread each one's K over 16 waves, many
 // workgroups keep 4 longer-running waves each so that more of them are resident.  Scheduling only: bits do not move.
@@ -472,11 +473,14 @@ extern "C" int tf_qmm(const uint16_t* x, int64_t ldx, const float* xs, const uin
   const int tiles = (n + 63) / 64, rts = (m + bm - 1) / bm, per = kg / sk;
   const size_t smem = sizeof(float) * ((size_t)QMM_WAVES * RBMAX * 64);
   TF_REQUIRE((int64_t)tiles * rts <= 0x7FFFFFFF && sk <= 65535, "qmm: grid too large");
-  if (reduce && m <= RBMAX && (sk == 2 || sk == 4 || sk == 8 || sk == 16)) {
-    // one pass of rows: split and reduce in one launch, a workgroup of 8 or 16 waves a tile taking every slice (same
-    // bits).  With more passes the split launch is better: its waves keep their one or two groups in registers from
-    // pass to pass, these would stream theirs again.
-    const dim3 fat((unsigned)(tiles * rts));
+  const int64_t fat_blocks = (int64_t)((n + 63) / 64) * ((m + RBMAX - 1) / RBMAX);
+  if (reduce && (m <= RBMAX || (m <= FAT_ROWS && fat_blocks <= 512)) && (sk == 2 || sk == 4 || sk == 8 || sk == 16)) {
+    // few rows: split and reduce in one launch, a workgroup of 8 or 16 waves taking every slice of a tile for RBMAX
+    // rows in one pass (same bits), while those workgroups fit the chip at once (512 of 16 waves).  Past that, and
+    // with many rows, the split launch is better: its waves keep their one or two groups in registers from pass to
+    // pass.
+    bm = RBMAX;
+    const dim3 fat((unsigned)(tiles * ((m + RBMAX - 1) / RBMAX)));
     const size_t fat_smem = sizeof(float) * ((size_t)4 * sk * RBMAX * 64);
 #define TF_FAT(GS_, FW_) \
   qmm_fat_kernel<GS_, FW_><<<fat, FW_ * 64, fat_smem, s>>>(x, ldx, xs, weight, scales, biases, sb_stride, out, m, n, kg, sk, bm, f32)
