@@ -231,13 +231,13 @@ __device__ __forceinline__ void qmm_fat_pass(const uint16_t* __restrict__ X, int
 }
 
 template <int GS, int FW>
-__global__ void __launch_bounds__(FW * 64)
-    qmm_fat_kernel(const uint16_t* __restrict__ X, int64_t ldx, const float* __restrict__ XS,
-                   const uint32_t* __restrict__ W, const uint16_t* __restrict__ S, const uint16_t* __restrict__ B,
-                   int64_t sb_stride, void* __restrict__ out, int M, int N, int KG, int SK, int BM, int f32) {
-  extern __shared__ float lds[];            // sub-slice sums [4 * SK][RBMAX][64]
+__device__ __forceinline__ void qmm_fat_block(const uint16_t* __restrict__ X, int64_t ldx, const float* __restrict__ XS,
+                                              const uint32_t* __restrict__ W, const uint16_t* __restrict__ S,
+                                              const uint16_t* __restrict__ B, int64_t sb_stride,
+                                              void* __restrict__ out, int M, int N, int KG, int SK, int BM, int f32,
+                                              int block, float* lds) {
   const int tiles = (N + 63) >> 6;
-  const int tile = blockIdx.x % tiles, rt = blockIdx.x / tiles;
+  const int tile = block % tiles, rt = block / tiles;
   const int per = KG / SK;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   constexpr int CH = GS / 32;
@@ -263,6 +263,15 @@ __global__ void __launch_bounds__(FW * 64)
     loaded = gB - gA <= DEPTH;
   }
   if (r0 < m_end) qmm_fat_pass<GS, FW, 1>(X, ldx, XS, wq, sb, r0, tile, per, SK, gA, gB, out, N, KG, f32, lds, st, loaded);
+}
+
+template <int GS, int FW>
+__global__ void __launch_bounds__(FW * 64)
+    qmm_fat_kernel(const uint16_t* __restrict__ X, int64_t ldx, const float* __restrict__ XS,
+                   const uint32_t* __restrict__ W, const uint16_t* __restrict__ S, const uint16_t* __restrict__ B,
+                   int64_t sb_stride, void* __restrict__ out, int M, int N, int KG, int SK, int BM, int f32) {
+  extern __shared__ float lds[];            // sub-slice sums [4 * SK][RBMAX][64]
+  qmm_fat_block<GS, FW>(X, ldx, XS, W, S, B, sb_stride, out, M, N, KG, SK, BM, f32, blockIdx.x, lds);
 }
 
 // Up to four weights against one x in one launch (and one reduce launch): workgroups [first[w], first[w + 1]) take
@@ -292,6 +301,20 @@ __global__ void __launch_bounds__(WAVES * 64)
   if ((int)blockIdx.z >= a.sk[w]) return;
   qmm_block<GS, WAVES>(X, ldx, XS, a.w[w], a.s[w], a.b[w], a.sb_stride[w], a.out[w], a.part[w], M, a.n[w], KG, a.sk[w],
                        BM, f32, blockIdx.x - a.first[w], blockIdx.z, lds);
+}
+
+// The grouped launch in the one-launch form (see qmm_fat_block): every weight's K split is 4, 8 or 16.
+template <int GS>
+__global__ void __launch_bounds__(1024)
+    qmm_group_fat_kernel(const uint16_t* __restrict__ X, int64_t ldx, const float* __restrict__ XS, GroupArgs a, int M,
+                         int KG, int BM, int f32) {
+  extern __shared__ float lds[];
+  int w = 0;
+#pragma unroll
+  for (int i = 1; i < GROUP_MAX; ++i)
+    if (i < a.count && (int)blockIdx.x >= a.first[i]) w = i;
+  qmm_fat_block<GS, 16>(X, ldx, XS, a.w[w], a.s[w], a.b[w], a.sb_stride[w], a.out[w], M, a.n[w], KG, a.sk[w], BM, f32,
+                        blockIdx.x - a.first[w], lds);
 }
 
 __global__ void qmm_group_reduce_kernel(GroupArgs a, int M, int f32) {
@@ -524,7 +547,17 @@ extern "C" int tf_qmm_group(const uint16_t* x, int64_t ldx, const float* xs, int
   TF_REQUIRE(aligned16(x) && (m == 1 || ldx % 8 == 0), "x rows must start on 16-byte boundaries");
   TF_REQUIRE(ldx >= k || m == 1, "x: (M, K) bf16 with contiguous rows");
   TF_REQUIRE(k % gs == 0, "K splits into whole groups a slice");
-  const int kg = k / gs, rts = (m + bm - 1) / bm;
+  const int kg = k / gs;
+  // few rows and every K split 4, 8 or 16: the one-launch form (two rows a workgroup), as tf_qmm
+  bool fat = m <= FAT_ROWS;
+  int64_t fat_blocks = 0;
+  for (int i = 0; i < count && fat; ++i) {
+    fat = ns && sks && ns[i] >= 1 && (sks[i] == 4 || sks[i] == 8 || sks[i] == 16);
+    if (fat) fat_blocks += (int64_t)((ns[i] + 63) / 64) * ((m + RBMAX - 1) / RBMAX);
+  }
+  fat = fat && (m <= RBMAX || fat_blocks <= 512);
+  if (fat) bm = RBMAX;
+  const int rts = (m + bm - 1) / bm;
   GroupArgs a{}, r{};
   int max_sk = 1;
   int64_t blocks = 0, chunks = 0;
@@ -555,6 +588,13 @@ extern "C" int tf_qmm_group(const uint16_t* x, int64_t ldx, const float* xs, int
   a.count = count;
   a.first[count] = (int)blocks;
   hipStream_t s = as_stream(stream);
+  if (fat) {
+    const size_t fat_smem = sizeof(float) * ((size_t)4 * max_sk * RBMAX * 64);
+    if (gs == 64) qmm_group_fat_kernel<64><<<(unsigned)blocks, 1024, fat_smem, s>>>(x, ldx, xs, a, m, kg, bm, f32);
+    else qmm_group_fat_kernel<32><<<(unsigned)blocks, 1024, fat_smem, s>>>(x, ldx, xs, a, m, kg, bm, f32);
+    TF_LAUNCH_OK("tf_qmm_group");
+    return 0;
+  }
   const size_t smem = sizeof(float) * ((size_t)QMM_WAVES * RBMAX * 64);
   const dim3 grid((unsigned)blocks, 1, (unsigned)max_sk);
   if (gs == 64) qmm_group_kernel<64, QMM_WAVES><<<grid, QMM_WAVES * 64, smem, s>>>(x, ldx, xs, a, m, kg, bm, f32);
