@@ -53,13 +53,14 @@ int tf_qmm_unpack(const uint32_t* weight, const uint16_t* scales_t, const uint16
 int tf_group_sums(const uint16_t* x, int64_t ldx, int m, int k, int gs, float* xs, tf_stream_t stream);
 /* Decode-form matmul: per group in order acc = fma(xs, b, fma(P, s, acc)), P = sum x*q with exact q; K in `sk`
  * slices summed in slice order; one rounding to bf16 (or fp32 with f32).  `part` fp32 [sk, m, n] is required when
- * sk > 1 (with reduce == 0 the slices are left there unadded).  sb_stride = elements between scale rows (>= npad).
- * Replaces kernels/qmm.cpp:18-48 `qmm`. */
+ * sk > 1 (with reduce == 0 the slices are left there unadded; with few rows and reduce != 0 the slices are added
+ * inside the one launch, in the same order, and `part` goes unused).  sb_stride = elements between scale rows
+ * (>= npad).  Replaces kernels/qmm.cpp:18-48 `qmm`. */
 int tf_qmm(const uint16_t* x, int64_t ldx, const float* xs, const uint32_t* weight, const uint16_t* scales,
            const uint16_t* biases, int64_t sb_stride, void* out, float* part, int m, int n, int k, int sk, int gs,
            int bm, int f32, int reduce, tf_stream_t stream);
-/* `count` (1 to 4) weights against one x in one launch (plus one reduce launch when any K is split): the bits of
- * tf_qmm on each.  The arrays are host arrays of `count` entries, read during the call: packed weights, transposed
+/* `count` (1 to 4) weights against one x in one launch (plus one reduce launch when any K is split and the rows are
+ * many): the bits of tf_qmm on each.  The arrays are host arrays of `count` entries, read during the call: packed weights, transposed
  * scales and biases with their row strides, outputs, parts (fp32 [sks[i], m, ns[i]], may be NULL where sks[i] == 1),
  * column counts and slice counts.  Replaces kernels/qmm.cpp:51-80 `qmm_group`. */
 int tf_qmm_group(const uint16_t* x, int64_t ldx, const float* xs, int count, const uint32_t* const* weights,
