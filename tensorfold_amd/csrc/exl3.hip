@@ -301,11 +301,22 @@ __global__ void __launch_bounds__(WK * 64)
       if (last) {
         for (int r = wave; r < R; r += WK) {
           const size_t at = (size_t)(m0 + r) * N + col0 + 2 * lane;
-          float sx = __hip_atomic_load(Z + at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          float sy = __hip_atomic_load(Z + at + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          for (int q = 1; q < SK; ++q) {
-            sx += __hip_atomic_load(Z + (size_t)q * M * N + at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            sy += __hip_atomic_load(Z + (size_t)q * M * N + at + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          // eight splits' loads go out together (one trip to memory, not eight), then the sums in split order
+          float sx = 0.f, sy = 0.f;
+          for (int q0 = 0; q0 < SK; q0 += 8) {
+            float vx[8], vy[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const float* zq = Z + (size_t)(q0 + j < SK ? q0 + j : SK - 1) * M * N + at;
+              vx[j] = __hip_atomic_load(zq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              vy[j] = __hip_atomic_load(zq + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+              if (q0 + j < SK) {
+                sx = q0 + j ? sx + vx[j] : vx[j];
+                sy = q0 + j ? sy + vy[j] : vy[j];
+              }
           }
           finish_row(sx, sy, lane, svh, bias, col0 + 2 * lane, y, y_dtype, at);
         }

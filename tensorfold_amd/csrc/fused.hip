@@ -64,9 +64,18 @@ __device__ __forceinline__ void combine_cells(const int* pairs, int* last, int c
     if (!last[r] || col >= D) continue;
     const int token = pairs[r] / slots;
     float a = 0.f;
-    for (int k = 0; k < slots; ++k) {
-      const float w = wts[(size_t)token * slots + k];
-      a = fmaf(w, ld_agent(y + ((size_t)token * slots + k) * D + col), a);
+    // eight slots' loads go out together (one trip to memory instead of eight), then the sum in slot order
+    for (int k0 = 0; k0 < slots; k0 += 8) {
+      float v[8], w[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int k = k0 + j < slots ? k0 + j : slots - 1;
+        w[j] = wts[(size_t)token * slots + k];
+        v[j] = ld_agent(y + ((size_t)token * slots + k) * D + col);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (k0 + j < slots) a = fmaf(w[j], v[j], a);
     }
     out[(size_t)token * D + col] = (uint16_t)f32_bf16_bits(a);
   }
