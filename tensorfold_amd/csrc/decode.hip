@@ -317,6 +317,20 @@ __global__ void __launch_bounds__(1024)
                         blockIdx.x - a.first[w], lds);
 }
 
+// p[0] + p[stride] + ... (n terms, in that order); eight loads go out together before they are added
+__device__ __forceinline__ float ordered_sum(const float* __restrict__ p, long long stride, int n) {
+  float acc = 0.f;
+  for (int s0 = 0; s0 < n; s0 += 8) {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = p[(long long)(s0 + j < n ? s0 + j : n - 1) * stride];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (s0 + j < n) acc = s0 + j ? acc + v[j] : v[j];
+  }
+  return acc;
+}
+
 __global__ void qmm_group_reduce_kernel(GroupArgs a, int M, int f32) {
   int w = 0;
 #pragma unroll
@@ -327,8 +341,7 @@ __global__ void qmm_group_reduce_kernel(GroupArgs a, int M, int f32) {
   const long long i = (long long)(blockIdx.x - a.first[w]) * blockDim.x + threadIdx.x;
   if (i >= total) return;
   const float* part = a.part[w];
-  float acc = part[i];
-  for (int s = 1; s < a.sk[w]; ++s) acc = acc + part[s * total + i];
+  const float acc = ordered_sum(part + i, total, a.sk[w]);
   if (f32) reinterpret_cast<float*>(a.out[w])[i] = acc;
   else reinterpret_cast<uint16_t*>(a.out[w])[i] = (uint16_t)f32_bf16_bits(acc);
 }
@@ -338,8 +351,7 @@ __global__ void qmm_reduce_kernel(const float* __restrict__ part, void* __restri
                                   int f32) {
   const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= total) return;
-  float acc = part[i];
-  for (int s = 1; s < SK; ++s) acc = acc + part[s * total + i];
+  const float acc = ordered_sum(part + i, total, SK);
   if (f32) reinterpret_cast<float*>(out)[i] = acc;
   else reinterpret_cast<uint16_t*>(out)[i] = (uint16_t)f32_bf16_bits(acc);
 }

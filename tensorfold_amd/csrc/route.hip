@@ -227,18 +227,30 @@ __global__ void __launch_bounds__(256)
   const int d = (blockIdx.y * 256 + threadIdx.x) * 2;
   if (d >= D) return;
   float a0 = 0.f, a1 = 0.f;
-  for (int k = 0; k < S; ++k) {
-    const float w = Wt[(size_t)r * S + k];
-    const size_t at = ((size_t)r * S + k) * D + d;
-    if (YBF16) {
-      const uint32_t v = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(Y) + at);
-      a0 = fmaf(w, bf16_lo(v), a0);
-      a1 = fmaf(w, bf16_hi(v), a1);
-    } else {
-      const float2 v = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(Y) + at);
-      a0 = fmaf(w, v.x, a0);
-      a1 = fmaf(w, v.y, a1);
+  // eight slots' loads go out together, then the sum in slot order
+  for (int k0 = 0; k0 < S; k0 += 8) {
+    float w[8], v0[8], v1[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int k = k0 + j < S ? k0 + j : S - 1;
+      w[j] = Wt[(size_t)r * S + k];
+      const size_t at = ((size_t)r * S + k) * D + d;
+      if (YBF16) {
+        const uint32_t v = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(Y) + at);
+        v0[j] = bf16_lo(v);
+        v1[j] = bf16_hi(v);
+      } else {
+        const float2 v = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(Y) + at);
+        v0[j] = v.x;
+        v1[j] = v.y;
+      }
     }
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (k0 + j < S) {
+        a0 = fmaf(w[j], v0[j], a0);
+        a1 = fmaf(w[j], v1[j], a1);
+      }
   }
   *reinterpret_cast<uint32_t*>(out + (size_t)r * D + d) = pack_bf16(a0, a1);
 }
@@ -251,14 +263,23 @@ __global__ void __launch_bounds__(256)
   if (d >= D) return;
   float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
   const float* y = Y + (size_t)r * S * D + d;
-#pragma unroll 4
-  for (int k = 0; k < S; ++k) {
-    const float w = Wt[(size_t)r * S + k];
-    const f32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(y + (size_t)k * D));
-    a0 = fmaf(w, v[0], a0);
-    a1 = fmaf(w, v[1], a1);
-    a2 = fmaf(w, v[2], a2);
-    a3 = fmaf(w, v[3], a3);
+  for (int k0 = 0; k0 < S; k0 += 8) {
+    float w[8];
+    f32x4_t v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int k = k0 + j < S ? k0 + j : S - 1;
+      w[j] = Wt[(size_t)r * S + k];
+      v[j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(y + (size_t)k * D));
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (k0 + j < S) {
+        a0 = fmaf(w[j], v[j][0], a0);
+        a1 = fmaf(w[j], v[j][1], a1);
+        a2 = fmaf(w[j], v[j][2], a2);
+        a3 = fmaf(w[j], v[j][3], a3);
+      }
   }
   *reinterpret_cast<uint2*>(out + (size_t)r * D + d) = make_uint2(pack_bf16(a0, a1), pack_bf16(a2, a3));
 }
