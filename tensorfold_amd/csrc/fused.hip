@@ -21,7 +21,10 @@
 namespace tf {
 namespace {
 
-int fused_waves(int64_t grid) { return grid < 768 ? 16 : grid < 1536 ? 8 : 4; }
+// Waves a workgroup from a launch's size (measured on config 1): few workgroups want many waves each to keep enough
+// loads in flight; past about 1,300 workgroups of the routing launch (about 1,700 of the down launch) eight waves
+// each no longer fit the chip at once and four are faster.
+int fused_waves(int64_t grid) { return grid < 768 ? 16 : grid < 2560 ? 8 : 4; }
 
 struct WaitItem {
   const int* flag;
@@ -441,7 +444,7 @@ extern "C" int tf_moe_down_combine(int gs, const uint16_t* act, int rows, int sl
 #define TF_GO(GS_, W_)                                                                                             \
   down_combine_kernel<GS_, W_><<<g, W_ * 64, smem, s>>>(act, slots, down, d, ni, desc, wts, xs_act, y, out, arrive)
 #define TF_GS(GS_)                      \
-  switch (fused_waves(2 * grid)) {      \
+  switch (fused_waves(grid + grid / 2)) {      \
     case 16: TF_GO(GS_, 16); break;     \
     case 8: TF_GO(GS_, 8); break;       \
     default: TF_GO(GS_, 4);             \
