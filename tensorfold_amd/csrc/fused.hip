@@ -49,23 +49,22 @@ struct WaitItem {
 // unit that completes a (token, 64 columns) cell adds the token's slots in slot order (fp32 fma, as tf_moe_combine)
 // and writes bf16.  `arrive` [tokens * NB2d] starts at zero.
 template <int WAVES>
-__device__ __forceinline__ void combine_cells(const int* pairs, int* last, int cnt, int slots, int cb2, int NB2d, int D,
+__device__ __forceinline__ void combine_cells(const int* pairs, int cnt, int slots, int cb2, int NB2d, int D,
                                               const float* __restrict__ wts, const float* __restrict__ y,
                                               uint16_t* __restrict__ out, int* __restrict__ arrive) {
-  const int tid = threadIdx.x;
   __builtin_amdgcn_s_waitcnt(0);      // every store of this wave is acknowledged ...
   __syncthreads();                    // ... of every wave ...
-  if (tid < cnt) {                    // ... then the unit counts itself in
-    const int token = pairs[tid] / slots;
-    last[tid] = __hip_atomic_fetch_add(arrive + (size_t)token * NB2d + cb2, 1, __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT) == slots - 1;
-  }
-  __syncthreads();
-  const int lane = tid & 63, wave = tid >> 6;
+  // ... then wave r counts the unit in for its row r and, if that completes the cell, sums it; the other waves
+  // are done (an item has at most as many rows as a workgroup has waves)
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int col = cb2 * 64 + lane;
   for (int r = wave; r < cnt; r += WAVES) {
-    if (!last[r] || col >= D) continue;
     const int token = pairs[r] / slots;
+    int done = 0;
+    if (lane == 0)
+      done = __hip_atomic_fetch_add(arrive + (size_t)token * NB2d + cb2, 1, __ATOMIC_RELAXED,
+                                    __HIP_MEMORY_SCOPE_AGENT) == slots - 1;
+    if (!__builtin_amdgcn_readfirstlane(done) || col >= D) continue;
     float a = 0.f;
     // eight slots' loads go out together (one trip to memory instead of eight), then the sum in slot order
     for (int k0 = 0; k0 < slots; k0 += 8) {
@@ -92,7 +91,6 @@ __global__ void __launch_bounds__(WAVES * 64)
                         float* __restrict__ y, uint16_t* __restrict__ out, int* __restrict__ arrive) {
   extern __shared__ float lds[];
   __shared__ int pairs[16];
-  __shared__ int last[16];
   const int NB = D / 32, NB2d = (NB + 1) >> 1;
   const int it = blockIdx.x / NB2d, cb2 = blockIdx.x - it * NB2d;
   if (it >= desc[0]) return;
@@ -103,7 +101,7 @@ __global__ void __launch_bounds__(WAVES * 64)
   NoHook none;
   expert_unit<GS, 1, 0, WAVES, true, COH_OUT>(act, NI, 0, Wdown, NI / GS, NB, e, cnt, pairs, cb2, y, D, 0.f, xs_act,
                                               nullptr, lds, none);
-  combine_cells<WAVES>(pairs, last, cnt, slots, cb2, NB2d, D, wts, y, out, arrive);
+  combine_cells<WAVES>(pairs, cnt, slots, cb2, NB2d, D, wts, y, out, arrive);
 }
 
 template <int GS, int NM, int EPI_UP, int WAVES>
@@ -116,7 +114,6 @@ __global__ void __launch_bounds__(WAVES * 64)
                      int* __restrict__ status, float limit, int max_items, int spins) {
   extern __shared__ float lds[];
   __shared__ int pairs[16];
-  __shared__ int last[16];
   const int NB2u = (NI / 32 + 1) >> 1, NB2d = (D / 32 + 1) >> 1;
   const int U = max_items * NB2u;
   const int b = blockIdx.x, tid = threadIdx.x;
@@ -142,7 +139,7 @@ __global__ void __launch_bounds__(WAVES * 64)
   if (!expert_unit<GS, 1, 0, WAVES, true, DCOH>(act, NI, 0, Wdown, NI / GS, D / 32, e, cnt, pairs, cb2, y, D,
                                                             0.f, xs_act, nullptr, lds, wait))
     return;                     // the wait ran out: status is set, nothing is published
-  combine_cells<WAVES>(pairs, last, cnt, slots, cb2, NB2d, D, wts, y, out, arrive);
+  combine_cells<WAVES>(pairs, cnt, slots, cb2, NB2d, D, wts, y, out, arrive);
 }
 
 
