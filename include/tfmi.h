@@ -101,7 +101,8 @@ int tf_experts_run(int gs, int epi, const uint16_t* x, int64_t x_stride, int slo
  * TF_DESC_INTS; row 0 holds the number of descriptors, row 1 + i = {expert, count, first member, 0, pairs[..]}: the plan
  * cut into items of at most TF_DESC_TILE pairs, every full item first (expert order), then the experts' short last
  * items (expert order).  A buffer for P pairs over E experts needs
- * 1 + min(P, E) + P / TF_DESC_TILE rows; that bound is the max_items of the calls that read descriptors. */
+ * 1 + min(P, min(P, E) + P / TF_DESC_TILE) rows (no item is empty); that bound is the max_items of the calls that
+ * read descriptors. */
 #define TF_DESC_INTS 8
 #define TF_DESC_TILE 2
 

@@ -117,9 +117,10 @@ def make(up: list[tuple], down: tuple, gs: int, *, limit: float = 0.0) -> Expert
 
 def max_items(pairs: int, experts: int, tile: int = TILE) -> int:
     """Upper bound on the items of any plan over ``pairs`` pairs: each used expert opens one item and every full
-    ``tile`` pairs can open one more.  Grids are sized with it; the live count stays on the device."""
+    ``tile`` pairs can open one more, and no item is empty.  Grids are sized with it (a launch's surplus workgroups
+    still route before they find they have no item); the live count stays on the device."""
 
-    return min(pairs, experts) + pairs // tile
+    return min(pairs, min(pairs, experts) + pairs // tile)
 
 
 class Plan:
