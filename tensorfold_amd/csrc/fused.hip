@@ -206,9 +206,21 @@ __global__ void __launch_bounds__(WAVES * 64)
                                               act, NI, limit, nullptr, xs_act, lds, none);
     return;
   }
+  // the pairs are counted by expert as they are found (find_item's histogram, without its two barriers)
+  for (int e = tid; e < E; e += threads) item.cnt[e] = 0;
+  if (tid < 6) item.sel[tid] = tid == 0 ? -1 : 0;
+  __syncthreads();
+  auto count = [&](int id) {
+    if ((unsigned)id >= (unsigned)E || writer) return;
+    const int old = atomicAdd(&item.cnt[id], 1);
+    if (old % DTILE == DTILE - 1) atomicAdd(&item.sel[5], 1);
+  };
   if (!L) {
     // the picks are given (a top-k launch ran before): only the plan is made here
-    for (int p = tid; p < P; p += threads) pk[p] = (unsigned)pick[p] < (unsigned)E ? pick[p] : -1;
+    for (int p = tid; p < P; p += threads) {
+      pk[p] = (unsigned)pick[p] < (unsigned)E ? pick[p] : -1;
+      count(pk[p]);
+    }
   } else if (NE <= 128 && slots <= 16 && R > WAVES) {
     // more rows than waves: four logits rows a wave, each on a row of 16 lanes
     for (int r0 = 4 * wave; r0 < R; r0 += 4 * WAVES) {
@@ -218,6 +230,7 @@ __global__ void __launch_bounds__(WAVES * 64)
       topk_row16(r < R ? L + (size_t)r * ldl : nullptr, NE, TOPK, shared, lane, id, w);
       if (r < R && (lane & 15) < slots) {
         pk[r * slots + (lane & 15)] = (unsigned)id < (unsigned)E ? id : -1;
+        count(id);
         if (writer) {
           pick[r * slots + (lane & 15)] = id;
           wts[r * slots + (lane & 15)] = w;
@@ -230,6 +243,7 @@ __global__ void __launch_bounds__(WAVES * 64)
       float w;
       topk_lane(L + (size_t)r * ldl, NE, TOPK, shared, lane, id, w);
       keep(r, id, w);
+      if (lane < slots) count(id);
     }
   }
   __syncthreads();
@@ -300,7 +314,7 @@ __global__ void __launch_bounds__(WAVES * 64)
     }
     return;
   }
-  if (!find_item<DTILE>(item, pk, P, E, it)) return;
+  if (!find_item<DTILE, true>(item, pk, P, E, it)) return;
   NoHook none;
   // the item's rows are summed group by group inside the unit (a pass at a time), under its first weight loads
   expert_unit<GS, NM, EPI, WAVES, false, 0>(X, x_stride, slots, Wup, D / GS, NI / 32, item.sel[0], item.sel[2],

@@ -297,18 +297,22 @@ struct ItemLds {
 //
 // Every thread of the workgroup calls this (it has barriers); pk holds P expert ids (negative = none).
 // Returns false when there is no item `it`.  On return L.sel and L.pairs describe the item.
-template <int TILE>
+// COUNTED: the caller has already cleared L.sel, counted the pairs into L.cnt and the full tiles into L.sel[5] (as the
+// loop below does) and passed a barrier.
+template <int TILE, bool COUNTED = false>
 __device__ __forceinline__ bool find_item(ItemLds& L, const int* pk, int P, int E, int it) {
   const int tid = threadIdx.x, threads = blockDim.x, lane = tid & 63;
-  for (int e = tid; e < E; e += threads) L.cnt[e] = 0;
-  if (tid < 6) L.sel[tid] = tid == 0 ? -1 : 0;
-  __syncthreads();
-  for (int p = tid; p < P; p += threads)
-    if (pk[p] >= 0) {
-      const int old = atomicAdd(&L.cnt[pk[p]], 1);
-      if (old % TILE == TILE - 1) atomicAdd(&L.sel[5], 1);     // this pair completes a tile
-    }
-  __syncthreads();
+  if constexpr (!COUNTED) {
+    for (int e = tid; e < E; e += threads) L.cnt[e] = 0;
+    if (tid < 6) L.sel[tid] = tid == 0 ? -1 : 0;
+    __syncthreads();
+    for (int p = tid; p < P; p += threads)
+      if (pk[p] >= 0) {
+        const int old = atomicAdd(&L.cnt[pk[p]], 1);
+        if (old % TILE == TILE - 1) atomicAdd(&L.sel[5], 1);     // this pair completes a tile
+      }
+    __syncthreads();
+  }
   if (tid < 64) {
     const int F = L.sel[5];
     int full_before = 0, short_before = 0, pairs_before = 0;
