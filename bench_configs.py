@@ -1,7 +1,7 @@
 """Kernel timings of the benchmark configurations that are not bench.py's headline: 0 (dense 4-bit projection),
 2 (verify-window MoE layer), 3 (prompt chunk, grouped MFMA) and 4 (EXL3 projections).
 
-    python bench_configs.py [c0] [c2] [c3] [c4]
+    python bench_configs.py [c0] [c2] [c3] [c4] [c4p]
 
 One JSON line a configuration: time of one pass (hipGraph of back-to-back passes cycling over enough weight copies to
 miss the 256 MB Infinity Cache, HIP events around the replay), algorithmic bytes or flops, and the fraction of the
@@ -212,11 +212,40 @@ def c4() -> dict:
             "bound": "hbm", "rows": out}
 
 
+def c4p() -> dict:
+    """Prompt form of configuration 4's gate projection: input rotation, W_q decoded once a chunk, MFMA GEMM."""
+
+    from tensorfold_amd.exl3 import prefill
+
+    gen = torch.Generator(device=DEV).manual_seed(5)
+    k, n = 5120, 17408
+    trellis = torch.randint(-2 ** 15, 2 ** 15, (k // 16, n // 16, 48), generator=gen, device=DEV,
+                            dtype=torch.int32).to(torch.int16)
+    sc = lambda size: (torch.rand(size, generator=gen, device=DEV) * 1.5 + 0.5).half()
+    layer = exl3.Exl3Linear.from_tensors(trellis, sc(k), sc(n), "3inst", device=DEV)
+    ws = prefill.Workspace()
+    out = {}
+    for m in (512, 4096):
+        x = synthetic.activations(m, k, 4400 + m, dtype=torch.float16).to(DEV)
+        y = torch.empty((m, n), dtype=torch.float16, device=DEV)
+        prefill.matmul(layer, x, y, ws)
+        wt = prefill.decode(layer, ws)
+        whole = graph_us(lambda i: prefill.matmul(layer, x, y, ws), 8)
+        gemm = graph_us(lambda i: prefill.matmul(layer, x, y, ws, wt=wt), 8)
+        dec = graph_us(lambda i: prefill.decode(layer, ws), 8)
+        flops = 2.0 * m * k * n
+        out[m] = {"matmul_us": whole, "decode_us": dec, "rot_gemm_us": gemm, "tflops": flops / whole * 1e-6,
+                  "frac": flops / whole * 1e-6 / MFMA, "gemm_tflops": flops / gemm * 1e-6,
+                  "decode_gbs": (k * n * 3 // 8 + k * n * 2) / dec * 1e-3}
+    return {"config": "c4p: EXL3 3.0 bpw gate projection 5120 -> 17408 on a prompt chunk (rotation + decode + MFMA GEMM)",
+            "bound": "mfma", "rows": out}
+
+
 def main() -> int:
     torch.cuda.set_device(0)
     which = sys.argv[1:] or ["c0", "c2", "c3", "c4"]
     for name in which:
-        res = {"c0": c0, "c2": c2, "c3": c3, "c4": c4}[name]()
+        res = {"c0": c0, "c2": c2, "c3": c3, "c4": c4, "c4p": c4p}[name]()
         torch.cuda.empty_cache()
         print(json.dumps(res, default=lambda v: round(v, 4)), flush=True)
     return 0

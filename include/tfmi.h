@@ -188,6 +188,20 @@ int tf_exl3_linear(const uint16_t* xh, const uint32_t* T, int64_t stride_k, int6
 int tf_exl3_unpack(const uint32_t* T, uint16_t* W, int k, int n, int64_t stride_k, int64_t stride_nb, int k2, int cb,
                    tf_stream_t stream);
 
+/* ---- EXL3 prompt matmul (exl3/prefill.py:15-95; Triton `_gemm` in the reference) ----------------------------------- */
+
+/* W8[k / 8][n][8] fp16 = the decoded trellis in the order an MFMA B operand is read (tf_exl3_unpack's values:
+ * W8[k / 8][c][k % 8] = W[k][c]; the 8 consecutive inputs of a lane are 16 bytes, a tile's 16 columns side by side).
+ * The reference decodes W_q [K, N] with `unpack` once a chunk (exl3/prefill.py:88-89). */
+int tf_exl3_unpack_k8(const uint32_t* T, uint16_t* W8, int k, int n, int64_t stride_k, int64_t stride_nb, int k2,
+                      int cb, tf_stream_t stream);
+/* y[m, block] = ((xh[m] @ W_q[:, block]) H / sqrt(128)) * svh + bias for any m: xh fp16 [m, k] from tf_exl3_rot_in,
+ * w8 from tf_exl3_unpack_k8 (k * n < 2^31), K added in order in fp32 (a row's bits do not depend on m or on the
+ * rows beside it), the rotation exact in fp32.  y rows are y_stride elements apart.  Replaces exl3/prefill.py:16-44
+ * `_gemm`. */
+int tf_exl3_gemm(const uint16_t* xh, const uint16_t* w8, const uint16_t* svh, const uint16_t* bias, void* y, int y_dtype,
+                 int64_t y_stride, int m, int k, int n, tf_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

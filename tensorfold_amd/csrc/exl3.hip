@@ -341,6 +341,171 @@ __global__ void __launch_bounds__(64)
   }
 }
 
+// W_q as [K / 8][N][8] fp16, the order an MFMA B operand is read in: the 8 consecutive inputs a lane holds are 16
+// bytes, and the 16 columns of a tile lie side by side, so a wave's operand load is four runs of 256 bytes.  A lane's
+// four values are two pairs of consecutive inputs of one column: two 4-byte stores, a wave's a run of 256 bytes each.
+template <int K2, int CB>
+__global__ void __launch_bounds__(64)
+    unpack_k8_kernel(const uint32_t* __restrict__ T, uint16_t* __restrict__ W8, int N, int64_t stride_k,
+                     int64_t stride_nb) {
+  const int kt = blockIdx.y, nt = blockIdx.x, lane = threadIdx.x, L = lane & 31, h = lane >> 5;
+  const uint32_t* tile = T + (size_t)kt * stride_k + (size_t)(nt >> 3) * stride_nb + (nt & 7) * tile_words<K2>();
+  uint16_t v[4];
+  values4<K2, CB>(tile, L, h, v);
+  const int col = (L >> 2) + 8 * h;                      // values j = 0, 1: inputs 2 (L & 3), + 1; j = 2, 3: those + 8
+  uint32_t* dst = reinterpret_cast<uint32_t*>(W8) + ((size_t)(2 * kt) * N + nt * 16 + col) * 4 + (L & 3);
+  dst[0] = (uint32_t)v[0] | ((uint32_t)v[1] << 16);
+  dst[(size_t)N * 4] = (uint32_t)v[2] | ((uint32_t)v[3] << 16);
+}
+
+// ---- prompt matmul: y = ((xh @ W_q) H / sqrt(128)) * svh + bias on decoded weights (exl3/prefill.py:15-95) -----------
+//
+// xh fp16 [M, K] (rot_in's output), W8 fp16 [K / 8][N][8] (unpack_k8's).  A workgroup of eight waves takes 128 rows x
+// 512 columns; a wave owns 64 columns = four B operands and all eight 16-row tiles, so one B operand feeds eight MFMAs
+// and one LDS read of xh four: per 32 inputs a wave issues 32 MFMAs against 8 LDS reads and 4 global loads.  B
+// operands come straight from W8 into registers (16 bytes a lane, 16 neighbouring lanes one 256-byte run: the cache
+// sees 8 full lines a load, not 64 lanes' separate pieces), requested two steps of 64 inputs ahead; xh goes a step
+// ahead through registers into LDS (two stages, 144-byte rows), one barrier a step.
+// The epilogue is linear_kernel's: a row tile's sums through LDS, a wave a (row, 128-column block): FWHT, scale, bias.
+// A row's arithmetic does not depend on the other rows, on M or on the tile it falls in.
+//
+// Workgroups reach the XCDs round-robin (blockIdx % 8) and each XCD has its own L2: an XCD's 32 consecutive workgroups
+// take an RG x CG block of tiles (RG * CG = 32), so what they stream in step from beyond L2 is RG tiles of xh and CG of
+// W8, not 32 of either.
+constexpr int GEMM_KSTEP = 64, GEMM_AROW = 2 * GEMM_KSTEP + 16, GEMM_STAGE = 128 * GEMM_AROW;     // bytes
+constexpr int GEMM_LDS = 2 * GEMM_STAGE;         // two stages of xh; the epilogue's 16 x 516 floats fit too
+constexpr int GEMM_RED = 516;                    // floats from one row of the epilogue's tile to the next
+static_assert(16 * GEMM_RED * 4 <= GEMM_LDS, "the epilogue's tile must fit the staging buffers");
+
+__global__ void __launch_bounds__(512, 1)
+    gemm_kernel(const uint16_t* __restrict__ xh, const uint16_t* __restrict__ W8, const uint16_t* __restrict__ svh,
+                const uint16_t* __restrict__ bias, void* __restrict__ y, int y_dtype, int64_t y_stride, int M, int K,
+                int N, int rts, int cts, int rg_log2) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int RG = 1 << rg_log2, CG = 32 >> rg_log2;
+  const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+  const int super = (local >> 5) * 8 + xcd, place = local & 31;
+  const int rgs = (rts + RG - 1) >> rg_log2;
+  const int sc = super / rgs, sr = super - sc * rgs;
+  const int rt = sr * RG + (place & (RG - 1)), ct = sc * CG + (place >> rg_log2);
+  if (rt >= rts || ct >= cts) return;
+  const int m0 = rt * 128, col0 = ct * 512;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 15, kq = lane >> 4;
+  const bool wok = col0 + 64 * wave < N;                   // N is a multiple of 128: a pair of waves falls out together
+  const int steps = K / GEMM_KSTEP, last = steps - 1;
+
+  // B: W8 from the workgroup's first column on as one buffer; the lane's octet and column as the vector offset, the
+  // step's and chunk's octet as the scalar offset
+  const int ncols = min(512, N - col0);
+  const uint32_t octet = (uint32_t)N * 16u;                // bytes from one octet of inputs to the next
+  const __amdgpu_buffer_rsrc_t wsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(W8 + (size_t)col0 * 8), 0, (uint32_t)(K / 8 - 1) * octet + (uint32_t)ncols * 16u, 0x00020000);
+  uint32_t boff[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) boff[j] = (uint32_t)kq * octet + (uint32_t)((wok ? 64 * wave : 0) + 16 * j + c) * 16u;
+  typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+  u32x4_t b[2][4][2];
+  auto load_b = [&](int step, int i, u32x4_t (&dst)[4][2]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      dst[j][i] = __builtin_amdgcn_raw_buffer_load_b128(wsrc, boff[j], (step * 8 + 4 * i) * octet, 0);
+  };
+  // A: the workgroup's rows of xh as one buffer; this thread's two 16-byte pieces of a step: piece q = (row q / 8,
+  // 8 inputs q % 8); rows past M read the last row and are dropped at the end
+  const int nrows = min(128, M - m0);
+  const __amdgpu_buffer_rsrc_t asrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(xh + (size_t)m0 * K), 0, (uint32_t)nrows * (uint32_t)K * 2u, 0x00020000);
+  uint32_t aoff[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int q = tid + 512 * j;
+    aoff[j] = ((uint32_t)min(q >> 3, nrows - 1) * (uint32_t)K + (q & 7) * 8) * 2u;
+  }
+  u32x4_t ar[2];
+  auto load_a = [&](int step) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) ar[j] = __builtin_amdgcn_raw_buffer_load_b128(asrc, aoff[j], step * (GEMM_KSTEP * 2), 0);
+  };
+  auto store_a = [&](int buf) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int q = tid + 512 * j;
+      *reinterpret_cast<u32x4_t*>(smem + buf * GEMM_STAGE + (q >> 3) * GEMM_AROW + (q & 7) * 16) = ar[j];
+    }
+  };
+
+  f32x4_t acc[4][8];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int r = 0; r < 8; ++r) acc[j][r] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+
+  load_b(0, 0, b[0]);
+  load_b(0, 1, b[0]);
+  load_a(0);
+  load_b(min(1, last), 0, b[1]);
+  load_b(min(1, last), 1, b[1]);
+  store_a(0);
+  __syncthreads();
+  // K is a multiple of 128, so the steps come in pairs: the loop body is one block with nothing conditional in it
+  for (int step0 = 0; step0 < steps; step0 += 2) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int step = step0 + u;
+      load_a(min(step + 1, last));
+      __builtin_amdgcn_sched_barrier(0);                // the request leaves now, not when its registers are needed
+      const unsigned char* abuf = smem + u * GEMM_STAGE + c * GEMM_AROW + kq * 16;
+      // operand t of the step is (chunk t / 8, row tile t % 8), requested two row tiles before its MFMAs
+      auto read_a = [&](int t) {
+        return *reinterpret_cast<const f16x8_t*>(abuf + 16 * (t & 7) * GEMM_AROW + (t >> 3) * 64);
+      };
+      f16x8_t a = read_a(0), a1 = read_a(1);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          const int t = 8 * i + r;
+          f16x8_t a2 = a1;
+          if (t + 2 < 16) a2 = read_a(t + 2);
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            acc[j][r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, __builtin_bit_cast(f16x8_t, b[u][j][i]), acc[j][r], 0, 0, 0);
+          a = a1;
+          a1 = a2;
+          // keep the order written here: one LDS read two row tiles ahead of the four MFMAs it feeds
+          if (t == 0) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+          if (t + 2 < 16) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        load_b(min(step + 2, last), i, b[u]);           // this chunk's registers are free again
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      store_a(1 - u);
+      __syncthreads();
+    }
+  }
+  // D[row 4 kq + e][column c] of tile (j, r) -> LDS [16 rows][516] a row tile at a time, then a wave a (row, block)
+  float* red = reinterpret_cast<float*>(smem);
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    if (r) __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) red[(4 * kq + e) * GEMM_RED + 64 * wave + 16 * j + c] = acc[j][r][e];
+    __syncthreads();
+    for (int unit = wave; unit < 64; unit += 8) {
+      const int row = unit >> 2, blk = unit & 3;
+      const int grow = m0 + 16 * r + row, col = col0 + 128 * blk + 2 * lane;
+      if (grow < M && col0 + 128 * blk < N) {
+        const float2 v = *reinterpret_cast<const float2*>(red + row * GEMM_RED + 128 * blk + 2 * lane);
+        finish_row(v.x, v.y, lane, svh, bias, col, y, y_dtype, (size_t)grow * y_stride + col);
+      }
+    }
+  }
+}
+
 // every width ExLlamaV3 writes: k2 = 2 * bits; half-integer widths exist with the mul1 codebook only
 #define TF_EXL3_WIDTHS(X, CB) X(2, CB) X(4, CB) X(6, CB) X(8, CB) X(10, CB) X(12, CB) X(14, CB) X(16, CB)
 #define TF_EXL3_ALL(X) TF_EXL3_WIDTHS(X, 0) TF_EXL3_WIDTHS(X, 1) TF_EXL3_WIDTHS(X, 2) X(3, 2) X(5, 2) X(7, 2)
@@ -412,4 +577,46 @@ extern "C" int tf_exl3_unpack(const uint32_t* T, uint16_t* W, int k, int n, int6
 #undef TF_LAUNCH
   set_error("unsupported EXL3 width/codebook: K2=%d codebook=%d", k2, cb);
   return 1;
+}
+
+extern "C" int tf_exl3_unpack_k8(const uint32_t* T, uint16_t* W8, int k, int n, int64_t stride_k, int64_t stride_nb,
+                                 int k2, int cb, tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(T && W8 && aligned16(W8), "unpack_k8: null or unaligned pointer argument");
+  TF_REQUIRE(k >= 128 && n >= 128 && k % 128 == 0 && n % 128 == 0, "W must be [K, N], multiples of 128");
+  TF_REQUIRE(k / 16 <= 65535, "unpack_k8: K too large for one launch");
+  const dim3 grid((unsigned)(n / 16), (unsigned)(k / 16));
+  hipStream_t s = as_stream(stream);
+#define TF_LAUNCH(K2_, CB_)                                                            \
+  if (k2 == K2_ && cb == CB_) {                                                        \
+    unpack_k8_kernel<K2_, CB_><<<grid, 64, 0, s>>>(T, W8, n, stride_k, stride_nb);     \
+    TF_LAUNCH_OK("tf_exl3_unpack_k8");                                                 \
+    return 0;                                                                          \
+  }
+  TF_EXL3_ALL(TF_LAUNCH)
+#undef TF_LAUNCH
+  set_error("unsupported EXL3 width/codebook: K2=%d codebook=%d", k2, cb);
+  return 1;
+}
+
+extern "C" int tf_exl3_gemm(const uint16_t* xh, const uint16_t* w8, const uint16_t* svh, const uint16_t* bias, void* y,
+                            int y_dtype, int64_t y_stride, int m, int k, int n, tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(xh && w8 && svh && y, "gemm: null pointer argument");
+  TF_REQUIRE(m >= 1 && k >= 128 && n >= 128 && k % 128 == 0 && n % 128 == 0, "xh [M, K], W8 [K / 8, N, 8]: multiples of 128");
+  TF_REQUIRE((int64_t)k * n < (1LL << 31), "gemm: K * N must stay below 2^31 (buffer offsets are 32-bit)");
+  TF_REQUIRE(y_dtype == TF_F16 || y_dtype == TF_BF16 || y_dtype == TF_F32, "y: expected fp16, bf16 or fp32");
+  TF_REQUIRE(y_stride >= n && y_stride % 2 == 0, "y rows hold at least N values, an even stride apart");
+  TF_REQUIRE(aligned16(xh) && aligned16(w8) && ((uintptr_t)y & 7) == 0, "xh, W8 16-byte and y 8-byte aligned");
+  const int64_t rts = ((int64_t)m + 127) / 128, cts = (n + 511) / 512;
+  TF_REQUIRE(rts <= 0x3FFFFF, "gemm: too many rows for one launch");
+  int rg_log2 = 0;                                  // an XCD's 32 workgroups: 2^rg_log2 row tiles x the rest column tiles
+  while (rg_log2 < 3 && (1 << rg_log2) < rts) ++rg_log2;
+  const int64_t supers = ((rts + (1 << rg_log2) - 1) >> rg_log2) * ((cts + (32 >> rg_log2) - 1) / (32 >> rg_log2));
+  const int64_t grid = (supers + 7) / 8 * 256;
+  TF_REQUIRE(grid <= 0x7FFFFFFF, "gemm: %lld workgroups exceed the grid limit", (long long)grid);
+  gemm_kernel<<<dim3((unsigned)grid), 512, GEMM_LDS, as_stream(stream)>>>(xh, w8, svh, bias, y, y_dtype, y_stride, m, k, n,
+                                                                          (int)rts, (int)cts, rg_log2);
+  TF_LAUNCH_OK("tf_exl3_gemm");
+  return 0;
 }
