@@ -153,20 +153,34 @@ __device__ __forceinline__ void store2(void* p, int dtype, size_t i, float a, fl
   }
 }
 
-// xh = fp16(((x * suh) H) / sqrt(128)), a wave a (row, block of 128)
+// xh = fp16(((x * suh) H) / sqrt(128)), a wave a (row, block of 128); a workgroup walks rows blockIdx.y, + gridDim.y, ...
 __global__ void __launch_bounds__(256)
     rot_in_kernel(const void* __restrict__ x, int x_dtype, const uint16_t* __restrict__ suh, uint16_t* __restrict__ xh,
-                  int K) {
-  const int blk = blockIdx.x * 4 + (threadIdx.x >> 6), row = blockIdx.y, lane = threadIdx.x & 63;
+                  int M, int K) {
+  const int blk = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (blk * 128 >= K) return;
   const int k = blk * 128 + 2 * lane;
-  float a, b, sa, sb;
-  load2(x, x_dtype, (size_t)row * K + k, a, b);
+  float sa, sb;
   load2(suh, TF_F16, k, sa, sb);
-  a *= sa;
-  b *= sb;
-  fwht128(a, b, lane);
-  store2(xh, TF_F16, (size_t)row * K + k, a * HAD_SCALE, b * HAD_SCALE);
+  // four rows' loads are in flight together
+  for (int row0 = blockIdx.y; row0 < M; row0 += 4 * gridDim.y) {
+    float a[4], b[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int row = row0 + u * gridDim.y;
+      if (row < M) load2(x, x_dtype, (size_t)row * K + k, a[u], b[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int row = row0 + u * gridDim.y;
+      if (row < M) {
+        a[u] *= sa;
+        b[u] *= sb;
+        fwht128(a[u], b[u], lane);
+        store2(xh, TF_F16, (size_t)row * K + k, a[u] * HAD_SCALE, b[u] * HAD_SCALE);
+      }
+    }
+  }
 }
 
 // the finished outputs of one row's 128 columns from their fp32 sums: H / sqrt(128), * svh, + bias
@@ -344,24 +358,28 @@ __global__ void __launch_bounds__(64)
 // W_q as [K / 8][N][8] fp16, the order an MFMA B operand is read in: the 8 consecutive inputs a lane holds are 16
 // bytes, and the 16 columns of a tile lie side by side, so a wave's operand load is four runs of 256 bytes.  A lane's
 // four values are two pairs of consecutive inputs of one column: two 4-byte stores, a wave's a run of 256 bytes each.
+// A workgroup takes four k-tiles of a 128-column block, a wave the eight tiles of one of them.
 template <int K2, int CB>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(256)
     unpack_k8_kernel(const uint32_t* __restrict__ T, uint16_t* __restrict__ W8, int N, int64_t stride_k,
                      int64_t stride_nb) {
-  const int kt = blockIdx.y, nt = blockIdx.x, lane = threadIdx.x, L = lane & 31, h = lane >> 5;
-  const uint32_t* tile = T + (size_t)kt * stride_k + (size_t)(nt >> 3) * stride_nb + (nt & 7) * tile_words<K2>();
-  uint16_t v[4];
-  values4<K2, CB>(tile, L, h, v);
+  const int kt = 4 * blockIdx.y + (threadIdx.x >> 6), nb = blockIdx.x, lane = threadIdx.x & 63, L = lane & 31, h = lane >> 5;
+  const uint32_t* tiles = T + (size_t)kt * stride_k + (size_t)nb * stride_nb;
   const int col = (L >> 2) + 8 * h;                      // values j = 0, 1: inputs 2 (L & 3), + 1; j = 2, 3: those + 8
-  uint32_t* dst = reinterpret_cast<uint32_t*>(W8) + ((size_t)(2 * kt) * N + nt * 16 + col) * 4 + (L & 3);
-  dst[0] = (uint32_t)v[0] | ((uint32_t)v[1] << 16);
-  dst[(size_t)N * 4] = (uint32_t)v[2] | ((uint32_t)v[3] << 16);
+  uint32_t* dst = reinterpret_cast<uint32_t*>(W8) + ((size_t)(2 * kt) * N + nb * 128 + col) * 4 + (L & 3);
+#pragma unroll
+  for (int t = 0; t < 8; ++t) {
+    uint16_t v[4];
+    values4<K2, CB>(tiles + t * tile_words<K2>(), L, h, v);
+    dst[t * 64] = (uint32_t)v[0] | ((uint32_t)v[1] << 16);
+    dst[(size_t)N * 4 + t * 64] = (uint32_t)v[2] | ((uint32_t)v[3] << 16);
+  }
 }
 
 // ---- prompt matmul: y = ((xh @ W_q) H / sqrt(128)) * svh + bias on decoded weights (exl3/prefill.py:15-95) -----------
 //
-// xh fp16 [M, K] (rot_in's output), W8 fp16 [K / 8][N][8] (unpack_k8's).  A workgroup of eight waves takes 128 rows x
-// 512 columns; a wave owns 64 columns = four B operands and all eight 16-row tiles, so one B operand feeds eight MFMAs
+// xh fp16 [M, K] (rot_in's output), W8 fp16 [K / 8][N][8] (unpack_k8's).  A workgroup of WAVES waves takes 128 rows x
+// 64 WAVES columns; a wave owns 64 columns = four B operands and all eight 16-row tiles, so one B operand feeds eight MFMAs
 // and one LDS read of xh four: per 32 inputs a wave issues 32 MFMAs against 8 LDS reads and 4 global loads.  B
 // operands come straight from W8 into registers (16 bytes a lane, 16 neighbouring lanes one 256-byte run: the cache
 // sees 8 full lines a load, not 64 lanes' separate pieces), requested two steps of 64 inputs ahead; xh goes a step
@@ -369,34 +387,35 @@ __global__ void __launch_bounds__(64)
 // The epilogue is linear_kernel's: a row tile's sums through LDS, a wave a (row, 128-column block): FWHT, scale, bias.
 // A row's arithmetic does not depend on the other rows, on M or on the tile it falls in.
 //
-// Workgroups reach the XCDs round-robin (blockIdx % 8) and each XCD has its own L2: an XCD's 32 consecutive workgroups
-// take an RG x CG block of tiles (RG * CG = 32), so what they stream in step from beyond L2 is RG tiles of xh and CG of
-// W8, not 32 of either.
+// Workgroups reach the XCDs round-robin (blockIdx % 8) and each XCD has its own L2: the workgroups an XCD runs
+// together (2^g_log2 consecutive ones) take an RG x CG block of tiles, so what they stream in step from beyond L2 is
+// RG tiles of xh and CG of W8, not one of each a workgroup.
 constexpr int GEMM_KSTEP = 64, GEMM_AROW = 2 * GEMM_KSTEP + 16, GEMM_STAGE = 128 * GEMM_AROW;     // bytes
 constexpr int GEMM_LDS = 2 * GEMM_STAGE;         // two stages of xh; the epilogue's 16 x 516 floats fit too
-constexpr int GEMM_RED = 516;                    // floats from one row of the epilogue's tile to the next
-static_assert(16 * GEMM_RED * 4 <= GEMM_LDS, "the epilogue's tile must fit the staging buffers");
+static_assert(16 * 516 * 4 <= GEMM_LDS, "the epilogue's tile must fit the staging buffers");
 
-__global__ void __launch_bounds__(512, 1)
+template <int WAVES>
+__global__ void __launch_bounds__(64 * WAVES, 8 / WAVES)
     gemm_kernel(const uint16_t* __restrict__ xh, const uint16_t* __restrict__ W8, const uint16_t* __restrict__ svh,
                 const uint16_t* __restrict__ bias, void* __restrict__ y, int y_dtype, int64_t y_stride, int M, int K,
-                int N, int rts, int cts, int rg_log2) {
+                int N, int rts, int cts, int rg_log2, int g_log2) {
+  constexpr int THREADS = 64 * WAVES, COLS = 64 * WAVES, RED = COLS + 4;     // RED: floats a row of the epilogue's tile
   extern __shared__ __align__(16) unsigned char smem[];
-  const int RG = 1 << rg_log2, CG = 32 >> rg_log2;
+  const int RG = 1 << rg_log2, CG = 1 << (g_log2 - rg_log2);
   const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
-  const int super = (local >> 5) * 8 + xcd, place = local & 31;
+  const int super = (local >> g_log2) * 8 + xcd, place = local & ((1 << g_log2) - 1);
   const int rgs = (rts + RG - 1) >> rg_log2;
   const int sc = super / rgs, sr = super - sc * rgs;
   const int rt = sr * RG + (place & (RG - 1)), ct = sc * CG + (place >> rg_log2);
   if (rt >= rts || ct >= cts) return;
-  const int m0 = rt * 128, col0 = ct * 512;
+  const int m0 = rt * 128, col0 = ct * COLS;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 15, kq = lane >> 4;
   const bool wok = col0 + 64 * wave < N;                   // N is a multiple of 128: a pair of waves falls out together
   const int steps = K / GEMM_KSTEP, last = steps - 1;
 
   // B: W8 from the workgroup's first column on as one buffer; the lane's octet and column as the vector offset, the
   // step's and chunk's octet as the scalar offset
-  const int ncols = min(512, N - col0);
+  const int ncols = min(COLS, N - col0);
   const uint32_t octet = (uint32_t)N * 16u;                // bytes from one octet of inputs to the next
   const __amdgpu_buffer_rsrc_t wsrc = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint16_t*>(W8 + (size_t)col0 * 8), 0, (uint32_t)(K / 8 - 1) * octet + (uint32_t)ncols * 16u, 0x00020000);
@@ -410,26 +429,27 @@ __global__ void __launch_bounds__(512, 1)
     for (int j = 0; j < 4; ++j)
       dst[j][i] = __builtin_amdgcn_raw_buffer_load_b128(wsrc, boff[j], (step * 8 + 4 * i) * octet, 0);
   };
-  // A: the workgroup's rows of xh as one buffer; this thread's two 16-byte pieces of a step: piece q = (row q / 8,
+  // A: the workgroup's rows of xh as one buffer; this thread's 16-byte pieces of a step: piece q = (row q / 8,
   // 8 inputs q % 8); rows past M read the last row and are dropped at the end
+  constexpr int PPT = 1024 / THREADS;
   const int nrows = min(128, M - m0);
   const __amdgpu_buffer_rsrc_t asrc = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<uint16_t*>(xh + (size_t)m0 * K), 0, (uint32_t)nrows * (uint32_t)K * 2u, 0x00020000);
-  uint32_t aoff[2];
+  uint32_t aoff[PPT];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int q = tid + 512 * j;
+  for (int j = 0; j < PPT; ++j) {
+    const int q = tid + THREADS * j;
     aoff[j] = ((uint32_t)min(q >> 3, nrows - 1) * (uint32_t)K + (q & 7) * 8) * 2u;
   }
-  u32x4_t ar[2];
+  u32x4_t ar[PPT];
   auto load_a = [&](int step) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) ar[j] = __builtin_amdgcn_raw_buffer_load_b128(asrc, aoff[j], step * (GEMM_KSTEP * 2), 0);
+    for (int j = 0; j < PPT; ++j) ar[j] = __builtin_amdgcn_raw_buffer_load_b128(asrc, aoff[j], step * (GEMM_KSTEP * 2), 0);
   };
   auto store_a = [&](int buf) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int q = tid + 512 * j;
+    for (int j = 0; j < PPT; ++j) {
+      const int q = tid + THREADS * j;
       *reinterpret_cast<u32x4_t*>(smem + buf * GEMM_STAGE + (q >> 3) * GEMM_AROW + (q & 7) * 16) = ar[j];
     }
   };
@@ -485,7 +505,7 @@ __global__ void __launch_bounds__(512, 1)
       __syncthreads();
     }
   }
-  // D[row 4 kq + e][column c] of tile (j, r) -> LDS [16 rows][516] a row tile at a time, then a wave a (row, block)
+  // D[row 4 kq + e][column c] of tile (j, r) -> LDS [16 rows][RED] a row tile at a time, then a wave a (row, block)
   float* red = reinterpret_cast<float*>(smem);
 #pragma unroll
   for (int r = 0; r < 8; ++r) {
@@ -493,13 +513,13 @@ __global__ void __launch_bounds__(512, 1)
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) red[(4 * kq + e) * GEMM_RED + 64 * wave + 16 * j + c] = acc[j][r][e];
+      for (int e = 0; e < 4; ++e) red[(4 * kq + e) * RED + 64 * wave + 16 * j + c] = acc[j][r][e];
     __syncthreads();
-    for (int unit = wave; unit < 64; unit += 8) {
-      const int row = unit >> 2, blk = unit & 3;
+    for (int unit = wave; unit < 8 * WAVES; unit += WAVES) {
+      const int row = unit / (WAVES / 2), blk = unit % (WAVES / 2);
       const int grow = m0 + 16 * r + row, col = col0 + 128 * blk + 2 * lane;
       if (grow < M && col0 + 128 * blk < N) {
-        const float2 v = *reinterpret_cast<const float2*>(red + row * GEMM_RED + 128 * blk + 2 * lane);
+        const float2 v = *reinterpret_cast<const float2*>(red + row * RED + 128 * blk + 2 * lane);
         finish_row(v.x, v.y, lane, svh, bias, col, y, y_dtype, (size_t)grow * y_stride + col);
       }
     }
@@ -522,8 +542,7 @@ extern "C" int tf_exl3_rot_in(const void* x, int x_dtype, const uint16_t* suh, u
   TF_REQUIRE(x_dtype == TF_F16 || x_dtype == TF_BF16 || x_dtype == TF_F32, "x: expected fp16, bf16 or fp32");
   TF_REQUIRE(m >= 1 && k >= 128 && k % 128 == 0, "x and xh must be [M, K], K a multiple of 128, suh [K]");
   TF_REQUIRE(aligned16(x) && aligned16(xh), "x: must be 16-byte aligned");
-  TF_REQUIRE(m <= 65535, "rot_in: at most 65535 rows");
-  rot_in_kernel<<<dim3((k / 128 + 3) / 4, m), 256, 0, as_stream(stream)>>>(x, x_dtype, suh, xh, k);
+  rot_in_kernel<<<dim3((k / 128 + 3) / 4, m < 1024 ? m : 1024), 256, 0, as_stream(stream)>>>(x, x_dtype, suh, xh, m, k);
   TF_LAUNCH_OK("tf_exl3_rot_in");
   return 0;
 }
@@ -584,12 +603,12 @@ extern "C" int tf_exl3_unpack_k8(const uint32_t* T, uint16_t* W8, int k, int n, 
   clear_error();
   TF_REQUIRE(T && W8 && aligned16(W8), "unpack_k8: null or unaligned pointer argument");
   TF_REQUIRE(k >= 128 && n >= 128 && k % 128 == 0 && n % 128 == 0, "W must be [K, N], multiples of 128");
-  TF_REQUIRE(k / 16 <= 65535, "unpack_k8: K too large for one launch");
-  const dim3 grid((unsigned)(n / 16), (unsigned)(k / 16));
+  TF_REQUIRE(k / 64 <= 65535, "unpack_k8: K too large for one launch");
+  const dim3 grid((unsigned)(n / 128), (unsigned)(k / 64));
   hipStream_t s = as_stream(stream);
 #define TF_LAUNCH(K2_, CB_)                                                            \
   if (k2 == K2_ && cb == CB_) {                                                        \
-    unpack_k8_kernel<K2_, CB_><<<grid, 64, 0, s>>>(T, W8, n, stride_k, stride_nb);     \
+    unpack_k8_kernel<K2_, CB_><<<grid, 256, 0, s>>>(T, W8, n, stride_k, stride_nb);    \
     TF_LAUNCH_OK("tf_exl3_unpack_k8");                                                 \
     return 0;                                                                          \
   }
@@ -608,15 +627,26 @@ extern "C" int tf_exl3_gemm(const uint16_t* xh, const uint16_t* w8, const uint16
   TF_REQUIRE(y_dtype == TF_F16 || y_dtype == TF_BF16 || y_dtype == TF_F32, "y: expected fp16, bf16 or fp32");
   TF_REQUIRE(y_stride >= n && y_stride % 2 == 0, "y rows hold at least N values, an even stride apart");
   TF_REQUIRE(aligned16(xh) && aligned16(w8) && ((uintptr_t)y & 7) == 0, "xh, W8 16-byte and y 8-byte aligned");
-  const int64_t rts = ((int64_t)m + 127) / 128, cts = (n + 511) / 512;
+  // 128 x 256 tiles, four waves, two workgroups a CU: one workgroup's first loads and its epilogue run under the
+  // other's MFMAs, and the last, part-filled round of tiles is spread thinner
+  constexpr int WAVES = 4, COLS = 64 * WAVES;
+  const int64_t rts = ((int64_t)m + 127) / 128, cts = (n + COLS - 1) / COLS;
   TF_REQUIRE(rts <= 0x3FFFFF, "gemm: too many rows for one launch");
-  int rg_log2 = 0;                                  // an XCD's 32 workgroups: 2^rg_log2 row tiles x the rest column tiles
-  while (rg_log2 < 3 && (1 << rg_log2) < rts) ++rg_log2;
-  const int64_t supers = ((rts + (1 << rg_log2) - 1) >> rg_log2) * ((cts + (32 >> rg_log2) - 1) / (32 >> rg_log2));
-  const int64_t grid = (supers + 7) / 8 * 256;
+  // an XCD's 2^g_log2 consecutive workgroups: 2^rg_log2 row tiles x the rest column tiles; smaller groups when the
+  // whole grid would not give every XCD two of them
+  int g_log2 = WAVES == 4 ? 6 : 5, rg_log2 = 0;
+  int64_t supers = 0;
+  for (;; --g_log2) {
+    rg_log2 = 0;
+    while (rg_log2 < 3 && rg_log2 < g_log2 && (1 << rg_log2) < rts) ++rg_log2;
+    const int64_t cg = 1 << (g_log2 - rg_log2);
+    supers = ((rts + (1 << rg_log2) - 1) >> rg_log2) * ((cts + cg - 1) / cg);
+    if (supers >= 16 || g_log2 == 3) break;
+  }
+  const int64_t grid = (supers + 7) / 8 * (8 << g_log2);
   TF_REQUIRE(grid <= 0x7FFFFFFF, "gemm: %lld workgroups exceed the grid limit", (long long)grid);
-  gemm_kernel<<<dim3((unsigned)grid), 512, GEMM_LDS, as_stream(stream)>>>(xh, w8, svh, bias, y, y_dtype, y_stride, m, k, n,
-                                                                          (int)rts, (int)cts, rg_log2);
+  gemm_kernel<WAVES><<<dim3((unsigned)grid), 64 * WAVES, GEMM_LDS, as_stream(stream)>>>(
+      xh, w8, svh, bias, y, y_dtype, y_stride, m, k, n, (int)rts, (int)cts, rg_log2, g_log2);
   TF_LAUNCH_OK("tf_exl3_gemm");
   return 0;
 }

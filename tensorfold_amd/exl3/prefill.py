@@ -18,7 +18,7 @@ def tiles(k: int, n: int) -> tuple[int, int]:
     """(rows, columns) a workgroup takes: the shape's alone, so a row never depends on its chunk
     (exl3/prefill.py:47-50)."""
 
-    return 128, 512
+    return 128, 256
 
 
 class Workspace:
