@@ -1,7 +1,7 @@
 """Kernel timings of the benchmark configurations that are not bench.py's headline: 0 (dense 4-bit projection),
 2 (verify-window MoE layer), 3 (prompt chunk, grouped MFMA) and 4 (EXL3 projections).
 
-    python bench_configs.py [c0] [c2] [c3] [c4] [c4p]
+    python bench_configs.py [c0] [c2] [c3] [c4] [c4p] [glue]
 
 One JSON line a configuration: time of one pass (hipGraph of back-to-back passes cycling over enough weight copies to
 miss the 256 MB Infinity Cache, HIP events around the replay), algorithmic bytes or flops, and the fraction of the
@@ -241,11 +241,34 @@ def c4p() -> dict:
             "bound": "mfma", "rows": out}
 
 
+def glue_() -> dict:
+    """The fused producers either side of the MoE layer: pair outputs -> residual + RMSNorm + group sums."""
+
+    from tensorfold_amd import glue
+
+    gen = torch.Generator(device=DEV).manual_seed(6)
+    out = {}
+    for name, rows, d, slots, top_k, ydt in (("decode_8x7x2688_f32", 8, 2688, 7, 6, torch.float32),
+                                             ("window_32x11x2048_f32", 32, 2048, 11, 10, torch.float32),
+                                             ("prompt_4096x9x2048_bf16", 4096, 2048, 9, 8, torch.bfloat16),
+                                             ("prompt_4096x7x2688_bf16", 4096, 2688, 7, 6, torch.bfloat16)):
+        copies = 1 if rows <= 32 else 3
+        h = [torch.randn((rows, d), generator=gen, device=DEV).bfloat16() for _ in range(copies)]
+        y = [(torch.randn((rows * slots, d), generator=gen, device=DEV) * 0.5).to(ydt) for _ in range(copies)]
+        wt = torch.rand((rows, slots), generator=gen, device=DEV)
+        w = (torch.rand((d,), generator=gen, device=DEV) + 0.5).bfloat16()
+        us = graph_us(lambda i: glue.add_moe_norm(h[i % copies], y[i % copies], wt, w, 1e-5, top_k), 24)
+        nbytes = rows * d * (slots * y[0].element_size() + 3 * 2) + rows * (d // 64 + slots) * 4 + d * 2
+        out[name] = {"us": us, "bytes": nbytes, "gbs": nbytes / us * 1e-3, "frac": nbytes / us * 1e-3 / HBM}
+    return {"config": "glue: add_moe_norm (weighted pair outputs + residual + RMSNorm + group sums), one launch",
+            "bound": "hbm", "rows": out}
+
+
 def main() -> int:
     torch.cuda.set_device(0)
     which = sys.argv[1:] or ["c0", "c2", "c3", "c4"]
     for name in which:
-        res = {"c0": c0, "c2": c2, "c3": c3, "c4": c4, "c4p": c4p}[name]()
+        res = {"c0": c0, "c2": c2, "c3": c3, "c4": c4, "c4p": c4p, "glue": glue_}[name]()
         torch.cuda.empty_cache()
         print(json.dumps(res, default=lambda v: round(v, 4)), flush=True)
     return 0

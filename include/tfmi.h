@@ -133,6 +133,20 @@ int tf_moe_topk(const float* logits, int64_t ldl, int rows, int experts, int top
 int tf_moe_combine(const void* y, int y_bf16, const float* wts, uint16_t* out, int rows, int slots, int d,
                    tf_stream_t stream);
 
+/* The producers of a 4-bit matmul's input in one launch, a row's bits depending on that row alone:
+ *   hn = x                                   (delta_kind 0; h is not written and may be NULL)
+ *      = bf16(x + delta)                     (1: delta bf16 [rows, d])
+ *      = bf16(x + bf16(routed + shared))     (2, 3: delta = pair outputs [rows * slots, d], fp32 or bf16;
+ *                                             routed = sum over slots < `routed` of wts[r, k] * y[r, k], shared = sum
+ *                                             of the other slots' y[r, k], fp32 in slot order)
+ *   y  = bf16(hn / sqrt(mean(hn^2) + eps) * w),  xs[r, g] = fp32 sum of y over group g of `gs` columns.
+ * x, w, h, y bf16; xs fp32 [rows, d / gs]; d <= 16384, whole groups of gs = 32, 64 or 128.
+ * Replaces families/qwen3_5/cuda/glue.py:10-41 `add_rmsnorm` and families/nemotron_h/cuda/glue.py:103-141
+ * `add_moe_norm`. */
+int tf_add_norm(const uint16_t* x, const void* delta, int delta_kind, const float* wts, int slots, int routed,
+                const uint16_t* w, float eps, uint16_t* h, uint16_t* y, float* xs, int rows, int d, int gs,
+                tf_stream_t stream);
+
 /* Routing and the up projection of the decode layer in ONE launch, for rows * (top_k + shared) <= 1024: workgroup 0
  * writes what tf_moe_topk and tf_experts_plan (tile 16) would (pick, wts, members, items, counts) plus the item
  * descriptors that tf_experts_run_desc reads; every other workgroup finds its own item from the

@@ -140,3 +140,46 @@ def combine(y: np.ndarray, wts: np.ndarray) -> np.ndarray:
     for k in range(slots):
         acc = acc + wts[:, k:k + 1].astype(np.float32) * y[:, k].astype(np.float32)
     return bf16(acc)
+
+
+# -- fused producers: residual add, RMSNorm, group sums ---------------------------------------------------------------
+#
+# Pins (tests/test_oracle_affine.py): zero delta leaves h = x; the group sums equal sums of the returned y; a float64
+# evaluation of the formulas agrees to bf16 rounding; moving one slot across the routed/shared boundary or dropping
+# its weight changes the result (the routed slots are weighted, the rest are not).
+
+def add_rmsnorm(x: np.ndarray, r: np.ndarray | None, w: np.ndarray, eps: float, gs: int = 64):
+    """h = bf16(x + r) (x itself without r), y = bf16(h / sqrt(mean(h^2) + eps) * w), xs = y's sums over groups of
+    ``gs`` columns in fp32.  x, r, w hold bf16 values as float32.  Returns (h, y, xs)
+    (families/qwen3_5/cuda/glue.py:10-41)."""
+
+    x = np.asarray(x, dtype=np.float32)
+    h = bf16(x + np.asarray(r, dtype=np.float32)) if r is not None else x
+    d = h.shape[1]
+    ss = (h.astype(np.float64) ** 2).sum(axis=1, keepdims=True)
+    inv = (np.float32(1) / np.sqrt((ss / d).astype(np.float32) + np.float32(eps), dtype=np.float32)).astype(np.float32)
+    y = bf16((h * inv) * np.asarray(w, dtype=np.float32)[None, :])
+    xs = y.reshape(y.shape[0], d // gs, gs).astype(np.float64).sum(axis=2).astype(np.float32)
+    return h, y, xs
+
+
+def moe_delta(y: np.ndarray, wts: np.ndarray, top_k: int) -> np.ndarray:
+    """delta[r] = bf16(sum over the first ``top_k`` slots of w[r, k] * y[r, k] + sum of the remaining slots' y[r, k]),
+    each sum in slot order in fp32, products rounded before they are added
+    (families/nemotron_h/cuda/glue.py:111-118)."""
+
+    rows, slots, d = y.shape
+    routed = np.zeros((rows, d), dtype=np.float32)
+    for k in range(top_k):
+        routed = routed + wts[:, k:k + 1].astype(np.float32) * y[:, k].astype(np.float32)
+    shared = np.zeros((rows, d), dtype=np.float32)
+    for k in range(top_k, slots):
+        shared = shared + y[:, k].astype(np.float32)
+    return bf16(routed + shared)
+
+
+def add_moe_norm(h: np.ndarray, y: np.ndarray, wts: np.ndarray, w: np.ndarray, eps: float, top_k: int, gs: int = 64):
+    """(bf16(h + delta), its RMSNorm times w, the group sums) with ``delta = moe_delta(y, wts, top_k)``
+    (families/nemotron_h/cuda/glue.py:103-141)."""
+
+    return add_rmsnorm(h, moe_delta(y, wts, top_k), w, eps, gs)

@@ -118,3 +118,63 @@ def test_c_layer_agrees_with_the_numpy_pairs(swiglu, gs):
     a_c = ora.bf16_from_bits(act_c)
     assert np.abs(a_c - act).max() <= 2 ** -7 * np.abs(act).max()          # summation order may move a bf16 step
     assert np.abs(ora.bf16_from_bits(out) - want).max() <= 2 ** -7 * np.abs(want).max()
+
+
+# -- fused producers (add_rmsnorm, add_moe_norm) ----------------------------------------------------------------------
+
+def _norm_case(rows, d, slots, seed):
+    rng = np.random.default_rng(seed)
+    h = ora.bf16(rng.standard_normal((rows, d)).astype(np.float32))
+    y = (rng.standard_normal((rows, slots, d)) * 0.5).astype(np.float32)
+    wts = ora.bf16(rng.random((rows, slots)).astype(np.float32) * 0.5 + 0.05)
+    w = ora.bf16((rng.random(d) + 0.5).astype(np.float32))
+    return h, y, wts, w
+
+
+def test_rmsnorm_closed_forms():
+    """A row of +-c has mean square c^2: with eps = 0 and w = 1 the normed row is +-1 and every group of 64 sums to
+    its count of +1 minus its count of -1; without a residual h is x itself."""
+
+    d = 256
+    sign = np.where(np.arange(d) % 3 == 0, -1.0, 1.0).astype(np.float32)
+    x = (sign * np.float32(0.75))[None, :]
+    h, y, xs = ora.add_rmsnorm(x, None, np.ones(d, dtype=np.float32), 0.0)
+    assert h is x or np.array_equal(h, x)
+    assert np.array_equal(y, sign[None, :])
+    assert np.array_equal(xs[0], sign.reshape(4, 64).sum(axis=1))
+    # eps enters under the root: x = 3, eps = 16 -> 3 / sqrt(9 + 16) = 0.6 -> bf16
+    _, y, _ = ora.add_rmsnorm(np.full((1, 64), 3.0, dtype=np.float32), None, np.ones(64, dtype=np.float32), 16.0)
+    assert np.array_equal(y, ora.bf16(np.full((1, 64), 0.6, dtype=np.float32)))
+
+
+def test_add_rmsnorm_against_float64_and_its_own_outputs():
+    h, y3, _, w = _norm_case(5, 384, 1, 11)
+    r = ora.bf16(y3[:, 0])
+    hn, out, xs = ora.add_rmsnorm(h, r, w, 1e-5, gs=64)
+    assert np.array_equal(hn, ora.bf16(h + r))
+    h64 = hn.astype(np.float64)
+    want = h64 / np.sqrt((h64 ** 2).mean(axis=1, keepdims=True) + 1e-5) * w.astype(np.float64)
+    assert np.abs(out - want).max() <= 2 ** -8 * np.abs(want).max()              # one bf16 step
+    assert np.allclose(xs, out.reshape(5, 6, 64).sum(axis=2), rtol=1e-6, atol=1e-6)
+    _, _, xs32 = ora.add_rmsnorm(h, r, w, 1e-5, gs=32)
+    assert np.allclose(xs32.reshape(5, 6, 2).sum(axis=2), xs, rtol=1e-6, atol=1e-5)
+
+
+def test_moe_delta_weights_the_routed_slots_only():
+    """Slots below top_k are weighted, the rest are added as they are; with weights of one the split does not matter;
+    moving the boundary or zeroing a routed weight changes the result by that slot's share."""
+
+    h, y, wts, w = _norm_case(3, 128, 5, 12)
+    want = (wts[:, :3, None].astype(np.float64) * y[:, :3]).sum(axis=1) + y[:, 3:].astype(np.float64).sum(axis=1)
+    got = ora.moe_delta(y, wts, 3)
+    assert np.abs(got - want).max() <= 2 ** -8 * np.abs(want).max()
+    ones = np.ones_like(wts)
+    assert np.array_equal(ora.moe_delta(y, ones, 0), ora.moe_delta(y, ones, 5))
+    moved = ora.moe_delta(y, wts, 4)
+    step = ((wts[:, 3, None] - 1).astype(np.float64) * y[:, 3])
+    assert np.abs((moved - got) - step).max() <= 2 ** -6 * np.abs(want).max()
+    assert np.abs(moved - got).max() > 0.05
+    hn, out, xs = ora.add_moe_norm(h, y, wts, w, 1e-5, 3)
+    assert np.array_equal(hn, ora.bf16(h + got))
+    h2, out2, xs2 = ora.add_rmsnorm(h, got, w, 1e-5)
+    assert np.array_equal(out, out2) and np.array_equal(xs, xs2) and np.array_equal(hn, h2)
