@@ -1,7 +1,7 @@
 """Kernel timings of the benchmark configurations that are not bench.py's headline: 0 (dense 4-bit projection),
 2 (verify-window MoE layer), 3 (prompt chunk, grouped MFMA) and 4 (EXL3 projections).
 
-    python bench_configs.py [c0] [c2] [c3] [c4] [c4p] [glue]
+    python bench_configs.py [c0] [c2] [c3] [c4] [c4p] [glue] [c4x]
 
 One JSON line a configuration: time of one pass (hipGraph of back-to-back passes cycling over enough weight copies to
 miss the 256 MB Infinity Cache, HIP events around the replay), algorithmic bytes or flops, and the fraction of the
@@ -264,11 +264,49 @@ def glue_() -> dict:
             "bound": "hbm", "rows": out}
 
 
+def c4x() -> dict:
+    """EXL3 routed experts at decode: GLM-shaped layer (288 experts, 4096 -> 2048 -> 4096, 4.0 bpw mcg, top-8)."""
+
+    from tensorfold_amd.exl3 import experts as xexp
+
+    gen = torch.Generator(device=DEV).manual_seed(7)
+    n_exp, d, width, top_k = 288, 4096, 2048, 8
+
+    def trellis(k, n):
+        return torch.randint(-2 ** 15, 2 ** 15, (n_exp, k // 16, n // 16, 64), generator=gen, device=DEV,
+                             dtype=torch.int32).to(torch.int16)
+
+    sc = lambda n, m: (torch.randn((n_exp, n), generator=gen, device=DEV) * m).half()
+    ex = xexp.prepare_stacked(trellis(d, width), trellis(d, width), trellis(width, d), sc(d, 0.02), sc(d, 0.02),
+                              sc(width, 0.5), sc(width, 0.5), sc(width, 0.05), sc(d, 0.2), "mcg")
+    out = {}
+    for rows in (1, 8):
+        scratch = xexp.Scratch(ex, rows, top_k + 1)
+        x = synthetic.activations(rows, d, 4500 + rows).to(DEV)
+        y = torch.empty((rows, d), dtype=torch.float32, device=DEV)
+        sets = []
+        for i in range(4):                                  # four draws of experts, cycled: no draw finds the last one's weights cached
+            sel = torch.stack([torch.randperm(n_exp, generator=gen, device=DEV)[:top_k] for _ in range(rows)]).int()
+            sel = torch.cat([sel, torch.full((rows, 1), n_exp, dtype=torch.int32, device=DEV)], 1).contiguous()
+            w = torch.cat([torch.rand((rows, top_k), generator=gen, device=DEV) * 0.2 + 0.05,
+                           torch.ones((rows, 1), device=DEV)], 1).contiguous()
+            sets.append((sel, w, len(set(sel[:, :top_k].flatten().tolist()))))
+        us = graph_us(lambda i: xexp.routed(x, sets[i % 4][0], sets[i % 4][1], ex, scratch, y, rows, limit=10.0,
+                                            act_mode=xexp.ACT_BF16), 16)
+        distinct = sum(s[2] for s in sets) / 4
+        nbytes = distinct * (3 * d * width // 2 + 2 * (3 * d + 3 * width)) + rows * d * 6
+        out[rows] = {"layer_us": us, "distinct_experts": distinct, "bytes": nbytes, "gbs": nbytes / us * 1e-3,
+                     "frac": nbytes / us * 1e-3 / HBM}
+    return {"config": "c4x: EXL3 routed experts at decode, 288 experts 4096 -> 2048 -> 4096, 4.0 bpw mcg, top-8 (group, "
+                      "rotation, gate/up, SwiGLU epilogue, down, rotation + combine: six launches)",
+            "bound": "hbm", "rows": out}
+
+
 def main() -> int:
     torch.cuda.set_device(0)
     which = sys.argv[1:] or ["c0", "c2", "c3", "c4"]
     for name in which:
-        res = {"c0": c0, "c2": c2, "c3": c3, "c4": c4, "c4p": c4p, "glue": glue_}[name]()
+        res = {"c0": c0, "c2": c2, "c3": c3, "c4": c4, "c4p": c4p, "glue": glue_, "c4x": c4x}[name]()
         torch.cuda.empty_cache()
         print(json.dumps(res, default=lambda v: round(v, 4)), flush=True)
     return 0

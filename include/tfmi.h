@@ -216,6 +216,34 @@ int tf_exl3_unpack_k8(const uint32_t* T, uint16_t* W8, int k, int n, int64_t str
 int tf_exl3_gemm(const uint16_t* xh, const uint16_t* w8, const uint16_t* svh, const uint16_t* bias, void* y, int y_dtype,
                  int64_t y_stride, int m, int k, int n, tf_stream_t stream);
 
+/* ---- EXL3 routed experts (exl3/experts.py:173-202 `routed`; pybind `tensorfold_exl3_experts_v1`, experts.cpp:132-141) --
+ * Pairs p = row * slots + slot; a pick outside [0, experts) is not a routed expert and is skipped everywhere.  The
+ * pairs are grouped by tf_experts_plan (tile 16, ids up to and including `experts`): items, counts, members. */
+
+/* out0[p] = fp16(((x[p / slots] * suh0[pick[p]]) H) / sqrt(128)), and out1 from suh1 when given: fp16 [pairs, k];
+ * suh fp16 [experts, k]; x rows x_stride elements apart.  Replaces experts.cpp `rot_in` (experts.cu:96-117). */
+int tf_exl3x_rot_in(const void* x, int x_dtype, int64_t x_stride, const int32_t* pick, const uint16_t* suh0,
+                    const uint16_t* suh1, uint16_t* out0, uint16_t* out1, int rows, int slots, int k, int experts,
+                    tf_stream_t stream);
+/* z[(mat * sk + split), p, :] = the split's share of x_mat[p] @ W_q of pick[p]'s matrix `mat`, fp32 [mats * sk, pairs,
+ * n]: tp int64 [experts] the address of each expert's trellis (the checkpoint's [k/16, n/16, 16 * bits] int16), k2
+ * int32 [experts] its half-bits a value (2..16 even; 3, 5, 7 with codebook 2), one width per expert and matrix.
+ * Replaces experts.cpp `grouped` (experts_grouped.cuh:190-284). */
+int tf_exl3x_grouped(const uint16_t* x0, const uint16_t* x1, const int64_t* tp0, const int64_t* tp1, const int32_t* k2_0,
+                     const int32_t* k2_1, const int32_t* items, const int32_t* counts, const int32_t* members, float* z,
+                     int mats, int k, int n, int pairs, int sk, int cb, int experts, int max_items, tf_stream_t stream);
+/* gate and up of a pair: splits added in order, H / sqrt(128), * svh; SwiGLU clipped at `limit` (act_mode 0 with the
+ * bf16 roundings of exl3/experts.cu:141-146, 1 in fp32); xd[p] = fp16(((act * suh_d) H) / sqrt(128)), fp16 [pairs, n].
+ * Replaces experts.cpp `gateup_epilogue` (experts.cu:121-157). */
+int tf_exl3x_gateup_epilogue(const float* z, const int32_t* pick, const uint16_t* svh_g, const uint16_t* svh_u,
+                             const uint16_t* suh_d, uint16_t* xd, int pairs, int n, int sk, int experts, float limit,
+                             int act_mode, tf_stream_t stream);
+/* y[p] = ((splits added in order) H / sqrt(128)) * svh_d for routed pairs, fp32 [pairs, d] (other pairs keep the
+ * caller's y); with wts: out[r] = fma chain over the slots in order of wts[r, k] * y[r * slots + k], fp32 [rows, d].
+ * Replaces experts.cpp `down_epilogue`, `combine` and `down_combine` (experts.cu:160-237). */
+int tf_exl3x_down_combine(const float* z, const int32_t* pick, const uint16_t* svh_d, float* y, const float* wts,
+                          float* out, int rows, int slots, int d, int sk, int experts, tf_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -148,3 +148,55 @@ def forward(x, trellis, suh, svh, bits: float, name: str, bias=None, *, half_inp
         xh = xh.astype(np.float16).astype(np.float64)
     y = rotate(xh @ unpack(trellis, bits, name).astype(np.float64), -1) * np.asarray(svh, dtype=np.float64)
     return y if bias is None else y + np.asarray(bias, dtype=np.float64)
+
+
+# -- routed experts (cuda/exl3/experts.py:173-202, experts.cu:96-237) --------------------------------------------------
+#
+# Pins (tests/test_oracle_exl3.py): without the fp16 input roundings the pair output equals the dense float64
+# formula on dequantize()'s W (an independent path through the same decode); the clip and the bf16 roundings against
+# hand-computed values; skipped picks contribute nothing; the combine is linear in the weights.
+
+def swiglu_pair(g: np.ndarray, u: np.ndarray, limit: float = np.inf, act_bf16: bool = False) -> np.ndarray:
+    """min(g, limit) * sigmoid(min(g, limit)) * clip(u, -limit, limit); with ``act_bf16`` g, u, the SiLU and the
+    product are each rounded to bf16 first, in fp32 as the kernel computes them (experts.cu:141-151)."""
+
+    if not act_bf16:
+        gg = np.minimum(np.asarray(g, dtype=np.float64), limit)
+        uu = np.clip(np.asarray(u, dtype=np.float64), -limit, limit)
+        return gg / (1.0 + np.exp(-gg)) * uu
+    from .affine import bf16
+
+    gg = np.minimum(bf16(np.asarray(g, dtype=np.float32)), np.float32(min(limit, 3.0e38)))
+    uu = np.clip(bf16(np.asarray(u, dtype=np.float32)), -np.float32(min(limit, 3.0e38)), np.float32(min(limit, 3.0e38)))
+    silu = bf16((gg / (np.float32(1) + np.exp(-gg, dtype=np.float32))).astype(np.float32))
+    return bf16((silu * uu).astype(np.float32)).astype(np.float64)
+
+
+def routed(x, pick, wts, gate, up, down, name: str, *, limit: float = np.inf, act_bf16: bool = False,
+           half_input: bool = True) -> tuple[np.ndarray, np.ndarray]:
+    """Routed experts: ``gate``, ``up``, ``down`` are per-expert (trellis int16, suh, svh) triples, each trellis at
+    its own width; pick [R, slots] int, wts [R, slots].  Pair (r, k) with 0 <= pick < E gives
+    y[r, k] = down(swiglu(gate(x[r]), up(x[r]))), every projection a ``forward`` (``half_input`` rounds its rotated
+    input to fp16 as the kernels do); other pairs are skipped (zeros).  Returns (y [R, slots, D], out [R, D] =
+    sum over the routed slots of wts * y), float64."""
+
+    x = np.asarray(x, dtype=np.float64)
+    pick = np.asarray(pick)
+    rows, slots = pick.shape
+    n_exp = len(gate)
+    y = np.zeros((rows, slots, x.shape[1]), dtype=np.float64)
+
+    def lin(v, m):
+        t, suh, svh = m
+        return forward(v[None, :], np.asarray(t), np.asarray(suh), np.asarray(svh), t.shape[-1] / 16, name,
+                       half_input=half_input)[0]
+
+    for r in range(rows):
+        for k in range(slots):
+            e = int(pick[r, k])
+            if e < 0 or e >= n_exp:
+                continue
+            a = swiglu_pair(lin(x[r], gate[e]), lin(x[r], up[e]), limit, act_bf16)
+            y[r, k] = lin(a, down[e])
+    out = (np.asarray(wts, dtype=np.float64)[:, :, None] * y).sum(axis=1)
+    return y, out

@@ -147,3 +147,63 @@ def test_weight_and_rotated_forward_agree():
         c = native.exl3_linear(xh, t, suh, svh, int(2 * bits), ore.CODEBOOK_IDS[cb], bias)
         want = ore.forward(xh, t, suh, svh, bits, cb, bias, half_input=True)
         assert np.abs(c - want).max() <= 1e-5 * np.abs(want).max()
+
+
+# -- routed experts ----------------------------------------------------------------------------------------------------
+
+def _experts(n_exp, d, width, cb, widths, seed):
+    rng = np.random.default_rng(seed)
+
+    def mat(k, n, bits, s_in, s_out):
+        t = rng.integers(-2 ** 15, 2 ** 15, size=(k // 16, n // 16, int(16 * bits)), dtype=np.int64).astype(np.int16)
+        return t, (rng.standard_normal(k) * s_in).astype(np.float16), (rng.standard_normal(n) * s_out).astype(np.float16)
+
+    gate = [mat(d, width, widths[e % len(widths)], 1 / np.sqrt(d), 1.0) for e in range(n_exp)]
+    up = [mat(d, width, widths[(e + 1) % len(widths)], 1 / np.sqrt(d), 1.0) for e in range(n_exp)]
+    down = [mat(width, d, widths[(e + 2) % len(widths)], 1 / np.sqrt(width), 0.25) for e in range(n_exp)]
+    return gate, up, down
+
+
+def test_swiglu_pair_known_answers():
+    """silu(0) = 0; silu(g) * u at g = ln 3: g / (1 + 1/3) = 0.75 g; the clip caps g from above only and u both ways;
+    the bf16 mode rounds g, u, the SiLU and the product in turn."""
+
+    g = np.array([0.0, np.log(3.0), 50.0, -50.0, 2.0])
+    u = np.array([5.0, 2.0, -30.0, 30.0, 1.0])
+    got = ore.swiglu_pair(g, u)
+    assert np.allclose(got[:2], [0.0, 0.75 * np.log(3.0) * 2.0], atol=1e-15)
+    clipped = ore.swiglu_pair(g, u, limit=10.0)
+    assert np.isclose(clipped[2], 10.0 / (1 + np.exp(-10.0)) * -10.0)
+    assert np.isclose(clipped[3], -50.0 / (1 + np.exp(50.0)) * 10.0)             # g is not clipped from below
+    from oracle.affine import bf16
+    b = ore.swiglu_pair(np.array([1.2345678]), np.array([0.7654321]), act_bf16=True)
+    gg, uu = bf16(np.float32([1.2345678]))[0], bf16(np.float32([0.7654321]))[0]
+    silu = bf16(np.float32([gg / (1 + np.exp(-np.float64(gg)))]))[0]
+    assert b[0] == bf16(np.float32([silu * uu]))[0]
+
+
+def test_routed_experts_against_the_dense_weights():
+    """Without the fp16 input roundings a pair's output is the textbook MLP on dequantize()'s W; a pick outside
+    [0, E) contributes nothing; the combine is the weighted sum."""
+
+    n_exp, d, width = 5, 256, 128
+    gate, up, down = _experts(n_exp, d, width, "mul1", (2, 2.5, 4), 21)
+    rng = np.random.default_rng(22)
+    x = rng.standard_normal((3, d))
+    pick = np.array([[0, 3, 5], [4, 4, -1], [2, 1, 0]], dtype=np.int32)
+    wts = rng.random((3, 3)) + 0.1
+    y, out = ore.routed(x, pick, wts, gate, up, down, "mul1", half_input=False)
+    for r in range(3):
+        for k in range(3):
+            e = int(pick[r, k])
+            if not 0 <= e < n_exp:
+                assert not y[r, k].any()
+                continue
+            w = [ore.dequantize(m[e][0], m[e][1], m[e][2], m[e][0].shape[-1] / 16, "mul1") for m in (gate, up, down)]
+            g, u = x[r] @ w[0], x[r] @ w[1]
+            want = (g / (1 + np.exp(-g)) * u) @ w[2]
+            assert np.allclose(y[r, k], want, rtol=1e-9, atol=1e-9 * np.abs(want).max())
+    assert np.allclose(out, np.einsum("rk,rkd->rd", wts, y))
+    # the fp16 roundings of the rotated inputs move the result by about 2^-11 a value, not more
+    y16, _ = ore.routed(x, pick, wts, gate, up, down, "mul1")
+    assert 0 < np.abs(y16 - y).max() <= 4e-3 * np.abs(y).max()
