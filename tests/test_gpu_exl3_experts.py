@@ -184,3 +184,21 @@ def test_bad_arguments_raise():
         experts.prepare([], [], [], "mcg")
     with pytest.raises(ValueError):
         experts.codebook_id("nope")
+
+
+def test_more_than_1024_pairs():
+    """Past 1,024 pairs the pair sort runs on several workgroups and an expert's pairs span many items of 16."""
+
+    n_exp, d, width, top_k, rows = 12, 256, 128, 7, 160
+    ex, mats = make_layer(n_exp, d, width, "mcg", lambda e: (2 + e % 3, 3, 4), 71)
+    x = torch.randn((rows, d), generator=torch.Generator().manual_seed(5)).to(torch.bfloat16).to(DEV)
+    sel, w = picks(n_exp, rows, top_k, 6, shared=True)
+    scratch = experts.Scratch(ex, rows, top_k + 1)
+    scratch.y.zero_()
+    full = experts.routed(x, sel, w, ex, scratch, None, rows).clone()
+    small = experts.Scratch(ex, 3, top_k + 1)
+    for r0 in (0, 77, rows - 3):
+        part = experts.routed(x[r0:r0 + 3], sel[r0:r0 + 3].contiguous(), w[r0:r0 + 3].contiguous(), ex, small, None, 3)
+        assert torch.equal(part, full[r0:r0 + 3])
+    _, want = ore.routed(x[:3].float().cpu().numpy(), sel[:3].cpu().numpy(), w[:3].cpu().numpy(), *mats, "mcg")
+    assert rel_l2(full[:3].double().cpu().numpy(), want) <= TOL
