@@ -97,14 +97,38 @@ __device__ __forceinline__ uint16_t code_value(uint32_t s) {
   }
 }
 
+// The hashed word of a state of the 3inst and mcg codebooks: the value is the fp16 sum of its two halves.
+template <int CB>
+__device__ __forceinline__ uint32_t code_word(uint32_t s) {
+  const uint32_t x = CB == 1 ? s * 0xCBAC1FEDu : s * 89226354u + 64248484u;
+  return (x & 0x8FFF8FFFu) ^ 0x3B603B60u;
+}
+
+// (half(xa.lo) + half(xa.hi)) | (half(xb.lo) + half(xb.hi)) << 16.  The second add writes the upper half of the
+// register the first one wrote and keeps the lower: two instructions for two values, where the compiler's own
+// pairing pads each result and ORs them (a third).  The same IEEE add as __hadd.
+__device__ __forceinline__ uint32_t half_sums(uint32_t xa, uint32_t xb) {
+  uint32_t r;
+  asm("v_add_f16_sdwa %0, %1, %1 dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1" : "=v"(r) : "v"(xa));
+  asm("v_add_f16_sdwa %0, %1, %1 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_0 src1_sel:WORD_1"
+      : "+v"(r)
+      : "v"(xb));
+  return r;
+}
+
 // the fp16 bits of the lane's four values of one tile, as two packed words
 template <int K2, int CB>
 __device__ __forceinline__ void decode4(const Windows<K2>& win, const uint32_t (&w)[Windows<K2>::NW], uint32_t& lo,
                                         uint32_t& hi) {
   uint32_t s[4];
   win.states(w, s);
-  lo = (uint32_t)code_value<CB>(s[0]) | ((uint32_t)code_value<CB>(s[1]) << 16);
-  hi = (uint32_t)code_value<CB>(s[2]) | ((uint32_t)code_value<CB>(s[3]) << 16);
+  if constexpr (CB == 2) {
+    lo = (uint32_t)code_value<CB>(s[0]) | ((uint32_t)code_value<CB>(s[1]) << 16);
+    hi = (uint32_t)code_value<CB>(s[2]) | ((uint32_t)code_value<CB>(s[3]) << 16);
+  } else {
+    lo = half_sums(code_word<CB>(s[0]), code_word<CB>(s[1]));
+    hi = half_sums(code_word<CB>(s[2]), code_word<CB>(s[3]));
+  }
 }
 
 template <int K2, int CB>
