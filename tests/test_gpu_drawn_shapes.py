@@ -122,3 +122,27 @@ def test_exl3_layer(seed):
         assert torch.equal(layer(xd[r:r + 1], out_dtype=torch.float32)[0], got[r]), split
         assert int(layer.counters.abs().sum()) == 0
     assert ran >= 2
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_drawn_exl3_prompt_matmuls(seed):
+    """Shapes off the benchmark's grid through the decode-once GEMM: any M, N of 1 to 5 blocks of 128 (part-filled
+    256-column tiles), K down to one block, every codebook."""
+
+    from tensorfold_amd.exl3 import prefill
+
+    rng = np.random.default_rng(900 + seed)
+    codebook = ("3inst", "mcg", "mul1")[seed % 3]
+    bits = (2, 3, 4, 5, 6, 8)[int(rng.integers(6))] if codebook != "mul1" else (1.5, 2.5, 3.5, 4)[int(rng.integers(4))]
+    kt, nt, m = 8 * int(rng.integers(1, 6)), 8 * int(rng.integers(1, 6)), int(rng.integers(1, 300))
+    trellis = torch.from_numpy(rng.integers(-2 ** 15, 2 ** 15, size=(kt, nt, int(16 * bits))).astype(np.int16))
+    k, n = 16 * kt, 16 * nt
+    suh = torch.from_numpy((rng.standard_normal(k) * 0.05).astype(np.float16))
+    svh = torch.from_numpy((rng.standard_normal(n) * 0.05).astype(np.float16))
+    layer = linear.Exl3Linear.from_tensors(trellis, suh, svh, codebook)
+    x = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float16))
+    out = torch.full((m + 1, n + 2), 7.0, dtype=torch.float32, device=DEV)          # strided rows, a guard row below
+    prefill.matmul(layer, x.to(DEV), out[:m, :n], prefill.Workspace())
+    want = ore.forward(x.numpy(), trellis.numpy(), suh.numpy(), svh.numpy(), bits, codebook, half_input=True)
+    assert rel_l2(out[:m, :n].cpu().numpy(), want) < TOL, (codebook, bits, k, n, m)
+    assert (out[m] == 7.0).all() and (out[:, n:] == 7.0).all()
