@@ -202,3 +202,23 @@ def test_more_than_1024_pairs():
         assert torch.equal(part, full[r0:r0 + 3])
     _, want = ore.routed(x[:3].float().cpu().numpy(), sel[:3].cpu().numpy(), w[:3].cpu().numpy(), *mats, "mcg")
     assert rel_l2(full[:3].double().cpu().numpy(), want) <= TOL
+
+
+def test_no_routed_pick_at_all():
+    """Every slot outside [0, E): nothing is grouped, y stays the caller's and the combine is its weighted sum."""
+
+    n_exp, d, width, rows, slots = 5, 256, 128, 3, 4
+    ex, _ = make_layer(n_exp, d, width, "mcg", lambda e: (4, 4, 4), 81)
+    x = torch.randn((rows, d), generator=torch.Generator().manual_seed(1)).to(torch.bfloat16).to(DEV)
+    sel = torch.tensor([[5, 7, -1, 5]] * rows, dtype=torch.int32, device=DEV)
+    w = torch.rand((rows, slots), generator=torch.Generator().manual_seed(2)).to(DEV)
+    scratch = experts.Scratch(ex, rows, slots)
+    mine = torch.randn((rows * slots, d), generator=torch.Generator().manual_seed(3)).to(DEV)
+    scratch.y.copy_(mine)
+    out = experts.routed(x, sel, w, ex, scratch, None, rows)
+    assert torch.equal(scratch.y, mine)
+    want = np.zeros((rows, d), dtype=np.float32)
+    wn, yn = w.cpu().numpy(), mine.view(rows, slots, d).cpu().numpy()
+    for k in range(slots):
+        want = (wn[:, k:k + 1].astype(np.float64) * yn[:, k].astype(np.float64) + want.astype(np.float64)).astype(np.float32)
+    assert np.array_equal(out.cpu().numpy(), want)
