@@ -149,6 +149,122 @@ __device__ __forceinline__ void topk_row16(const float* __restrict__ row, int NE
 #undef TF_ROW_I
 }
 
+// The k-th pick of a row alone: passes 0 .. k of topk_pick's selection (value descending, ties to the lower id), no
+// weights.  The same value in every lane.
+template <int VPL>
+__device__ __forceinline__ int topk_kth(float (&v)[VPL], int k, int lane) {
+  const float NEG = -__builtin_inff();
+  int idx = 0;
+  for (int pass = 0; pass <= k; ++pass) {
+    float bv = v[0];
+    int bi = lane;
+#pragma unroll
+    for (int i = 1; i < VPL; ++i)
+      if (v[i] > bv) {
+        bv = v[i];
+        bi = lane + 64 * i;
+      }
+    const float m = wave_max(bv);
+    unsigned long long cand = __ballot(bv == m);
+    idx = 0x7FFFFFFF;
+    while (cand) {
+      const int l = __builtin_ctzll(cand);
+      idx = min(idx, __builtin_amdgcn_readlane(bi, l));
+      cand &= cand - 1;
+    }
+    if ((idx & 63) == lane) {
+#pragma unroll
+      for (int i = 0; i < VPL; ++i)
+        if (i == (idx >> 6)) v[i] = NEG;
+    }
+  }
+  return idx;
+}
+
+// The slot expert e would take in a row (v as topk_load leaves it): the number of experts that the selection takes
+// before it, i.e. with a larger logit, or an equal one and a lower id.  e is picked iff this is below TOPK, and
+// then it is the pick's slot, since the passes of topk_pick take the experts in exactly that order.
+template <int VPL>
+__device__ __forceinline__ int topk_slot_of(const float (&v)[VPL], int e, int lane) {
+  float c = v[0];
+#pragma unroll
+  for (int i = 1; i < VPL; ++i)
+    if (i == (e >> 6)) c = v[i];
+  const float val = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, c), e & 63));
+  int rank = 0;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) rank += __popcll(__ballot(v[i] > val || (v[i] == val && lane + 64 * i < e)));
+  return rank;
+}
+
+// A workgroup that takes ONE pair p = (row r, slot k) finds its item without the other rows' top-k: wave 0 runs
+// k + 1 selection passes over row r to learn the expert; every wave then asks of its share of the rows whether the
+// expert is among their picks (topk_slot_of); the expert's pairs, in pair order, go two an item, and the workgroup
+// of an item's first pair takes the item, the workgroup of its second pair leaves.  Items and their pairs are those
+// of the plan's descriptors (DTILE = 2).  R <= 64.  memb: R ints of LDS, sel: one, wp: this wave's two.
+// Every thread calls this (two barriers).  False: this workgroup has nothing to do.
+template <int VPL, int WAVES>
+__device__ __forceinline__ bool pair_item(const float* __restrict__ L, int64_t ldl, int R, int NE, int TOPK, int shared,
+                                          int slots, int p, int* memb, int* sel, int* wp, int& e_out, int& cnt_out) {
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r = p / slots, k = p - r * slots;
+  const bool always = shared && k == TOPK;         // the shared expert: every row, slot TOPK
+  constexpr int PRE = VPL <= 2 ? 2 : 1;     // rows a wave requests before the selection, to wait for them under it
+  float v[PRE][VPL];
+  if (!always) {
+#pragma unroll
+    for (int i = 0; i < PRE; ++i)
+      if (wave + i * WAVES < R) topk_load<VPL>(L + (size_t)(wave + i * WAVES) * ldl, NE, lane, v[i]);
+  }
+  if (wave == 0) {
+    int e = NE;
+    if (!always) {
+      float t[VPL];
+      topk_load<VPL>(L + (size_t)r * ldl, NE, lane, t);
+      e = topk_kth<VPL>(t, k, lane);
+    }
+    if (lane == 0) sel[0] = e;
+  }
+  __syncthreads();
+  const int e = sel[0];
+#pragma unroll
+  for (int i = 0; i < PRE; ++i) {
+    const int q = wave + i * WAVES;
+    if (q >= R) break;
+    int m = TOPK;
+    if (!always) {
+      const int slot = topk_slot_of<VPL>(v[i], e, lane);
+      m = slot < TOPK ? slot : -1;
+    }
+    if (lane == 0) memb[q] = m;
+  }
+  for (int q = wave + PRE * WAVES; q < R; q += WAVES) {
+    int m = TOPK;
+    if (!always) {
+      topk_load<VPL>(L + (size_t)q * ldl, NE, lane, v[0]);
+      const int slot = topk_slot_of<VPL>(v[0], e, lane);
+      m = slot < TOPK ? slot : -1;
+    }
+    if (lane == 0) memb[q] = m;
+  }
+  __syncthreads();
+  const int m = lane < R ? memb[lane] : -1;
+  const unsigned long long mask = __ballot(m >= 0);
+  if (__popcll(mask & ((1ull << r) - 1ull)) & 1) return false;       // the second pair of an item
+  const unsigned long long rest = r < 63 ? mask >> (r + 1) : 0ull;
+  int p1 = p, cnt = 1;
+  if (rest) {
+    const int q = __builtin_amdgcn_readfirstlane(r + 1 + __builtin_ctzll(rest));
+    p1 = q * slots + __builtin_amdgcn_readlane(m, q);
+    cnt = 2;
+  }
+  wp[0] = p;
+  wp[1] = p1;
+  e_out = e;
+  cnt_out = cnt;
+  return true;
+}
+
 template <int VPL>
 __device__ __forceinline__ void topk_lane_n(const float* __restrict__ row, int NE, int TOPK, int shared, int lane,
                                             int& id, float& w) {

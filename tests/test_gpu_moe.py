@@ -278,7 +278,7 @@ def test_decode_replays_in_a_graph_with_new_logits_and_inputs():
         moe.decode(torch.cat([x, x]), torch.cat([l, l]), ex, buf, shape.top_k, ne)      # more rows than the buffers hold
 
 
-def check_decode_forms(shape, ne, rows, seed, oracle=True):
+def check_decode_forms(shape, ne, rows, seed, oracle=True, levels=0):
     """Every form of ``decode`` gives the bits of the separate kernels (twice in a row), ids equal the oracle's, and
     the output is within 2e-3 of the CPU oracle's layer."""
 
@@ -288,7 +288,10 @@ def check_decode_forms(shape, ne, rows, seed, oracle=True):
     cfg = type("c", (), dict(num_experts_per_tok=top_k, num_experts=ne, moe_intermediate_size=width,
                              hidden_size=hidden))
     x = synthetic.activations(rows, hidden, 4000 + seed).to(DEV)
-    l = synthetic.logits(rows, ne + int(shared), 5000 + seed).to(DEV)
+    l = synthetic.logits(rows, ne + int(shared), 5000 + seed)
+    if levels:
+        l = torch.round(l * levels) / levels          # few distinct values: ties inside every row
+    l = l.to(DEV)
     ref = moe.MoEBuffers(rows, cfg, DEV, shared=shared)
     moe.select(l, ref, top_k, ne)
     experts.gate_up(x, ex, ref.plan, ref.act.view(-1, ex.width), rows)
@@ -345,3 +348,13 @@ def test_random_shapes_of_the_decode_layer(seed):
 ])
 def test_the_decode_layer_at_its_limits(hidden, width, ne, top_k, gs, swiglu, shared, rows):
     check_decode_forms(synthetic.MoEShape("limit", hidden, ne, width, top_k, gs, swiglu, shared), ne, rows, 99)
+
+
+@pytest.mark.parametrize("ne,top_k,shared,rows,levels", [(128, 6, False, 8, 2), (40, 8, True, 13, 1), (300, 5, False, 6, 2),
+                                                         (16, 16, False, 64, 1), (700, 3, True, 2, 1)])
+def test_tied_logits_through_the_decode_layer(ne, top_k, shared, rows, levels):
+    """Logits on a grid of a few values, so every row holds runs of equal logits across its top-k boundary: a
+    workgroup that finds its item from its pair's own row and a rank test on the other rows must break the ties as
+    the selection passes do (lower id first)."""
+
+    check_decode_forms(synthetic.MoEShape("ties", 128, ne, 64, top_k, 64, False, shared), ne, rows, 7, levels=levels)
