@@ -149,10 +149,13 @@ def c3() -> dict:
     wts = torch.cat([torch.softmax(sel[:, :-1], 1), torch.sigmoid(sel[:, -1:])], 1).bfloat16().float().contiguous().to(DEV)
     slots = s.top_k + 1
     out = {}
-    for tile in (64, 128):
+    # items of 64 and of 128 with fp32 pair outputs (this build's default), then items of 128 with the reference's
+    # bf16 pair outputs (cuda/moe.py:99), which halve the traffic between the down projection and the combine
+    for tile, ydt in ((64, torch.float32), (128, torch.float32), ("128_y_bf16", torch.bfloat16)):
+        key, tile = tile, 128 if isinstance(tile, str) else tile
         plan = experts.Plan(rows, slots, s.experts + 1, DEV, prefill=True)
         act = torch.empty((rows * slots, s.width), dtype=torch.bfloat16, device=DEV)
-        y = torch.empty((rows * slots, s.hidden), dtype=torch.float32, device=DEV)
+        y = torch.empty((rows * slots, s.hidden), dtype=ydt, device=DEV)
         res = torch.empty((rows, s.hidden), dtype=torch.bfloat16, device=DEV)
 
         def step(i):
@@ -167,7 +170,8 @@ def c3() -> dict:
         down_us = graph_us(lambda i: experts.down(act, ex, plan, y, rows), 8)
         route_us = graph_us(lambda i: experts.route(picks, plan, tile), 8)
         flop = rows * slots * 3 * 2 * s.hidden * s.width
-        out[tile] = {"chunk_us": us, "tokens_per_s": rows / us * 1e6, "flop": flop, "tflops": flop / us * 1e-6,
+        combine_us = graph_us(lambda i: moe.combine(y.view(rows, slots, s.hidden), wts, res), 8)
+        out[key] = {"chunk_us": us, "combine_us": combine_us, "tokens_per_s": rows / us * 1e6, "flop": flop, "tflops": flop / us * 1e-6,
                      "frac": flop / us * 1e-6 / MFMA, "route_us": route_us, "up_us": up_us, "down_us": down_us,
                      "up_tflops": flop * 2 / 3 / up_us * 1e-6, "down_tflops": flop / 3 / down_us * 1e-6,
                      "items": int(plan.counts[0])}
