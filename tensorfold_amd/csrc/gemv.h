@@ -150,15 +150,6 @@ __device__ __forceinline__ void chunk_dot(float (&p)[NM][RB], const Stage<GS, NM
 //   xsum(r, g)      -> row r's sum over group g (wave-uniform)
 //   flush(g, acc)   -> called after group g has been added (wave-uniform); may park and clear acc
 // `st` holds the weights of groups gA .. gA + DEPTH - 1 on entry when `loaded`.
-__device__ __forceinline__ void set_prio(int q) {
-  switch (q) {
-    case 3: __builtin_amdgcn_s_setprio(3); break;
-    case 2: __builtin_amdgcn_s_setprio(2); break;
-    case 1: __builtin_amdgcn_s_setprio(1); break;
-    default: __builtin_amdgcn_s_setprio(0);
-  }
-}
-
 template <int GS, int NM, int RB, int COH, class WQ, class SB, class XS, class FLUSH>
 __device__ __forceinline__ void gemv_stream(float (&acc)[NM][RB], Stage<GS, NM> (&st)[DEPTH], bool loaded,
                                             const WQ& wq, const SB& sb, const uint32_t* const (&xl)[RB],
@@ -173,13 +164,7 @@ __device__ __forceinline__ void gemv_stream(float (&acc)[NM][RB], Stage<GS, NM> 
     }
   const int n = gB - gA;
   for (int gb = gA; gb < gB; gb += DEPTH) {
-    // A wave that is behind issues first: priority 3 in the first quarter of its groups, down to 0 in the last.
-    // (Left alone, the oldest wave of a SIMD issues first, the workgroups dispatched first finish microseconds before
-    // the others, and the launch ends on a few late ones that cannot fill the memory system by themselves.)
-    if (n > DEPTH) {                          // (a wave that makes one trip through this loop has nobody to yield to)
-      const int left4 = 4 * (gB - gb);
-      set_prio(left4 > 3 * n ? 3 : left4 > 2 * n ? 2 : left4 > n ? 1 : 0);
-    }
+    if (n > DEPTH) prio_by_progress(gB - gb, n);      // (one trip through this loop: nobody to yield to)
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
       const int g = gb + d;

@@ -78,6 +78,22 @@ __device__ __forceinline__ float swiglu(float g, float u, float limit) {
   return round_bf16(gv / (1.f + __expf(-gv))) * uv;
 }
 
+// ---- issue priority by progress ------------------------------------------------------------------------------------
+//
+// A wave with `left` of its `n` loop trips to go takes priority 3 in the first quarter of them, down to 0 in the
+// last: a wave that is behind issues first.  Left alone, the oldest wave of a SIMD issues first, the workgroups
+// dispatched first finish microseconds before the others, and the launch ends on a few late ones that cannot fill
+// the memory system by themselves.  (s_setprio takes an immediate, hence the switch.)
+__device__ __forceinline__ void prio_by_progress(int left, int n) {
+  const int left4 = 4 * left;
+  switch (left4 > 3 * n ? 3 : left4 > 2 * n ? 2 : left4 > n ? 1 : 0) {
+    case 3: __builtin_amdgcn_s_setprio(3); break;
+    case 2: __builtin_amdgcn_s_setprio(2); break;
+    case 1: __builtin_amdgcn_s_setprio(1); break;
+    default: __builtin_amdgcn_s_setprio(0);
+  }
+}
+
 // ---- 4-bit blocks -------------------------------------------------------------------------------------------------
 
 constexpr uint32_t NIB_MASK = 0x000F000Fu;
