@@ -91,6 +91,7 @@ __global__ void __launch_bounds__(WAVES * 64)
                         float* __restrict__ y, uint16_t* __restrict__ out, int* __restrict__ arrive) {
   extern __shared__ float lds[];
   __shared__ int pairs[16];
+  __builtin_amdgcn_s_setprio(3);       // the descriptor and the first requests issue ahead of the workgroups that already stream
   const int NB = D / 32, NB2d = (NB + 1) >> 1;
   const int it = blockIdx.x / NB2d, cb2 = blockIdx.x - it * NB2d;
   if (it >= desc[0]) return;
@@ -161,6 +162,7 @@ __global__ void __launch_bounds__(WAVES * 64)
   extern __shared__ float lds[];
   __shared__ int pk[PLAN_THREADS];
   __shared__ ItemLds item;
+  __builtin_amdgcn_s_setprio(3);       // the lookup issues ahead of the workgroups that already stream
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, threads = WAVES * 64;
   const int slots = TOPK + (shared ? 1 : 0), P = R * slots, E = NE + (shared ? 1 : 0);
   const bool writer = blockIdx.x == 0;
