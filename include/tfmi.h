@@ -150,10 +150,11 @@ int tf_add_norm(const uint16_t* x, const void* delta, int delta_kind, const floa
 /* Routing and the up projection of the decode layer in ONE launch, for rows * (top_k + shared) <= 1024: workgroup 0
  * writes what tf_moe_topk and tf_experts_plan (tile 16) would (pick, wts, members, items, counts) plus the item
  * descriptors that tf_experts_run_desc reads; every other workgroup finds its own item from the
- * logits and runs the up unit of tf_experts_run (epilogue relu^2, or SwiGLU when swiglu != 0): act bf16 [pairs, ni] and
+ * logits (with 2 to 64 rows a workgroup a pair: its own row's selection up to its slot, then a rank test of that
+ * expert on the other rows) and runs the up unit of tf_experts_run (epilogue relu^2, or SwiGLU when swiglu != 0): act bf16 [pairs, ni] and
  * its group sums xs_act fp32 [pairs, ni / gs]; it also zeroes `zero` (n_zero ints: the next launch's counters).  Same
  * bits as the separate calls.  logits may be NULL: pick and wts are then inputs (tf_moe_topk ran before, the better
- * order past about 2,048 logits, where repeating the top-k in every workgroup costs more than a launch) and only the
+ * order past about 2,048 logits, where reading the rows in every workgroup costs more than a launch) and only the
  * plan is made here.  No counterpart in the reference (moe.py:88-128 issues them one by one). */
 int tf_moe_route_up(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared, int gs, int swiglu,
                     const uint16_t* x, int64_t x_stride, const uint32_t* up, int d, int ni, int32_t* pick, float* wts,
