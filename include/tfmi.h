@@ -105,6 +105,8 @@ int tf_experts_run(int gs, int epi, const uint16_t* x, int64_t x_stride, int slo
  * read descriptors. */
 #define TF_DESC_INTS 8
 #define TF_DESC_TILE 2
+/* ints between two descriptors' arrival counters in tf_moe_decode_experts' `done` (each alone in 256 bytes) */
+#define TF_DONE_STRIDE 64
 
 /* tf_experts_run with the items given as descriptors; xs is required; counts is not read (kept for symmetry).
  * Same bits as tf_experts_run on the same plan.  Same reference counterpart (experts.cpp:43-48 `run`); the
@@ -179,7 +181,7 @@ int tf_moe_route_decode(const float* logits, int64_t ldl, int rows, int experts,
 /* The decode layer's experts in one launch: up (+ relu^2 or SwiGLU), down and the weighted combine, with the bits
  * of tf_experts_run, tf_experts_run and tf_moe_combine run in turn.  desc, counts, wts, xs_x as left by
  * tf_moe_route_decode; scratch act bf16 [pairs, ni], xs_act fp32 [pairs, ni/gs], y fp32 [pairs, d]; counters done
- * [max_items] (one a descriptor) and arrive [rows * d/64] zero on entry; status[0] is set to 1 if a bounded wait ran out (the output
+ * [max_items * 64] (one a descriptor, each alone in 256 bytes: TF_DONE_STRIDE ints apart) and arrive [rows * d/64] zero on entry; status[0] is set to 1 if a bounded wait ran out (the output
  * is then invalid).  d and ni multiples of 64.  Fuses experts.cpp:43-48 `run` (twice) and moe.py:131-151 `combine`. */
 int tf_moe_decode_experts(int gs, int swiglu, const uint16_t* x, int64_t x_stride, int rows, int slots,
                           const uint32_t* up, const uint32_t* down, int d, int ni, const int32_t* desc,

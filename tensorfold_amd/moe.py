@@ -29,6 +29,7 @@ ROUTING_LAUNCH = os.environ.get("TENSORFOLD_AMD_ROUTING_LAUNCH", "0") == "1"
 # Item descriptors the routing launches leave for the decode expert kernels: rows of DESC_INTS int32, row 0 the
 # count; items of at most DESC_TILE pairs (TF_DESC_INTS / TF_DESC_TILE of the C header).
 DESC_INTS, DESC_TILE = 8, 2
+DONE_STRIDE = 64     # ints between the arrival counters of two descriptors (the one-launch form): one a 256-byte block
 
 
 def router(x: torch.Tensor, rows: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
@@ -80,11 +81,11 @@ class MoEBuffers:
             items = grouped.max_items(pairs, cfg.num_experts + int(self.shared), DESC_TILE)
             cells = self.rows * (cfg.hidden_size // 64)
             self._fused = dict(
-                items=items,
+                items=items * DONE_STRIDE,          # ints the descriptors' arrival counters take
                 desc=torch.zeros((1 + items, DESC_INTS), dtype=torch.int32, device=dev),
                 xs_x=torch.empty((self.rows, cfg.hidden_size // gs), dtype=torch.float32, device=dev),
                 xs_act=torch.empty((pairs, cfg.moe_intermediate_size // gs), dtype=torch.float32, device=dev),
-                counters=torch.zeros((1 + items + cells,), dtype=torch.int32, device=dev),
+                counters=torch.zeros((1 + items * DONE_STRIDE + cells,), dtype=torch.int32, device=dev),
                 out=torch.empty((self.rows, cfg.hidden_size), dtype=torch.bfloat16, device=dev))
         return self._fused
 
