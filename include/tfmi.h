@@ -107,6 +107,8 @@ int tf_experts_run(int gs, int epi, const uint16_t* x, int64_t x_stride, int slo
 #define TF_DESC_TILE 2
 /* ints between two descriptors' arrival counters in tf_moe_decode_experts' `done` (each alone in 256 bytes) */
 #define TF_DONE_STRIDE 64
+/* ints between two cells' arrival counters in `arrive` when rows <= 64 (each alone in 64 bytes); 1 past 64 rows */
+#define TF_ARRIVE_STRIDE 16
 
 /* tf_experts_run with the items given as descriptors; xs is required; counts is not read (kept for symmetry).
  * Same bits as tf_experts_run on the same plan.  Same reference counterpart (experts.cpp:43-48 `run`); the
@@ -164,7 +166,8 @@ int tf_moe_route_up(const float* logits, int64_t ldl, int rows, int experts, int
                     float limit, int max_items, int32_t* zero, int n_zero, tf_stream_t stream);
 /* The down projection from item descriptors with the weighted combine folded in: y fp32 [pairs, d] as
  * tf_experts_run_desc (epilogue 0) writes it, and out bf16 [rows, d] with the bits of tf_moe_combine, written by
- * whichever workgroup completes a (token, 64 columns) cell.  `arrive` int32 [rows * ceil(d / 64)] must be zero on
+ * whichever workgroup completes a (token, 64 columns) cell.  `arrive` int32 [rows * ceil(d / 64) * s], s =
+ * TF_ARRIVE_STRIDE with rows <= 64 and 1 past that, must be zero on
  * entry (tf_moe_route_up and tf_moe_route_decode clear a `zero` range for this) and is left non-zero.  Fuses
  * experts.cpp:43-48 `run` and moe.py:131-151 `combine`. */
 int tf_moe_down_combine(int gs, const uint16_t* act, int rows, int slots, const uint32_t* down, int d, int ni,
@@ -181,7 +184,7 @@ int tf_moe_route_decode(const float* logits, int64_t ldl, int rows, int experts,
 /* The decode layer's experts in one launch: up (+ relu^2 or SwiGLU), down and the weighted combine, with the bits
  * of tf_experts_run, tf_experts_run and tf_moe_combine run in turn.  desc, counts, wts, xs_x as left by
  * tf_moe_route_decode; scratch act bf16 [pairs, ni], xs_act fp32 [pairs, ni/gs], y fp32 [pairs, d]; counters done
- * [max_items * 64] (one a descriptor, each alone in 256 bytes: TF_DONE_STRIDE ints apart) and arrive [rows * d/64] zero on entry; status[0] is set to 1 if a bounded wait ran out (the output
+ * [max_items * 64] (one a descriptor, each alone in 256 bytes: TF_DONE_STRIDE ints apart) and arrive [rows * d/64 * s] (s as in tf_moe_down_combine) zero on entry; status[0] is set to 1 if a bounded wait ran out (the output
  * is then invalid).  d and ni multiples of 64.  Fuses experts.cpp:43-48 `run` (twice) and moe.py:131-151 `combine`. */
 int tf_moe_decode_experts(int gs, int swiglu, const uint16_t* x, int64_t x_stride, int rows, int slots,
                           const uint32_t* up, const uint32_t* down, int d, int ni, const int32_t* desc,

@@ -50,11 +50,15 @@ struct WaitItem {
   }
 };
 
+// Ints between the arrival counters of two (token, 64 columns) cells: with few rows each counter sits alone in 64
+// bytes (at one token the 252 units of a launch arrive within a microsecond on 42 counters).
+int arrive_stride(int rows) { return rows <= 64 ? TF_ARRIVE_STRIDE : 1; }
+
 // A down unit has written its 64 columns of y (agent-scope stores) for its rows: count it in each row's token; the
 // unit that completes a (token, 64 columns) cell adds the token's slots in slot order (fp32 fma, as tf_moe_combine)
-// and writes bf16.  `arrive` [tokens * NB2d] starts at zero.
+// and writes bf16.  `arrive` [tokens * NB2d * astride] starts at zero.
 template <int WAVES>
-__device__ __forceinline__ void combine_cells(const int* pairs, int cnt, int slots, int cb2, int NB2d, int D,
+__device__ __forceinline__ void combine_cells(const int* pairs, int cnt, int slots, int cb2, int NB2d, int D, int astride,
                                               const float* __restrict__ wts, const float* __restrict__ y,
                                               uint16_t* __restrict__ out, int* __restrict__ arrive) {
   __builtin_amdgcn_s_waitcnt(0);      // every store of this wave is acknowledged ...
@@ -67,7 +71,7 @@ __device__ __forceinline__ void combine_cells(const int* pairs, int cnt, int slo
     const int token = pairs[r] / slots;
     int done = 0;
     if (lane == 0)
-      done = __hip_atomic_fetch_add(arrive + (size_t)token * NB2d + cb2, 1, __ATOMIC_RELAXED,
+      done = __hip_atomic_fetch_add(arrive + ((size_t)token * NB2d + cb2) * astride, 1, __ATOMIC_RELAXED,
                                     __HIP_MEMORY_SCOPE_AGENT) == slots - 1;
     if (!__builtin_amdgcn_readfirstlane(done) || col >= D) continue;
     float a = 0.f;
@@ -93,7 +97,7 @@ template <int GS, int WAVES>
 __global__ void __launch_bounds__(WAVES * 64)
     down_combine_kernel(const uint16_t* __restrict__ act, int slots, const uint32_t* __restrict__ Wdown, int D, int NI,
                         const int* __restrict__ desc, const float* __restrict__ wts, const float* __restrict__ xs_act,
-                        float* __restrict__ y, uint16_t* __restrict__ out, int* __restrict__ arrive) {
+                        float* __restrict__ y, uint16_t* __restrict__ out, int* __restrict__ arrive, int astride) {
   extern __shared__ float lds[];
   __shared__ int pairs[16];
   __builtin_amdgcn_s_setprio(3);       // the descriptor and the first requests issue ahead of the workgroups that already stream
@@ -107,7 +111,7 @@ __global__ void __launch_bounds__(WAVES * 64)
   NoHook none;
   expert_unit<GS, 1, 0, WAVES, true, COH_OUT>(act, NI, 0, Wdown, NI / GS, NB, e, cnt, pairs, cb2, y, D, 0.f, xs_act,
                                               nullptr, lds, none);
-  combine_cells<WAVES>(pairs, cnt, slots, cb2, NB2d, D, wts, y, out, arrive);
+  combine_cells<WAVES>(pairs, cnt, slots, cb2, NB2d, D, astride, wts, y, out, arrive);
 }
 
 template <int GS, int NM, int EPI_UP, int WAVES>
@@ -117,7 +121,7 @@ __global__ void __launch_bounds__(WAVES * 64)
                      const int* __restrict__ counts, const float* __restrict__ wts, const float* __restrict__ xs_x,
                      uint16_t* __restrict__ act, float* __restrict__ xs_act, float* __restrict__ y,
                      uint16_t* __restrict__ out, int* __restrict__ done, int* __restrict__ arrive,
-                     int* __restrict__ status, float limit, int max_items, int spins) {
+                     int* __restrict__ status, float limit, int max_items, int spins, int astride) {
   extern __shared__ float lds[];
   __shared__ int pairs[16];
   const int NB2u = (NI / 32 + 1) >> 1, NB2d = (D / 32 + 1) >> 1;
@@ -145,7 +149,7 @@ __global__ void __launch_bounds__(WAVES * 64)
   if (!expert_unit<GS, 1, 0, WAVES, true, DCOH>(act, NI, 0, Wdown, NI / GS, D / 32, e, cnt, pairs, cb2, y, D,
                                                             0.f, xs_act, nullptr, lds, wait))
     return;                     // the wait ran out: status is set, nothing is published
-  combine_cells<WAVES>(pairs, cnt, slots, cb2, NB2d, D, wts, y, out, arrive);
+  combine_cells<WAVES>(pairs, cnt, slots, cb2, NB2d, D, astride, wts, y, out, arrive);
 }
 
 
@@ -376,7 +380,7 @@ template <int GS, int NM, int EPI_UP>
 int launch_fused(const uint16_t* x, int64_t x_stride, int slots, const uint32_t* wup, const uint32_t* wdown, int d,
                  int ni, const int* desc, const int* counts, const float* wts, const float* xs_x, uint16_t* act,
                  float* xs_act, float* y, uint16_t* out, int* done, int* arrive, int* status, float limit,
-                 int max_items, hipStream_t stream) {
+                 int max_items, int astride, hipStream_t stream) {
   const int nb2u = (ni / 32 + 1) / 2, nb2d = (d / 32 + 1) / 2;
   const int64_t grid = (int64_t)max_items * (nb2u + nb2d);
   if (grid < 1) return 0;
@@ -387,7 +391,7 @@ int launch_fused(const uint16_t* x, int64_t x_stride, int slots, const uint32_t*
 #define TF_GO(W_)                                                                                                 \
   moe_fused_kernel<GS, NM, EPI_UP, W_><<<g, W_ * 64, smem, stream>>>(x, x_stride, slots, wup, wdown, d, ni, desc, \
                                                                      counts, wts, xs_x, act, xs_act, y, out, done, \
-                                                                     arrive, status, limit, max_items, spins)
+                                                                     arrive, status, limit, max_items, spins, astride)
   switch (fused_waves(grid)) {
     case 16: TF_GO(16); break;
     case 8: TF_GO(8); break;
@@ -420,13 +424,13 @@ extern "C" int tf_moe_decode_experts(int gs, int swiglu, const uint16_t* x, int6
   hipStream_t s = as_stream(stream);
   if (gs == 64)
     return swiglu ? launch_fused<64, 2, 2>(x, x_stride, slots, up, down, d, ni, desc, counts, wts, xs_x, act, xs_act, y,
-                                           out, done, arrive, status, limit, max_items, s)
+                                           out, done, arrive, status, limit, max_items, arrive_stride(rows), s)
                   : launch_fused<64, 1, 1>(x, x_stride, slots, up, down, d, ni, desc, counts, wts, xs_x, act, xs_act, y,
-                                           out, done, arrive, status, limit, max_items, s);
+                                           out, done, arrive, status, limit, max_items, arrive_stride(rows), s);
   return swiglu ? launch_fused<32, 2, 2>(x, x_stride, slots, up, down, d, ni, desc, counts, wts, xs_x, act, xs_act, y,
-                                         out, done, arrive, status, limit, max_items, s)
+                                         out, done, arrive, status, limit, max_items, arrive_stride(rows), s)
                 : launch_fused<32, 1, 1>(x, x_stride, slots, up, down, d, ni, desc, counts, wts, xs_x, act, xs_act, y,
-                                         out, done, arrive, status, limit, max_items, s);
+                                         out, done, arrive, status, limit, max_items, arrive_stride(rows), s);
 }
 
 extern "C" int tf_moe_route_up(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared, int gs,
@@ -478,7 +482,8 @@ extern "C" int tf_moe_down_combine(int gs, const uint16_t* act, int rows, int sl
   hipStream_t s = as_stream(stream);
   const dim3 g((unsigned)grid);
 #define TF_GO(GS_, W_)                                                                                             \
-  down_combine_kernel<GS_, W_><<<g, W_ * 64, smem, s>>>(act, slots, down, d, ni, desc, wts, xs_act, y, out, arrive)
+  down_combine_kernel<GS_, W_><<<g, W_ * 64, smem, s>>>(act, slots, down, d, ni, desc, wts, xs_act, y, out, arrive, \
+                                                        arrive_stride(rows))
 #define TF_GS(GS_)                      \
   switch (fused_waves(grid + grid / 2)) {      \
     case 16: TF_GO(GS_, 16); break;     \

@@ -29,6 +29,11 @@ ROUTING_LAUNCH = os.environ.get("TENSORFOLD_AMD_ROUTING_LAUNCH", "0") == "1"
 # Item descriptors the routing launches leave for the decode expert kernels: rows of DESC_INTS int32, row 0 the
 # count; items of at most DESC_TILE pairs (TF_DESC_INTS / TF_DESC_TILE of the C header).
 DESC_INTS, DESC_TILE = 8, 2
+ARRIVE_STRIDE = 16   # ints between the arrival counters of two (token, 64 columns) cells with at most 64 rows, else 1
+
+
+def arrive_stride(rows: int) -> int:
+    return ARRIVE_STRIDE if rows <= 64 else 1
 DONE_STRIDE = 64     # ints between the arrival counters of two descriptors (the one-launch form): one a 256-byte block
 
 
@@ -79,7 +84,7 @@ class MoEBuffers:
         if self._fused is None:
             cfg, dev, pairs = self.cfg, self.device, self.rows * self.slots
             items = grouped.max_items(pairs, cfg.num_experts + int(self.shared), DESC_TILE)
-            cells = self.rows * (cfg.hidden_size // 64)
+            cells = max(min(self.rows, 64) * ARRIVE_STRIDE, self.rows) * (cfg.hidden_size // 64)
             self._fused = dict(
                 items=items * DONE_STRIDE,          # ints the descriptors' arrival counters take
                 desc=torch.zeros((1 + items, DESC_INTS), dtype=torch.int32, device=dev),
@@ -157,7 +162,7 @@ def decode(x: torch.Tensor, logits: torch.Tensor, ex: grouped.Experts, buf: MoEB
     plan = buf.plan
     plan.tile = grouped.TILE
     items = grouped.max_items(n * buf.slots, experts + int(buf.shared), DESC_TILE)
-    cells = n * (ex.dims // 64)
+    cells = n * (ex.dims // 64) * arrive_stride(n)
     ctr = f["counters"]
     if FUSED_DECODE:
         _lib.call("tf_moe_route_decode", _lib.ptr(logits), logits.stride(0), n, experts, top_k, int(buf.shared),
