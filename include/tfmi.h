@@ -192,6 +192,8 @@ int tf_moe_decode_experts(int gs, int swiglu, const uint16_t* x, int64_t x_strid
                           float* y, uint16_t* out, int32_t* done, int32_t* arrive, int32_t* status, float limit,
                           int max_items, tf_stream_t stream);
 
+#define TF_EXL3_COUNTER_STRIDE 16
+
 /* ---- EXL3 linear (exl3/linear.cpp:70-74, module tensorfold_exl3_linear_v3) ---------------------------------------- */
 
 /* xh[m, k] fp16 = fp16(((x * suh) @ H) / sqrt(128)) per block of 128; x is fp16, bf16 or fp32 (TF_* code).
@@ -199,7 +201,8 @@ int tf_moe_decode_experts(int gs, int swiglu, const uint16_t* x, int64_t x_strid
 int tf_exl3_rot_in(const void* x, int x_dtype, const uint16_t* suh, uint16_t* xh, int m, int k, tf_stream_t stream);
 /* y[m, n] = ((xh @ W_q) @ H / sqrt(128)) * svh + bias, 1 <= m <= 128.  T: trellis words, tile (kt, nt) at
  * kt*stride_k + (nt/8)*stride_nb + (nt%8)*4*k2 words; k2 = 2*bits; cb 0 3inst, 1 mcg, 2 mul1; sk K splits (Z fp32
- * [sk, m, n] and zeroed int32 counters [8 * n/128] needed when sk > 1; counters are left zero); wk waves a block.
+ * [sk, m, n] and zeroed int32 counters [8 * n/128 * TF_EXL3_COUNTER_STRIDE] needed when sk > 1 (each counter alone in
+ * 64 bytes); counters are left zero); wk waves a block.
  * Replaces exl3/linear.cpp:36-58 `linear`. */
 int tf_exl3_linear(const uint16_t* xh, const uint32_t* T, int64_t stride_k, int64_t stride_nb, const uint16_t* svh,
                    const uint16_t* bias, void* y, int y_dtype, float* Z, int32_t* counters, int m, int k, int n,

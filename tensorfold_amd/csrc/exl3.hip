@@ -93,7 +93,7 @@ __global__ void __launch_bounds__(WK * 64)
       __builtin_amdgcn_s_waitcnt(0);        // this wave's stores are acknowledged ...
       __syncthreads();                      // ... every wave's are ...
       if (threadIdx.x == 0)                 // ... then the block counts itself in
-        last = __hip_atomic_fetch_add(counters + pass * NB + nb, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == SK - 1;
+        last = __hip_atomic_fetch_add(counters + (size_t)(pass * NB + nb) * TF_EXL3_COUNTER_STRIDE, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == SK - 1;
       __syncthreads();
       if (last) {
         for (int r = wave; r < R; r += WK) {
@@ -117,7 +117,7 @@ __global__ void __launch_bounds__(WK * 64)
           }
           finish_row(sx, sy, lane, svh, bias, col0 + 2 * lane, y, y_dtype, at);
         }
-        if (threadIdx.x == 0) counters[pass * NB + nb] = 0;     // every block of the column has arrived
+        if (threadIdx.x == 0) counters[(size_t)(pass * NB + nb) * TF_EXL3_COUNTER_STRIDE] = 0;     // every block of the column has arrived
       }
     }
   }

@@ -16,6 +16,7 @@ from .. import _lib
 from . import format as fmt
 
 CODEBOOK_IDS = fmt.CODEBOOK_IDS
+COUNTER_STRIDE = 16       # ints between two K-split arrival counters (TF_EXL3_COUNTER_STRIDE): each alone in 64 bytes
 _DTYPES = {torch.float16: 0, torch.bfloat16: 1, torch.float32: 2}
 
 
@@ -120,7 +121,7 @@ class Exl3Linear:
         """Arrival counters of the K splits, zero between calls."""
 
         if self._counters is None:
-            self._counters = torch.zeros((8 * (self.n // 128),), dtype=torch.int32, device=self.words.device)
+            self._counters = torch.zeros((8 * (self.n // 128) * COUNTER_STRIDE,), dtype=torch.int32, device=self.words.device)
         return self._counters
 
     def __call__(self, x: torch.Tensor, out: torch.Tensor | None = None, out_dtype: torch.dtype | None = None,
