@@ -37,6 +37,20 @@ def test_ctypes_table_covers_the_header():
         assert len(args) == decl.count(",") + 1, name
 
 
+def test_host_constants_are_the_headers():
+    """The counter layouts the host allocates are the ones the kernels index: the header's defines and the Python
+    constants agree."""
+
+    from tensorfold_amd import moe
+
+    define = lambda name: int(re.search(r"^#define " + name + r" (\d+)", HEADER, flags=re.M).group(1))
+    assert define("TF_DESC_TILE") == moe.DESC_TILE
+    assert define("TF_DONE_STRIDE") == moe.DONE_STRIDE
+    assert define("TF_ARRIVE_STRIDE") == moe.ARRIVE_STRIDE
+    assert define("TF_EXL3_COUNTER_STRIDE") == linear.COUNTER_STRIDE
+    assert [moe.arrive_stride(r) for r in (1, 64, 65, 1024)] == [moe.ARRIVE_STRIDE, moe.ARRIVE_STRIDE, 1, 1]
+
+
 def test_no_gpu_means_a_loud_error_not_a_fallback():
     if torch.cuda.is_available():
         pytest.skip("a GPU is present")
