@@ -158,8 +158,8 @@ int tf_add_norm(const uint16_t* x, const void* delta, int delta_kind, const floa
  * expert on the other rows) and runs the up unit of tf_experts_run (epilogue relu^2, or SwiGLU when swiglu != 0): act bf16 [pairs, ni] and
  * its group sums xs_act fp32 [pairs, ni / gs]; it also zeroes `zero` (n_zero ints: the next launch's counters).  Same
  * bits as the separate calls.  logits may be NULL: pick and wts are then inputs (tf_moe_topk ran before, the better
- * order past about 2,048 logits, where reading the rows in every workgroup costs more than a launch) and only the
- * plan is made here.  No counterpart in the reference (moe.py:88-128 issues them one by one). */
+ * order past about 2,048 logits, where reading the rows in every workgroup costs more than a launch) and every
+ * workgroup finds its item from the picks.  No counterpart in the reference (moe.py:88-128 issues them one by one). */
 int tf_moe_route_up(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared, int gs, int swiglu,
                     const uint16_t* x, int64_t x_stride, const uint32_t* up, int d, int ni, int32_t* pick, float* wts,
                     int32_t* members, int32_t* items, int32_t* counts, int32_t* desc, uint16_t* act, float* xs_act,

@@ -232,7 +232,17 @@ __global__ void __launch_bounds__(WAVES * 64)
                                               NI, limit, nullptr, xs_act, lds, none);
     return;
   }
-  // the pairs are counted by expert as they are found (find_item's histogram, without its two barriers)
+  if (!L && !writer) {
+    // the picks are given: a workgroup a pair, its item from the picks alone
+    __shared__ int wavepairs[WAVES][2];
+    if (it >= P) return;
+    int e = 0, cnt = 0;
+    if (!pair_item_given(pick, P, E, it, wavepairs[wave], e, cnt)) return;
+    NoHook none;
+    expert_unit<GS, NM, EPI, WAVES, false, 0>(X, x_stride, slots, Wup, D / GS, NI / 32, e, cnt, wavepairs[wave], cb2, act,
+                                              NI, limit, nullptr, xs_act, lds, none);
+    return;
+  }
   for (int e = tid; e < E; e += threads) item.cnt[e] = 0;
   if (tid < 6) item.sel[tid] = tid == 0 ? -1 : 0;
   __syncthreads();
@@ -353,9 +363,9 @@ int launch_route_up(const float* logits, int64_t ldl, int rows, int experts, int
                     int* items, int* counts, int* desc, uint16_t* act, float* xs_act, float limit, int max_items,
                     int* zero, int n_zero, hipStream_t stream) {
   const int nb2 = (ni / 32 + 1) / 2;
-  // with logits and 2 to 64 rows the workgroups go a pair (route_up_kernel), else an item
+  // with the picks given, or logits of 2 to 64 rows, the workgroups go a pair (route_up_kernel), else an item
   const int64_t pairs = (int64_t)rows * (top_k + (shared ? 1 : 0));
-  const int64_t units = logits && rows > 1 && rows <= 64 ? pairs : max_items;
+  const int64_t units = !logits || (rows > 1 && rows <= 64) ? pairs : max_items;
   const int64_t grid = 1 + units * nb2;
   TF_REQUIRE(grid <= 0x7FFFFFFF, "moe: %lld workgroups exceed the grid limit", (long long)grid);
   const size_t floats = expert_lds_floats(NM, d / GS, false);

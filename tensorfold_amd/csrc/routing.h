@@ -471,5 +471,41 @@ __device__ __forceinline__ bool find_item(ItemLds& L, const int* pk, int P, int 
   return true;
 }
 
+// pair_item with the picks given (a top-k launch ran before): pair p's expert is pick[p], the expert's pairs are
+// the equal picks, in pair order, two an item.  Every wave works it out for itself from the picks alone (up to 1,024,
+// all requested at once), so there is no barrier and no LDS.  An id outside [0, E) joins no item.
+__device__ __forceinline__ bool pair_item_given(const int* __restrict__ pick, int P, int E, int p, int* wp, int& e_out,
+                                                int& cnt_out) {
+  const int lane = threadIdx.x & 63;
+  int v[PLAN_THREADS / 64];
+#pragma unroll
+  for (int i = 0; i < PLAN_THREADS / 64; ++i) v[i] = 64 * i + lane < P ? pick[64 * i + lane] : -1;
+  const int e = __builtin_amdgcn_readfirstlane(pick[p]);
+  if ((unsigned)e >= (unsigned)E) return false;
+  int before = 0, partner = -1;
+#pragma unroll
+  for (int i = 0; i < PLAN_THREADS / 64; ++i) {
+    const int q0 = 64 * i;
+    if (q0 >= P) break;
+    const unsigned long long m = __ballot(v[i] == e);
+    if (q0 + 64 <= p) {
+      before += __popcll(m);
+    } else if (q0 <= p) {
+      const int b = p - q0;
+      before += __popcll(m & ((1ull << b) - 1ull));
+      const unsigned long long after = b < 63 ? m >> (b + 1) : 0ull;
+      if (after) partner = p + 1 + __builtin_ctzll(after);
+    } else if (m && partner < 0) {
+      partner = q0 + __builtin_ctzll(m);
+    }
+  }
+  if (before & 1) return false;       // the second pair of an item
+  wp[0] = p;
+  wp[1] = partner >= 0 ? partner : p;
+  e_out = e;
+  cnt_out = partner >= 0 ? 2 : 1;
+  return true;
+}
+
 }  // namespace
 }  // namespace tf
