@@ -187,28 +187,32 @@ __global__ void __launch_bounds__(WAVES * 64)
   const int NB2 = (NI / 32 + 1) >> 1;
   const int u = blockIdx.x - 1, it = u / NB2, cb2 = u - it * NB2;
   if (R == 1 && !writer) {
-    // one row: every pick is its own item and the items go in expert order, so the item is the pick whose id
-    // ranks `it` among the picks; wave 0 finds it in registers
+    // one row: every pick is its own item, so unit `it` takes slot `it`, and needs the selection only up to it
     if (it >= slots) return;
     if (wave == 0) {
       int id;
-      float w;
-      if (L) topk_lane(L, NE, TOPK, shared, lane, id, w);
-      else id = lane < slots ? pick[lane] : -1;
-      const int mine = lane < slots && (unsigned)id < (unsigned)E ? id : 0x7FFFFFFF;
-      int rank = 0;
-      for (int i = 0; i < slots; ++i) {
-        const int other = __builtin_amdgcn_readlane(mine, i);
-        rank += other < mine || (other == mine && i < lane);
+      if (!L) {
+        id = pick[it];
+      } else if (shared && it == TOPK) {
+        id = NE;
+      } else if (NE <= 128) {
+        float v[2];
+        topk_load<2>(L, NE, lane, v);
+        id = topk_kth<2>(v, it, lane);
+      } else if (NE <= 512) {
+        float v[8];
+        topk_load<8>(L, NE, lane, v);
+        id = topk_kth<8>(v, it, lane);
+      } else {
+        float v[TOPK_VPL];
+        topk_load<TOPK_VPL>(L, NE, lane, v);
+        id = topk_kth<TOPK_VPL>(v, it, lane);
       }
-      const bool found = mine != 0x7FFFFFFF && rank == it;
-      if (found) {
-        item.sel[0] = mine;
+      if (lane == 0) {
+        item.sel[0] = (unsigned)id < (unsigned)E ? id : -1;
         item.sel[2] = 1;
-        item.pairs[0] = lane;
+        item.pairs[0] = it;
       }
-      const unsigned long long any = __ballot(found);
-      if (lane == 0 && !any) item.sel[0] = -1;
     }
     __syncthreads();
     if (item.sel[0] < 0) return;
