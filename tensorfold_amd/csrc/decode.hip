@@ -61,10 +61,11 @@ __global__ void __launch_bounds__(WAVES * 64)
   __shared__ int pairs[16];
   const int NB2 = (NB + 1) >> 1;
   const int it = blockIdx.x / NB2, cb2 = blockIdx.x - it * NB2;
-  if (it >= desc[0]) return;
+  // the descriptor's words are requested with the count, not after it (a row past the count exists and is ignored)
   const int* d = desc + (size_t)(1 + it) * DESC;
-  const int e = d[0], cnt = d[1];
-  if (threadIdx.x < DTILE) pairs[threadIdx.x] = d[4 + threadIdx.x];
+  const int n_items = desc[0], e = d[0], cnt = d[1], p0 = d[4], p1 = d[5];
+  if (it >= n_items) return;
+  if (threadIdx.x < DTILE) pairs[threadIdx.x] = threadIdx.x ? p1 : p0;
   __syncthreads();
   NoHook none;
   expert_unit<GS, NM, EPI, WAVES, true, 0>(X, x_stride, slots, W, KG, NB, e, cnt, pairs, cb2, out, N, limit, xs_in,

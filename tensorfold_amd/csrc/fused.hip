@@ -131,10 +131,11 @@ __global__ void __launch_bounds__(WAVES * 64)
   const bool up = b < U;
   const int it = up ? b / NB2u : (b - U) / NB2d;
   const int cb2 = up ? b - it * NB2u : (b - U) - it * NB2d;
-  if (it >= desc[0]) return;
+  // the descriptor's words are requested with the count, not after it (a row past the count exists and is ignored)
   const int* d = desc + (size_t)(1 + it) * DESC;
-  const int e = d[0], cnt = d[1];
-  if (tid < DTILE) pairs[tid] = d[4 + tid];
+  const int n_items = desc[0], e = d[0], cnt = d[1], p0 = d[4], p1 = d[5];
+  if (it >= n_items) return;
+  if (tid < DTILE) pairs[tid] = tid ? p1 : p0;
   __syncthreads();
   if (up) {
     NoHook none;
