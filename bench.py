@@ -26,9 +26,9 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes a launch of the expert kernels on this (seeded) workload, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
 # (KiB a dispatch; FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0, the factors a plain 256 MiB elementwise kernel gives).
 # Keyed by (projection, tokens); measured with --steps 20 --warmup 2 --copy-probe, independent of the step count.
-MEASURED_TRAFFIC = {("up", 8): (2 * 56797.7 + 219.8) * 1024, ("down", 8): (2 * 57638.4 + 609.0) * 1024,
-                    ("up", 4): (2 * 30411.2 + 110.1) * 1024, ("down", 4): (2 * 30761.4 + 304.5) * 1024,
-                    ("up", 1): (2 * 8335.0 + 27.5) * 1024, ("down", 1): (2 * 8406.3 + 76.1) * 1024}
+MEASURED_TRAFFIC = {("up", 8): (2 * 56818.7 + 225.8) * 1024, ("down", 8): (2 * 57634.3 + 609.0) * 1024,
+                    ("up", 4): (2 * 30405.4 + 113.1) * 1024, ("down", 4): (2 * 30762.0 + 304.5) * 1024,
+                    ("up", 1): (2 * 8327.7 + 28.4) * 1024, ("down", 1): (2 * 8404.8 + 76.1) * 1024}
 SHAPE = synthetic.C1
 LAYERS = 4          # 4 x 718 MB of expert tables
 POOL = 64           # distinct routing draws
