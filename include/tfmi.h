@@ -59,6 +59,18 @@ int tf_group_sums(const uint16_t* x, int64_t ldx, int m, int k, int gs, float* x
 int tf_qmm(const uint16_t* x, int64_t ldx, const float* xs, const uint32_t* weight, const uint16_t* scales,
            const uint16_t* biases, int64_t sb_stride, void* out, float* part, int m, int n, int k, int sk, int gs,
            int bm, int f32, int reduce, tf_stream_t stream);
+/* tf_qmm (reduce != 0) for callers that cannot allocate or pass a workspace: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  The K slices that tf_qmm keeps in `part` live in a fixed array
+ * inside the library's device image (TF_QMM_STATIC_FLOATS fp32 = 16 MiB, held by every GPU the library runs on
+ * until the process ends); sk * m * n beyond that is refused with a message.  Nothing is allocated or freed by the
+ * call.  Same kernels and bits as tf_qmm.  Every call on a GPU shares that GPU's array: calls that overlap on one
+ * GPU (two streams, two threads) race; calls on one stream are ordered.  Nothing in the array needs to start at
+ * zero (each slice is written in full before the reduce reads it).  No counterpart in the reference, whose `qmm`
+ * allocates `part` itself when none is given (kernels/qmm.cpp:40-45). */
+#define TF_QMM_STATIC_FLOATS (4u << 20)
+int tf_qmm_static(const uint16_t* x, int64_t ldx, const float* xs, const uint32_t* weight, const uint16_t* scales,
+                  const uint16_t* biases, int64_t sb_stride, void* out, int m, int n, int k, int sk, int gs, int bm,
+                  int f32, tf_stream_t stream);
 /* `count` (1 to 4) weights against one x in one launch (plus one reduce launch when any K is split and the rows are
  * many): the bits of tf_qmm on each.  The arrays are host arrays of `count` entries, read during the call: packed weights, transposed
  * scales and biases with their row strides, outputs, parts (fp32 [sks[i], m, ns[i]], may be NULL where sks[i] == 1),

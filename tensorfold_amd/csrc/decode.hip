@@ -19,6 +19,7 @@
 // P = fma(-128, xs, that).
 
 #include <cstdlib>
+#include <mutex>
 
 #include "gemv.h"
 #include "routing.h"
@@ -491,10 +492,10 @@ extern "C" int tf_group_sums(const uint16_t* x, int64_t ldx, int m, int k, int g
   return 0;
 }
 
-extern "C" int tf_qmm(const uint16_t* x, int64_t ldx, const float* xs, const uint32_t* weight, const uint16_t* scales,
+// tf_qmm and tf_qmm_static: the checks and launches of the decode-form matmul; `part` holds the K slices.
+static int qmm_launch(const uint16_t* x, int64_t ldx, const float* xs, const uint32_t* weight, const uint16_t* scales,
                       const uint16_t* biases, int64_t sb_stride, void* out, float* part, int m, int n, int k, int sk,
                       int gs, int bm, int f32, int reduce, tf_stream_t stream) {
-  clear_error();
   TF_REQUIRE(gs == 32 || gs == 64, "groups of 32 or 64");
   TF_REQUIRE(bm == 16 || bm == 32 || bm == 64, "row tile 16, 32 or 64");
   TF_REQUIRE(x && xs && weight && scales && biases && out && m >= 1 && n >= 1, "qmm: null pointer or empty shape");
@@ -545,6 +546,53 @@ extern "C" int tf_qmm(const uint16_t* x, int64_t ldx, const float* xs, const uin
     TF_LAUNCH_OK("tf_qmm reduce");
   }
   return 0;
+}
+
+extern "C" int tf_qmm(const uint16_t* x, int64_t ldx, const float* xs, const uint32_t* weight, const uint16_t* scales,
+                      const uint16_t* biases, int64_t sb_stride, void* out, float* part, int m, int n, int k, int sk,
+                      int gs, int bm, int f32, int reduce, tf_stream_t stream) {
+  clear_error();
+  return qmm_launch(x, ldx, xs, weight, scales, biases, sb_stride, out, part, m, n, k, sk, gs, bm, f32, reduce, stream);
+}
+
+// The K slices of tf_qmm_static: one array a GPU, part of the loaded code object, so no call ever allocates it.
+// Host code may not use the array's name as an address; it asks the runtime once a device for where that device
+// holds its copy and passes that pointer to the kernels like any other buffer.
+static __device__ __align__(256) float scratch[TF_QMM_STATIC_FLOATS];
+
+static float* static_part() {
+  constexpr int MAX_DEVICES = 64;
+  static float* where[MAX_DEVICES];
+  static std::mutex guard;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+    set_error("tf_qmm_static: no current HIP device (or its index is %d or more)", MAX_DEVICES);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(guard);
+  if (!where[dev]) {
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      set_error("tf_qmm_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+      return nullptr;
+    }
+    where[dev] = static_cast<float*>(p);
+  }
+  return where[dev];
+}
+
+extern "C" int tf_qmm_static(const uint16_t* x, int64_t ldx, const float* xs, const uint32_t* weight,
+                             const uint16_t* scales, const uint16_t* biases, int64_t sb_stride, void* out, int m, int n,
+                             int k, int sk, int gs, int bm, int f32, tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(m >= 1 && n >= 1 && sk >= 1, "qmm: null pointer or empty shape");
+  TF_REQUIRE(sk == 1 || (int64_t)sk * m * n <= (int64_t)TF_QMM_STATIC_FLOATS,
+             "tf_qmm_static: %d slices x %d rows x %d columns = %lld fp32 partial sums exceed the built-in %lld; use "
+             "tf_qmm with a part buffer", sk, m, n, (long long)sk * m * n, (long long)TF_QMM_STATIC_FLOATS);
+  float* part = nullptr;
+  if (sk > 1 && !(part = static_part())) return 1;
+  return qmm_launch(x, ldx, xs, weight, scales, biases, sb_stride, out, part, m, n, k, sk, gs, bm, f32, 1, stream);
 }
 
 extern "C" int tf_qmm_group(const uint16_t* x, int64_t ldx, const float* xs, int count, const uint32_t* const* weights,

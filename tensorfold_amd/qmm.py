@@ -145,6 +145,37 @@ def matmul(x: torch.Tensor, q: Q4, xs: torch.Tensor | None = None, *, sk: int | 
     return part.reshape(-1)[:sk * m * q.n].view(sk, m, q.n)
 
 
+STATIC_FLOATS = 4 << 20          # TF_QMM_STATIC_FLOATS of include/tfmi.h
+
+
+def matmul_static(x: torch.Tensor, q: Q4, xs: torch.Tensor, out: torch.Tensor, *, sk: int | None = None,
+                  f32: bool = False) -> torch.Tensor:
+    """``matmul`` into the caller's ``out`` with nothing allocated on the way: the K slices go to an array built into
+    the library (one a GPU, 16 MiB), so ``sk * M * n`` may not exceed ``STATIC_FLOATS``.  x must already have
+    16-byte aligned rows and ``xs`` its group sums.  Same bits as ``matmul``; calls that overlap on one GPU share
+    that array and race.  No counterpart in the reference (for callers that cannot allocate)."""
+
+    if x.dtype != torch.bfloat16 or x.dim() != 2 or x.shape[1] != q.k:
+        raise ValueError(f"matmul_static: x must be (M, {q.k}) bf16")
+    _lib.on_gpu(x, xs, out)
+    m = int(x.shape[0])
+    if x.stride(1) != 1 or x.data_ptr() % 16 or (m > 1 and x.stride(0) % 8):
+        raise ValueError("matmul_static: x rows must be contiguous and start on 16-byte boundaries (nothing is copied)")
+    sk = split_k(q.n, q.k, q.gs) if not sk else sk
+    if sk > 1 and sk * m * q.n > STATIC_FLOATS:
+        raise ValueError(f"matmul_static: {sk} x {m} x {q.n} partial sums exceed the built-in {STATIC_FLOATS}; "
+                         "use matmul with a part buffer")
+    if tuple(out.shape) != (m, q.n) or out.dtype != (torch.float32 if f32 else torch.bfloat16) \
+            or not out.is_contiguous() or out.device != x.device:
+        raise ValueError(f"matmul_static: out must be contiguous ({m}, {q.n}) {'fp32' if f32 else 'bf16'} on x's device")
+    if xs.dtype != torch.float32 or tuple(xs.shape) != (m, q.k // q.gs) or not xs.is_contiguous() \
+            or xs.device != x.device:
+        raise ValueError(f"matmul_static: xs must be contiguous fp32 ({m}, {q.k // q.gs}), the group sums of x")
+    _lib.call("tf_qmm_static", _lib.ptr(x), x.stride(0), _lib.ptr(xs), _lib.ptr(q.weight), _lib.ptr(q.scales),
+              _lib.ptr(q.biases), q.scales.stride(0), _lib.ptr(out), m, q.n, q.k, sk, q.gs, bucket(m), int(f32))
+    return out
+
+
 def matmul_group(x: torch.Tensor, qs: list[Q4], xs: torch.Tensor | None = None, *, f32: bool = False,
                  sks: list[int] | None = None, outs: list[torch.Tensor] | None = None,
                  parts: list[torch.Tensor | None] | None = None) -> list[torch.Tensor]:
