@@ -23,12 +23,6 @@ import torch
 from tensorfold_amd import _lib, experts, moe, synthetic
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes a launch of the expert kernels on this (seeded) workload, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
-# (KiB a dispatch; FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0, the factors a plain 256 MiB elementwise kernel gives).
-# Keyed by (projection, tokens); measured with --steps 20 --warmup 2 --copy-probe, independent of the step count.
-MEASURED_TRAFFIC = {("up", 8): (2 * 56818.7 + 225.8) * 1024, ("down", 8): (2 * 57634.3 + 609.0) * 1024,
-                    ("up", 4): (2 * 30405.4 + 113.1) * 1024, ("down", 4): (2 * 30762.0 + 304.5) * 1024,
-                    ("up", 1): (2 * 8327.7 + 28.4) * 1024, ("down", 1): (2 * 8404.8 + 76.1) * 1024}
 SHAPE = synthetic.C1
 LAYERS = 4          # 4 x 718 MB of expert tables
 POOL = 64           # distinct routing draws
@@ -234,7 +228,7 @@ def cpu_baseline(keep, tokens: int, dev: str) -> dict:
     upc, downc = cpu(up), cpu(down)
     native.moe_layer(b16(x), remap[picks], wts, None, upc, downc, s.gs)             # warm-up
     times = []
-    for _ in range(3):
+    for _ in range(5):
         t0 = time.perf_counter()
         out = native.moe_layer(b16(x), remap[picks], wts, None, upc, downc, s.gs)
         times.append(time.perf_counter() - t0)
@@ -252,8 +246,38 @@ def cpu_baseline(keep, tokens: int, dev: str) -> dict:
     ids_ok = bool(np.array_equal(buf.pick.cpu().numpy(), picks))
     med = float(np.median(times))
     return {"value": med / tokens * 1e6, "unit": "us/token", "cores": native.threads(), "kind": "port",
-            "sample": f"one layer pass, {tokens} tokens x top-{s.top_k} ({len(used)} experts), median of 3",
+            "sample": f"one layer pass, {tokens} tokens x top-{s.top_k} ({len(used)} experts), median of 5",
             "parity_rel_l2": rel, "parity_ids_exact": ids_ok}
+
+
+def other_configs() -> dict:
+    """Short legs of the benchmark's other configurations (bench_configs.py's functions): the dense projection (0),
+    the verify window (2), the prompt chunk on the matrix cores (3: chunk time and TFLOP/s) and the EXL3 MLP (4)."""
+
+    import bench_configs as bc
+
+    rnd = lambda v: round(v, 4) if isinstance(v, float) else v
+    out = {}
+    r = bc.c0()
+    out["c0"] = {"workload": r["config"],
+                 "rows": {str(m): {k: rnd(v) for k, v in d.items()} for m, d in r["rows"].items()},
+                 "prompt_form": {k: rnd(v) for k, v in r["prompt_form"].items()}}
+    torch.cuda.empty_cache()
+    r = bc.c2()
+    out["c2"] = {k: rnd(v) for k, v in r.items() if k != "config"} | {"workload": r["config"]}
+    torch.cuda.empty_cache()
+    r = bc.c3(tiles=((128, torch.float32),))
+    t = r["tiles"][128]
+    out["c3"] = {"workload": r["config"], "bound": "mfma", "chunk_us": rnd(t["chunk_us"]),
+                 "tokens_per_s": rnd(t["tokens_per_s"]), "tflops": rnd(t["tflops"]), "peak_tflops": bc.MFMA,
+                 "frac": rnd(t["frac"]), "flop": t["flop"], "route_us": rnd(t["route_us"]), "up_us": rnd(t["up_us"]),
+                 "down_us": rnd(t["down_us"]), "combine_us": rnd(t["combine_us"]), "items": t["items"]}
+    torch.cuda.empty_cache()
+    r = bc.c4()
+    out["c4"] = {"workload": r["config"], "bound": "hbm",
+                 "rows": {str(m): {k: rnd(v) for k, v in d.items()} for m, d in r["rows"].items()}}
+    torch.cuda.empty_cache()
+    return out
 
 
 def main() -> int:
@@ -263,6 +287,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--tokens", type=int, default=8, help="batch of the headline value (1, 4 and 8 are all reported)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the short legs of configurations 0, 2, 3 and 4 (the `configs` key of the line)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB in / 256 MiB out elementwise kernel three times: the known-size "
                          "dispatch that FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
@@ -276,6 +302,9 @@ def main() -> int:
     tables, keep = device_tables(SHAPE, LAYERS, dev)
     results = {t: run_batch(t, tables, args.steps, args.warmup, dev) for t in sorted({1, 4, 8, args.tokens})}
     head = results[args.tokens]
+    # HBM bytes a launch are counter readings (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE) of this same command, not
+    # something a timing run can see: the line carries null and the summary of those two runs is kept beside the
+    # kernel trace (profiles/expert_kernel_c1_decode_traffic.txt).
     traffic = None
     if moe.FUSED_DECODE:
         dom_us, dom_bytes = head["fused_kernel_us"], 2 * head["kernel_bytes"]
@@ -284,7 +313,6 @@ def main() -> int:
         which = "up" if head["up_kernel_us"] >= head["down_kernel_us"] else "down"
         dom_us, dom_bytes = head[f"{which}_kernel_us"], head["kernel_bytes"]
         dom = ("route_up_kernel (routing + up projection" if which == "up" else "down_combine_kernel (down projection + combine")
-        traffic = MEASURED_TRAFFIC.get((which, args.tokens))
     achieved = dom_bytes / dom_us * 1e-3
     line = {
         "metric": "moe_decode_layer_us_per_token", "value": head["us_per_token"], "unit": "us/token", "n_gpus": 1,
@@ -310,10 +338,14 @@ def main() -> int:
             torch.mul(a, 2.0, out=b)
         torch.cuda.synchronize()
         del a, b
+    del tables
+    torch.cuda.empty_cache()
     if not args.no_cpu:
-        del tables
-        torch.cuda.empty_cache()
         line["cpu_baseline"] = cpu_baseline(keep, args.tokens, dev)
+    del keep
+    torch.cuda.empty_cache()
+    if not args.no_configs:
+        line["configs"] = other_configs()
     print(json.dumps(line))
     return 0
 

@@ -138,7 +138,7 @@ def c2() -> dict:
             "down_gbs": uniq[0] * per_expert / 3 / down_us * 1e-3}
 
 
-def c3() -> dict:
+def c3(tiles=((64, torch.float32), (128, torch.float32), ("128_y_bf16", torch.bfloat16))) -> dict:
     s, rows = synthetic.C2, 4096
     gen = torch.Generator(device=DEV).manual_seed(3)
     ex = moe_tables(s, 1, gen)[0]
@@ -151,7 +151,7 @@ def c3() -> dict:
     out = {}
     # items of 64 and of 128 with fp32 pair outputs (this build's default), then items of 128 with the reference's
     # bf16 pair outputs (cuda/moe.py:99), which halve the traffic between the down projection and the combine
-    for tile, ydt in ((64, torch.float32), (128, torch.float32), ("128_y_bf16", torch.bfloat16)):
+    for tile, ydt in tiles:
         key, tile = tile, 128 if isinstance(tile, str) else tile
         plan = experts.Plan(rows, slots, s.experts + 1, DEV, prefill=True)
         act = torch.empty((rows * slots, s.width), dtype=torch.bfloat16, device=DEV)
