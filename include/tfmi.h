@@ -36,6 +36,9 @@ enum { TF_F16 = 0, TF_BF16 = 1, TF_F32 = 2 };
 const char* tf_last_error(void);
 /* ABI version of this header. */
 int tf_version(void);
+/* Digest of the sources and compiler flags the library was built from (16 hex digits), "unknown" when the build gave
+ * none.  The Python loader compares it with the sources beside it before it loads the file. */
+const char* tf_build_id(void);
 /* 0 when the current HIP device is gfx950; otherwise non-zero with a message naming the device.
  * Replaces build.py:20-32 `arch_flags` (refusal of a GPU the kernels were not built for). */
 int tf_check_device(void);
@@ -79,10 +82,22 @@ int tf_qmm_group(const uint16_t* x, int64_t ldx, const float* xs, int count, con
                  const uint16_t* const* scales, const uint16_t* const* biases, const int64_t* sb_strides,
                  void* const* outs, float* const* parts, const int* ns, const int* sks, int m, int k, int gs, int bm,
                  int f32, tf_stream_t stream);
-/* Prompt-form matmul on f16 MFMA: each weight rounded once (256 w to fp16; the reference rounds w to bf16), one
- * fp32 chain over K.  Replaces kernels/qmm.cpp:83-102 `qmm_prefill`. */
+/* The arithmetic of the prompt-form (MFMA) matmuls.
+ *   TF_ARITH_F16: operands in fp16 - each weight rounded once as fp16(256 w), activations converted to fp16 (exact for a
+ *     bf16 value between 2^-14 and 65504 in magnitude; larger ones are clamped to +-65504, smaller ones keep 2^-24
+ *     absolute).  Valid when every |scale| and |bias| of the table is below 255.9 (256 x must stay finite in fp16)
+ *     and the activations stay within +-65504.  An eighth of the reference's weight rounding error: the form that
+ *     holds 2e-3 relative L2 against dequant-then-matmul in fp32, and the fast one.
+ *   TF_ARITH_BF16: the reference's own arithmetic - w = bf16(fma(q, s, b)) (round to nearest even), bf16 activations
+ *     untouched, bf16 MFMA (kernels/qmm_prefill.cu:116-117, experts_prefill.cu:130-131).  bf16's range on both
+ *     operands; runs on the four-wave kernel at every size, about half the speed.
+ * The Python wrappers choose TF_ARITH_BF16 by themselves for a table whose scales or biases do not fit the fp16 form. */
+enum { TF_ARITH_F16 = 0, TF_ARITH_BF16 = 1 };
+
+/* Prompt-form matmul on MFMA: each weight rounded once (see TF_ARITH_*), one fp32 chain over K.
+ * Replaces kernels/qmm.cpp:83-102 `qmm_prefill`. */
 int tf_qmm_prefill(const uint16_t* x, int64_t ldx, const uint32_t* weight, const uint16_t* scales,
-                   const uint16_t* biases, void* out, int m, int n, int k, int gs, int f32, int tile,
+                   const uint16_t* biases, void* out, int m, int n, int k, int gs, int f32, int tile, int arith,
                    tf_stream_t stream);
 
 /* ---- routed experts (experts.cpp:77-82, module tensorfold_experts_v7) ---------------------------------------------- */
@@ -128,11 +143,11 @@ int tf_experts_run(int gs, int epi, const uint16_t* x, int64_t x_stride, int slo
 int tf_experts_run_desc(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg,
                         int nb, const int32_t* desc, const int32_t* counts, void* out, int n, float limit,
                         int64_t max_items, const float* xs, float* xs_out, tf_stream_t stream);
-/* Prompt form on f16 MFMA, each weight rounded once as in tf_qmm_prefill; epi 3: bf16 out.  `tile` is the plan's
- * item size (16, 64 or 128).  Replaces experts.cpp:50-55 `prefill`. */
+/* Prompt form on MFMA, each weight rounded once as in tf_qmm_prefill (arith: TF_ARITH_*); epi 3: bf16 out.  `tile` is
+ * the plan's item size (16, 64 or 128).  Replaces experts.cpp:50-55 `prefill`. */
 int tf_experts_prefill(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg,
                        int nb, const int32_t* items, const int32_t* counts, const int32_t* members, void* out, int n,
-                       float limit, int64_t max_items, int tile, tf_stream_t stream);
+                       float limit, int64_t max_items, int tile, int arith, tf_stream_t stream);
 
 /* ---- MoE glue (moe.py:23-151; Triton kernels in the reference) ------------------------------------------------------ */
 

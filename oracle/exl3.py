@@ -11,7 +11,10 @@ import numpy as np
 
 CODEBOOKS = ("3inst", "mcg", "mul1")
 CODEBOOK_IDS = {"3inst": 0, "mcg": 1, "mul1": 2}
-WIDTHS = (1, 1.5, 2, 2.5, 3, 3.5, 4, 5, 6, 7, 8)
+WIDTHS = (1, 1.5, 2, 2.5, 3, 3.5, 4, 5, 6, 7, 8)            # what checkpoints hold (x.5 with mul1 only)
+# every half-bit count from 2 to 16: the bitstream rule is the same for all of them, and the reference's routed-expert
+# kernels take any of them with any codebook (cuda/exl3/experts.py:15-16, decode.cuh:19-22)
+EVERY_WIDTH = tuple(k2 / 2 for k2 in range(2, 17))
 
 _tables: dict[str, np.ndarray] = {}
 
@@ -46,8 +49,8 @@ def codebook(name: str) -> np.ndarray:
 
 def check_width(bits: float) -> float:
     b = float(bits)
-    if b not in WIDTHS:
-        raise ValueError(f"EXL3 bits must be one of {WIDTHS}, got {bits}")
+    if b not in EVERY_WIDTH:
+        raise ValueError(f"EXL3 bits must be one of {EVERY_WIDTH}, got {bits}")
     return b
 
 

@@ -64,8 +64,9 @@ def affine_dequant(words, scales_bits, biases_bits, gs: int) -> np.ndarray:
     return out
 
 
-def affine_linear(x_bits, words, scales_bits, biases_bits, gs: int, *, prefill: bool = False) -> np.ndarray:
-    """fp32 [M, N]; x, scales, biases as bf16 bit patterns (uint16)."""
+def affine_linear(x_bits, words, scales_bits, biases_bits, gs: int, *, prefill: bool | int = False) -> np.ndarray:
+    """fp32 [M, N]; x, scales, biases as bf16 bit patterns (uint16).  ``prefill`` 1 (True): every weight rounded once as
+    this build's fp16 prompt form does; 2: as the reference's bf16 prompt form does; 0: not at all."""
 
     x_bits, words = _u16(x_bits), _u32(words)
     m, k = x_bits.shape

@@ -107,7 +107,9 @@ static void dequant_row(const uint32_t* row, const uint16_t* s, const uint16_t* 
     for (int c = g * gs; c < (g + 1) * gs; ++c) {
       const float prod = (float)code_at(row, c) * sv;
       const float v = prod + bv;
-      w[c] = prefill ? (float)(half_to_double(double_to_half((double)v * 256.0)) / 256.0) : v;
+      /* prefill 1: this build's fp16 form; 2: the reference's bf16(fmaf(q, s, b)) (cuda/kernels/qmm_prefill.cu:116-117) */
+      if (prefill == 2) w[c] = round_bf16(fmaf((float)code_at(row, c), sv, bv));
+      else w[c] = prefill ? (float)(half_to_double(double_to_half((double)v * 256.0)) / 256.0) : v;
     }
   }
 }

@@ -8,7 +8,6 @@ time, in the tree, for the one target this package supports, and a GPU that is n
 from __future__ import annotations
 
 import ctypes
-import os
 import shutil
 import subprocess
 import sys
@@ -33,12 +32,34 @@ def hipcc() -> str | None:
     return shutil.which("hipcc") or (str(Path("/opt/rocm/bin/hipcc")) if Path("/opt/rocm/bin/hipcc").exists() else None)
 
 
-def stale() -> bool:
+def source_id() -> str:
+    """16 hex digits over every file the library is built from and the compiler flags."""
+
+    import hashlib
+
+    h = hashlib.sha256(" ".join(FLAGS).encode())
+    for path in [CSRC / s for s in SOURCES] + sorted(CSRC.glob("*.h")) + [HERE.parent / "include" / "tfmi.h"]:
+        h.update(path.name.encode())
+        h.update(path.read_bytes())
+    return h.hexdigest()[:16]
+
+
+def built_id() -> str | None:
+    """The digest the library file carries (``tf_build_id``), read from the file without loading it."""
+
     if not LIB.exists():
-        return True
-    built = LIB.stat().st_mtime
-    deps = [CSRC / s for s in SOURCES] + list(CSRC.glob("*.h")) + [HERE.parent / "include" / "tfmi.h"]
-    return any(d.stat().st_mtime > built for d in deps)
+        return None
+    blob, mark = LIB.read_bytes(), b"TFMI_BUILD_ID="
+    at = blob.find(mark)
+    return None if at < 0 else blob[at + len(mark):at + len(mark) + 16].decode(errors="replace")
+
+
+def stale() -> bool:
+    """Whether the library is missing or was built from other sources than the ones beside it."""
+
+    if LIB.exists() and not (CSRC / SOURCES[0]).exists():
+        return False                       # a library shipped without its sources is taken as it is
+    return built_id() != source_id()
 
 
 def compile(verbose: bool = False) -> Path:
@@ -61,7 +82,7 @@ def compile(verbose: bool = False) -> Path:
             raise RuntimeError(f"tensorfold-amd: hipcc failed:\n{err}")
         return err
 
-    compile_flags = [f for f in FLAGS if f != "-shared"]
+    compile_flags = [f for f in FLAGS if f != "-shared"] + [f'-DTF_BUILD_ID="{source_id()}"']
     with tempfile.TemporaryDirectory(prefix="tfmi-build-") as tmp:
         objects = [str(Path(tmp) / (Path(s).stem + ".o")) for s in SOURCES]
         with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
@@ -77,14 +98,13 @@ def compile(verbose: bool = False) -> Path:
 
 @lru_cache(maxsize=1)
 def load() -> ctypes.CDLL:
-    """The library, built first if it is missing and hipcc is here; a missing library never falls back to anything."""
+    """The library, built first if it is missing or out of date (its digest differs from the sources') and hipcc is
+    here; a missing or stale library never falls back to anything."""
 
-    override = os.environ.get("TENSORFOLD_AMD_LIB")        # a library built elsewhere (same ABI)
-    if override:
-        return ctypes.CDLL(override)
-    if not LIB.exists():
+    if stale():
         if hipcc() is None:
-            raise RuntimeError(f"tensorfold-amd: {LIB} is missing and there is no hipcc to build it; "
+            what = "is missing" if not LIB.exists() else "was built from other sources than the ones beside it"
+            raise RuntimeError(f"tensorfold-amd: {LIB} {what} and there is no hipcc to build it; "
                                "run `python -c 'import __graft_entry__ as g; g.build()'` where ROCm is installed")
         compile()
     return ctypes.CDLL(str(LIB))

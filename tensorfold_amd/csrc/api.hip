@@ -23,7 +23,17 @@ void clear_error() { g_error.clear(); }
 
 extern "C" const char* tf_last_error(void) { return tf::g_error.c_str(); }
 
-extern "C" int tf_version(void) { return 1; }
+extern "C" int tf_version(void) { return 2; }
+
+// A digest of the sources and flags this library was built from, given by the build (tensorfold_amd/build.py); the
+// loader compares it with the sources it sees and rebuilds or refuses a library that is out of date.
+#ifndef TF_BUILD_ID
+#define TF_BUILD_ID "unknown"
+#endif
+extern "C" const char* tf_build_id(void) {
+  static const char id[] = "TFMI_BUILD_ID=" TF_BUILD_ID;
+  return id + sizeof("TFMI_BUILD_ID=") - 1;
+}
 
 extern "C" int tf_check_device(void) {
   tf::clear_error();

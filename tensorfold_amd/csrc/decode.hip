@@ -371,14 +371,7 @@ constexpr int FAT_ROWS = 8;          // rows up to which tf_qmm runs the one-lau
 
 // Waves a workgroup of the expert GEMV: few workgroups (a small batch) spread each one's K over 16 waves, many
 // workgroups keep 4 longer-running waves each so that more of them are resident.  Scheduling only: bits do not move.
-int expert_waves(int64_t grid) {
-  static const int forced = [] {
-    const char* v = getenv("TENSORFOLD_AMD_EXPERT_WAVES");
-    return v ? atoi(v) : 0;
-  }();
-  if (forced == 4 || forced == 8 || forced == 16) return forced;
-  return grid < 384 ? 16 : grid < 768 ? 8 : 4;
-}
+int expert_waves(int64_t grid) { return grid < 384 ? 16 : grid < 768 ? 8 : 4; }
 
 template <int GS, int NM, int EPI, bool XSG>
 int launch_experts(const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg, int nb, const int* items,

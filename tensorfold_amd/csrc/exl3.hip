@@ -372,7 +372,7 @@ extern "C" int tf_exl3_unpack(const uint32_t* T, uint16_t* W, int k, int n, int6
     TF_LAUNCH_OK("tf_exl3_unpack");                                                  \
     return 0;                                                                        \
   }
-  TF_EXL3_ALL(TF_LAUNCH)
+  TF_EXL3_EVERY(TF_LAUNCH)
 #undef TF_LAUNCH
   set_error("unsupported EXL3 width/codebook: K2=%d codebook=%d", k2, cb);
   return 1;

@@ -266,6 +266,11 @@ __device__ __forceinline__ void wave_block(const uint16_t* xr, const uint32_t* t
 // every width ExLlamaV3 writes: k2 = 2 * bits; half-integer widths exist with the mul1 codebook only
 #define TF_EXL3_WIDTHS(X, CB) X(2, CB) X(4, CB) X(6, CB) X(8, CB) X(10, CB) X(12, CB) X(14, CB) X(16, CB)
 #define TF_EXL3_ALL(X) TF_EXL3_WIDTHS(X, 0) TF_EXL3_WIDTHS(X, 1) TF_EXL3_WIDTHS(X, 2) X(3, 2) X(5, 2) X(7, 2)
+// every half-bit count from 2 to 16 with every codebook: what the routed experts and the plain decode accept
+// (reference: cuda/exl3/experts.py:15-16, experts_grouped.cuh:184-187)
+#define TF_EXL3_ODD(X, CB) X(3, CB) X(5, CB) X(7, CB) X(9, CB) X(11, CB) X(13, CB) X(15, CB)
+#define TF_EXL3_EVERY(X) \
+  TF_EXL3_WIDTHS(X, 0) TF_EXL3_ODD(X, 0) TF_EXL3_WIDTHS(X, 1) TF_EXL3_ODD(X, 1) TF_EXL3_WIDTHS(X, 2) TF_EXL3_ODD(X, 2)
 
 }  // namespace
 }  // namespace tf

@@ -101,13 +101,8 @@ __global__ void __launch_bounds__(XWK * 64) grouped_kernel(const GroupedArgs g) 
   case K2_:          \
     grouped_body<K2_, CB>(g, T, xh, first, cnt, mat, red); \
     break;
-    TF_CASE(2) TF_CASE(4) TF_CASE(6) TF_CASE(8) TF_CASE(10) TF_CASE(12) TF_CASE(14) TF_CASE(16)
-#undef TF_CASE
-#define TF_CASE(K2_)                                                                  \
-  case K2_:                                                                           \
-    if constexpr (CB == 2) grouped_body<K2_, CB>(g, T, xh, first, cnt, mat, red);     \
-    break;
-    TF_CASE(3) TF_CASE(5) TF_CASE(7)
+    TF_CASE(2) TF_CASE(3) TF_CASE(4) TF_CASE(5) TF_CASE(6) TF_CASE(7) TF_CASE(8) TF_CASE(9) TF_CASE(10) TF_CASE(11)
+    TF_CASE(12) TF_CASE(13) TF_CASE(14) TF_CASE(15) TF_CASE(16)
 #undef TF_CASE
     default: break;                                         // widths are checked on the host
   }

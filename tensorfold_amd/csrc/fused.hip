@@ -345,14 +345,15 @@ __global__ void __launch_bounds__(WAVES * 64)
         d[3] = 0;
       }
     }
-    for (int p = tid; p < P; p += threads) {
-      const int e = pk[p];
-      if (e < 0) continue;
-      int rank = 0;
-      for (int q = 0; q < p; ++q) rank += pk[q] == e;
-      members[off[e] + rank] = p;
-      const int j = rank / DTILE, row = DTILE * (j + 1) <= item.cnt[e] ? dtoff[e] + j : F + shoff[e];
-      desc[(size_t)(1 + row) * DESC + 4 + rank % DTILE] = p;
+    // a wave an expert that has pairs: its members in pair order, and their places in its descriptors
+    for (int e = wave; e < E; e += WAVES) {
+      const int c = item.cnt[e];
+      if (!c) continue;
+      expert_pairs(pk, P, e, c, lane, [&](int rank, int p) {
+        members[off[e] + rank] = p;
+        const int j = rank / DTILE, row = DTILE * (j + 1) <= c ? dtoff[e] + j : F + shoff[e];
+        desc[(size_t)(1 + row) * DESC + 4 + rank % DTILE] = p;
+      });
     }
     return;
   }

@@ -70,6 +70,40 @@ __device__ __forceinline__ f16x8_t dequant8h(uint32_t w, uint32_t sb) {
   return r;
 }
 
+// ---- the reference's own prompt arithmetic (AR = 1): bf16 operands, w = bf16(fma(q, s, b)) ------------------------------
+//
+// cuda/kernels/qmm_prefill.cu:116-117 and cuda/experts_prefill.cu:130-131 round every dequantized weight to bf16 and
+// run a bf16 mma.  That form has bf16's range on both operands (no clamp at 65504, any scale or bias), at twice the
+// dequantization work and eight times the rounding error of the fp16 form above; it is what callers get when a
+// table's scales or biases do not fit fp16 after the 2^8 scaling, or when they ask for it.
+
+// eight consecutive bf16 inputs in the operand order (0, 4, 1, 5, 2, 6, 3, 7), unchanged
+__device__ __forceinline__ uint4 stage8_bf16(uint4 v) {
+  return make_uint4(__builtin_amdgcn_perm(v.z, v.x, 0x05040100u), __builtin_amdgcn_perm(v.z, v.x, 0x07060302u),
+                    __builtin_amdgcn_perm(v.w, v.y, 0x05040100u), __builtin_amdgcn_perm(v.w, v.y, 0x07060302u));
+}
+
+__device__ __forceinline__ uint32_t pack_bf16_rn(float lo, float hi) {
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf2;
+  bf2 r;
+  r[0] = (__bf16)lo;
+  r[1] = (__bf16)hi;
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+// one packed word -> the B operand in the same input order, each bf16(fma(q, s, b)) with s and b the stored bf16
+// values: round to nearest even, as the reference's __float2bfloat16_rn
+__device__ __forceinline__ bf16x8_t dequant8b(uint32_t w, uint32_t sb) {
+  const float s = bf16_lo(sb), b = bf16_hi(sb);
+  const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
+  auto q = [](uint32_t v, int byte) { return (float)((v >> (8 * byte)) & 0xFFu); };
+  const u32x4_t r = {pack_bf16_rn(fmaf(q(lo, 0), s, b), fmaf(q(lo, 1), s, b)),
+                     pack_bf16_rn(fmaf(q(lo, 2), s, b), fmaf(q(lo, 3), s, b)),
+                     pack_bf16_rn(fmaf(q(hi, 0), s, b), fmaf(q(hi, 1), s, b)),
+                     pack_bf16_rn(fmaf(q(hi, 2), s, b), fmaf(q(hi, 3), s, b))};
+  return __builtin_bit_cast(bf16x8_t, r);
+}
+
 // EPI 0: fp32; 1: bf16 relu(bf16 a)^2; 2: bf16 SwiGLU(matrix 0, matrix 1); 3: bf16
 template <int EPI>
 __device__ __forceinline__ void store_out(void* out, size_t at, float a, float u, float limit) {
@@ -83,7 +117,7 @@ __device__ __forceinline__ void store_out(void* out, size_t at, float a, float u
 // packed word and its column's scale and bias.
 //   word(g, m, i, t): group g, matrix m, chunk i (32 inputs) of the group, column tile t (16 columns) of the wave
 //   sb(g, m, t): that column's stored (scale | bias << 16) pair of group g
-template <int GS, int NM, int EPI, int RT, class WSRC>
+template <int GS, int NM, int EPI, int RT, int AR, class WSRC>
 __device__ __forceinline__ void mfma_body(const uint16_t* __restrict__ X, int64_t x_stride, int K, const WSRC& ws,
                                           const int* src_rows, int cnt, void* out, int N, int col0, int wave_cols_ok,
                                           const int* dst_rows, float limit, unsigned char* smem) {
@@ -119,7 +153,8 @@ __device__ __forceinline__ void mfma_body(const uint16_t* __restrict__ X, int64_
   auto store_a = [&](int buf, const uint4 (&v)[PPT]) {
 #pragma unroll
     for (int j = 0; j < PPT; ++j)
-      if (adst[j] >= 0) *reinterpret_cast<uint4*>(smem + buf * (ROWS * AROW) + adst[j]) = stage8(v[j]);
+      if (adst[j] >= 0)
+        *reinterpret_cast<uint4*>(smem + buf * (ROWS * AROW) + adst[j]) = AR ? stage8_bf16(v[j]) : stage8(v[j]);
   };
 
   uint32_t wcur[NM][CPS][2], wnxt[NM][CPS][2];
@@ -166,23 +201,30 @@ __device__ __forceinline__ void mfma_body(const uint16_t* __restrict__ X, int64_
 #pragma unroll
     for (int i = 0; i < CPS; ++i) {
       if (step * KSTEP + 32 * i >= K) break;
-      f16x8_t bfrag[NM][2];
+      u32x4_t bfrag[NM][2];
 #pragma unroll
       for (int m = 0; m < NM; ++m)
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
           const int gi = (32 * i) / GS;
-          bfrag[m][t] = dequant8h(wcur[m][i][t], sb_half2(scur[m][gi][t]));
+          if constexpr (AR) bfrag[m][t] = __builtin_bit_cast(u32x4_t, dequant8b(wcur[m][i][t], scur[m][gi][t]));
+          else bfrag[m][t] = __builtin_bit_cast(u32x4_t, dequant8h(wcur[m][i][t], sb_half2(scur[m][gi][t])));
         }
 #pragma unroll
       for (int r = 0; r < RT; ++r) {
         if (r >= nt) break;
-        const f16x8_t a = *reinterpret_cast<const f16x8_t*>(abuf + (16 * r + c) * AROW + i * 64 + kq * 16);
+        const u32x4_t a = *reinterpret_cast<const u32x4_t*>(abuf + (16 * r + c) * AROW + i * 64 + kq * 16);
 #pragma unroll
         for (int m = 0; m < NM; ++m)
 #pragma unroll
-          for (int t = 0; t < 2; ++t)
-            acc[m][r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bfrag[m][t], acc[m][r][t], 0, 0, 0);
+          for (int t = 0; t < 2; ++t) {
+            if constexpr (AR)
+              acc[m][r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                  __builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, bfrag[m][t]), acc[m][r][t], 0, 0, 0);
+            else
+              acc[m][r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                  __builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, bfrag[m][t]), acc[m][r][t], 0, 0, 0);
+          }
       }
     }
     if (more) {
@@ -215,7 +257,8 @@ __device__ __forceinline__ void mfma_body(const uint16_t* __restrict__ X, int64_
       for (int t = 0; t < 2; ++t) {
         const int col = col0 + 16 * t + c;
         if (col < N)
-          store_out<EPI>(out, base + col, acc[0][r][t][i] * WUNSCALE, acc[NM - 1][r][t][i] * WUNSCALE, limit);
+          store_out<EPI>(out, base + col, acc[0][r][t][i] * (AR ? 1.f : WUNSCALE),
+                         acc[NM - 1][r][t][i] * (AR ? 1.f : WUNSCALE), limit);
       }
     }
   }
@@ -235,7 +278,7 @@ struct ExpertWords {
   }
 };
 
-template <int GS, int NM, int EPI, int RT>
+template <int GS, int NM, int EPI, int RT, int AR>
 __global__ void __launch_bounds__(256)
     experts_prefill_kernel(const uint16_t* __restrict__ X, int64_t x_stride, int slots, const uint32_t* __restrict__ W,
                            int KG, int NB, const int* __restrict__ items, const int* __restrict__ counts,
@@ -259,7 +302,7 @@ __global__ void __launch_bounds__(256)
   const uint32_t* blk = W + (((size_t)e * NB + (ok ? nb : NB - 1)) * KG) * (size_t)(NM * block_words(GS));
   ws.base = blk + c * 4 + kq;
   ws.sbase = blk + 32 * GS / 8 + c;
-  mfma_body<GS, NM, EPI, RT>(X, x_stride, KG * GS, ws, src_rows, cnt, out, N, nb * 32, ok, dst_rows, limit, smem);
+  mfma_body<GS, NM, EPI, RT, AR>(X, x_stride, KG * GS, ws, src_rows, cnt, out, N, nb * 32, ok, dst_rows, limit, smem);
 }
 
 // ---- routed experts, big items ---------------------------------------------------------------------------------------
@@ -552,7 +595,7 @@ struct LaneWords {
   }
 };
 
-template <int GS, int EPI, int RT>
+template <int GS, int EPI, int RT, int AR>
 __global__ void __launch_bounds__(256)
     qmm_prefill_kernel(const uint16_t* __restrict__ X, int64_t ldx, const uint32_t* __restrict__ W,
                        const uint16_t* __restrict__ S, const uint16_t* __restrict__ B, void* __restrict__ out, int M,
@@ -574,7 +617,7 @@ __global__ void __launch_bounds__(256)
   ws.B = B + (ok ? col0 : 0) + c;
   ws.stride = npad;
   ws.KG = KG;
-  mfma_body<GS, 1, EPI, RT>(X, ldx, KG * GS, ws, rows, cnt, out, N, col0, ok, rows, 0.f, smem);
+  mfma_body<GS, 1, EPI, RT, AR>(X, ldx, KG * GS, ws, rows, cnt, out, N, col0, ok, rows, 0.f, smem);
 }
 
 template <int RT>
@@ -583,24 +626,27 @@ constexpr size_t stage_bytes() {
 }
 
 template <int GS, int NM, int EPI>
-int launch_experts_prefill(int tile, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg, int nb,
-                           const int* items, const int* counts, const int* members, void* out, int n, float limit,
-                           int64_t max_items, hipStream_t s) {
+int launch_experts_prefill(int tile, int arith, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w,
+                           int kg, int nb, const int* items, const int* counts, const int* members, void* out, int n,
+                           float limit, int64_t max_items, hipStream_t s) {
   const int64_t grid = max_items * ((nb + 3) / 4);
   if (grid < 1) return 0;
   TF_REQUIRE(grid <= 0x7FFFFFFF, "experts: %lld workgroups exceed the grid limit", (long long)grid);
   const dim3 g((unsigned)grid), b(256);
-  if (tile == 16) {
-    experts_prefill_kernel<GS, NM, EPI, 1><<<g, b, stage_bytes<1>(), s>>>(x, x_stride, slots, w, kg, nb, items, counts,
-                                                                         members, out, n, limit);
+#define TF_SMALL(RT_, AR_)                                                                                              \
+  experts_prefill_kernel<GS, NM, EPI, RT_, AR_><<<g, b, stage_bytes<RT_>(), s>>>(x, x_stride, slots, w, kg, nb, items, \
+                                                                               counts, members, out, n, limit)
+  if (arith) {
+    // the bf16 form runs on the four-wave kernel at every item size
+    if (tile == 16) TF_SMALL(1, 1);
+    else if (tile == 64) TF_SMALL(4, 1);
+    else TF_SMALL(8, 1);
+  } else if (tile == 16) {
+    TF_SMALL(1, 0);
   } else if ((kg * GS) % KSTEP) {
     // a K that is not whole steps of 64 (odd group counts at g32): the small kernel's tail handling
-    if (tile == 64)
-      experts_prefill_kernel<GS, NM, EPI, 4><<<g, b, stage_bytes<4>(), s>>>(x, x_stride, slots, w, kg, nb, items,
-                                                                           counts, members, out, n, limit);
-    else
-      experts_prefill_kernel<GS, NM, EPI, 8><<<g, b, stage_bytes<8>(), s>>>(x, x_stride, slots, w, kg, nb, items,
-                                                                           counts, members, out, n, limit);
+    if (tile == 64) TF_SMALL(4, 0);
+    else TF_SMALL(8, 0);
   } else {
     constexpr int NBW = big_blocks(NM);
     const int64_t big = max_items * ((nb + NBW - 1) / NBW);
@@ -608,31 +654,36 @@ int launch_experts_prefill(int tile, const uint16_t* x, int64_t x_stride, int sl
     experts_prefill_big_kernel<GS, NM, EPI><<<dim3((unsigned)big), BIG_THREADS, 2 * BIG_ROWS * AROW, s>>>(
         x, x_stride, slots, w, kg, nb, items, counts, members, out, n, limit);
   }
+#undef TF_SMALL
   TF_LAUNCH_OK("tf_experts_prefill");
   return 0;
 }
 
 template <int GS, int EPI>
-int launch_qmm_prefill(const uint16_t* x, int64_t ldx, const uint32_t* w, const uint16_t* s, const uint16_t* b,
-                       void* out, int m, int n, int kg, hipStream_t st) {
+int launch_qmm_prefill(int arith, const uint16_t* x, int64_t ldx, const uint32_t* w, const uint16_t* s,
+                       const uint16_t* b, void* out, int m, int n, int kg, hipStream_t st) {
   const int npad = (n + 127) / 128 * 128;
   const int ct = (n + 127) / 128;
-  if (m <= 16) {
-    qmm_prefill_kernel<GS, EPI, 1><<<(unsigned)(((m + 15) / 16) * ct), 256, stage_bytes<1>(), st>>>(x, ldx, w, s, b, out,
-                                                                                                   m, n, kg, npad);
+#define TF_SMALL(RT_, AR_)                                                                                       \
+  qmm_prefill_kernel<GS, EPI, RT_, AR_><<<(unsigned)(((m + 16 * RT_ - 1) / (16 * RT_)) * ct), 256, stage_bytes<RT_>(), \
+                                          st>>>(x, ldx, w, s, b, out, m, n, kg, npad)
+  TF_REQUIRE((int64_t)((m + 15) / 16) * ct <= 0x7FFFFFFF, "qmm_prefill: grid too large");
+  if (arith) {
+    if (m <= 16) TF_SMALL(1, 1);
+    else if (m <= 64) TF_SMALL(4, 1);
+    else TF_SMALL(8, 1);
+  } else if (m <= 16) {
+    TF_SMALL(1, 0);
   } else if (m <= 64) {
-    qmm_prefill_kernel<GS, EPI, 4><<<(unsigned)(((m + 63) / 64) * ct), 256, stage_bytes<4>(), st>>>(x, ldx, w, s, b, out,
-                                                                                                   m, n, kg, npad);
+    TF_SMALL(4, 0);
   } else if ((kg * GS) % KSTEP == 0 && (int64_t)npad * kg * GS / 2 < (1ll << 32)) {
     const int64_t grid = (int64_t)((m + BIG_ROWS - 1) / BIG_ROWS) * ((n + 511) / 512);
-    TF_REQUIRE(grid <= 0x7FFFFFFF, "qmm_prefill: grid too large");
     qmm_prefill_big_kernel<GS, EPI><<<(unsigned)grid, BIG_THREADS, 2 * BIG_ROWS * AROW, st>>>(x, ldx, w, s, b, out, m, n,
                                                                                             kg, npad);
   } else {
-    const int64_t grid = (int64_t)((m + 127) / 128) * ct;
-    TF_REQUIRE(grid <= 0x7FFFFFFF, "qmm_prefill: grid too large");
-    qmm_prefill_kernel<GS, EPI, 8><<<(unsigned)grid, 256, stage_bytes<8>(), st>>>(x, ldx, w, s, b, out, m, n, kg, npad);
+    TF_SMALL(8, 0);
   }
+#undef TF_SMALL
   TF_LAUNCH_OK("tf_qmm_prefill");
   return 0;
 }
@@ -644,8 +695,10 @@ using namespace tf;
 
 extern "C" int tf_experts_prefill(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w,
                                   int kg, int nb, const int32_t* items, const int32_t* counts, const int32_t* members,
-                                  void* out, int n, float limit, int64_t max_items, int tile, tf_stream_t stream) {
+                                  void* out, int n, float limit, int64_t max_items, int tile, int arith,
+                                  tf_stream_t stream) {
   clear_error();
+  TF_REQUIRE(arith == TF_ARITH_F16 || arith == TF_ARITH_BF16, "prefill arithmetic %d: TF_ARITH_F16 or TF_ARITH_BF16", arith);
   TF_REQUIRE(gs == 32 || gs == 64, "experts: groups of 32 or 64 inputs, not %d", gs);
   TF_REQUIRE(x && w && items && counts && members && out, "experts: null pointer argument");
   TF_REQUIRE(kg >= 1 && nb >= 1 && n == nb * 32, "experts: n (%d) must be the column blocks (%d) times 32", n, nb);
@@ -655,7 +708,7 @@ extern "C" int tf_experts_prefill(int gs, int epi, const uint16_t* x, int64_t x_
   hipStream_t s = as_stream(stream);
 #define TF_PRE(GS_, NM_, EPI_) \
   if (gs == GS_ && epi == EPI_) \
-    return launch_experts_prefill<GS_, NM_, EPI_>(tile, x, x_stride, slots, w, kg, nb, items, counts, members, out, n, limit, max_items, s);
+    return launch_experts_prefill<GS_, NM_, EPI_>(tile, arith, x, x_stride, slots, w, kg, nb, items, counts, members, out, n, limit, max_items, s);
   TF_PRE(32, 1, 0) TF_PRE(32, 1, 1) TF_PRE(32, 1, 3) TF_PRE(32, 2, 2)
   TF_PRE(64, 1, 0) TF_PRE(64, 1, 1) TF_PRE(64, 1, 3) TF_PRE(64, 2, 2)
 #undef TF_PRE
@@ -665,8 +718,9 @@ extern "C" int tf_experts_prefill(int gs, int epi, const uint16_t* x, int64_t x_
 
 extern "C" int tf_qmm_prefill(const uint16_t* x, int64_t ldx, const uint32_t* weight, const uint16_t* scales,
                               const uint16_t* biases, void* out, int m, int n, int k, int gs, int f32, int tile,
-                              tf_stream_t stream) {
+                              int arith, tf_stream_t stream) {
   clear_error();
+  TF_REQUIRE(arith == TF_ARITH_F16 || arith == TF_ARITH_BF16, "prefill arithmetic %d: TF_ARITH_F16 or TF_ARITH_BF16", arith);
   TF_REQUIRE(gs == 32 || gs == 64, "groups of 32 or 64");
   TF_REQUIRE(tile >= 0 && tile <= 11, "tile 0-11");
   TF_REQUIRE(x && weight && scales && biases && out && m >= 1 && n >= 1, "qmm_prefill: null pointer or empty shape");
@@ -674,8 +728,8 @@ extern "C" int tf_qmm_prefill(const uint16_t* x, int64_t ldx, const uint32_t* we
   TF_REQUIRE(k >= gs && k % gs == 0, "K splits into whole groups");
   hipStream_t s = as_stream(stream);
   const int kg = k / gs;
-  if (gs == 64) return f32 ? launch_qmm_prefill<64, 0>(x, ldx, weight, scales, biases, out, m, n, kg, s)
-                           : launch_qmm_prefill<64, 3>(x, ldx, weight, scales, biases, out, m, n, kg, s);
-  return f32 ? launch_qmm_prefill<32, 0>(x, ldx, weight, scales, biases, out, m, n, kg, s)
-             : launch_qmm_prefill<32, 3>(x, ldx, weight, scales, biases, out, m, n, kg, s);
+  if (gs == 64) return f32 ? launch_qmm_prefill<64, 0>(arith, x, ldx, weight, scales, biases, out, m, n, kg, s)
+                           : launch_qmm_prefill<64, 3>(arith, x, ldx, weight, scales, biases, out, m, n, kg, s);
+  return f32 ? launch_qmm_prefill<32, 0>(arith, x, ldx, weight, scales, biases, out, m, n, kg, s)
+             : launch_qmm_prefill<32, 3>(arith, x, ldx, weight, scales, biases, out, m, n, kg, s);
 }

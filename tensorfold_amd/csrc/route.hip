@@ -50,31 +50,25 @@ __global__ void __launch_bounds__(64)
 
 // ---- plan: stable counting sort of pairs by expert -------------------------------------------------------------------
 
-// up to 1024 pairs: one block does everything
+// up to 1024 pairs: one workgroup counts, scans and places; then a wave an expert that has pairs collects them in
+// pair order (ballots over the pairs, 64 a step)
 __global__ void __launch_bounds__(PLAN_THREADS)
     plan_small_kernel(const int* __restrict__ picks, int P, int E, int T, int* __restrict__ members,
                       int* __restrict__ items, int* __restrict__ counts) {
   __shared__ int pk[PLAN_THREADS];
-  __shared__ int cnt[EMAX];
-  __shared__ int off[EMAX];
-  const int tid = threadIdx.x;
-  cnt[tid] = 0;
+  __shared__ PlanLds plan;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  plan.cnt[tid] = 0;
   __syncthreads();
-  int e = -1;
-  if (tid < P) {
-    e = picks[tid];
-    if ((unsigned)e >= (unsigned)E) e = -1;          // an id outside the table joins no expert (and faults nothing)
-    pk[tid] = e;
-    if (e >= 0) atomicAdd(&cnt[e], 1);
-  }
+  int e = tid < P ? picks[tid] : -1;
+  if ((unsigned)e >= (unsigned)E) e = -1;            // an id outside the table joins no expert (and faults nothing)
+  pk[tid] = e;
+  if (e >= 0) atomicAdd(&plan.cnt[e], 1);
   __syncthreads();
-  const int o = place_items(tid < E ? cnt[tid] : 0, E, T, items, counts);
-  off[tid] = o;
-  __syncthreads();
-  if (tid < P && e >= 0) {
-    int rank = 0;
-    for (int q = 0; q < tid; ++q) rank += pk[q] == e;
-    members[off[e] + rank] = tid;
+  place_items(plan, tid < E ? plan.cnt[tid] : 0, E, T, items, counts);
+  for (int x = wave; x < E; x += PLAN_THREADS / 64) {
+    const int c = plan.cnt[x], at = plan.first[x];
+    if (c) expert_pairs(pk, P, x, c, lane, [&](int rank, int p) { members[at + rank] = p; });
   }
 }
 
@@ -89,12 +83,11 @@ __global__ void __launch_bounds__(PLAN_THREADS)
                         int* __restrict__ counts, int* __restrict__ desc, float* __restrict__ xs_x,
                         int* __restrict__ zero, int n_zero, int have_picks) {
   __shared__ int pk[PLAN_THREADS];
-  __shared__ int cnt[EMAX];
-  __shared__ int off[EMAX];
+  __shared__ PlanLds plan;
   __shared__ int mem[PLAN_THREADS];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int slots = TOPK + (shared ? 1 : 0), P = R * slots, E = NE + (shared ? 1 : 0), T = 16;
-  cnt[tid] = 0;
+  plan.cnt[tid] = 0;
   for (int i = tid; i < n_zero; i += PLAN_THREADS) zero[i] = 0;
   if (!have_picks) {      // else a launch before this one has left the picks, the weights and the group sums
     for (int r = wave; r < R; r += PLAN_THREADS / 64)
@@ -105,25 +98,24 @@ __global__ void __launch_bounds__(PLAN_THREADS)
   }
   __threadfence_block();
   __syncthreads();
-  int e = -1;
-  if (tid < P) {
-    e = pick[tid];
-    if ((unsigned)e >= (unsigned)E) e = -1;
-    pk[tid] = e;
-    if (e >= 0) atomicAdd(&cnt[e], 1);
-  }
+  int e = tid < P ? pick[tid] : -1;
+  if ((unsigned)e >= (unsigned)E) e = -1;
+  pk[tid] = e;
+  if (e >= 0) atomicAdd(&plan.cnt[e], 1);
   __syncthreads();
-  const int o = place_items(tid < E ? cnt[tid] : 0, E, T, items, counts);
-  off[tid] = o;
-  __syncthreads();
-  if (tid < P && e >= 0) {
-    int rank = 0;
-    for (int q = 0; q < tid; ++q) rank += pk[q] == e;
-    members[off[e] + rank] = tid;
-    mem[off[e] + rank] = tid;
+  place_items(plan, tid < E ? plan.cnt[tid] : 0, E, T, items, counts);
+  for (int x = wave; x < E; x += PLAN_THREADS / 64) {
+    const int c = plan.cnt[x], at = plan.first[x];
+    if (c)
+      expert_pairs(pk, P, x, c, lane, [&](int rank, int p) {
+        members[at + rank] = p;
+        mem[at + rank] = p;
+      });
   }
   __threadfence_block();
   __syncthreads();
+  const int* cnt = plan.cnt;
+  const int* off = plan.first;
   // the descriptors: the same members cut into items of DTILE, every full item first (they take longest), then the
   // experts' short last items
   const int c = tid < E ? cnt[tid] : 0, f = c / DTILE, r = c - DTILE * f > 0 ? 1 : 0;
@@ -194,7 +186,9 @@ __global__ void __launch_bounds__(PLAN_THREADS)
 #pragma unroll
       for (int i = 0; i < CH; ++i) c += v[i];
     }
-  int run = place_items(c, E, T, items, counts);
+  __shared__ PlanLds plan;
+  place_items(plan, c, E, T, items, counts);
+  int run = plan.first[tid];
   if (tid < E)
     for (int b0 = 0; b0 < nblk; b0 += CH) {
       int v[CH];

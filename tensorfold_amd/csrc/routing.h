@@ -351,24 +351,55 @@ __device__ void scan3(int (&val)[3], int (&excl)[3], int (&tot)[3]) {
   __syncthreads();
 }
 
-// thread e: expert e's pair count c -> its first member; writes the items (expert order) and counts
-__device__ int place_items(int c, int E, int T, int* __restrict__ items, int* __restrict__ counts) {
+// The plan's tables of a workgroup of PLAN_THREADS threads: a thread an expert.
+struct PlanLds {
+  int cnt[EMAX];       // pairs of expert e
+  int first[EMAX];     // its first member
+  int istart[EMAX];    // its first item
+};
+
+// Whole workgroup (PLAN_THREADS threads, barriers inside); thread e brings expert e's pair count c (0 past E).
+// Fills L and writes the plan's items and counts: experts ascending, an expert's pairs cut into runs of T.  The
+// items are written a thread an item (an expert that holds thousands of a prompt chunk's pairs has dozens): item i
+// belongs to the last expert whose first item is not past i, found by bisection of the non-decreasing istart.
+__device__ void place_items(PlanLds& L, int c, int E, int T, int* __restrict__ items, int* __restrict__ counts) {
   const int tid = threadIdx.x;
-  const int tiles = (c + T - 1) / T;
-  int val[3] = {c, tiles, c > 0 ? 1 : 0}, excl[3], tot[3];
+  int val[3] = {c, (c + T - 1) / T, c > 0 ? 1 : 0}, excl[3], tot[3];
   scan3(val, excl, tot);
+  L.cnt[tid] = c;
+  L.first[tid] = excl[0];
+  L.istart[tid] = excl[1];
   if (tid == 0) {
     counts[0] = tot[1];
     counts[1] = tot[2];
   }
-  if (tid < E)
-    for (int j = 0; j < tiles; ++j) {
-      int* it = items + 3 * (excl[1] + j);
-      it[0] = tid;
-      it[1] = excl[0] + T * j;
-      it[2] = min(T, c - T * j);
+  __syncthreads();
+  for (int i = tid; i < tot[1]; i += PLAN_THREADS) {
+    int lo = 0, hi = E - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (L.istart[mid] <= i) lo = mid;
+      else hi = mid - 1;
     }
-  return excl[0];
+    const int j = i - L.istart[lo];
+    items[3 * i] = lo;
+    items[3 * i + 1] = L.first[lo] + T * j;
+    items[3 * i + 2] = min(T, L.cnt[lo] - T * j);
+  }
+}
+
+// One wave hands expert e's `count` pairs among pk[0 .. P) to put(rank, pair) in pair order: it walks the pairs 64 at a
+// time and ranks the hits of a step with one ballot.
+template <class Put>
+__device__ __forceinline__ void expert_pairs(const int* pk, int P, int e, int count, int lane, Put&& put) {
+  int before = 0;
+  for (int p0 = 0; p0 < P && before < count; p0 += 64) {
+    const int p = p0 + lane;
+    const bool hit = p < P && pk[p] == e;
+    const unsigned long long m = __ballot(hit);
+    if (hit) put(before + __popcll(m & ((1ull << lane) - 1ull)), p);
+    before += __popcll(m);
+  }
 }
 
 // Inclusive prefix sums over the 64 lanes: shifts inside each row of 16 lanes through DPP, then the rows' totals

@@ -24,10 +24,13 @@ from .linear import CODEBOOK_IDS, _DTYPES
 
 CB_3INST, CB_MCG, CB_MUL1 = 0, 1, 2
 ACT_BF16, ACT_F32 = 0, 1          # SwiGLU with bf16 roundings after each step / in fp32
-# Half-bits a value the kernels decode: 1..8 bits with every codebook, 1.5, 2.5, 3.5 with mul1
-K2_SUPPORTED = {CB_3INST: (2, 4, 6, 8, 10, 12, 14, 16), CB_MCG: (2, 4, 6, 8, 10, 12, 14, 16),
-                CB_MUL1: (2, 3, 4, 5, 6, 7, 8, 10, 12, 14, 16)}
+# Half-bits a value the kernels decode: every count from 2 to 16 (1 to 8 bits in half-bit steps) with every codebook,
+# as the reference's module accepts them (cuda/exl3/experts.py:15-16); an odd count gives the odd stream positions
+# the extra bit.
+K2_SUPPORTED = {cb: tuple(range(2, 17)) for cb in (CB_3INST, CB_MCG, CB_MUL1)}
 WAVES = 4                         # waves a workgroup of the grouped kernel (each takes a share of a K split)
+GATE, UP, DOWN = 0, 1, 2          # rows of the per-layer address and width tables
+MAX_EXPERTS = 1024                # the pair sort's table
 
 
 def codebook_id(name: str) -> int:
@@ -49,96 +52,106 @@ def k2_of(trellis: torch.Tensor) -> int:
 
 @dataclass
 class Exl3RoutedExperts:
-    """One layer's routed experts: trellis addresses and widths per projection, stacked suh/svh, and the tensors that
-    keep the trellises alive."""
+    """One layer's routed experts as the kernels read them: a table of trellis addresses and one of widths (rows
+    ``GATE``, ``UP``, ``DOWN``; a column an expert) and the experts' sign-scale vectors stacked per projection."""
 
-    gate_ptr: torch.Tensor    # int64 [E]
-    up_ptr: torch.Tensor
-    down_ptr: torch.Tensor
-    gate_k2: torch.Tensor     # int32 [E], half-bits a value
-    up_k2: torch.Tensor
-    down_k2: torch.Tensor
-    suh_g: torch.Tensor       # fp16 [E, D]
-    suh_u: torch.Tensor
-    svh_g: torch.Tensor       # fp16 [E, I]
-    svh_u: torch.Tensor
-    suh_d: torch.Tensor       # fp16 [E, I]
-    svh_d: torch.Tensor       # fp16 [E, D]
-    count: int                # E
-    dims: int                 # D
-    width: int                # I
+    ptr: torch.Tensor             # int64 [3, E] on the GPU: where each expert's gate / up / down trellis starts
+    k2: torch.Tensor              # int32 [3, E] on the GPU: its half-bits a value
+    suh: tuple                    # fp16 input scales: gate [E, D], up [E, D], down [E, I]
+    svh: tuple                    # fp16 output scales: gate [E, I], up [E, I], down [E, D]
+    count: int                    # E
+    dims: int                     # D
+    width: int                    # I
     cb: int
-    trellis_bytes: torch.Tensor   # int64 [E] (host): gate + up + down trellis bytes of each expert
-    keep: list = field(default_factory=list, repr=False)
+    trellis_bytes: torch.Tensor   # int64 [E] on the host: bytes of an expert's three trellises
+    keep: list = field(default_factory=list, repr=False)     # whatever owns the memory ``ptr`` points into
 
     def nbytes_read(self, ids: Sequence[int]) -> int:
         return int(self.trellis_bytes[list(ids)].sum())
+
+
+def _codebook(codebook: int | str) -> int:
+    cb = codebook_id(codebook) if isinstance(codebook, str) else int(codebook)
+    if cb not in K2_SUPPORTED:
+        raise ValueError(f"unknown EXL3 codebook id {cb}")
+    return cb
+
+
+def _trellis_ok(t: torch.Tensor, k: int, n: int, cb: int) -> int:
+    """Checks one expert's trellis against the layer's K x N and returns its half-bits a value."""
+
+    if t.dtype != torch.int16 or not t.is_contiguous() or not t.is_cuda:
+        raise ValueError("trellis must be a contiguous GPU int16 tensor")
+    if t.dim() != 3 or 16 * t.shape[0] != k or 16 * t.shape[1] != n:
+        raise ValueError(f"expert shape {tuple(t.shape)} does not match [{k // 16}, {n // 16}, *]")
+    if t.data_ptr() % 4:
+        raise ValueError("trellis must start on a 4-byte boundary")
+    k2 = k2_of(t)
+    if k2 not in K2_SUPPORTED[cb]:
+        raise ValueError(f"unsupported EXL3 bit width {k2 / 2} for codebook {cb}")
+    return k2
+
+
+def _layer(ptr, k2, suh, svh, d: int, width: int, cb: int, keep: list, device) -> Exl3RoutedExperts:
+    """The layer from host-side [3][E] lists (or tensors) of addresses and widths and the stacked scale vectors."""
+
+    n_exp = len(ptr[0])
+    if d % fmt.HAD or width % fmt.HAD:
+        raise ValueError(f"D={d} and I={width} must be multiples of 128")
+    if n_exp > MAX_EXPERTS:
+        raise ValueError("at most 1024 experts a layer (the pair sort's table)")
+    widths = torch.as_tensor(k2, dtype=torch.int32).reshape(3, n_exp)
+    tile_bytes = 16 * widths.to(torch.int64).sum(0)                  # a 16 x 16 tile at k2 half-bits is 16 k2 bytes
+    for name, vs, sizes in (("suh", suh, (d, d, width)), ("svh", svh, (width, width, d))):
+        for v, size in zip(vs, sizes):
+            if tuple(v.shape) != (n_exp, size) or v.dtype != torch.float16 or not v.is_contiguous() or not v.is_cuda:
+                raise ValueError(f"{name}: contiguous GPU fp16 [{n_exp}, {size}] expected, got {tuple(v.shape)} {v.dtype}")
+    return Exl3RoutedExperts(torch.as_tensor(ptr, dtype=torch.int64).reshape(3, n_exp).to(device),
+                             widths.to(device), tuple(suh), tuple(svh), n_exp, d, width, cb,
+                             tile_bytes * (d * width // 256), keep)
 
 
 def prepare(gate: Sequence[tuple], up: Sequence[tuple], down: Sequence[tuple], codebook: int | str,
             device: str | torch.device = "cuda") -> Exl3RoutedExperts:
     """A layer from per-expert (trellis, suh, svh) triples, trellises referenced in place, each at its own width."""
 
-    cb = codebook_id(codebook) if isinstance(codebook, str) else int(codebook)
-    if cb not in K2_SUPPORTED:
-        raise ValueError(f"unknown EXL3 codebook id {cb}")
+    cb = _codebook(codebook)
+    projections = (gate, up, down)
     n_exp = len(gate)
-    if not (len(up) == len(down) == n_exp) or n_exp == 0:
+    if n_exp == 0 or any(len(p) != n_exp for p in projections):
         raise ValueError("gate, up and down need the same, non-zero number of experts")
-    d, width = int(gate[0][0].shape[0]) * 16, int(gate[0][0].shape[1]) * 16
-    if d % fmt.HAD or width % fmt.HAD:
-        raise ValueError(f"D={d} and I={width} must be multiples of 128")
-    if n_exp > 1024:
-        raise ValueError("at most 1024 experts a layer (the pair sort's table)")
-    keep: list = []
+    d, width = 16 * int(gate[0][0].shape[0]), 16 * int(gate[0][0].shape[1])
+    shapes = ((d, width), (d, width), (width, d))
+    k2 = [[_trellis_ok(m[0], k, n, cb) for m in mats] for mats, (k, n) in zip(projections, shapes)]
+    ptr = [[m[0].data_ptr() for m in mats] for mats in projections]
 
-    def table(mats, k, n):
-        ptrs, k2s = [], []
-        for t, _, _ in mats:
-            if t.dtype != torch.int16 or not t.is_contiguous() or not t.is_cuda:
-                raise ValueError("trellis must be a contiguous GPU int16 tensor")
-            if t.shape[0] * 16 != k or t.shape[1] * 16 != n:
-                raise ValueError(f"expert shape {tuple(t.shape)} does not match [{k // 16}, {n // 16}, *]")
-            k2 = k2_of(t)
-            if k2 not in K2_SUPPORTED[cb]:
-                raise ValueError(f"unsupported EXL3 bit width {k2 / 2} for codebook {cb}")
-            if t.data_ptr() % 4:
-                raise ValueError("trellis must start on a 4-byte boundary")
-            k2s.append(k2)
-            ptrs.append(t.data_ptr())
-            keep.append(t)
-        return (torch.tensor(ptrs, dtype=torch.int64, device=device),
-                torch.tensor(k2s, dtype=torch.int32, device=device), k2s)
+    def rows(mats, which: int) -> torch.Tensor:
+        return torch.stack([m[which].reshape(-1) for m in mats]).to(device=device, dtype=torch.float16).contiguous()
 
-    gp, gk, gks = table(gate, d, width)
-    upp, uk, uks = table(up, d, width)
-    dp, dk, dks = table(down, width, d)
-
-    def stack(mats, j, n):
-        out = torch.empty((n_exp, n), dtype=torch.float16, device=device)
-        for e, m in enumerate(mats):
-            out[e].copy_(m[j].reshape(-1))
-        return out
-
-    tb = torch.tensor([(d * width // 256) * (gks[e] + uks[e] + dks[e]) * 16 for e in range(n_exp)], dtype=torch.int64)
-    return Exl3RoutedExperts(gp, upp, dp, gk, uk, dk, stack(gate, 1, d), stack(up, 1, d), stack(gate, 2, width),
-                             stack(up, 2, width), stack(down, 1, width), stack(down, 2, d), n_exp, d, width, cb, tb,
-                             keep)
+    return _layer(ptr, k2, [rows(m, 1) for m in projections], [rows(m, 2) for m in projections], d, width, cb,
+                  [m[0] for mats in projections for m in mats], device)
 
 
 def prepare_stacked(gt: torch.Tensor, ut: torch.Tensor, dt: torch.Tensor, suh_g, suh_u, svh_g, svh_u, suh_d, svh_d,
                     codebook: int | str) -> Exl3RoutedExperts:
     """A uniform-width layer stacked per projection: trellis [E, K/16, N/16, 16 * bits] (int16, or the same bytes as
-    int32 words), suh/svh [E, n]."""
+    int32 words), suh/svh [E, n].  Nothing is copied: expert e's trellis is the stack's base plus e strides."""
 
-    def as16(t):
-        return t.view(torch.int16) if t.dtype == torch.int32 else t
-
-    gt, ut, dt = as16(gt), as16(ut), as16(dt)
-    n_exp = gt.shape[0]
-    return prepare([(gt[e], suh_g[e], svh_g[e]) for e in range(n_exp)],
-                   [(ut[e], suh_u[e], svh_u[e]) for e in range(n_exp)],
-                   [(dt[e], suh_d[e], svh_d[e]) for e in range(n_exp)], codebook, device=gt.device)
+    cb = _codebook(codebook)
+    stacks = [t.view(torch.int16) if t.dtype == torch.int32 else t for t in (gt, ut, dt)]
+    n_exp = int(stacks[0].shape[0])
+    if n_exp == 0 or any(t.dim() != 4 or t.shape[0] != n_exp for t in stacks):
+        raise ValueError("gate, up and down need the same, non-zero number of experts")
+    d, width = 16 * int(stacks[0].shape[1]), 16 * int(stacks[0].shape[2])
+    ptr, k2 = [], []
+    for t, (k, n) in zip(stacks, ((d, width), (d, width), (width, d))):
+        k2.append([_trellis_ok(t[0], k, n, cb)] * n_exp)
+        if not t.is_contiguous() or (t[0].numel() * 2) % 4:
+            raise ValueError("stacked trellises must be contiguous, every expert on a 4-byte boundary")
+        ptr.append((t.data_ptr() + torch.arange(n_exp, dtype=torch.int64) * (t[0].numel() * 2)).tolist())
+    half = lambda v: v.to(device=gt.device, dtype=torch.float16).contiguous()
+    return _layer(ptr, k2, [half(suh_g), half(suh_u), half(suh_d)], [half(svh_g), half(svh_u), half(svh_d)], d, width,
+                  cb, stacks, gt.device)
 
 
 def default_config(k: int, n: int, gateup: bool = True) -> int:
@@ -155,23 +168,28 @@ def default_config(k: int, n: int, gateup: bool = True) -> int:
 
 
 class Scratch:
-    """Buffers for up to ``rows`` rows of ``slots`` slots; slots whose pick is not a routed expert are left to the
-    caller (``y`` keeps what the caller wrote there)."""
+    """Device buffers of ``routed`` for up to ``rows`` rows of ``slots`` slots: the rotated inputs of the three
+    projections (``xg``, ``xu``, ``xd``, fp16 a pair), the K splits' fp32 partial sums ``z``, the pair outputs ``y``
+    and the pair sort's plan.  Pairs whose pick is not a routed expert touch none of them (their ``y`` rows stay as
+    the caller left them)."""
 
     def __init__(self, ex: Exl3RoutedExperts, rows: int, slots: int, sk_gu: int | None = None, sk_d: int | None = None,
                  device: str | torch.device = "cuda") -> None:
-        d, width = ex.dims, ex.width
-        self.sk_gu = sk_gu or default_config(d, width, True)
-        self.sk_d = sk_d or default_config(width, d, False)
-        p = rows * slots
-        self.xg = torch.zeros((p, d), dtype=torch.float16, device=device)
-        self.xu = torch.zeros((p, d), dtype=torch.float16, device=device)
-        self.xd = torch.zeros((p, width), dtype=torch.float16, device=device)
-        # gate and up write 2 * splits * P * I partials, down splits * P * D
-        self.z = torch.zeros((max(2 * self.sk_gu * width, self.sk_d * d) * p,), dtype=torch.float32, device=device)
-        self.y = torch.zeros((p, d), dtype=torch.float32, device=device)
-        self.plan = grouped.Plan(rows, slots, ex.count, device)          # ids outside [0, E) join no item
         self.rows, self.slots, self.count_experts = rows, slots, ex.count
+        self.sk_gu = sk_gu or default_config(ex.dims, ex.width, True)
+        self.sk_d = sk_d or default_config(ex.width, ex.dims, False)
+        pairs = rows * slots
+
+        def buffer(columns: int, dtype: torch.dtype) -> torch.Tensor:
+            return torch.zeros((pairs, columns), dtype=dtype, device=device)
+
+        self.xg, self.xu = buffer(ex.dims, torch.float16), buffer(ex.dims, torch.float16)
+        self.xd = buffer(ex.width, torch.float16)
+        self.y = buffer(ex.dims, torch.float32)
+        # one buffer serves both grouped launches: [2 matrices][sk_gu][pairs][I] first, [sk_d][pairs][D] after
+        self.z = torch.zeros((pairs * max(2 * self.sk_gu * ex.width, self.sk_d * ex.dims),), dtype=torch.float32,
+                             device=device)
+        self.plan = grouped.Plan(rows, slots, ex.count, device)          # ids outside [0, E) join no item
 
 
 def routed(x: torch.Tensor, pick: torch.Tensor, wts: torch.Tensor | None, ex: Exl3RoutedExperts, s: Scratch,
@@ -201,25 +219,25 @@ def routed(x: torch.Tensor, pick: torch.Tensor, wts: torch.Tensor | None, ex: Ex
         grouped.route(pick, plan)                         # the pair sort drops ids outside [0, E)
     items = grouped.max_items(p, n_exp, grouped.TILE)
     plan_args = (_lib.ptr(plan.items), _lib.ptr(plan.counts), _lib.ptr(plan.members))
-    _lib.call("tf_exl3x_rot_in", _lib.ptr(x), _DTYPES[x.dtype], x.stride(0), _lib.ptr(pick), _lib.ptr(ex.suh_g),
-              _lib.ptr(ex.suh_u), _lib.ptr(s.xg), _lib.ptr(s.xu), R, slots, d, n_exp)
-    _lib.call("tf_exl3x_grouped", _lib.ptr(s.xg), _lib.ptr(s.xu), _lib.ptr(ex.gate_ptr), _lib.ptr(ex.up_ptr),
-              _lib.ptr(ex.gate_k2), _lib.ptr(ex.up_k2), *plan_args, _lib.ptr(s.z), 2, d, width, p, s.sk_gu, ex.cb,
+    _lib.call("tf_exl3x_rot_in", _lib.ptr(x), _DTYPES[x.dtype], x.stride(0), _lib.ptr(pick), _lib.ptr(ex.suh[GATE]),
+              _lib.ptr(ex.suh[UP]), _lib.ptr(s.xg), _lib.ptr(s.xu), R, slots, d, n_exp)
+    _lib.call("tf_exl3x_grouped", _lib.ptr(s.xg), _lib.ptr(s.xu), _lib.ptr(ex.ptr[GATE]), _lib.ptr(ex.ptr[UP]),
+              _lib.ptr(ex.k2[GATE]), _lib.ptr(ex.k2[UP]), *plan_args, _lib.ptr(s.z), 2, d, width, p, s.sk_gu, ex.cb,
               n_exp, items)
-    _lib.call("tf_exl3x_gateup_epilogue", _lib.ptr(s.z), _lib.ptr(pick), _lib.ptr(ex.svh_g), _lib.ptr(ex.svh_u),
-              _lib.ptr(ex.suh_d), _lib.ptr(s.xd), p, width, s.sk_gu, n_exp,
+    _lib.call("tf_exl3x_gateup_epilogue", _lib.ptr(s.z), _lib.ptr(pick), _lib.ptr(ex.svh[GATE]), _lib.ptr(ex.svh[UP]),
+              _lib.ptr(ex.suh[DOWN]), _lib.ptr(s.xd), p, width, s.sk_gu, n_exp,
               float(min(limit, 3.0e38)), act_mode)
-    _lib.call("tf_exl3x_grouped", _lib.ptr(s.xd), None, _lib.ptr(ex.down_ptr), None, _lib.ptr(ex.down_k2), None,
+    _lib.call("tf_exl3x_grouped", _lib.ptr(s.xd), None, _lib.ptr(ex.ptr[DOWN]), None, _lib.ptr(ex.k2[DOWN]), None,
               *plan_args, _lib.ptr(s.z), 1, width, d, p, s.sk_d, ex.cb, n_exp, items)
     if wts is None:
-        _lib.call("tf_exl3x_down_combine", _lib.ptr(s.z), _lib.ptr(pick), _lib.ptr(ex.svh_d), _lib.ptr(s.y), None, None,
+        _lib.call("tf_exl3x_down_combine", _lib.ptr(s.z), _lib.ptr(pick), _lib.ptr(ex.svh[DOWN]), _lib.ptr(s.y), None, None,
                   R, slots, d, s.sk_d, n_exp)
         return s.y[:p]
     if out is None:
         out = torch.empty((R, d), dtype=torch.float32, device=x.device)
     elif out.dtype != torch.float32 or tuple(out.shape) != (R, d) or not out.is_contiguous():
         raise ValueError(f"out must be a contiguous fp32 [{R}, {d}]")
-    _lib.call("tf_exl3x_down_combine", _lib.ptr(s.z), _lib.ptr(pick), _lib.ptr(ex.svh_d), _lib.ptr(s.y), _lib.ptr(wts),
+    _lib.call("tf_exl3x_down_combine", _lib.ptr(s.z), _lib.ptr(pick), _lib.ptr(ex.svh[DOWN]), _lib.ptr(s.y), _lib.ptr(wts),
               _lib.ptr(out), R, slots, d, s.sk_d, n_exp)
     return out
 

@@ -48,8 +48,28 @@ def strips(words: torch.Tensor) -> torch.Tensor:
     """Trellis words [K/16, N/16, W] -> [N/128, K/16, 8, W] (a copy): each 128-column block's tiles in k order, the
     order a workgroup walks."""
 
-    kt, nt, w = words.shape
-    return words.reshape(kt, nt // 8, 8, w).transpose(0, 1).contiguous()
+    return words.unflatten(1, (-1, 8)).movedim(1, 0).contiguous()
+
+
+def _scale_vector(t: torch.Tensor, size: int, device) -> torch.Tensor:
+    """A layer's suh or svh as fp16 [size] on ``device``; older checkpoints store one sign bit an element instead
+    (int16 [size / 16]), which become +-1."""
+
+    if t.dtype == torch.int16 and 16 * t.numel() == size:
+        t = torch.from_numpy(fmt.unpack_signs(t))
+    if t.dtype != torch.float16 or t.numel() != size:
+        raise ValueError(f"scales must be fp16 [{size}] or int16 sign words [{size // 16}]")
+    return t.to(device).reshape(size).contiguous()
+
+
+def _decode(words: torch.Tensor, k: int, n: int, strides: tuple[int, int], k2: int, codebook: str,
+            out: torch.Tensor | None) -> torch.Tensor:
+    """W_q [K, N] fp16 from GPU trellis words laid out with ``strides`` (see ``Exl3Linear.strides``)."""
+
+    if out is None:
+        out = words.new_empty((k, n), dtype=torch.float16)
+    _lib.call("tf_exl3_unpack", _lib.ptr(words), _lib.ptr(out), k, n, *strides, k2, CODEBOOK_IDS[codebook])
+    return out
 
 
 @dataclasses.dataclass
@@ -79,26 +99,18 @@ class Exl3Linear:
         """Build from a checkpoint group: trellis int16 [K/16, N/16, 16 * bits]; suh / svh fp16, or the int16 sign
         words of older checkpoints; the codebook's name."""
 
-        bits = fmt.bits_of(trellis.shape)
-        fmt.check_pair(bits, codebook)
-        k, n = 16 * int(trellis.shape[0]), 16 * int(trellis.shape[1])
-        if k % fmt.HAD or n % fmt.HAD:
-            raise ValueError(f"K={k} and N={n} must be multiples of 128")
         if layout not in ("strips", "stored"):
             raise ValueError(f"layout must be 'strips' or 'stored', got {layout!r}")
-
-        def vector(t: torch.Tensor, size: int) -> torch.Tensor:
-            if t.dtype == torch.int16 and t.numel() * 16 == size:
-                t = torch.from_numpy(fmt.unpack_signs(t))
-            if t.dtype != torch.float16 or t.numel() != size:
-                raise ValueError(f"scales must be fp16 [{size}] or int16 sign words [{size // 16}]")
-            return t.reshape(size).to(device).contiguous()
-
+        bits = fmt.bits_of(trellis.shape)
+        fmt.check_pair(bits, codebook)
+        k, n = (16 * int(v) for v in trellis.shape[:2])
+        if k % fmt.HAD or n % fmt.HAD:
+            raise ValueError(f"K={k} and N={n} must be multiples of 128")
         words = trellis.to(device).contiguous().view(torch.int32)
-        if layout == "strips":
-            words = strips(words)
-        b = None if bias is None else bias.to(device=device, dtype=torch.float16).contiguous()
-        return cls(words, vector(suh, k), vector(svh, n), b, bits, codebook, k, n, layout)
+        return cls(words=strips(words) if layout == "strips" else words, suh=_scale_vector(suh, k, device),
+                   svh=_scale_vector(svh, n, device),
+                   bias=None if bias is None else bias.to(device=device, dtype=torch.float16).contiguous(),
+                   bits=bits, codebook=codebook, k=k, n=n, layout=layout)
 
     @property
     def k2(self) -> int:
@@ -108,10 +120,9 @@ class Exl3Linear:
     def strides(self) -> tuple[int, int]:
         """int32 words from one k tile to the next, and from one 128-column block to the next."""
 
-        tile = 4 * self.k2
-        if self.layout == "strips":
-            return 8 * tile, (self.k // 16) * 8 * tile
-        return (self.n // 16) * tile, 8 * tile
+        if self.layout == "strips":                       # [N/128, K/16, 8, W]
+            return self.words.stride(1), self.words.stride(0)
+        return self.words.stride(0), 8 * self.words.stride(1)       # [K/16, N/16, W]: a block is 8 tiles side by side
 
     def nbytes(self) -> int:
         return self.words.numel() * 4
@@ -162,10 +173,7 @@ class Exl3Linear:
     def unpack(self, out: torch.Tensor | None = None) -> torch.Tensor:
         """W_q [K, N] fp16, decoded on the GPU from either layout."""
 
-        w = out if out is not None else self.words.new_empty((self.k, self.n), dtype=torch.float16)
-        _lib.call("tf_exl3_unpack", _lib.ptr(self.words), _lib.ptr(w), self.k, self.n, *self.strides, self.k2,
-                  CODEBOOK_IDS[self.codebook])
-        return w
+        return _decode(self.words, self.k, self.n, self.strides, self.k2, self.codebook, out)
 
 
 def unpack_gpu(trellis: torch.Tensor, codebook: str) -> torch.Tensor:
@@ -174,12 +182,8 @@ def unpack_gpu(trellis: torch.Tensor, codebook: str) -> torch.Tensor:
     bits = fmt.bits_of(trellis.shape)
     fmt.check_pair(bits, codebook)
     words = trellis.cuda().contiguous().view(torch.int32)
-    k, n = 16 * int(trellis.shape[0]), 16 * int(trellis.shape[1])
-    w = words.new_empty((k, n), dtype=torch.float16)
-    tile = 4 * k2_of(bits)
-    _lib.call("tf_exl3_unpack", _lib.ptr(words), _lib.ptr(w), k, n, (n // 16) * tile, 8 * tile, k2_of(bits),
-              CODEBOOK_IDS[codebook])
-    return w
+    kt, nt, tile = words.shape
+    return _decode(words, 16 * kt, 16 * nt, (nt * tile, 8 * tile), k2_of(bits), codebook, None)
 
 
 unpack_cuda = unpack_gpu      # the name the reference's callers use (torch keeps the "cuda" device name on ROCm)

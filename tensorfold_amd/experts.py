@@ -21,6 +21,15 @@ TILE = 16             # largest decode item, in pairs
 PREFILL_TILE = 128    # default prompt item; the MFMA kernels also take 16 and 64
 SMALL = 1024          # a plan up to this many pairs is sorted by one workgroup
 _GROUPS = (32, 64)
+ARITH_F16, ARITH_BF16 = 0, 1      # TF_ARITH_* of the C header: the prompt form's operand arithmetic
+F16_TABLE_LIMIT = 255.9           # |scale| and |bias| below this ride the fp16 form (256 x stays finite in fp16)
+
+
+def fits_f16(*tensors: torch.Tensor) -> bool:
+    """Whether every scale and bias given is finite and small enough for the prompt form's fp16 arithmetic (one
+    reduction and a host read: for load time)."""
+
+    return all(bool(torch.isfinite(t).all()) and float(t.abs().max()) < F16_TABLE_LIMIT for t in tensors if t.numel())
 
 
 def block_words(gs: int) -> int:
@@ -91,6 +100,7 @@ class Experts:
     width: int           # NI
     dims: int            # D
     limit: float = 0.0   # SwiGLU clip, 0 for none
+    arith: int = ARITH_F16   # the prompt form's arithmetic: ARITH_BF16 when a scale or bias does not fit the fp16 form
 
     @property
     def count(self) -> int:
@@ -104,15 +114,22 @@ class Experts:
         return 4 * (self.up[0].numel() + self.down[0].numel())
 
 
-def make(up: list[tuple], down: tuple, gs: int, *, limit: float = 0.0) -> Experts:
-    """Pack a layer.  ``up`` = [(words, scales, biases)] for relu^2 or [gate, up] for SwiGLU; ``down`` one triple."""
+def make(up: list[tuple], down: tuple, gs: int, *, limit: float = 0.0, arith: int | None = None) -> Experts:
+    """Pack a layer.  ``up`` = [(words, scales, biases)] for relu^2 or [gate, up] for SwiGLU; ``down`` one triple.
+
+    ``arith`` fixes the prompt form's arithmetic; left None it is the fp16 form unless a scale or bias of the layer
+    is too large for it (``fits_f16``), in which case the layer takes the reference's bf16 form.  The fp16 form also
+    clamps activations beyond +-65504: a layer whose prompt activations can exceed that (a wide relu^2) should be made
+    with ``arith=ARITH_BF16``."""
 
     if len(up) not in (1, 2):
         raise ValueError("experts take a gate and an up projection, or an up projection alone")
     ni, d = int(up[0][0].shape[1]), 8 * int(up[0][0].shape[2])
     table_up = torch.stack([pack(w, s, b, gs) for (w, s, b) in up], dim=3)
     table_down = pack(*down, gs).unsqueeze(3)
-    return Experts(table_up, table_down, gs, ni, d, float(limit))
+    if arith is None:
+        arith = ARITH_F16 if fits_f16(*[t for m in (*up, down) for t in m[1:]]) else ARITH_BF16
+    return Experts(table_up, table_down, gs, ni, d, float(limit), int(arith))
 
 
 def max_items(pairs: int, experts: int, tile: int = TILE) -> int:
@@ -188,6 +205,22 @@ def _fits(plan: Plan, rows: int, x_rows: int | None, pair_rows: int) -> None:
         raise ValueError(f"buffers too small for {rows} rows x {plan.slots} slots")
 
 
+# Which call last wrote a pair-activation buffer through this library (address -> a running number).  ``gate_up`` notes
+# it and ``down`` trusts the group sums a plan kept only while its own ``gate_up`` is still the last writer: launches
+# made through ctypes do not move torch's version counter, so that counter alone would miss them.
+_writes: dict[int, int] = {}
+_epoch = 0
+
+
+def wrote(t: torch.Tensor) -> int:
+    """Note that a kernel of this library has just (re)written ``t``; returns the note's number."""
+
+    global _epoch
+    _epoch += 1
+    _writes[t.data_ptr()] = _epoch
+    return _epoch
+
+
 def _group_sums(x: torch.Tensor, gs: int, into: torch.Tensor) -> torch.Tensor:
     _lib.call("tf_group_sums", _lib.ptr(x), x.stride(0), int(x.shape[0]), int(x.shape[1]), gs, _lib.ptr(into))
     return into
@@ -195,12 +228,12 @@ def _group_sums(x: torch.Tensor, gs: int, into: torch.Tensor) -> torch.Tensor:
 
 def _launch(x: torch.Tensor, slots: int, table: torch.Tensor, gs: int, k: int, n: int, epi: int, plan: Plan,
             out: torch.Tensor, limit: float, rows: int, xs: torch.Tensor | None = None,
-            xs_out: torch.Tensor | None = None) -> None:
+            xs_out: torch.Tensor | None = None, arith: int = ARITH_F16) -> None:
     bound = max_items(rows * plan.slots, plan.experts, plan.tile)
     common = (gs, epi, _lib.ptr(x), x.stride(0), slots, _lib.ptr(table), k // gs, n // COLS, _lib.ptr(plan.items),
               _lib.ptr(plan.counts), _lib.ptr(plan.members), _lib.ptr(out), n, limit)
     if plan.prefill:
-        _lib.call("tf_experts_prefill", *common, bound, plan.tile)
+        _lib.call("tf_experts_prefill", *common, bound, plan.tile, arith)
     else:
         _lib.call("tf_experts_run", *common, bound * (n // COLS), _lib.ptr(xs), _lib.ptr(xs_out))
 
@@ -218,8 +251,9 @@ def gate_up(x: torch.Tensor, ex: Experts, plan: Plan, out: torch.Tensor, rows: i
     if not plan.prefill:
         xs = _group_sums(x, ex.gs, plan.sums("x", int(x.shape[0]), ex.dims // ex.gs))
         xs_out = plan.sums("act", int(out.shape[0]), ex.width // ex.gs)
-    _launch(x, plan.slots, ex.up, ex.gs, ex.dims, ex.width, epi, plan, out, ex.limit, rows, xs, xs_out)
-    plan._act_key = None if plan.prefill else (out.data_ptr(), out._version, rows, ex.width)
+    _launch(x, plan.slots, ex.up, ex.gs, ex.dims, ex.width, epi, plan, out, ex.limit, rows, xs, xs_out, ex.arith)
+    stamp = wrote(out)
+    plan._act_key = None if plan.prefill else (out.data_ptr(), out._version, rows, ex.width, stamp)
 
 
 def down(act: torch.Tensor, ex: Experts, plan: Plan, out: torch.Tensor, rows: int) -> None:
@@ -231,8 +265,8 @@ def down(act: torch.Tensor, ex: Experts, plan: Plan, out: torch.Tensor, rows: in
     _fits(plan, rows, None, min(act.shape[0], out.shape[0]))
     xs = None
     if not plan.prefill:
-        if plan._act_key == (act.data_ptr(), act._version, rows, ex.width):
+        if plan._act_key == (act.data_ptr(), act._version, rows, ex.width, _writes.get(act.data_ptr())):
             xs = plan.sums("act", int(act.shape[0]), ex.width // ex.gs)        # left there by gate_up
         else:
             xs = _group_sums(act, ex.gs, plan.sums("act2", int(act.shape[0]), ex.width // ex.gs))
-    _launch(act, 0, ex.down, ex.gs, ex.width, ex.dims, epi, plan, out, 0.0, rows, xs)
+    _launch(act, 0, ex.down, ex.gs, ex.width, ex.dims, epi, plan, out, 0.0, rows, xs, None, ex.arith)

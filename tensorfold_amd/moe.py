@@ -10,7 +10,6 @@ the optional shared expert rides in the last slot with a sigmoid gate.
 from __future__ import annotations
 
 import dataclasses
-import os
 
 import torch
 
@@ -19,13 +18,13 @@ from . import experts as grouped
 
 # ``run`` issues a decode-sized layer as routing + up + down + combine launches; with this set it issues the routing
 # launch and the one fused experts launch (``decode``) instead.  Same bits either way.
-FUSED_DECODE = os.environ.get("TENSORFOLD_AMD_FUSED_DECODE", "0") == "1"
+FUSED_DECODE = False
 # Up to this many router logits (rows x experts) a call, the up projection's workgroups each repeat the top-k
 # instead of waiting for a launch; past it the top-k runs once, a launch before, and they rebuild only the plan.
 ROUTE_UP_LOGITS = 2048
 # With this set ``decode`` makes the whole routing (top-k, plan, group sums, descriptors) in launches of its own and
 # runs the up projection from its descriptors: one launch more, for callers that want the plan before the experts.
-ROUTING_LAUNCH = os.environ.get("TENSORFOLD_AMD_ROUTING_LAUNCH", "0") == "1"
+ROUTING_LAUNCH = False
 # Item descriptors the routing launches leave for the decode expert kernels: rows of DESC_INTS int32, row 0 the
 # count; items of at most DESC_TILE pairs (TF_DESC_INTS / TF_DESC_TILE of the C header).
 DESC_INTS, DESC_TILE = 8, 2
@@ -75,29 +74,29 @@ class MoEBuffers:
         # rounding alone costs 1.1e-3 relative L2 at the combine, most of a 2e-3 budget.  ``experts.down`` still
         # writes bf16 into a bf16 ``out`` on a prompt plan for callers that want the smaller buffer.)
         self.y = torch.empty((rows, self.slots, cfg.hidden_size), device=device, dtype=torch.float32)
-        self.cfg, self.device, self._fused = cfg, device, None
+        self.cfg, self.device, self._fused = cfg, device, {}
 
     def fused(self, gs: int) -> dict:
-        """Scratch of ``decode``, made on first use: item descriptors, group sums, the counters of the one-launch
+        """Scratch of ``decode`` for tables of group size ``gs``, made on first use: item descriptors, group sums, the counters of the one-launch
         form (status, then an arrival count a descriptor, then one a (token, 64 columns) cell) and the output."""
 
-        if self._fused is None:
+        if gs not in self._fused:
             cfg, dev, pairs = self.cfg, self.device, self.rows * self.slots
             items = grouped.max_items(pairs, cfg.num_experts + int(self.shared), DESC_TILE)
             cells = max(min(self.rows, 64) * ARRIVE_STRIDE, self.rows) * (cfg.hidden_size // 64)
-            self._fused = dict(
+            self._fused[gs] = dict(
                 items=items * DONE_STRIDE,          # ints the descriptors' arrival counters take
                 desc=torch.zeros((1 + items, DESC_INTS), dtype=torch.int32, device=dev),
                 xs_x=torch.empty((self.rows, cfg.hidden_size // gs), dtype=torch.float32, device=dev),
                 xs_act=torch.empty((pairs, cfg.moe_intermediate_size // gs), dtype=torch.float32, device=dev),
                 counters=torch.zeros((1 + items * DONE_STRIDE + cells,), dtype=torch.int32, device=dev),
                 out=torch.empty((self.rows, cfg.hidden_size), dtype=torch.bfloat16, device=dev))
-        return self._fused
+        return self._fused[gs]
 
     def check(self) -> None:
         """Host-side look at the fused layer's status flag (synchronises): raises if a bounded wait ran out."""
 
-        if self._fused is not None and int(self._fused["counters"][0]):
+        if any(int(f["counters"][0]) for f in self._fused.values()):
             raise RuntimeError("tensorfold-amd: the fused decode layer timed out waiting for its activations")
 
 
@@ -157,6 +156,7 @@ def decode(x: torch.Tensor, logits: torch.Tensor, ex: grouped.Experts, buf: MoEB
     if logits.dtype != torch.float32 or logits.stride(1) != 1:
         raise ValueError("select: logits must be fp32 with unit-stride rows")
     f = buf.fused(ex.gs)
+    grouped.wrote(buf.act)          # the launches below rewrite the pair activations: sums a plan kept of them are void
     if out is None:
         out = f["out"][:n]
     plan = buf.plan
@@ -247,7 +247,7 @@ def run(x: torch.Tensor, m: Routed, *, prefill: bool = False) -> torch.Tensor:
 
     n = int(x.shape[0])
     cap = max(16, 1 << (n - 1).bit_length())
-    key = (cap, m.count, m.top_k, m.experts.width, m.experts.dims, prefill, x.device)
+    key = (cap, m.count, m.top_k, m.experts.width, m.experts.dims, m.experts.gs, prefill, x.device)
     if key not in _pool:
         _pool[key] = MoEBuffers(cap, _Dims(m), x.device, prefill=prefill)
     buf, x = _pool[key], x.contiguous()

@@ -29,6 +29,7 @@ class Q4:
     n: int
     k: int
     gs: int
+    arith: int = 0       # the prompt form's arithmetic (TF_ARITH_*): 1 when a scale or bias does not fit the fp16 form
 
     def nbytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in (self.weight, self.scales, self.biases))
@@ -52,6 +53,9 @@ def pack(weight: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, gs: i
     _lib.call("tf_qmm_pack", _lib.ptr(words.contiguous()), _lib.ptr(scales.to(torch.bfloat16).contiguous()),
               _lib.ptr(biases.to(torch.bfloat16).contiguous()), n, k, gs, _lib.ptr(q.weight), _lib.ptr(q.scales),
               _lib.ptr(q.biases))
+    from .experts import ARITH_BF16, ARITH_F16, fits_f16
+
+    q.arith = ARITH_F16 if fits_f16(scales, biases) else ARITH_BF16
     return q
 
 
@@ -220,9 +224,11 @@ def matmul_group(x: torch.Tensor, qs: list[Q4], xs: torch.Tensor | None = None, 
 
 
 def prefill_matmul(x: torch.Tensor, q: Q4, *, f32: bool = False, tile: int = 0,
-                   out: torch.Tensor | None = None) -> torch.Tensor:
-    """Prompt-form x @ W.T on f16 MFMA: every weight is rounded once (256 w to fp16) and K is one fp32 chain, so
-    chunking a prompt never changes a row's bits (they differ from ``matmul``'s)."""
+                   out: torch.Tensor | None = None, arith: int | None = None) -> torch.Tensor:
+    """Prompt-form x @ W.T on MFMA: every weight is rounded once and K is one fp32 chain, so chunking a prompt never
+    changes a row's bits (they differ from ``matmul``'s).  ``arith`` 0: fp16 operands (256 w rounded to fp16;
+    activations beyond +-65504 are clamped); 1: the reference's bf16 operands (w rounded to bf16), slower, with
+    bf16's range; None: what ``pack`` found the weight's scales and biases to need."""
 
     x = _check_x(x, q, "prefill_matmul")
     m = int(x.shape[0])
@@ -232,5 +238,6 @@ def prefill_matmul(x: torch.Tensor, q: Q4, *, f32: bool = False, tile: int = 0,
             or not out.is_contiguous() or out.device != x.device:
         raise ValueError(f"prefill_matmul: out must be contiguous ({m}, {q.n}) {'fp32' if f32 else 'bf16'}")
     _lib.call("tf_qmm_prefill", _lib.ptr(x), x.stride(0), _lib.ptr(q.weight), _lib.ptr(q.scales.contiguous()),
-              _lib.ptr(q.biases.contiguous()), _lib.ptr(out), m, q.n, q.k, q.gs, int(f32), tile)
+              _lib.ptr(q.biases.contiguous()), _lib.ptr(out), m, q.n, q.k, q.gs, int(f32), tile,
+              q.arith if arith is None else int(arith))
     return out

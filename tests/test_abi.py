@@ -20,17 +20,20 @@ DECLARED = re.findall(r"^(?:int|const char\*)\s+(tf_\w+)\(", HEADER, flags=re.M)
 
 def test_library_exports_the_header():
     assert len(DECLARED) >= 19
-    so = ctypes.CDLL(str(build.LIB)) if build.LIB.exists() else build.load()
+    so = build.load()
     for name in DECLARED:
         assert hasattr(so, name), name
     so.tf_version.restype = ctypes.c_int
-    assert so.tf_version() == 1
+    assert so.tf_version() == 2
+    # the library says which sources it was built from, and the loader only hands out one built from these
+    so.tf_build_id.restype = ctypes.c_char_p
+    assert so.tf_build_id().decode() == build.source_id() == build.built_id() and not build.stale()
     so.tf_last_error.restype = ctypes.c_char_p
     assert so.tf_last_error() == b""
 
 
 def test_ctypes_table_covers_the_header():
-    compute = [n for n in DECLARED if n not in ("tf_last_error", "tf_version", "tf_check_device")]
+    compute = [n for n in DECLARED if n not in ("tf_last_error", "tf_version", "tf_build_id", "tf_check_device")]
     assert sorted(compute) == sorted(_lib.PROTOTYPES)
     for name, args in _lib.PROTOTYPES.items():                 # argument counts against the header's text
         decl = re.search(name + r"\((.*?)\);", HEADER, flags=re.S).group(1)
@@ -78,7 +81,7 @@ def test_argument_errors_come_before_the_gpu():
     with pytest.raises(ValueError, match="gate and an up"):
         experts.make([], (), 64)
     with pytest.raises(ValueError):
-        fmt.check_bits(4.5)
+        fmt.check_bits(4.5)                       # a dense layer's checkpoint never holds it (the routed experts take it)
     with pytest.raises(ValueError):
         fmt.bits_of((4, 4, 36))
 

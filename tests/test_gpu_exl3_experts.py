@@ -52,6 +52,10 @@ MIXED = [
     ("mul1", lambda e: ((1, 1.5, 2.5, 3, 3.5, 4, 5, 6, 7, 8)[e % 10],) * 2 + ((1.5, 2.5, 3.5, 4, 8)[e % 5],)),
     ("mcg", lambda e: ((1, 2, 3, 4, 5, 6, 7, 8)[e % 8],) * 2 + ((2, 3, 4)[e % 3],)),
     ("3inst", lambda e: ((1, 2, 3, 4, 5, 6, 7, 8)[(e + 3) % 8],) * 2 + ((4, 3, 8)[e % 3],)),
+    # the half-bit widths past 3.5 and half-bit widths off the mul1 codebook (the reference's experts take every count)
+    ("3inst", lambda e: ((4.5, 5.5, 6.5, 7.5, 1.5, 2.5, 3.5)[e % 7],) * 2 + ((4.5, 7.5, 2.5)[e % 3],)),
+    ("mcg", lambda e: ((7.5, 6.5, 5.5, 4.5)[e % 4],) * 2 + ((5.5, 6.5)[e % 2],)),
+    ("mul1", lambda e: ((4.5, 5.5, 6.5, 7.5)[e % 4],) * 2 + ((7.5, 4.5, 6.5)[e % 3],)),
 ]
 
 
@@ -176,10 +180,11 @@ def test_bad_arguments_raise():
         experts.routed(x, sel, w.double(), ex, scratch, None, 2)
     with pytest.raises(ValueError):
         experts.routed(x, sel, w, ex, scratch, None, 2, act_mode=5)
-    t = torch.zeros((16, 8, 16 * 3 + 8), dtype=torch.int16, device=DEV)          # 3.5 bits needs mul1
     v = torch.ones(256, dtype=torch.float16, device=DEV)
-    with pytest.raises(ValueError):
-        experts.prepare([(t, v, v[:128])], [(t, v, v[:128])], [(t.reshape(8, 16, -1), v[:128], v)], "mcg")
+    for last in (16 * 3 + 4, 8 * 17, 8):                # not whole half-bits; 8.5 bits; half a bit
+        t = torch.zeros((16, 8, last), dtype=torch.int16, device=DEV)
+        with pytest.raises(ValueError):
+            experts.prepare([(t, v, v[:128])], [(t, v, v[:128])], [(t.reshape(8, 16, -1), v[:128], v)], "mcg")
     with pytest.raises(ValueError):
         experts.prepare([], [], [], "mcg")
     with pytest.raises(ValueError):

@@ -273,3 +273,64 @@ def test_bad_arguments_raise():
         experts.route(torch.zeros((5, 3), dtype=torch.int32, device=DEV), plan)
     with pytest.raises(ValueError):
         experts.make([w, w, w], w, 64)
+
+
+def test_prompt_experts_beyond_the_range_of_fp16():
+    """A layer whose scales do not fit the fp16 prompt form is made for the bf16 form (the reference's arithmetic) and
+    its prompt plan runs in it: against the oracle with the same once-rounded weights, every item size the same bits."""
+
+    from oracle import native
+    from tests.helpers import bits16
+
+    gs, e, d, ni, rows = 32, 9, 256, 128, 150
+    g = torch.Generator().manual_seed(17)
+
+    def table(n, k, lo):
+        words = synthetic.affine_general(n, k, gs, n + k, (e,))[0]
+        scales = (torch.rand((e, n, k // gs), generator=g) * lo + lo).bfloat16()
+        return words, scales, (scales.float() * -7.5).bfloat16()
+
+    up, down = [table(ni, d, 150.0)], table(d, ni, 0.01)                 # only the up table is out of range
+    ex = experts.make([tuple(t.to(DEV) for t in m) for m in up], tuple(t.to(DEV) for t in down), gs)
+    assert ex.arith == experts.ARITH_BF16
+    fits = experts.make([tuple(t.to(DEV) for t in down)], tuple(t.to(DEV) for t in table(ni, ni, 0.01)), gs)
+    assert fits.arith == experts.ARITH_F16
+    x = (synthetic.activations(rows, d, 18).float() * 300).bfloat16()
+    picks = torch.stack([torch.randperm(e, generator=g)[:3] for _ in range(rows)]).to(torch.int32)
+    wts = torch.full((rows, 3), 1 / 3)
+    got = {t: run(ex, x.to(DEV), picks, prefill=True, tile=t) for t in (16, 64, 128)}
+    for t in (64, 128):
+        assert torch.equal(got[16][0], got[t][0]) and torch.equal(got[16][1], got[t][1]), t
+    act, y, _ = got[128]
+    assert torch.isfinite(y).all()
+    tab = lambda m: (u32(m[0]), bits16(m[1]), bits16(m[2]))
+    _, act_ref, y_ref = native.moe_layer(bits16(x), picks.numpy(), wts.numpy(), None, tab(up[0]), tab(down), gs,
+                                         prefill=2, want_pairs=True)
+    assert rel_l2(f32(act), ora.bf16_from_bits(act_ref)) <= 2e-3          # relu^2 on bf16 roundings: a few flipped steps
+    assert rel_l2(f32(y), y_ref) <= 2e-3
+    print(f"bf16 prompt form: act rel-L2 {rel_l2(f32(act), ora.bf16_from_bits(act_ref)):.2e}, "
+          f"y rel-L2 {rel_l2(f32(y), y_ref):.2e}, max-abs {max_abs(f32(y), y_ref):.3e}")
+
+
+def test_group_sums_kept_by_a_plan_are_dropped_when_the_activations_are_rewritten():
+    """``down`` reuses the group sums ``gate_up`` left in its plan only while that call is still the last one to have
+    written the activation buffer: a second ``gate_up`` into the same buffer under another plan voids them."""
+
+    case = CASES[2]
+    ex, _, _ = build(case, 53)
+    rows = 6
+    picks = picks_for(rows, case, 54).to(DEV).contiguous()
+    slots = picks.shape[1]
+    x1 = synthetic.activations(rows, ex.dims, 55, 0.5).to(DEV)
+    x2 = synthetic.activations(rows, ex.dims, 56, 2.0).to(DEV)
+    a, b = experts.Plan(rows, slots, ex.count, DEV), experts.Plan(rows, slots, ex.count, DEV)
+    experts.route(picks, a)
+    experts.route(picks, b)
+    act = torch.empty((rows * slots, ex.width), dtype=torch.bfloat16, device=DEV)
+    experts.gate_up(x1, ex, a, act, rows)
+    experts.gate_up(x2, ex, b, act, rows)             # the buffer now holds x2's activations; a's sums are x1's
+    ya = torch.empty((rows * slots, ex.dims), dtype=torch.float32, device=DEV)
+    yb = torch.empty_like(ya)
+    experts.down(act, ex, a, ya, rows)
+    experts.down(act, ex, b, yb, rows)
+    assert torch.equal(ya, yb)

@@ -170,3 +170,62 @@ def test_bad_arguments_raise():
         qmm.matmul(x, q, sk=4, part=torch.empty((2, 2, 64), device=DEV))       # room for 2 of the 4 slices
     with pytest.raises(ValueError, match="out must be"):
         qmm.matmul(x, q, out=torch.empty((1, 64), device=DEV, dtype=torch.bfloat16))
+
+
+def test_the_bf16_prompt_form_is_the_references_arithmetic():
+    """``arith=1``: every weight bf16(fma(q, s, b)), bf16 activations, bf16 MFMA, one fp32 chain (the reference's
+    kernels/qmm_prefill.cu:116-117).  Equal to the oracle with the same once-rounded weights to fp32 rounding, rows
+    independent of the row count, and (with eight times the fp16 form's weight rounding) further from the fp32-weight
+    oracle than the fp16 form is."""
+
+    for n, k, gs in ((512, 2048, 32), (200, 1024, 64)):
+        w = synthetic.affine_general(n, k, gs, 5 * n + k)
+        x = synthetic.activations(70, k, 6)
+        q = qmm.pack(*gpu(*w), gs)
+        assert q.arith == 0                                     # these scales and biases fit the fp16 form
+        want = native.affine_linear(bits16(x), u32(w[0]), bits16(w[1]), bits16(w[2]), gs, prefill=2)
+        got = qmm.prefill_matmul(x.to(DEV), q, f32=True, arith=1)
+        assert rel_l2(f32(got), want) <= 1e-5
+        exact = native.affine_linear(bits16(x), u32(w[0]), bits16(w[1]), bits16(w[2]), gs)
+        e16, e_bf = rel_l2(f32(qmm.prefill_matmul(x.to(DEV), q, f32=True)), exact), rel_l2(f32(got), exact)
+        print(f"{n}x{k} g{gs}: fp16 form {e16:.2e}, bf16 form {e_bf:.2e} from the fp32-weight oracle")
+        assert e16 < e_bf <= 8e-3
+        for m in (1, 16, 17, 64, 65):
+            assert torch.equal(qmm.prefill_matmul(x[:m].to(DEV), q, f32=True, arith=1), got[:m]), m
+
+
+def test_prompt_form_beyond_the_range_of_fp16():
+    """Scales around 300 and activations around 1e5: 256 x scale has no fp16 value, so ``pack`` marks the weight for
+    the bf16 form and ``prefill_matmul`` takes it by itself; the result matches the oracle (2e-3 against the oracle
+    with the same once-rounded weights is loose: it measures 1e-6; against fp32 weights the bf16 rounding shows).
+    With a table that fits, the fp16 form clamps activations beyond +-65504, no more and no less."""
+
+    n, k, gs = 256, 1024, 64
+    g = torch.Generator().manual_seed(91)
+    words = synthetic.affine_general(n, k, gs, 92)[0]
+    scales = (torch.rand((n, k // gs), generator=g) * 200 + 200).bfloat16()               # 200 to 400
+    biases = (scales.float() * -7.5).bfloat16()
+    x = (torch.randn((40, k), generator=g) * 1e5).bfloat16()
+    q = qmm.pack(words.to(DEV), scales.to(DEV), biases.to(DEV), gs)
+    assert q.arith == 1
+    got = qmm.prefill_matmul(x.to(DEV), q, f32=True)
+    assert torch.isfinite(got).all()
+    same = native.affine_linear(bits16(x), u32(words), bits16(scales), bits16(biases), gs, prefill=2)
+    exact = native.affine_linear(bits16(x), u32(words), bits16(scales), bits16(biases), gs)
+    err, err_exact = rel_l2(f32(got), same), rel_l2(f32(got), exact)
+    print(f"beyond fp16: rel-L2 {err:.2e} (same rounded weights), {err_exact:.2e} (fp32 weights), "
+          f"max-abs {max_abs(f32(got), same):.3e} of {np.abs(same).max():.3e}")
+    assert err <= 1e-5 and err_exact <= 8e-3
+    assert rel_l2(f32(qmm.matmul(x.to(DEV), q, f32=True)), exact) <= 1e-5            # the decode form never minded
+    # a table that fits fp16 with activations that do not: the fp16 form is the matmul of the clamped activations
+    small = synthetic.affine_general(n, k, gs, 93)
+    q2 = qmm.pack(*gpu(*small), gs)
+    assert q2.arith == 0
+    clamped = x.float().clamp(-65504, 65504).bfloat16()
+    assert not torch.equal(clamped, x)
+    want = native.affine_linear(bits16(clamped), u32(small[0]), bits16(small[1]), bits16(small[2]), gs, prefill=True)
+    unclamped = native.affine_linear(bits16(x), u32(small[0]), bits16(small[1]), bits16(small[2]), gs, prefill=2)
+    got16 = f32(qmm.prefill_matmul(x.to(DEV), q2, f32=True))
+    # (the oracle's clamp lands on bf16's 65536, the kernel's on fp16's 65504: 5e-4 apart)
+    assert rel_l2(got16, want) <= 1e-3 and rel_l2(got16, unclamped) > 0.1
+    assert rel_l2(f32(qmm.prefill_matmul(x.to(DEV), q2, f32=True, arith=1)), unclamped) <= 1e-5
