@@ -243,6 +243,19 @@ __device__ __forceinline__ void wave_block(const uint16_t* xr, const uint32_t* t
     __builtin_amdgcn_wave_barrier();         // the wave's LDS accesses run in program order: no wait beyond the data's
     fetch(pr + 1 < pr1 ? pr + 1 : pr, g, an);
     const f16x8_t a = __builtin_bit_cast(f16x8_t, av);
+    // 3inst and mcg: a value is the sum of the two fp16 halves of its hashed word.  The matrix unit adds them: the
+    // four hashed words of a tile are the B operand as they stand (eight fp16 numbers) against every input twice
+    // over, so the add costs no vector instruction.  The products are exact in fp32, so each weight enters as the
+    // exact sum of its halves (the stored value is that sum rounded to fp16: at most 2^-12 relative apart).
+    f16x8_t a0, a1;
+    if constexpr (CB != 2) {
+      const u32x4_t lo = {__builtin_amdgcn_perm(av[0], av[0], 0x01000100u), __builtin_amdgcn_perm(av[0], av[0], 0x03020302u),
+                          __builtin_amdgcn_perm(av[1], av[1], 0x01000100u), __builtin_amdgcn_perm(av[1], av[1], 0x03020302u)};
+      const u32x4_t hi = {__builtin_amdgcn_perm(av[2], av[2], 0x01000100u), __builtin_amdgcn_perm(av[2], av[2], 0x03020302u),
+                          __builtin_amdgcn_perm(av[3], av[3], 0x01000100u), __builtin_amdgcn_perm(av[3], av[3], 0x03020302u)};
+      a0 = __builtin_bit_cast(f16x8_t, lo);
+      a1 = __builtin_bit_cast(f16x8_t, hi);
+    }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       uint32_t w0[NW], w1[NW];
@@ -251,12 +264,22 @@ __device__ __forceinline__ void wave_block(const uint16_t* xr, const uint32_t* t
         w0[q] = stage[j * TWP + win.wi + q];
         w1[q] = stage[(8 + j) * TWP + win.wi + q];
       }
-      uint32_t b0, b1, b2, b3;
-      decode4<K2, CB>(win, w0, b0, b1);
-      decode4<K2, CB>(win, w1, b2, b3);
-      const u32x4_t bw = {b0, b1, b2, b3};
-      const f16x8_t b = __builtin_bit_cast(f16x8_t, bw);
-      acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[j], 0, 0, 0);
+      if constexpr (CB != 2) {
+        uint32_t s0[4], s1[4];
+        win.states(w0, s0);
+        win.states(w1, s1);
+        const u32x4_t x0 = {code_word<CB>(s0[0]), code_word<CB>(s0[1]), code_word<CB>(s0[2]), code_word<CB>(s0[3])};
+        const u32x4_t x1 = {code_word<CB>(s1[0]), code_word<CB>(s1[1]), code_word<CB>(s1[2]), code_word<CB>(s1[3])};
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, __builtin_bit_cast(f16x8_t, x0), acc[j], 0, 0, 0);
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, __builtin_bit_cast(f16x8_t, x1), acc[j], 0, 0, 0);
+      } else {
+        uint32_t b0, b1, b2, b3;
+        decode4<K2, CB>(win, w0, b0, b1);
+        decode4<K2, CB>(win, w1, b2, b3);
+        const u32x4_t bw = {b0, b1, b2, b3};
+        const f16x8_t b = __builtin_bit_cast(f16x8_t, bw);
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[j], 0, 0, 0);
+      }
     }
     __builtin_amdgcn_wave_barrier();
     av = an;

@@ -26,22 +26,20 @@ def k2_of(bits: float) -> int:
     return int(2 * fmt.check_bits(bits))
 
 
-def plan(k: int, n: int, waves: int = 4608, min_pairs: int = 4) -> tuple[int, int]:
+def plan(k: int, n: int, waves: int = 4096, min_pairs: int = 4) -> tuple[int, int]:
     """(K splits, waves a workgroup) of a K x N layer, from the shape alone so that a layer keeps one reduction
-    order at every row count.  The decode is arithmetic-bound and wants about four waves on each of an MI355X's
-    1,024 SIMDs: K is split while N/128 * splits * 4 stays within ``waves`` and every wave keeps ``min_pairs`` pairs
-    of k tiles."""
+    order at every row count.  The decode is bound by vector arithmetic, every wave of a launch is resident at once,
+    and the launch ends with the busiest SIMD: a column block of 128 gets as many waves (splits x waves a workgroup)
+    as put just under four on each of an MI355X's 1,024 SIMDs, none of them with fewer than ``min_pairs`` pairs of k
+    tiles.  Many waves a block go eight a workgroup, so that the splits' partial sums stay few."""
 
     pairs, nb = k // 32, n // 128
-    wk = 4
-    while wk > 2 and pairs // wk < min_pairs:
+    slots = max(2, min(waves // max(nb, 1), pairs // min_pairs, 512))
+    wk = 8 if slots >= 64 else (4 if slots >= 8 else 2)
+    sk = max(1, min(64, slots // wk))
+    while wk > 2 and sk * wk > pairs:
         wk //= 2
-    sk = 1
-    while sk < 64 and nb * 2 * sk * wk <= waves and pairs // (2 * sk * wk) >= min_pairs:
-        sk *= 2
-    if wk == 4 and nb * sk * 8 <= 5120 and pairs // (sk * 8) >= min_pairs:
-        wk = 8              # few column blocks: five waves a SIMD (the kernel's register budget) still fit
-    return sk, wk
+    return min(sk, max(1, pairs // wk)), wk
 
 
 def strips(words: torch.Tensor) -> torch.Tensor:
