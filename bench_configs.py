@@ -1,7 +1,7 @@
 """Kernel timings of the benchmark configurations that are not bench.py's headline: 0 (dense 4-bit projection),
 2 (verify-window MoE layer), 3 (prompt chunk, grouped MFMA) and 4 (EXL3 projections).
 
-    python bench_configs.py [c0] [c2] [c3] [c4] [c4p] [glue] [c4x]
+    python bench_configs.py [c0] [c2] [c3] [c4] [c4p] [glue] [c4x] [mfma]
 
 One JSON line a configuration: time of one pass (hipGraph of back-to-back passes cycling over enough weight copies to
 miss the 256 MB Infinity Cache, HIP events around the replay), algorithmic bytes or flops, and the fraction of the
@@ -306,11 +306,27 @@ def c4x() -> dict:
             "bound": "hbm", "rows": out}
 
 
+def mfma() -> dict:
+    """Issue rates of the candidate matrix instructions (f16, fp8, block-scaled fp8), bare and with the per-group fma
+    of an 8-bit prompt path: the stand-alone probe built beside the library (csrc/probe_mfma.hip), its table as text."""
+
+    import subprocess
+
+    from tensorfold_amd import build
+
+    if not build.PROBE.exists():
+        raise RuntimeError(f"{build.PROBE} is missing: run `python -c 'import __graft_entry__ as g; g.build()'`")
+    done = subprocess.run([str(build.PROBE)], capture_output=True, text=True, timeout=120)
+    if done.returncode:
+        raise RuntimeError(f"probe_mfma failed: {done.stderr}")
+    return {"config": "mfma: issue rates of the matrix instructions (probe_mfma)", "lines": done.stdout.splitlines()}
+
+
 def main() -> int:
     torch.cuda.set_device(0)
     which = sys.argv[1:] or ["c0", "c2", "c3", "c4"]
     for name in which:
-        res = {"c0": c0, "c2": c2, "c3": c3, "c4": c4, "c4p": c4p, "glue": glue_, "c4x": c4x}[name]()
+        res = {"mfma": mfma, "c0": c0, "c2": c2, "c3": c3, "c4": c4, "c4p": c4p, "glue": glue_, "c4x": c4x}[name]()
         torch.cuda.empty_cache()
         print(json.dumps(res, default=lambda v: round(v, 4)), flush=True)
     return 0

@@ -18,6 +18,7 @@ ARCH = "gfx950"
 HERE = Path(__file__).resolve().parent
 CSRC = HERE / "csrc"
 LIB = HERE / "libtfmi.so"
+PROBE = HERE / "probe_mfma"          # stand-alone measurement of the matrix instructions' issue rates (csrc/probe_mfma.hip)
 SOURCES = ("api.hip", "pack.hip", "decode.hip", "fused.hip", "route.hip", "norm.hip", "prefill.hip", "exl3.hip", "exl3_experts.hip")
 # packed-fp32 VALU forms are switched off for the device pass (the host pass warns that it does not know the feature)
 FLAGS = ("-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",
@@ -89,6 +90,7 @@ def compile(verbose: bool = False) -> Path:
             logs = list(pool.map(lambda so: run([cc, *compile_flags, "-c", str(CSRC / so[0]), "-o", so[1]]),
                                  zip(SOURCES, objects)))
         logs.append(run([cc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", str(LIB), *objects]))
+        logs.append(run([cc, "-O3", f"--offload-arch={ARCH}", "-o", str(PROBE), str(CSRC / "probe_mfma.hip")]))
     if verbose:
         for text in logs:
             if text:
