@@ -50,6 +50,13 @@ __device__ __forceinline__ uint32_t sb_half2(uint32_t v) {
   return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(__uint_as_float(u << 16), __uint_as_float(u & 0xFFFF0000u)));
 }
 
+// The same from a scale and a bias still apart (each a bf16 in the low half of its register): the dense layout keeps
+// them in two arrays, and joining them when they are loaded would make every step wait for loads it has just issued.
+__device__ __forceinline__ uint32_t sb_half2(uint2 v) {
+  return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(__uint_as_float((v.x + 0x0400u) << 16),
+                                                                  __uint_as_float((v.y + 0x0400u) << 16)));
+}
+
 // q * s + b on two fp16 lanes, s and b being the low and high half of one register (the splats fold into the
 // packed instruction's operand selects)
 __device__ __forceinline__ f16x2_t fma_sb(f16x2_t q, uint32_t sb) {
@@ -324,16 +331,17 @@ constexpr int BIG_THREADS = BIG_WAVES * 64;
 // chunks of the step, and the stored (scale | bias << 16) pair of each operand and group of the step.  Buffer loads:
 // the base in scalar registers, the step as the scalar offset, the lane's part as the vector offset and the chunk or
 // group as the immediate, so no address arithmetic is left on the vector unit.
-template <int GS, int NM>
+template <int GS, int NM, int TJ = 4>
 struct ExpertSource {
   static constexpr int CPS = KSTEP / 32, GPS = KSTEP / GS;
   static constexpr uint32_t GSTRIDE = NM * block_words(GS);      // words from one group to the next
+  typedef uint32_t SB;                                            // a column's stored (scale | bias << 16)
   __amdgpu_buffer_rsrc_t rsrc;                                    // one expert's matrices
-  uint32_t wp[4], sp[4];                                          // word offsets inside the expert: below 2^32
-  __device__ __forceinline__ void load(int step, uint32_t (&w)[4][CPS], uint32_t (&sb)[4][GPS]) const {
+  uint32_t wp[TJ], sp[TJ];                                        // word offsets inside the expert: below 2^32
+  __device__ __forceinline__ void load(int step, uint32_t (&w)[TJ][CPS], uint32_t (&sb)[TJ][GPS]) const {
     const int soff = step * (int)(GPS * GSTRIDE * 4);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < TJ; ++j) {
 #pragma unroll
       for (int i = 0; i < CPS; ++i)
         w[j][i] = __builtin_amdgcn_raw_buffer_load_b32(
@@ -346,60 +354,61 @@ struct ExpertSource {
 };
 
 // The dense layout: codes [n / 64][K / gs][gs / 32][64][4] words, scales and biases bf16 [K / gs][npad].
-template <int GS>
+template <int GS, int TJ = 4>
 struct DenseSource {
   static constexpr int CPS = KSTEP / 32, GPS = KSTEP / GS;
+  typedef uint2 SB;                                               // a column's scale and bias, joined where they are used
   __amdgpu_buffer_rsrc_t codes, scales, biases;
-  uint32_t wp[4], cp[4];                                          // byte offsets: the lane's word; its column's bf16
+  uint32_t wp[TJ], cp[TJ];                                        // byte offsets: the lane's word; its column's bf16
   int row_bytes;                                                  // bytes from one group's scales to the next
-  __device__ __forceinline__ void load(int step, uint32_t (&w)[4][CPS], uint32_t (&sb)[4][GPS]) const {
+  __device__ __forceinline__ void load(int step, uint32_t (&w)[TJ][CPS], SB (&sb)[TJ][GPS]) const {
     const int soff = step * (KSTEP / 32) * 1024;                  // 32 inputs of a 64-column tile are 1 KB of codes
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < TJ; ++j) {
 #pragma unroll
       for (int i = 0; i < CPS; ++i) w[j][i] = __builtin_amdgcn_raw_buffer_load_b32(codes, wp[j] + i * 1024, soff, 0);
 #pragma unroll
       for (int gi = 0; gi < GPS; ++gi) {
         const int goff = (step * GPS + gi) * row_bytes;
-        const uint32_t sv = __builtin_amdgcn_raw_buffer_load_b16(scales, cp[j], goff, 0);
-        const uint32_t bv = __builtin_amdgcn_raw_buffer_load_b16(biases, cp[j], goff, 0);
-        sb[j][gi] = sv | (bv << 16);
+        sb[j][gi].x = __builtin_amdgcn_raw_buffer_load_b16(scales, cp[j], goff, 0);
+        sb[j][gi].y = __builtin_amdgcn_raw_buffer_load_b16(biases, cp[j], goff, 0);
       }
     }
   }
 };
 
-template <int GS, int NM, int EPI, int RT, class WS>
+template <int GS, int NM, int EPI, int RT, class WS, int TJ = 4, int NTHREADS = BIG_THREADS>
 __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t x_stride, const WS& ws,
-                                         const int (&ocol)[4], const bool (&jok)[4],
+                                         const int (&ocol)[TJ], const bool (&jok)[TJ],
                                          int K, const int* src_rows, const int* dst_rows, int cnt,
                                          void* __restrict__ out, int N, float limit, unsigned char* smem) {
-  constexpr int TJ = 4, CPS = KSTEP / 32, GPS = KSTEP / GS;
+  constexpr int CPS = KSTEP / 32, GPS = KSTEP / GS;
   constexpr int ROWS = 16 * RT;
   constexpr int PIECES = ROWS * 8;                // 16-byte pieces of a staged tile
-  constexpr int PPT = (PIECES + BIG_THREADS - 1) / BIG_THREADS;
+  constexpr int PPT = (PIECES + NTHREADS - 1) / NTHREADS;
   constexpr int STAGE = BIG_ROWS * AROW;
   const int tid = threadIdx.x, lane = tid & 63, c = lane & 15, kq = lane >> 4;
   const int steps = K / KSTEP;
-  auto load_w = [&](int step, uint32_t (&w)[TJ][CPS], uint32_t (&sb)[TJ][GPS]) { ws.load(step, w, sb); };
+  typedef typename WS::SB SB;
+  auto load_w = [&](int step, uint32_t (&w)[TJ][CPS], SB (&sb)[TJ][GPS]) { ws.load(step, w, sb); };
   // this thread's pieces of the activation tile: piece q = (row q / 8, 16 bytes q % 8)
   const uint16_t* asrc[PPT];
 #pragma unroll
   for (int j = 0; j < PPT; ++j) {
-    const int q = tid + j * BIG_THREADS, r = q >> 3, ch = q & 7;
+    const int q = tid + j * NTHREADS, r = q >> 3, ch = q & 7;
     asrc[j] = X + (size_t)src_rows[r < cnt ? r : 0] * x_stride + ch * 8;
   }
   auto load_a = [&](int step, uint4 (&v)[PPT]) {
 #pragma unroll
     for (int j = 0; j < PPT; ++j)
-      if (PIECES % BIG_THREADS == 0 || tid + j * BIG_THREADS < PIECES)
+      if (PIECES % NTHREADS == 0 || tid + j * NTHREADS < PIECES)
         v[j] = *reinterpret_cast<const uint4*>(asrc[j] + (size_t)step * KSTEP);
   };
   auto store_a = [&](int buf, const uint4 (&v)[PPT]) {
 #pragma unroll
     for (int j = 0; j < PPT; ++j) {
-      const int q = tid + j * BIG_THREADS;
-      if (PIECES % BIG_THREADS == 0 || q < PIECES)
+      const int q = tid + j * NTHREADS;
+      if (PIECES % NTHREADS == 0 || q < PIECES)
         *reinterpret_cast<uint4*>(smem + buf * STAGE + (q >> 3) * AROW + (q & 7) * 16) = stage8(v[j]);
     }
   };
@@ -410,7 +419,8 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
 #pragma unroll
     for (int r = 0; r < RT; ++r) acc[j][r] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
-  uint32_t wr[2][TJ][CPS], sr[2][TJ][GPS];
+  uint32_t wr[2][TJ][CPS];
+  SB sr[2][TJ][GPS];
   uint4 ar[PPT];
   const int last = steps - 1;
   load_w(0, wr[0], sr[0]);
@@ -482,9 +492,9 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
       const size_t base = (size_t)dst_rows[row] * N;
       if constexpr (NM == 2) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TJ / 2; ++j)
           if (jok[j])
-            store_out<EPI>(out, base + ocol[j], acc[j][r][i] * WUNSCALE, acc[j + 2][r][i] * WUNSCALE, limit);
+            store_out<EPI>(out, base + ocol[j], acc[j][r][i] * WUNSCALE, acc[j + TJ / 2][r][i] * WUNSCALE, limit);
       } else {
 #pragma unroll
         for (int j = 0; j < TJ; ++j)
