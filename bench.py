@@ -74,19 +74,18 @@ class Layer:
         _lib.call("tf_moe_route_up", _lib.ptr(l), l.stride(0), self.tokens, SHAPE.experts, SHAPE.top_k, 0, ex.gs,
                   int(ex.swiglu), _lib.ptr(x), x.stride(0), _lib.ptr(ex.up), ex.dims, ex.width, _lib.ptr(buf.pick),
                   _lib.ptr(buf.wts), _lib.ptr(buf.plan.members), _lib.ptr(buf.plan.items), _lib.ptr(buf.plan.counts),
-                  _lib.ptr(f["desc"]), _lib.ptr(buf.act), _lib.ptr(f["xs_act"]), ex.limit, items, None, 0)
+                  _lib.ptr(f["desc"]), _lib.ptr(buf.act), ex.limit, items, None, 0)
 
     def down(self, i: int, buf=None) -> None:
-        """The down projection + combine launch alone (its arrival counters are cleared by a small fill, which the
-        routing launch does in a layer pass; the fill's own time is measured and taken off)."""
+        """The down projection + combine launch alone (the unit that completes a cell leaves its arrival counter at
+        zero, so launches can follow one another)."""
 
         ex, buf = self.tables[i % len(self.tables)], buf or self.buf
         f = buf.fused(SHAPE.gs)
         items = experts.max_items(self.tokens * buf.slots, SHAPE.experts, moe.DESC_TILE)
         ctr = f["counters"]
-        ctr.zero_()
         _lib.call("tf_moe_down_combine", ex.gs, _lib.ptr(buf.act), self.tokens, buf.slots, _lib.ptr(ex.down), ex.dims,
-                  ex.width, _lib.ptr(f["desc"]), _lib.ptr(buf.wts), _lib.ptr(f["xs_act"]), _lib.ptr(buf.y),
+                  ex.width, _lib.ptr(f["desc"]), _lib.ptr(buf.wts), _lib.ptr(buf.y),
                   _lib.ptr(self.out), ctr.data_ptr() + 4 * (1 + f["items"]), items)
 
     def route_plans(self) -> float:
@@ -110,7 +109,8 @@ class Layer:
                    SHAPE.experts, self.out)
 
     def fused_experts(self, i: int, buf) -> None:
-        """The fused experts launch alone, on a pre-routed buffer (its counters are cleared by a small fill)."""
+        """The fused experts launch alone, on a pre-routed buffer, with the small fill that clears its counters (the
+        figure includes the fill)."""
 
         ex, f = self.tables[i % len(self.tables)], buf.fused(SHAPE.gs)
         f["counters"].zero_()
@@ -119,8 +119,8 @@ class Layer:
         ctr = f["counters"]
         _lib.call("tf_moe_decode_experts", ex.gs, int(ex.swiglu), _lib.ptr(self.x[i % 4]), self.x[i % 4].stride(0), n,
                   buf.slots, _lib.ptr(ex.up), _lib.ptr(ex.down), ex.dims, ex.width, _lib.ptr(f["desc"]),
-                  _lib.ptr(buf.plan.counts), _lib.ptr(buf.wts), _lib.ptr(f["xs_x"]), _lib.ptr(buf.act),
-                  _lib.ptr(f["xs_act"]), _lib.ptr(buf.y), _lib.ptr(self.out), ctr.data_ptr() + 4,
+                  _lib.ptr(buf.plan.counts), _lib.ptr(buf.wts), _lib.ptr(buf.act),
+                  _lib.ptr(buf.y), _lib.ptr(self.out), ctr.data_ptr() + 4,
                   ctr.data_ptr() + 4 * (1 + f["items"]), _lib.ptr(ctr), ex.limit, items)
 
     def unique_experts(self, i: int) -> int:
@@ -188,9 +188,8 @@ def run_batch(tokens: int, tables, steps: int, warmup: int, dev: str) -> dict:
         return a.elapsed_time(b) * 1e3 / reps
 
     u0 = layer.route_plans()
-    fill_us = kernel_us(lambda i, b: b.fused(SHAPE.gs)["counters"].zero_())
-    up_us, down_us = kernel_us(layer.up), kernel_us(layer.down) - fill_us
-    fused_us = kernel_us(layer.fused_experts) - fill_us
+    up_us, down_us = kernel_us(layer.up), kernel_us(layer.down)
+    fused_us = kernel_us(layer.fused_experts)
     layer.buf.check()
     half = bytes_per_expert(s) // 2
     act_bytes = tokens * s.top_k * (s.hidden + s.width) * 2
@@ -256,7 +255,11 @@ def other_configs() -> dict:
 
     import bench_configs as bc
 
-    rnd = lambda v: round(v, 4) if isinstance(v, float) else v
+    def rnd(v):
+        if isinstance(v, dict):
+            return {k: rnd(u) for k, u in v.items()}
+        return round(v, 4) if isinstance(v, float) else v
+
     out = {}
     r = bc.c0()
     out["c0"] = {"workload": r["config"],
@@ -274,7 +277,9 @@ def other_configs() -> dict:
                  "down_us": rnd(t["down_us"]), "combine_us": rnd(t["combine_us"]), "items": t["items"]}
     torch.cuda.empty_cache()
     r = bc.c4()
-    out["c4"] = {"workload": r["config"], "bound": "hbm",
+    # two rooflines: the stream of trellis words against HBM, and the decode's vector instructions against the
+    # vector units, which is the one that binds (`roofline_valu`, of the 1-row pass)
+    out["c4"] = {"workload": r["config"], "bound": "hbm", "roofline_valu": rnd(r["rows"][1]["valu"]),
                  "rows": {str(m): {k: rnd(v) for k, v in d.items()} for m, d in r["rows"].items()}}
     torch.cuda.empty_cache()
     return out

@@ -1,7 +1,7 @@
 """Kernel timings of the benchmark configurations that are not bench.py's headline: 0 (dense 4-bit projection),
 2 (verify-window MoE layer), 3 (prompt chunk, grouped MFMA) and 4 (EXL3 projections).
 
-    python bench_configs.py [c0] [c2] [c3] [c4] [c4p] [glue] [c4x] [mfma]
+    python bench_configs.py [c0] [c2] [c3] [c4] [c4p] [glue] [c4x] [mfma] [floor]
 
 One JSON line a configuration: time of one pass (hipGraph of back-to-back passes cycling over enough weight copies to
 miss the 256 MB Infinity Cache, HIP events around the replay), algorithmic bytes or flops, and the fraction of the
@@ -20,6 +20,12 @@ from tensorfold_amd.exl3 import linear as exl3
 
 DEV = "cuda:0"
 HBM, MFMA = 8000.0, 2500.0          # GB/s, TFLOP/s
+# Vector-unit peak in lane-operations a second: 256 CUs x 4 SIMDs x 16 lanes a cycle at the 2.4 GHz peak clock.
+VALU = 256 * 4 * 16 * 2.4e9
+# Vector instructions the EXL3 linear kernel spends on a weight: its loop over a pair of k tiles decodes 64 weights a
+# lane (4,096 a wave) in 310 vector instructions beside 16 matrix ones (counted in the compiled loop of
+# linear_kernel<6, 0, 8>; the 3INST hash alone is a bit-field extract, a multiply, an add and a bit operation).
+EXL3_VALU_PER_WEIGHT = 310 / 64
 
 
 def graph_us(step, reps: int) -> float:
@@ -209,9 +215,13 @@ def c4() -> dict:
         down_us = graph_us(lambda i: mlps[i % 4][2](h, yd, xh=hh, z=z), 48)
         per = 5120 * 17408 * 3 // 8
         nbytes = 3 * per + 3 * 2 * (5120 + 17408) + m * (2 * 5120 + 17408 + 17408 * 2 + 5120) * 2
+        ops = 3 * 5120 * 17408 * EXL3_VALU_PER_WEIGHT          # lane-operations of one MLP's decode
         out[m] = {"mlp_us": us, "bytes": nbytes, "gbs": nbytes / us * 1e-3, "frac": nbytes / us * 1e-3 / HBM,
                   "gate_us": gate_us, "gate_gbs": per / gate_us * 1e-3, "down_us": down_us,
-                  "down_gbs": per / down_us * 1e-3}
+                  "down_gbs": per / down_us * 1e-3,
+                  "valu": {"bound": "valu", "achieved": ops / us * 1e-6, "peak": VALU * 1e-12, "unit": "Tlane-op/s",
+                           "frac": ops / us * 1e6 / VALU, "ops_per_weight": EXL3_VALU_PER_WEIGHT,
+                           "floor_us": ops / VALU * 1e6}}
     return {"config": "c4: EXL3 3.0 bpw MLP, gate/up 5120 -> 17408, down 17408 -> 5120 (input rotation + linear kernel each)",
             "bound": "hbm", "rows": out}
 
@@ -322,11 +332,38 @@ def mfma() -> dict:
     return {"config": "mfma: issue rates of the matrix instructions (probe_mfma)", "lines": done.stdout.splitlines()}
 
 
+def floor() -> dict:
+    """What a launch costs and how fast a short stream runs: a graph of one-workgroup kernels (the gap a launch adds
+    to a layer of two launches), and plain streaming reads of the sizes a decode launch moves (17, 34, 113 MB)."""
+
+    from tensorfold_amd import _lib
+
+    x = synthetic.activations(1, 64, 1).to(DEV)
+    xs = torch.empty((1, 1), dtype=torch.float32, device=DEV)
+
+    def tiny(i):
+        _lib.call("tf_group_sums", _lib.ptr(x), x.stride(0), 1, 64, 64, _lib.ptr(xs))
+
+    def pair(i):
+        tiny(i)
+        tiny(i)
+
+    out = {"config": "floor: launch gap in a graph and the streaming rate of short reads",
+           "one_tiny_kernel_us": graph_us(tiny, 200), "two_tiny_kernels_us": graph_us(pair, 100), "reads": {}}
+    for mb in (17, 34, 113):
+        ts = [torch.empty(mb * 1024 * 1024 // 4, dtype=torch.float32, device=DEV).normal_() for _ in range(4)]
+        o = torch.empty((), device=DEV)
+        us = graph_us(lambda i: torch.sum(ts[i % 4], dim=0, out=o), 40)
+        out["reads"][f"{mb}MB"] = {"us": us, "gbs": mb * 1.048576 / us * 1e3}
+        del ts
+    return out
+
+
 def main() -> int:
     torch.cuda.set_device(0)
     which = sys.argv[1:] or ["c0", "c2", "c3", "c4"]
     for name in which:
-        res = {"mfma": mfma, "c0": c0, "c2": c2, "c3": c3, "c4": c4, "c4p": c4p, "glue": glue_, "c4x": c4x}[name]()
+        res = {"mfma": mfma, "c0": c0, "c2": c2, "c3": c3, "c4": c4, "c4p": c4p, "glue": glue_, "c4x": c4x, "floor": floor}[name]()
         torch.cuda.empty_cache()
         print(json.dumps(res, default=lambda v: round(v, 4)), flush=True)
     return 0

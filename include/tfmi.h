@@ -117,13 +117,11 @@ int tf_experts_plan(const int32_t* picks, int64_t pairs, int experts, int tile, 
                     int32_t* counts, int32_t* rank, int32_t* hist, tf_stream_t stream);
 /* Decode form.  epi 0: fp32 out; 1: bf16 relu(bf16 a)^2; 2: bf16 SwiGLU(matrix 0, matrix 1) with clip `limit`.
  * Pair p reads x row p / slots when slots > 0, row p when slots == 0.  max_units = max items * nb bounds the grid;
- * the live item count is read on the device.  xs (may be NULL): fp32 [x rows, kg] group sums of x, as
- * tf_group_sums or a previous call's xs_out gives them; without it each workgroup sums its rows itself.
- * xs_out (may be NULL; epi 1 and 2): receives fp32 [pairs, n / gs], the group sums of the activations written,
- * which is the xs of the down projection over the same pairs.  Replaces experts.cpp:43-48 `run`. */
+ * the live item count is read on the device.  The group sums of the inputs that the affine form needs are taken
+ * by each wave from the inputs it streams (no separate pass, no buffer).  Replaces experts.cpp:43-48 `run`. */
 int tf_experts_run(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg, int nb,
                    const int32_t* items, const int32_t* counts, const int32_t* members, void* out, int n, float limit,
-                   int64_t max_units, const float* xs, float* xs_out, tf_stream_t stream);
+                   int64_t max_units, tf_stream_t stream);
 /* Item descriptors, written by tf_moe_route_decode and tf_moe_route_up for the decode expert kernels: int32 rows of
  * TF_DESC_INTS; row 0 holds the number of descriptors, row 1 + i = {expert, count, first member, 0, pairs[..]}: the plan
  * cut into items of at most TF_DESC_TILE pairs, every full item first (expert order), then the experts' short last
@@ -137,12 +135,12 @@ int tf_experts_run(int gs, int epi, const uint16_t* x, int64_t x_stride, int slo
 /* ints between two cells' arrival counters in `arrive` when rows <= 64 (each alone in 64 bytes); 1 past 64 rows */
 #define TF_ARRIVE_STRIDE 16
 
-/* tf_experts_run with the items given as descriptors; xs is required; counts is not read (kept for symmetry).
+/* tf_experts_run with the items given as descriptors; counts is not read (kept for symmetry).
  * Same bits as tf_experts_run on the same plan.  Same reference counterpart (experts.cpp:43-48 `run`); the
  * descriptor form has none. */
 int tf_experts_run_desc(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg,
                         int nb, const int32_t* desc, const int32_t* counts, void* out, int n, float limit,
-                        int64_t max_items, const float* xs, float* xs_out, tf_stream_t stream);
+                        int64_t max_items, tf_stream_t stream);
 /* Prompt form on MFMA, each weight rounded once as in tf_qmm_prefill (arith: TF_ARITH_*); epi 3: bf16 out.  `tile` is
  * the plan's item size (16, 64 or 128).  Replaces experts.cpp:50-55 `prefill`. */
 int tf_experts_prefill(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg,
@@ -182,42 +180,42 @@ int tf_add_norm(const uint16_t* x, const void* delta, int delta_kind, const floa
  * writes what tf_moe_topk and tf_experts_plan (tile 16) would (pick, wts, members, items, counts) plus the item
  * descriptors that tf_experts_run_desc reads; every other workgroup finds its own item from the
  * logits (with 2 to 64 rows a workgroup a pair: its own row's selection up to its slot, then a rank test of that
- * expert on the other rows) and runs the up unit of tf_experts_run (epilogue relu^2, or SwiGLU when swiglu != 0): act bf16 [pairs, ni] and
- * its group sums xs_act fp32 [pairs, ni / gs]; it also zeroes `zero` (n_zero ints: the next launch's counters).  Same
+ * expert on the other rows) and runs the up unit of tf_experts_run (epilogue relu^2, or SwiGLU when swiglu != 0): act
+ * bf16 [pairs, ni]; it also zeroes `zero` (n_zero ints: the next launch's counters).  Same
  * bits as the separate calls.  logits may be NULL: pick and wts are then inputs (tf_moe_topk ran before, the better
  * order past about 2,048 logits, where reading the rows in every workgroup costs more than a launch) and every
  * workgroup finds its item from the picks.  No counterpart in the reference (moe.py:88-128 issues them one by one). */
 int tf_moe_route_up(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared, int gs, int swiglu,
                     const uint16_t* x, int64_t x_stride, const uint32_t* up, int d, int ni, int32_t* pick, float* wts,
-                    int32_t* members, int32_t* items, int32_t* counts, int32_t* desc, uint16_t* act, float* xs_act,
-                    float limit, int max_items, int32_t* zero, int n_zero, tf_stream_t stream);
+                    int32_t* members, int32_t* items, int32_t* counts, int32_t* desc, uint16_t* act, float limit,
+                    int max_items, int32_t* zero, int n_zero, tf_stream_t stream);
 /* The down projection from item descriptors with the weighted combine folded in: y fp32 [pairs, d] as
  * tf_experts_run_desc (epilogue 0) writes it, and out bf16 [rows, d] with the bits of tf_moe_combine, written by
  * whichever workgroup completes a (token, 64 columns) cell.  `arrive` int32 [rows * ceil(d / 64) * s], s =
  * TF_ARRIVE_STRIDE with rows <= 64 and 1 past that, must be zero on
- * entry (tf_moe_route_up and tf_moe_route_decode clear a `zero` range for this) and is left non-zero.  Fuses
+ * entry (tf_moe_route_up and tf_moe_route_decode clear a `zero` range for this); the workgroup that completes a cell
+ * sets its counter back to zero, so a cell every slot of which held a valid expert is left at zero.  Fuses
  * experts.cpp:43-48 `run` and moe.py:131-151 `combine`. */
 int tf_moe_down_combine(int gs, const uint16_t* act, int rows, int slots, const uint32_t* down, int d, int ni,
-                        const int32_t* desc, const float* wts, const float* xs_act, float* y, uint16_t* out,
-                        int32_t* arrive, int max_items, tf_stream_t stream);
+                        const int32_t* desc, const float* wts, float* y, uint16_t* out, int32_t* arrive,
+                        int max_items, tf_stream_t stream);
 /* The decode layer's routing in one launch (two past 16 rows: the top-k then runs a workgroup a row first), for
- * rows * (top_k + shared) <= 1024: tf_moe_topk, tf_experts_plan (tile 16) and tf_group_sums of x, plus the item
- * descriptors and the zeroing of `zero` (n_zero ints: the counters of tf_moe_down_combine or tf_moe_decode_experts).  No counterpart in the reference, which
- * launches `_topk_rows`, `plan` and its group sums separately (moe.py:103-116, kernels/qmm.py:148-154). */
-int tf_moe_route_decode(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared,
-                        const uint16_t* x, int64_t ldx, int d, int gs, int32_t* pick, float* wts, int32_t* members,
-                        int32_t* items, int32_t* counts, int32_t* desc, float* xs_x, int32_t* zero, int n_zero,
-                        tf_stream_t stream);
+ * rows * (top_k + shared) <= 1024: tf_moe_topk and tf_experts_plan (tile 16), plus the item descriptors and the
+ * zeroing of `zero` (n_zero ints: the counters of tf_moe_down_combine or tf_moe_decode_experts).  No counterpart in
+ * the reference, which launches `_topk_rows` and `plan` separately (moe.py:103-116). */
+int tf_moe_route_decode(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared, int32_t* pick,
+                        float* wts, int32_t* members, int32_t* items, int32_t* counts, int32_t* desc, int32_t* zero,
+                        int n_zero, tf_stream_t stream);
 /* The decode layer's experts in one launch: up (+ relu^2 or SwiGLU), down and the weighted combine, with the bits
- * of tf_experts_run, tf_experts_run and tf_moe_combine run in turn.  desc, counts, wts, xs_x as left by
- * tf_moe_route_decode; scratch act bf16 [pairs, ni], xs_act fp32 [pairs, ni/gs], y fp32 [pairs, d]; counters done
+ * of tf_experts_run, tf_experts_run and tf_moe_combine run in turn.  desc, counts, wts as left by
+ * tf_moe_route_decode; scratch act bf16 [pairs, ni], y fp32 [pairs, d]; counters done
  * [max_items * 64] (one a descriptor, each alone in 256 bytes: TF_DONE_STRIDE ints apart) and arrive [rows * d/64 * s] (s as in tf_moe_down_combine) zero on entry; status[0] is set to 1 if a bounded wait ran out (the output
  * is then invalid).  d and ni multiples of 64.  Fuses experts.cpp:43-48 `run` (twice) and moe.py:131-151 `combine`. */
 int tf_moe_decode_experts(int gs, int swiglu, const uint16_t* x, int64_t x_stride, int rows, int slots,
                           const uint32_t* up, const uint32_t* down, int d, int ni, const int32_t* desc,
-                          const int32_t* counts, const float* wts, const float* xs_x, uint16_t* act, float* xs_act,
-                          float* y, uint16_t* out, int32_t* done, int32_t* arrive, int32_t* status, float limit,
-                          int max_items, tf_stream_t stream);
+                          const int32_t* counts, const float* wts, uint16_t* act, float* y, uint16_t* out,
+                          int32_t* done, int32_t* arrive, int32_t* status, float limit, int max_items,
+                          tf_stream_t stream);
 
 #define TF_EXL3_COUNTER_STRIDE 16
 

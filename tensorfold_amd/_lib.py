@@ -24,13 +24,13 @@ PROTOTYPES = {
     "tf_experts_pack": [P, P, P, I, I, I, I, P, P],
     "tf_experts_unpack": [P, L, I, I, I, I, P, P, P, P],
     "tf_experts_plan": [P, L, I, I, P, P, P, P, P, P],
-    "tf_experts_run": [I, I, P, L, I, P, I, I, P, P, P, P, I, F, L, P, P, P],
-    "tf_experts_run_desc": [I, I, P, L, I, P, I, I, P, P, P, I, F, L, P, P, P],
+    "tf_experts_run": [I, I, P, L, I, P, I, I, P, P, P, P, I, F, L, P],
+    "tf_experts_run_desc": [I, I, P, L, I, P, I, I, P, P, P, I, F, L, P],
     "tf_experts_prefill": [I, I, P, L, I, P, I, I, P, P, P, P, I, F, L, I, I, P],
-    "tf_moe_route_up": [P, L, I, I, I, I, I, I, P, L, P, I, I, P, P, P, P, P, P, P, P, F, I, P, I, P],
-    "tf_moe_down_combine": [I, P, I, I, P, I, I, P, P, P, P, P, P, I, P],
-    "tf_moe_route_decode": [P, L, I, I, I, I, P, L, I, I, P, P, P, P, P, P, P, P, I, P],
-    "tf_moe_decode_experts": [I, I, P, L, I, I, P, P, I, I, P, P, P, P, P, P, P, P, P, P, P, F, I, P],
+    "tf_moe_route_up": [P, L, I, I, I, I, I, I, P, L, P, I, I, P, P, P, P, P, P, P, F, I, P, I, P],
+    "tf_moe_down_combine": [I, P, I, I, P, I, I, P, P, P, P, P, I, P],
+    "tf_moe_route_decode": [P, L, I, I, I, I, P, P, P, P, P, P, P, I, P],
+    "tf_moe_decode_experts": [I, I, P, L, I, I, P, P, I, I, P, P, P, P, P, P, P, P, P, F, I, P],
     "tf_moe_router": [P, L, P, P, I, I, I, P],
     "tf_moe_topk": [P, L, I, I, I, I, P, P, P],
     "tf_moe_combine": [P, I, P, P, I, I, I, P],

@@ -30,12 +30,11 @@ namespace {
 // A workgroup takes (item, pair of 32-column blocks, RBMAX of the item's rows): one pass over its weights, as with
 // item descriptors.  (Taking all of an item's up to 16 rows made it stream the same weights up to eight times, and
 // a compute unit's workgroups together overflow the L2 between passes.)  blockIdx.y picks the rows; see expert_unit.
-template <int GS, int NM, int EPI, int WAVES, bool XSG>
+template <int GS, int NM, int EPI, int WAVES>
 __global__ void __launch_bounds__(WAVES * 64)
     expert_kernel(const uint16_t* __restrict__ X, int64_t x_stride, int slots, const uint32_t* __restrict__ W, int KG,
                   int NB, const int* __restrict__ items, const int* __restrict__ counts,
-                  const int* __restrict__ members, void* __restrict__ out, int N, float limit,
-                  const float* __restrict__ xs_in, float* __restrict__ xs_out) {
+                  const int* __restrict__ members, void* __restrict__ out, int N, float limit) {
   extern __shared__ float lds[];
   const int NB2 = (NB + 1) >> 1;
   const int it = blockIdx.x / NB2, cb2 = blockIdx.x - it * NB2;
@@ -45,8 +44,8 @@ __global__ void __launch_bounds__(WAVES * 64)
   // rows RBMAX y .. of every 16 (a decode item holds at most 16, so this runs once)
   for (int skip = RBMAX * blockIdx.y; skip < total; skip += RBMAX * gridDim.y) {
     if (skip != RBMAX * (int)blockIdx.y) __syncthreads();
-    expert_unit<GS, NM, EPI, WAVES, XSG, 0>(X, x_stride, slots, W, KG, NB, e, min(RBMAX, total - skip),
-                                            members + first + skip, cb2, out, N, limit, xs_in, xs_out, lds, none);
+    expert_unit<GS, NM, EPI, WAVES, 0>(X, x_stride, slots, W, KG, NB, e, min(RBMAX, total - skip),
+                                       members + first + skip, cb2, out, N, limit, lds, none);
   }
 }
 
@@ -56,8 +55,7 @@ template <int GS, int NM, int EPI, int WAVES>
 __global__ void __launch_bounds__(WAVES * 64)
     expert_desc_kernel(const uint16_t* __restrict__ X, int64_t x_stride, int slots, const uint32_t* __restrict__ W,
                        int KG, int NB, const int* __restrict__ desc, const int* __restrict__ counts,
-                       void* __restrict__ out, int N, float limit, const float* __restrict__ xs_in,
-                       float* __restrict__ xs_out) {
+                       void* __restrict__ out, int N, float limit) {
   extern __shared__ float lds[];
   __shared__ int pairs[16];
   const int NB2 = (NB + 1) >> 1;
@@ -69,8 +67,7 @@ __global__ void __launch_bounds__(WAVES * 64)
   if (threadIdx.x < DTILE) pairs[threadIdx.x] = threadIdx.x ? p1 : p0;
   __syncthreads();
   NoHook none;
-  expert_unit<GS, NM, EPI, WAVES, true, 0>(X, x_stride, slots, W, KG, NB, e, cnt, pairs, cb2, out, N, limit, xs_in,
-                                           xs_out, lds, none);
+  expert_unit<GS, NM, EPI, WAVES, 0>(X, x_stride, slots, W, KG, NB, e, cnt, pairs, cb2, out, N, limit, lds, none);
 }
 
 // ---- dense lane matmul ---------------------------------------------------------------------------------------------
@@ -373,21 +370,21 @@ constexpr int FAT_ROWS = 8;          // rows up to which tf_qmm runs the one-lau
 // workgroups keep 4 longer-running waves each so that more of them are resident.  Scheduling only: bits do not move.
 int expert_waves(int64_t grid) { return grid < 384 ? 16 : grid < 768 ? 8 : 4; }
 
-template <int GS, int NM, int EPI, bool XSG>
+template <int GS, int NM, int EPI>
 int launch_experts(const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg, int nb, const int* items,
                    const int* counts, const int* members, void* out, int n, float limit, int64_t max_units,
-                   const float* xs_in, float* xs_out, hipStream_t stream) {
+                   hipStream_t stream) {
   const int nb2 = (nb + 1) / 2;
   const int64_t max_items = (max_units + nb - 1) / nb;
   const int64_t grid = max_items * nb2;
   if (grid < 1) return 0;
   TF_REQUIRE(grid <= 0x7FFFFFFF, "experts: %lld workgroups exceed the grid limit", (long long)grid);
-  const size_t smem = sizeof(float) * expert_lds_floats(NM, kg, XSG);
+  const size_t smem = sizeof(float) * expert_lds_floats(NM);
   TF_REQUIRE(smem <= 64 * 1024, "experts: K/gs = %d groups need %zu bytes of LDS (limit 65536)", kg, smem);
   const dim3 g((unsigned)grid, 16 / RBMAX);          // decode items hold at most 16 pairs
 #define TF_GO(W_)                                                                                                  \
-  expert_kernel<GS, NM, EPI, W_, XSG><<<g, W_ * 64, smem, stream>>>(x, x_stride, slots, w, kg, nb, items, counts, \
-                                                                    members, out, n, limit, xs_in, xs_out)
+  expert_kernel<GS, NM, EPI, W_><<<g, W_ * 64, smem, stream>>>(x, x_stride, slots, w, kg, nb, items, counts, members, \
+                                                               out, n, limit)
   switch (expert_waves(grid)) {
     case 16: TF_GO(16); break;
     case 8: TF_GO(8); break;
@@ -401,16 +398,16 @@ int launch_experts(const uint16_t* x, int64_t x_stride, int slots, const uint32_
 template <int GS, int NM, int EPI>
 int launch_experts_desc(const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg, int nb,
                         const int* desc, const int* counts, void* out, int n, float limit, int64_t max_items,
-                        const float* xs_in, float* xs_out, hipStream_t stream) {
+                        hipStream_t stream) {
   const int nb2 = (nb + 1) / 2;
   const int64_t grid = max_items * nb2;
   if (grid < 1) return 0;
   TF_REQUIRE(grid <= 0x7FFFFFFF, "experts: %lld workgroups exceed the grid limit", (long long)grid);
-  const size_t smem = sizeof(float) * expert_lds_floats(NM, kg, true);
+  const size_t smem = sizeof(float) * expert_lds_floats(NM);
   const dim3 g((unsigned)grid);
 #define TF_GO(W_)                                                                                                 \
   expert_desc_kernel<GS, NM, EPI, W_><<<g, W_ * 64, smem, stream>>>(x, x_stride, slots, w, kg, nb, desc, counts, out, n, \
-                                                                    limit, xs_in, xs_out)
+                                                                    limit)
   switch (expert_waves(grid)) {
     case 16: TF_GO(16); break;
     case 8: TF_GO(8); break;
@@ -428,12 +425,10 @@ using namespace tf;
 
 extern "C" int tf_experts_run_desc(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w,
                                    int kg, int nb, const int32_t* desc, const int32_t* counts, void* out, int n,
-                                   float limit, int64_t max_items, const float* xs, float* xs_out,
-                                   tf_stream_t stream) {
+                                   float limit, int64_t max_items, tf_stream_t stream) {
   clear_error();
   TF_REQUIRE(gs == 32 || gs == 64, "experts: groups of 32 or 64 inputs, not %d", gs);
-  TF_REQUIRE(x && w && desc && counts && out && xs, "experts: null pointer argument");
-  TF_REQUIRE(!xs_out || (epi != 0 && n % gs == 0), "experts: xs_out goes with an activation epilogue and whole groups");
+  TF_REQUIRE(x && w && desc && counts && out, "experts: null pointer argument");
   TF_REQUIRE(kg >= 1 && nb >= 1 && n == nb * 32, "experts: n (%d) must be the column blocks (%d) times 32", n, nb);
   TF_REQUIRE(aligned16(x) && x_stride % 8 == 0, "x: rows of K = groups * group size inputs, 16-byte aligned");
   TF_REQUIRE(aligned16(w), "w must be 16-byte aligned");
@@ -441,8 +436,7 @@ extern "C" int tf_experts_run_desc(int gs, int epi, const uint16_t* x, int64_t x
   hipStream_t s = as_stream(stream);
 #define TF_RUN(GS_, NM_, EPI_)            \
   if (gs == GS_ && epi == EPI_)           \
-    return launch_experts_desc<GS_, NM_, EPI_>(x, x_stride, slots, w, kg, nb, desc, counts, out, n, limit, max_items, \
-                                               xs, xs_out, s);
+    return launch_experts_desc<GS_, NM_, EPI_>(x, x_stride, slots, w, kg, nb, desc, counts, out, n, limit, max_items, s);
   TF_RUN(32, 1, 0) TF_RUN(32, 1, 1) TF_RUN(32, 2, 2) TF_RUN(64, 1, 0) TF_RUN(64, 1, 1) TF_RUN(64, 2, 2)
 #undef TF_RUN
   set_error("experts: no kernel for group %d and epilogue %d", gs, epi);
@@ -451,23 +445,19 @@ extern "C" int tf_experts_run_desc(int gs, int epi, const uint16_t* x, int64_t x
 
 extern "C" int tf_experts_run(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w,
                               int kg, int nb, const int32_t* items, const int32_t* counts, const int32_t* members,
-                              void* out, int n, float limit, int64_t max_units, const float* xs, float* xs_out,
-                              tf_stream_t stream) {
+                              void* out, int n, float limit, int64_t max_units, tf_stream_t stream) {
   clear_error();
   TF_REQUIRE(gs == 32 || gs == 64, "experts: groups of 32 or 64 inputs, not %d", gs);
   TF_REQUIRE(x && w && items && counts && members && out, "experts: null pointer argument");
-  TF_REQUIRE(!xs_out || (epi != 0 && n % gs == 0), "experts: xs_out goes with an activation epilogue and whole groups");
   TF_REQUIRE(kg >= 1 && nb >= 1 && n == nb * 32, "experts: n (%d) must be the column blocks (%d) times 32", n, nb);
   TF_REQUIRE(aligned16(x) && x_stride % 8 == 0, "x: rows of K = groups * group size inputs, 16-byte aligned");
   TF_REQUIRE(aligned16(w), "w must be 16-byte aligned");
   TF_REQUIRE(slots >= 0 && max_units >= 0, "experts: negative slots or max_units");
   hipStream_t s = as_stream(stream);
-#define TF_RUN(GS_, NM_, EPI_)                                                                                       \
-  if (gs == GS_ && epi == EPI_)                                                                                      \
-    return xs ? launch_experts<GS_, NM_, EPI_, true>(x, x_stride, slots, w, kg, nb, items, counts, members, out, n,  \
-                                                     limit, max_units, xs, xs_out, s)                                \
-              : launch_experts<GS_, NM_, EPI_, false>(x, x_stride, slots, w, kg, nb, items, counts, members, out, n, \
-                                                      limit, max_units, xs, xs_out, s);
+#define TF_RUN(GS_, NM_, EPI_)                                                                                    \
+  if (gs == GS_ && epi == EPI_)                                                                                   \
+    return launch_experts<GS_, NM_, EPI_>(x, x_stride, slots, w, kg, nb, items, counts, members, out, n, limit, \
+                                          max_units, s);
   TF_RUN(32, 1, 0) TF_RUN(32, 1, 1) TF_RUN(32, 2, 2) TF_RUN(64, 1, 0) TF_RUN(64, 1, 1) TF_RUN(64, 2, 2)
 #undef TF_RUN
   set_error("experts: no kernel for group %d and epilogue %d", gs, epi);

@@ -56,7 +56,7 @@ int arrive_stride(int rows) { return rows <= 64 ? TF_ARRIVE_STRIDE : 1; }
 
 // A down unit has written its 64 columns of y (agent-scope stores) for its rows: count it in each row's token; the
 // unit that completes a (token, 64 columns) cell adds the token's slots in slot order (fp32 fma, as tf_moe_combine)
-// and writes bf16.  `arrive` [tokens * NB2d * astride] starts at zero.
+// and writes bf16.  `arrive` [tokens * NB2d * astride] starts at zero and is left at zero.
 template <int WAVES>
 __device__ __forceinline__ void combine_cells(const int* pairs, int cnt, int slots, int cb2, int NB2d, int D, int astride,
                                               const float* __restrict__ wts, const float* __restrict__ y,
@@ -70,9 +70,11 @@ __device__ __forceinline__ void combine_cells(const int* pairs, int cnt, int slo
   for (int r = wave; r < cnt; r += WAVES) {
     const int token = pairs[r] / slots;
     int done = 0;
-    if (lane == 0)
-      done = __hip_atomic_fetch_add(arrive + ((size_t)token * NB2d + cb2) * astride, 1, __ATOMIC_RELAXED,
-                                    __HIP_MEMORY_SCOPE_AGENT) == slots - 1;
+    if (lane == 0) {
+      int* cell = arrive + ((size_t)token * NB2d + cb2) * astride;
+      done = __hip_atomic_fetch_add(cell, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == slots - 1;
+      if (done) __hip_atomic_store(cell, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // every unit has arrived: ready for the next launch
+    }
     if (!__builtin_amdgcn_readfirstlane(done) || col >= D) continue;
     float a = 0.f;
     // eight slots' loads go out together (one trip to memory instead of eight), then the sum in slot order
@@ -96,8 +98,7 @@ __device__ __forceinline__ void combine_cells(const int* pairs, int cnt, int slo
 template <int GS, int WAVES>
 __global__ void __launch_bounds__(WAVES * 64)
     down_combine_kernel(const uint16_t* __restrict__ act, int slots, const uint32_t* __restrict__ Wdown, int D, int NI,
-                        const int* __restrict__ desc, const float* __restrict__ wts, const float* __restrict__ xs_act,
-                        float* __restrict__ y, uint16_t* __restrict__ out, int* __restrict__ arrive, int astride) {
+                        const int* __restrict__ desc, const float* __restrict__ wts, float* __restrict__ y, uint16_t* __restrict__ out, int* __restrict__ arrive, int astride) {
   extern __shared__ float lds[];
   __shared__ int pairs[16];
   __builtin_amdgcn_s_setprio(3);       // the descriptor and the first requests issue ahead of the workgroups that already stream
@@ -110,8 +111,7 @@ __global__ void __launch_bounds__(WAVES * 64)
   if (threadIdx.x < DTILE) pairs[threadIdx.x] = threadIdx.x ? p1 : p0;
   __syncthreads();
   NoHook none;
-  expert_unit<GS, 1, 0, WAVES, true, COH_OUT>(act, NI, 0, Wdown, NI / GS, NB, e, cnt, pairs, cb2, y, D, 0.f, xs_act,
-                                              nullptr, lds, none);
+  expert_unit<GS, 1, 0, WAVES, COH_OUT>(act, NI, 0, Wdown, NI / GS, NB, e, cnt, pairs, cb2, y, D, 0.f, lds, none);
   combine_cells<WAVES>(pairs, cnt, slots, cb2, NB2d, D, astride, wts, y, out, arrive);
 }
 
@@ -119,8 +119,8 @@ template <int GS, int NM, int EPI_UP, int WAVES>
 __global__ void __launch_bounds__(WAVES * 64)
     moe_fused_kernel(const uint16_t* __restrict__ X, int64_t x_stride, int slots, const uint32_t* __restrict__ Wup,
                      const uint32_t* __restrict__ Wdown, int D, int NI, const int* __restrict__ desc,
-                     const int* __restrict__ counts, const float* __restrict__ wts, const float* __restrict__ xs_x,
-                     uint16_t* __restrict__ act, float* __restrict__ xs_act, float* __restrict__ y,
+                     const int* __restrict__ counts, const float* __restrict__ wts, uint16_t* __restrict__ act,
+                     float* __restrict__ y,
                      uint16_t* __restrict__ out, int* __restrict__ done, int* __restrict__ arrive,
                      int* __restrict__ status, float limit, int max_items, int spins, int astride) {
   extern __shared__ float lds[];
@@ -139,8 +139,8 @@ __global__ void __launch_bounds__(WAVES * 64)
   __syncthreads();
   if (up) {
     NoHook none;
-    expert_unit<GS, NM, EPI_UP, WAVES, true, COH_OUT>(X, x_stride, slots, Wup, D / GS, NI / 32, e, cnt, pairs, cb2, act,
-                                                      NI, limit, xs_x, xs_act, lds, none);
+    expert_unit<GS, NM, EPI_UP, WAVES, COH_OUT>(X, x_stride, slots, Wup, D / GS, NI / 32, e, cnt, pairs, cb2, act, NI,
+                                                limit, lds, none);
     __builtin_amdgcn_s_waitcnt(0);      // every store of this wave is acknowledged ...
     __syncthreads();                    // ... of every wave ...
     if (tid == 0) __hip_atomic_fetch_add(done + (size_t)it * DONE_STRIDE, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ... then it counts
@@ -148,8 +148,7 @@ __global__ void __launch_bounds__(WAVES * 64)
   }
   WaitItem wait{done + (size_t)it * DONE_STRIDE, NB2u, spins, status};
   constexpr int DCOH = COH_IN | COH_OUT;
-  if (!expert_unit<GS, 1, 0, WAVES, true, DCOH>(act, NI, 0, Wdown, NI / GS, D / 32, e, cnt, pairs, cb2, y, D,
-                                                            0.f, xs_act, nullptr, lds, wait))
+  if (!expert_unit<GS, 1, 0, WAVES, DCOH>(act, NI, 0, Wdown, NI / GS, D / 32, e, cnt, pairs, cb2, y, D, 0.f, lds, wait))
     return;                     // the wait ran out: status is set, nothing is published
   combine_cells<WAVES>(pairs, cnt, slots, cb2, NB2d, D, astride, wts, y, out, arrive);
 }
@@ -168,8 +167,7 @@ __global__ void __launch_bounds__(WAVES * 64)
                     const uint16_t* __restrict__ X, int64_t x_stride, const uint32_t* __restrict__ Wup, int D, int NI,
                     int* __restrict__ pick, float* __restrict__ wts, int* __restrict__ members,
                     int* __restrict__ items, int* __restrict__ counts, int* __restrict__ desc,
-                    uint16_t* __restrict__ act, float* __restrict__ xs_act, float limit, int* __restrict__ zero,
-                    int n_zero) {
+                    uint16_t* __restrict__ act, float limit, int* __restrict__ zero, int n_zero) {
   extern __shared__ float lds[];
   __shared__ int pk[PLAN_THREADS];
   __shared__ ItemLds item;
@@ -219,8 +217,8 @@ __global__ void __launch_bounds__(WAVES * 64)
     __syncthreads();
     if (item.sel[0] < 0) return;
     NoHook none;
-    expert_unit<GS, NM, EPI, WAVES, false, 0>(X, x_stride, slots, Wup, D / GS, NI / 32, item.sel[0], 1, item.pairs, cb2,
-                                              act, NI, limit, nullptr, xs_act, lds, none);
+    expert_unit<GS, NM, EPI, WAVES, 0>(X, x_stride, slots, Wup, D / GS, NI / 32, item.sel[0], 1, item.pairs, cb2,
+                                              act, NI, limit, lds, none);
     return;
   }
   if (L && !writer && R <= 64) {
@@ -234,8 +232,8 @@ __global__ void __launch_bounds__(WAVES * 64)
                     : pair_item<TOPK_VPL, WAVES>(L, ldl, R, NE, TOPK, shared, slots, it, pk, item.sel, wavepairs[wave], e, cnt);
     if (!live) return;
     NoHook none;
-    expert_unit<GS, NM, EPI, WAVES, false, 0>(X, x_stride, slots, Wup, D / GS, NI / 32, e, cnt, wavepairs[wave], cb2, act,
-                                              NI, limit, nullptr, xs_act, lds, none);
+    expert_unit<GS, NM, EPI, WAVES, 0>(X, x_stride, slots, Wup, D / GS, NI / 32, e, cnt, wavepairs[wave], cb2, act,
+                                              NI, limit, lds, none);
     return;
   }
   if (!L && !writer) {
@@ -245,8 +243,8 @@ __global__ void __launch_bounds__(WAVES * 64)
     int e = 0, cnt = 0;
     if (!pair_item_given(pick, P, E, it, wavepairs[wave], e, cnt)) return;
     NoHook none;
-    expert_unit<GS, NM, EPI, WAVES, false, 0>(X, x_stride, slots, Wup, D / GS, NI / 32, e, cnt, wavepairs[wave], cb2, act,
-                                              NI, limit, nullptr, xs_act, lds, none);
+    expert_unit<GS, NM, EPI, WAVES, 0>(X, x_stride, slots, Wup, D / GS, NI / 32, e, cnt, wavepairs[wave], cb2, act,
+                                              NI, limit, lds, none);
     return;
   }
   for (int e = tid; e < E; e += threads) item.cnt[e] = 0;
@@ -360,29 +358,29 @@ __global__ void __launch_bounds__(WAVES * 64)
   if (!find_item<DTILE, true>(item, pk, P, E, it)) return;
   NoHook none;
   // the item's rows are summed group by group inside the unit (a pass at a time), under its first weight loads
-  expert_unit<GS, NM, EPI, WAVES, false, 0>(X, x_stride, slots, Wup, D / GS, NI / 32, item.sel[0], item.sel[2],
-                                            item.pairs, cb2, act, NI, limit, nullptr, xs_act, lds, none);
+  expert_unit<GS, NM, EPI, WAVES, 0>(X, x_stride, slots, Wup, D / GS, NI / 32, item.sel[0], item.sel[2],
+                                            item.pairs, cb2, act, NI, limit, lds, none);
 }
 
 template <int GS, int NM, int EPI>
 int launch_route_up(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared, const uint16_t* x,
                     int64_t x_stride, const uint32_t* wup, int d, int ni, int* pick, float* wts, int* members,
-                    int* items, int* counts, int* desc, uint16_t* act, float* xs_act, float limit, int max_items,
-                    int* zero, int n_zero, hipStream_t stream) {
+                    int* items, int* counts, int* desc, uint16_t* act, float limit, int max_items, int* zero,
+                    int n_zero, hipStream_t stream) {
   const int nb2 = (ni / 32 + 1) / 2;
   // with the picks given, or logits of 2 to 64 rows, the workgroups go a pair (route_up_kernel), else an item
   const int64_t pairs = (int64_t)rows * (top_k + (shared ? 1 : 0));
   const int64_t units = !logits || (rows > 1 && rows <= 64) ? pairs : max_items;
   const int64_t grid = 1 + units * nb2;
   TF_REQUIRE(grid <= 0x7FFFFFFF, "moe: %lld workgroups exceed the grid limit", (long long)grid);
-  const size_t floats = expert_lds_floats(NM, d / GS, false);
+  const size_t floats = expert_lds_floats(NM);
   const size_t smem = sizeof(float) * (floats > 4 * EMAX ? floats : 4 * EMAX);
   TF_REQUIRE(smem <= 48 * 1024, "moe: %d input groups need %zu bytes of LDS", d / GS, smem);
   const dim3 g((unsigned)grid);
 #define TF_GO(W_)                                                                                                  \
   route_up_kernel<GS, NM, EPI, W_><<<g, W_ * 64, smem, stream>>>(logits, ldl, rows, experts, top_k, shared, x, x_stride, \
                                                                  wup, d, ni, pick, wts, members, items, counts, desc,  \
-                                                                 act, xs_act, limit, zero, n_zero)
+                                                                 act, limit, zero, n_zero)
   switch (fused_waves(2 * grid)) {
     case 16: TF_GO(16); break;
     case 8: TF_GO(8); break;
@@ -395,19 +393,18 @@ int launch_route_up(const float* logits, int64_t ldl, int rows, int experts, int
 
 template <int GS, int NM, int EPI_UP>
 int launch_fused(const uint16_t* x, int64_t x_stride, int slots, const uint32_t* wup, const uint32_t* wdown, int d,
-                 int ni, const int* desc, const int* counts, const float* wts, const float* xs_x, uint16_t* act,
-                 float* xs_act, float* y, uint16_t* out, int* done, int* arrive, int* status, float limit,
+                 int ni, const int* desc, const int* counts, const float* wts, uint16_t* act, float* y, uint16_t* out, int* done, int* arrive, int* status, float limit,
                  int max_items, int astride, hipStream_t stream) {
   const int nb2u = (ni / 32 + 1) / 2, nb2d = (d / 32 + 1) / 2;
   const int64_t grid = (int64_t)max_items * (nb2u + nb2d);
   if (grid < 1) return 0;
   TF_REQUIRE(grid <= 0x7FFFFFFF, "moe: %lld workgroups exceed the grid limit", (long long)grid);
-  const size_t smem = sizeof(float) * expert_lds_floats(NM, 0, true);
+  const size_t smem = sizeof(float) * expert_lds_floats(NM);
   const int spins = 1 << 16;     // polls of about a microsecond: far past any real wait, short enough to drain fast
   const dim3 g((unsigned)grid);
 #define TF_GO(W_)                                                                                                 \
   moe_fused_kernel<GS, NM, EPI_UP, W_><<<g, W_ * 64, smem, stream>>>(x, x_stride, slots, wup, wdown, d, ni, desc, \
-                                                                     counts, wts, xs_x, act, xs_act, y, out, done, \
+                                                                     counts, wts, act, y, out, done,              \
                                                                      arrive, status, limit, max_items, spins, astride)
   switch (fused_waves(grid)) {
     case 16: TF_GO(16); break;
@@ -426,12 +423,12 @@ using namespace tf;
 
 extern "C" int tf_moe_decode_experts(int gs, int swiglu, const uint16_t* x, int64_t x_stride, int rows, int slots,
                                      const uint32_t* up, const uint32_t* down, int d, int ni, const int32_t* desc,
-                                     const int32_t* counts, const float* wts, const float* xs_x, uint16_t* act,
-                                     float* xs_act, float* y, uint16_t* out, int32_t* done, int32_t* arrive,
+                                     const int32_t* counts, const float* wts, uint16_t* act, float* y,
+                                     uint16_t* out, int32_t* done, int32_t* arrive,
                                      int32_t* status, float limit, int max_items, tf_stream_t stream) {
   clear_error();
   TF_REQUIRE(gs == 32 || gs == 64, "moe: groups of 32 or 64 inputs, not %d", gs);
-  TF_REQUIRE(x && up && down && desc && counts && wts && xs_x && act && xs_act && y && out && done && arrive && status,
+  TF_REQUIRE(x && up && down && desc && counts && wts && act && y && out && done && arrive && status,
              "moe: null pointer argument");
   TF_REQUIRE(d % 64 == 0 && ni % 64 == 0 && d % gs == 0 && ni % gs == 0,
              "moe: the fused decode layer takes hidden and intermediate sizes that are multiples of 64");
@@ -440,25 +437,24 @@ extern "C" int tf_moe_decode_experts(int gs, int swiglu, const uint16_t* x, int6
   TF_REQUIRE(rows >= 1 && slots >= 1 && max_items >= 1, "moe: empty call");
   hipStream_t s = as_stream(stream);
   if (gs == 64)
-    return swiglu ? launch_fused<64, 2, 2>(x, x_stride, slots, up, down, d, ni, desc, counts, wts, xs_x, act, xs_act, y,
+    return swiglu ? launch_fused<64, 2, 2>(x, x_stride, slots, up, down, d, ni, desc, counts, wts, act, y,
                                            out, done, arrive, status, limit, max_items, arrive_stride(rows), s)
-                  : launch_fused<64, 1, 1>(x, x_stride, slots, up, down, d, ni, desc, counts, wts, xs_x, act, xs_act, y,
+                  : launch_fused<64, 1, 1>(x, x_stride, slots, up, down, d, ni, desc, counts, wts, act, y,
                                            out, done, arrive, status, limit, max_items, arrive_stride(rows), s);
-  return swiglu ? launch_fused<32, 2, 2>(x, x_stride, slots, up, down, d, ni, desc, counts, wts, xs_x, act, xs_act, y,
+  return swiglu ? launch_fused<32, 2, 2>(x, x_stride, slots, up, down, d, ni, desc, counts, wts, act, y,
                                          out, done, arrive, status, limit, max_items, arrive_stride(rows), s)
-                : launch_fused<32, 1, 1>(x, x_stride, slots, up, down, d, ni, desc, counts, wts, xs_x, act, xs_act, y,
+                : launch_fused<32, 1, 1>(x, x_stride, slots, up, down, d, ni, desc, counts, wts, act, y,
                                          out, done, arrive, status, limit, max_items, arrive_stride(rows), s);
 }
 
 extern "C" int tf_moe_route_up(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared, int gs,
                                int swiglu, const uint16_t* x, int64_t x_stride, const uint32_t* up, int d, int ni,
                                int32_t* pick, float* wts, int32_t* members, int32_t* items, int32_t* counts,
-                               int32_t* desc, uint16_t* act, float* xs_act, float limit, int max_items,
-                               int32_t* zero, int n_zero, tf_stream_t stream) {
+                               int32_t* desc, uint16_t* act, float limit, int max_items, int32_t* zero, int n_zero,
+                               tf_stream_t stream) {
   clear_error();
   TF_REQUIRE(gs == 32 || gs == 64, "moe: groups of 32 or 64 inputs, not %d", gs);
-  TF_REQUIRE(x && up && pick && wts && members && items && counts && desc && act && xs_act,
-             "moe: null pointer argument");
+  TF_REQUIRE(x && up && pick && wts && members && items && counts && desc && act, "moe: null pointer argument");
   TF_REQUIRE(experts >= 1 && experts + (shared ? 1 : 0) <= EMAX && experts <= 64 * TOPK_VPL,
              "route: at most %d experts", EMAX - 1);
   TF_REQUIRE(top_k >= 1 && top_k + (shared ? 1 : 0) <= 64 && top_k <= experts, "route: 1 to 64 slots a row, not %d",
@@ -474,32 +470,32 @@ extern "C" int tf_moe_route_up(const float* logits, int64_t ldl, int rows, int e
   hipStream_t s = as_stream(stream);
   if (gs == 64)
     return swiglu ? launch_route_up<64, 2, 2>(logits, ldl, rows, experts, top_k, shared, x, x_stride, up, d, ni, pick,
-                                              wts, members, items, counts, desc, act, xs_act, limit, max_items, zero, n_zero, s)
+                                              wts, members, items, counts, desc, act, limit, max_items, zero, n_zero, s)
                   : launch_route_up<64, 1, 1>(logits, ldl, rows, experts, top_k, shared, x, x_stride, up, d, ni, pick,
-                                              wts, members, items, counts, desc, act, xs_act, limit, max_items, zero, n_zero, s);
+                                              wts, members, items, counts, desc, act, limit, max_items, zero, n_zero, s);
   return swiglu ? launch_route_up<32, 2, 2>(logits, ldl, rows, experts, top_k, shared, x, x_stride, up, d, ni, pick, wts,
-                                            members, items, counts, desc, act, xs_act, limit, max_items, zero, n_zero, s)
+                                            members, items, counts, desc, act, limit, max_items, zero, n_zero, s)
                 : launch_route_up<32, 1, 1>(logits, ldl, rows, experts, top_k, shared, x, x_stride, up, d, ni, pick, wts,
-                                            members, items, counts, desc, act, xs_act, limit, max_items, zero, n_zero, s);
+                                            members, items, counts, desc, act, limit, max_items, zero, n_zero, s);
 }
 
 extern "C" int tf_moe_down_combine(int gs, const uint16_t* act, int rows, int slots, const uint32_t* down, int d, int ni,
-                                   const int32_t* desc, const float* wts, const float* xs_act, float* y, uint16_t* out,
-                                   int32_t* arrive, int max_items, tf_stream_t stream) {
+                                   const int32_t* desc, const float* wts, float* y, uint16_t* out, int32_t* arrive,
+                                   int max_items, tf_stream_t stream) {
   clear_error();
   TF_REQUIRE(gs == 32 || gs == 64, "moe: groups of 32 or 64 inputs, not %d", gs);
-  TF_REQUIRE(act && down && desc && wts && xs_act && y && out && arrive, "moe: null pointer argument");
+  TF_REQUIRE(act && down && desc && wts && y && out && arrive, "moe: null pointer argument");
   TF_REQUIRE(d % 32 == 0 && ni % gs == 0 && ni >= gs && rows >= 1 && slots >= 1 && max_items >= 1,
              "moe: hidden size in 32-column blocks, intermediate size in whole groups");
   TF_REQUIRE(aligned16(act) && ni % 8 == 0 && aligned16(down), "act: rows of whole groups, 16-byte aligned");
   const int nb2 = (d / 32 + 1) / 2;
   const int64_t grid = (int64_t)max_items * nb2;
   TF_REQUIRE(grid <= 0x7FFFFFFF, "moe: %lld workgroups exceed the grid limit", (long long)grid);
-  const size_t smem = sizeof(float) * expert_lds_floats(1, 0, true);
+  const size_t smem = sizeof(float) * expert_lds_floats(1);
   hipStream_t s = as_stream(stream);
   const dim3 g((unsigned)grid);
 #define TF_GO(GS_, W_)                                                                                             \
-  down_combine_kernel<GS_, W_><<<g, W_ * 64, smem, s>>>(act, slots, down, d, ni, desc, wts, xs_act, y, out, arrive, \
+  down_combine_kernel<GS_, W_><<<g, W_ * 64, smem, s>>>(act, slots, down, d, ni, desc, wts, y, out, arrive, \
                                                         arrive_stride(rows))
 #define TF_GS(GS_)                      \
   switch (fused_waves(grid + grid / 2)) {      \

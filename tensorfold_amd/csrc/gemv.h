@@ -97,6 +97,29 @@ __device__ __forceinline__ void load_weights(Stage<GS, NM>& st, const WQ& wq, co
   }
 }
 
+// The sum of a row of 16 lanes, left in every one of them: the two quad swaps, then the mirrored halves of 8 and of
+// 16 lanes.  Both sides of each step add the same two numbers, so all sixteen lanes end with the same bits.
+__device__ __forceinline__ float row16_sum(float s) {
+#define TF_DPP_ADD(CTRL_) \
+  s += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, s), CTRL_, 0xF, 0xF, true))
+  TF_DPP_ADD(0xB1);        // quad_perm [1, 0, 3, 2]
+  TF_DPP_ADD(0x4E);        // quad_perm [2, 3, 0, 1]
+  TF_DPP_ADD(0x141);       // row_half_mirror
+  TF_DPP_ADD(0x140);       // row_mirror
+#undef TF_DPP_ADD
+  return s;
+}
+
+// Row r's sum over the staged group, from the dwords the dot products read anyway: a lane adds its two inputs of
+// each chunk in chunk order (a dot product against ones), then the sixteen lanes that share the row add up.
+template <int GS, int NM>
+__device__ __forceinline__ float stage_row_sum(const Stage<GS, NM>& st, int r) {
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < GS / 32; ++i) s = dot2(st.x[r][i], BF16_ONES, s);
+  return row16_sum(s);
+}
+
 // xl[r]: row r's inputs as dwords, already offset by (lane % 16)
 template <int GS, int NM, int RB, int COH>
 __device__ __forceinline__ void load_inputs(Stage<GS, NM>& st, const uint32_t* const (&xl)[RB], int g) {
@@ -147,10 +170,10 @@ __device__ __forceinline__ void chunk_dot(float (&p)[NM][RB], const Stage<GS, NM
 //   wq(g, m, i)     -> the lane's 16 bytes of chunk i of group g of matrix m
 //   sb(g, m, s, b)  -> the lane's column's scale and bias of that group
 //   xl[r]           -> row r's inputs as dwords, offset by lane % 16
-//   xsum(r, g)      -> row r's sum over group g (wave-uniform)
+//   xsum(r, g)      -> row r's sum over group g (wave-uniform); with XIN the sums are taken from the staged inputs
 //   flush(g, acc)   -> called after group g has been added (wave-uniform); may park and clear acc
 // `st` holds the weights of groups gA .. gA + DEPTH - 1 on entry when `loaded`.
-template <int GS, int NM, int RB, int COH, class WQ, class SB, class XS, class FLUSH>
+template <int GS, int NM, int RB, int COH, bool XIN = false, class WQ, class SB, class XS, class FLUSH>
 __device__ __forceinline__ void gemv_stream(float (&acc)[NM][RB], Stage<GS, NM> (&st)[DEPTH], bool loaded,
                                             const WQ& wq, const SB& sb, const uint32_t* const (&xl)[RB],
                                             const XS& xsum, int gA, int gB, FLUSH& flush) {
@@ -184,7 +207,9 @@ __device__ __forceinline__ void gemv_stream(float (&acc)[NM][RB], Stage<GS, NM> 
           for (int r = 0; r < RB; ++r) asm volatile("s_nop 2" : "+v"(p[m][r]));
 #pragma unroll
         for (int r = 0; r < RB; ++r) {
-          const float sc = xsum(r, g);
+          float sc;
+          if constexpr (XIN) sc = stage_row_sum<GS, NM>(st[d], r);
+          else sc = xsum(r, g);
 #pragma unroll
           for (int m = 0; m < NM; ++m) {
             const float pq = fmaf(-128.f, sc, p[m][r]);
@@ -206,31 +231,25 @@ __device__ __forceinline__ void gemv_stream(float (&acc)[NM][RB], Stage<GS, NM> 
 __device__ __forceinline__ int slice_begin(int s, int KG) { return (int)((long long)s * KG / SLICES); }
 
 // One pass of an item: RB of its rows (pairs[0 ..]) against the workgroup's 64 columns.
-// XSG: the rows' group sums come from `xs_in` (fp32 [x rows, KG], scalar loads); otherwise they are summed here
-// into LDS first.  `xs_out` (may be null; epilogues 1 and 2) receives the group sums of the activations written,
-// fp32 [pairs, N / GS]: what the down projection of the same pairs reads as its `xs_in`.
-template <int GS, int NM, int EPI, int WAVES, int RB, bool XSG, int COH, class WQ, class SB>
+// Each wave takes the sums of its groups' inputs from the dwords it reads for the dot products.
+template <int GS, int NM, int EPI, int WAVES, int RB, int COH, class WQ, class SB>
 __device__ __forceinline__ void expert_pass(const uint16_t* __restrict__ X, int64_t x_stride, int slots, const WQ& wq,
                                             const SB& sb, int KG, int NB, int cb2, const int* pairs,
-                                            void* __restrict__ out, int N, float limit, float* xs, float* part,
-                                            Stage<GS, NM> (&st)[DEPTH], bool loaded, bool first_pass,
-                                            const float* __restrict__ xs_in, float* __restrict__ xs_out) {
+                                            void* __restrict__ out, int N, float limit, float* part,
+                                            Stage<GS, NM> (&st)[DEPTH], bool loaded, bool first_pass) {
   constexpr int SPW = SLICES / WAVES;               // slices a wave
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   int pr[RB];
   const uint16_t* xrow[RB];
   const uint32_t* xl[RB];
-  const float* xsr[RB];
 #pragma unroll
   for (int r = 0; r < RB; ++r) {
     pr[r] = pairs[r];
     const int row = slots ? pr[r] / slots : pr[r];
     xrow[r] = X + (size_t)row * x_stride;
     xl[r] = reinterpret_cast<const uint32_t*>(xrow[r]) + (lane & 15);
-    xsr[r] = xs_in + (size_t)row * KG;
   }
-  if (!first_pass || !XSG) __syncthreads();         // the previous pass is done with xs and part
-  if constexpr (!XSG) group_sums_block<GS>(xrow, RB, KG, xs, tid, WAVES * 64);
+  if (!first_pass) __syncthreads();                 // the previous pass is done with part
   // slices with no group (K/gs < SLICES) still take part in the ordered sum: as zeros
   if (KG < SLICES) {
 #pragma unroll
@@ -240,7 +259,7 @@ __device__ __forceinline__ void expert_pass(const uint16_t* __restrict__ X, int6
 #pragma unroll
         for (int r = 0; r < RB; ++r) part[(((wave * SPW + q) * NM + m) * RB + r) * 64 + lane] = 0.f;
   }
-  if (!XSG || KG < SLICES) __syncthreads();
+  if (KG < SLICES) __syncthreads();
   float acc[NM][RB];
 #pragma unroll
   for (int m = 0; m < NM; ++m)
@@ -263,25 +282,8 @@ __device__ __forceinline__ void expert_pass(const uint16_t* __restrict__ X, int6
     slice_end = slice < SLICES ? slice_begin(slice + 1, KG) : -1;
   };
   const int gA = slice_begin(wave * SPW, KG), gB = slice_begin((wave + 1) * SPW, KG);
-  // with sums from memory, lane i keeps the sums of group gA + i (64 groups at a time) and readlane hands them out
-  float xsv[RB];
-  int xs_base = gA;
-  auto fetch_sums = [&](int base) {
-#pragma unroll
-    for (int r = 0; r < RB; ++r)
-      xsv[r] = base + lane < gB ? ((COH & COH_IN) ? ld_agent(xsr[r] + base + lane) : xsr[r][base + lane]) : 0.f;
-    xs_base = base;
-  };
-  if constexpr (XSG) fetch_sums(gA);
-  auto xsum = [&](int r, int g) {
-    if constexpr (XSG) {
-      if (g - xs_base >= 64) fetch_sums(g);
-      return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, xsv[r]), g - xs_base));
-    } else {
-      return xs[r * KG + g];
-    }
-  };
-  gemv_stream<GS, NM, RB, COH>(acc, st, loaded, wq, sb, xl, xsum, gA, gB, flush);
+  auto no_sums = [](int, int) { return 0.f; };
+  gemv_stream<GS, NM, RB, COH, true>(acc, st, loaded, wq, sb, xl, no_sums, gA, gB, flush);
   __syncthreads();
   // a wave a row, a lane a column: the slices' sums in slice order, then the epilogue
   for (int r = wave; r < RB; r += WAVES) {
@@ -315,17 +317,6 @@ __device__ __forceinline__ void expert_pass(const uint16_t* __restrict__ X, int6
       } else if (ok) {
         reinterpret_cast<uint16_t*>(out)[at] = (uint16_t)bits;
       }
-      if (xs_out) {
-        // group sums of the rounded activations: a fixed xor tree over the group's lanes
-        float t = ok ? o : 0.f;
-#pragma unroll
-        for (int m = 1; m < GS; m <<= 1) t += __shfl_xor(t, m);
-        if (ok && (l & (GS - 1)) == 0) {
-          float* dst = xs_out + (size_t)prow * (N / GS) + (cb2 * 64 + l) / GS;
-          if (COH & COH_OUT) st_agent(dst, t);
-          else *dst = t;
-        }
-      }
     }
   }
 }
@@ -339,13 +330,12 @@ struct NoHook {
 // through in passes of 2 or 1; a row's arithmetic is the same in each, so its bits do not depend on the pass it
 // lands in.  `ready()` runs after the wave's first weights have been requested and before any activation is read
 // (the fused layer waits there for the item's activations); returning false abandons the unit.
-// lds: xs [RBMAX][KG] when !XSG, then the slices' sums [SLICES][NM][RBMAX][64].
-template <int GS, int NM, int EPI, int WAVES, bool XSG, int COH, class HOOK>
+// lds: the slices' sums [SLICES][NM][RBMAX][64].
+template <int GS, int NM, int EPI, int WAVES, int COH, class HOOK>
 __device__ __forceinline__ bool expert_unit(const uint16_t* __restrict__ X, int64_t x_stride, int slots,
                                             const uint32_t* __restrict__ W, int KG, int NB, int e, int cnt,
                                             const int* pairs, int cb2, void* __restrict__ out, int N, float limit,
-                                            const float* __restrict__ xs_in, float* __restrict__ xs_out, float* lds,
-                                            HOOK& ready) {
+                                            float* lds, HOOK& ready) {
   constexpr int BW = block_words(GS);
   constexpr int SPW = SLICES / WAVES;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -361,8 +351,7 @@ __device__ __forceinline__ bool expert_unit(const uint16_t* __restrict__ X, int6
     b = bf16_hi(v);
   };
   const int gA = slice_begin(wave * SPW, KG), gB = slice_begin((wave + 1) * SPW, KG);
-  float* xs = lds;
-  float* part = lds + (XSG ? 0 : RBMAX * KG);
+  float* part = lds;
   // the wave's first groups are on their way before anything else is read
   Stage<GS, NM> st[DEPTH];
 #pragma unroll
@@ -372,8 +361,8 @@ __device__ __forceinline__ bool expert_unit(const uint16_t* __restrict__ X, int6
   bool loaded = true, first_pass = true;
   int r0 = 0;
 #define TF_PASS(RB_)                                                                                                \
-  expert_pass<GS, NM, EPI, WAVES, RB_, XSG, COH>(X, x_stride, slots, wq, sb, KG, NB, cb2, pairs + r0, out, N, limit, xs, \
-                                            part, st, loaded, first_pass, xs_in, xs_out);                           \
+  expert_pass<GS, NM, EPI, WAVES, RB_, COH>(X, x_stride, slots, wq, sb, KG, NB, cb2, pairs + r0, out, N, limit, part, \
+                                            st, loaded, first_pass);                                                \
   first_pass = false;                                                                                               \
   loaded = gB - gA <= DEPTH   /* a run that fits the stages stays in registers for the next pass */
   for (; r0 + 2 <= cnt; r0 += 2) {
@@ -387,9 +376,7 @@ __device__ __forceinline__ bool expert_unit(const uint16_t* __restrict__ X, int6
 }
 
 // LDS floats a workgroup of expert_unit needs
-constexpr size_t expert_lds_floats(int nm, int kg, bool xsg) {
-  return (xsg ? 0 : (size_t)RBMAX * kg) + (size_t)SLICES * nm * RBMAX * 64;
-}
+constexpr size_t expert_lds_floats(int nm) { return (size_t)SLICES * nm * RBMAX * 64; }
 
 }  // namespace
 }  // namespace tf

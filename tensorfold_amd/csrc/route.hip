@@ -36,18 +36,6 @@ __global__ void __launch_bounds__(64)
   topk_row(L + (size_t)r * ldl, NE, TOPK, shared, threadIdx.x, pick + (size_t)r * slots, wts + (size_t)r * slots);
 }
 
-// A row's top-k and the group sums of its inputs: what the decode routing needs a row, spread a wave a row over the
-// chip when one workgroup would take too long over many rows.
-__global__ void __launch_bounds__(64)
-    topk_sums_kernel(const float* __restrict__ L, int64_t ldl, int NE, int TOPK, int shared, int* __restrict__ pick,
-                     float* __restrict__ wts, const uint16_t* __restrict__ X, int64_t ldx, int D, int gs,
-                     float* __restrict__ xs_x) {
-  const int r = blockIdx.x, slots = TOPK + (shared ? 1 : 0);
-  if (gs == 64) group_sums_rows<64>(X + (size_t)r * ldx, ldx, 1, D / 64, xs_x + (size_t)r * (D / 64), threadIdx.x, 64);
-  else group_sums_rows<32>(X + (size_t)r * ldx, ldx, 1, D / 32, xs_x + (size_t)r * (D / 32), threadIdx.x, 64);
-  topk_row(L + (size_t)r * ldl, NE, TOPK, shared, threadIdx.x, pick + (size_t)r * slots, wts + (size_t)r * slots);
-}
-
 // ---- plan: stable counting sort of pairs by expert -------------------------------------------------------------------
 
 // up to 1024 pairs: one workgroup counts, scans and places; then a wave an expert that has pairs collects them in
@@ -73,14 +61,13 @@ __global__ void __launch_bounds__(PLAN_THREADS)
 }
 
 // The decode layer's whole routing in one workgroup (rows * slots <= 1024): top-k of every row, the pair sort, one
-// descriptor an item for the fused expert kernel {expert, count, first, 0, pairs[16]}, the group sums of x, and the
-// zeroing of the fused kernel's counters.
+// descriptor an item for the fused expert kernel {expert, count, first, 0, pairs[16]}, and the zeroing of the fused
+// kernel's counters.
 
 __global__ void __launch_bounds__(PLAN_THREADS)
     route_decode_kernel(const float* __restrict__ L, int64_t ldl, int R, int NE, int TOPK, int shared,
-                        const uint16_t* __restrict__ X, int64_t ldx, int D, int gs, int* __restrict__ pick,
-                        float* __restrict__ wts, int* __restrict__ members, int* __restrict__ items,
-                        int* __restrict__ counts, int* __restrict__ desc, float* __restrict__ xs_x,
+                        int* __restrict__ pick, float* __restrict__ wts, int* __restrict__ members,
+                        int* __restrict__ items, int* __restrict__ counts, int* __restrict__ desc,
                         int* __restrict__ zero, int n_zero, int have_picks) {
   __shared__ int pk[PLAN_THREADS];
   __shared__ PlanLds plan;
@@ -89,12 +76,9 @@ __global__ void __launch_bounds__(PLAN_THREADS)
   const int slots = TOPK + (shared ? 1 : 0), P = R * slots, E = NE + (shared ? 1 : 0), T = 16;
   plan.cnt[tid] = 0;
   for (int i = tid; i < n_zero; i += PLAN_THREADS) zero[i] = 0;
-  if (!have_picks) {      // else a launch before this one has left the picks, the weights and the group sums
+  if (!have_picks) {      // else a launch before this one has left the picks and the weights
     for (int r = wave; r < R; r += PLAN_THREADS / 64)
       topk_row(L + (size_t)r * ldl, NE, TOPK, shared, lane, pick + (size_t)r * slots, wts + (size_t)r * slots);
-    // group sums of x, as tf_group_sums
-    if (gs == 64) group_sums_rows<64>(X, ldx, R, D / 64, xs_x, tid, PLAN_THREADS);
-    else group_sums_rows<32>(X, ldx, R, D / 32, xs_x, tid, PLAN_THREADS);
   }
   __threadfence_block();
   __syncthreads();
@@ -308,28 +292,22 @@ extern "C" int tf_moe_topk(const float* logits, int64_t ldl, int rows, int exper
 }
 
 extern "C" int tf_moe_route_decode(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared,
-                                   const uint16_t* x, int64_t ldx, int d, int gs, int32_t* pick, float* wts,
-                                   int32_t* members, int32_t* items, int32_t* counts, int32_t* desc, float* xs_x,
-                                   int32_t* zero, int n_zero, tf_stream_t stream) {
+                                   int32_t* pick, float* wts, int32_t* members, int32_t* items, int32_t* counts,
+                                   int32_t* desc, int32_t* zero, int n_zero, tf_stream_t stream) {
   clear_error();
-  TF_REQUIRE(logits && x && pick && wts && members && items && counts && desc && xs_x, "route: null pointer argument");
+  TF_REQUIRE(logits && pick && wts && members && items && counts && desc, "route: null pointer argument");
   TF_REQUIRE(experts >= 1 && experts + (shared ? 1 : 0) <= EMAX && experts <= 64 * TOPK_VPL,
              "route: at most %d experts", EMAX - 1);
   TF_REQUIRE(top_k >= 1 && top_k + (shared ? 1 : 0) <= 64 && top_k <= experts, "route: 1 to 64 slots a row, not %d", top_k);
   TF_REQUIRE(rows >= 1 && (int64_t)rows * (top_k + (shared ? 1 : 0)) <= PLAN_THREADS,
              "route: the fused decode routing takes at most %d pairs", PLAN_THREADS);
-  TF_REQUIRE(gs == 32 || gs == 64, "route: groups of 32 or 64 inputs");
-  TF_REQUIRE(d >= gs && d % gs == 0 && aligned16(x) && ldx % 8 == 0, "route: x rows of whole groups, 16-byte aligned");
   TF_REQUIRE(ldl >= experts + (shared ? 1 : 0), "route: logits rows are too short");
   TF_REQUIRE(n_zero >= 0 && (n_zero == 0 || zero), "route: bad counter range");
-  // more rows than the one workgroup has waves: top-k and group sums run first, a workgroup a row, spread over the chip
+  // more rows than the one workgroup has waves: the top-k runs first, a workgroup a row, spread over the chip
   const int spread = rows > PLAN_THREADS / 64;
-  if (spread)
-    topk_sums_kernel<<<rows, 64, 0, as_stream(stream)>>>(logits, ldl, experts, top_k, shared, pick, wts, x, ldx, d, gs,
-                                                         xs_x);
-  route_decode_kernel<<<1, PLAN_THREADS, 0, as_stream(stream)>>>(logits, ldl, rows, experts, top_k, shared, x, ldx, d,
-                                                                gs, pick, wts, members, items, counts, desc, xs_x, zero,
-                                                                n_zero, spread);
+  if (spread) topk_kernel<<<rows, 64, 0, as_stream(stream)>>>(logits, ldl, experts, top_k, shared, pick, wts);
+  route_decode_kernel<<<1, PLAN_THREADS, 0, as_stream(stream)>>>(logits, ldl, rows, experts, top_k, shared, pick, wts,
+                                                                members, items, counts, desc, zero, n_zero, spread);
   TF_LAUNCH_OK("tf_moe_route_decode");
   return 0;
 }

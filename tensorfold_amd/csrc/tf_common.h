@@ -97,6 +97,7 @@ __device__ __forceinline__ void prio_by_progress(int left, int n) {
 // ---- 4-bit blocks -------------------------------------------------------------------------------------------------
 
 constexpr uint32_t NIB_MASK = 0x000F000Fu;
+constexpr uint32_t BF16_ONES = 0x3F803F80u;  // the bf16 pair (1, 1)
 constexpr uint32_t BF16_128 = 0x43004300u;   // the bf16 pair (128, 128): OR-ing a nibble into the mantissa gives 128 + q
 
 // (word >> 4 i) & mask | 128.0: the bf16 pair (128 + q[2 i], 128 + q[2 i + 1]) of a packed word

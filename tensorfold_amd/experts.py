@@ -159,16 +159,6 @@ class Plan:
         blocks = -(-pairs // SMALL)
         self.rank = ints(pairs if pairs > SMALL else 1)            # the multi-workgroup sort's scratch
         self.hist = ints(blocks * experts if pairs > SMALL else 1)
-        self._sums: dict[str, torch.Tensor] = {}                   # fp32 group sums the decode kernels read
-        self._act_key: tuple | None = None                         # which activations ``act`` sums belong to
-
-    def sums(self, name: str, rows: int, groups: int) -> torch.Tensor:
-        """A [rows, groups] fp32 scratch for group sums, allocated on first use and kept."""
-
-        t = self._sums.get(name)
-        if t is None or t.numel() < rows * groups:
-            t = self._sums[name] = torch.empty((rows * groups,), dtype=torch.float32, device=self.members.device)
-        return t[:rows * groups]
 
 
 def route(picks: torch.Tensor, plan: Plan, tile: int = PREFILL_TILE) -> None:
@@ -205,55 +195,24 @@ def _fits(plan: Plan, rows: int, x_rows: int | None, pair_rows: int) -> None:
         raise ValueError(f"buffers too small for {rows} rows x {plan.slots} slots")
 
 
-# Which call last wrote a pair-activation buffer through this library (address -> a running number).  ``gate_up`` notes
-# it and ``down`` trusts the group sums a plan kept only while its own ``gate_up`` is still the last writer: launches
-# made through ctypes do not move torch's version counter, so that counter alone would miss them.
-_writes: dict[int, int] = {}
-_epoch = 0
-
-
-def wrote(t: torch.Tensor) -> int:
-    """Note that a kernel of this library has just (re)written ``t``; returns the note's number."""
-
-    global _epoch
-    _epoch += 1
-    _writes[t.data_ptr()] = _epoch
-    return _epoch
-
-
-def _group_sums(x: torch.Tensor, gs: int, into: torch.Tensor) -> torch.Tensor:
-    _lib.call("tf_group_sums", _lib.ptr(x), x.stride(0), int(x.shape[0]), int(x.shape[1]), gs, _lib.ptr(into))
-    return into
-
-
 def _launch(x: torch.Tensor, slots: int, table: torch.Tensor, gs: int, k: int, n: int, epi: int, plan: Plan,
-            out: torch.Tensor, limit: float, rows: int, xs: torch.Tensor | None = None,
-            xs_out: torch.Tensor | None = None, arith: int = ARITH_F16) -> None:
+            out: torch.Tensor, limit: float, rows: int, arith: int = ARITH_F16) -> None:
     bound = max_items(rows * plan.slots, plan.experts, plan.tile)
     common = (gs, epi, _lib.ptr(x), x.stride(0), slots, _lib.ptr(table), k // gs, n // COLS, _lib.ptr(plan.items),
               _lib.ptr(plan.counts), _lib.ptr(plan.members), _lib.ptr(out), n, limit)
     if plan.prefill:
         _lib.call("tf_experts_prefill", *common, bound, plan.tile, arith)
     else:
-        _lib.call("tf_experts_run", *common, bound * (n // COLS), _lib.ptr(xs), _lib.ptr(xs_out))
+        _lib.call("tf_experts_run", *common, bound * (n // COLS))
 
 
 def gate_up(x: torch.Tensor, ex: Experts, plan: Plan, out: torch.Tensor, rows: int) -> None:
-    """Token rows x bf16 [R, D] -> the activation of every pair, out bf16 [R * slots, NI].
-
-    On a decode plan the kernel also leaves, in the plan, the sum of every group of ``out``; ``down`` on the same
-    plan and the same (unmodified) ``out`` reads them instead of summing again."""
+    """Token rows x bf16 [R, D] -> the activation of every pair, out bf16 [R * slots, NI]."""
 
     epi = 2 if ex.swiglu else 1
     _check(x, ex.dims, out, ex.width, epi)
     _fits(plan, rows, x.shape[0], out.shape[0])
-    xs = xs_out = None
-    if not plan.prefill:
-        xs = _group_sums(x, ex.gs, plan.sums("x", int(x.shape[0]), ex.dims // ex.gs))
-        xs_out = plan.sums("act", int(out.shape[0]), ex.width // ex.gs)
-    _launch(x, plan.slots, ex.up, ex.gs, ex.dims, ex.width, epi, plan, out, ex.limit, rows, xs, xs_out, ex.arith)
-    stamp = wrote(out)
-    plan._act_key = None if plan.prefill else (out.data_ptr(), out._version, rows, ex.width, stamp)
+    _launch(x, plan.slots, ex.up, ex.gs, ex.dims, ex.width, epi, plan, out, ex.limit, rows, ex.arith)
 
 
 def down(act: torch.Tensor, ex: Experts, plan: Plan, out: torch.Tensor, rows: int) -> None:
@@ -263,10 +222,4 @@ def down(act: torch.Tensor, ex: Experts, plan: Plan, out: torch.Tensor, rows: in
     epi = 3 if (plan.prefill and out.dtype == torch.bfloat16) else 0
     _check(act, ex.width, out, ex.dims, epi)
     _fits(plan, rows, None, min(act.shape[0], out.shape[0]))
-    xs = None
-    if not plan.prefill:
-        if plan._act_key == (act.data_ptr(), act._version, rows, ex.width, _writes.get(act.data_ptr())):
-            xs = plan.sums("act", int(act.shape[0]), ex.width // ex.gs)        # left there by gate_up
-        else:
-            xs = _group_sums(act, ex.gs, plan.sums("act2", int(act.shape[0]), ex.width // ex.gs))
-    _launch(act, 0, ex.down, ex.gs, ex.width, ex.dims, epi, plan, out, 0.0, rows, xs, None, ex.arith)
+    _launch(act, 0, ex.down, ex.gs, ex.width, ex.dims, epi, plan, out, 0.0, rows, ex.arith)

@@ -77,7 +77,7 @@ class MoEBuffers:
         self.cfg, self.device, self._fused = cfg, device, {}
 
     def fused(self, gs: int) -> dict:
-        """Scratch of ``decode`` for tables of group size ``gs``, made on first use: item descriptors, group sums, the counters of the one-launch
+        """Scratch of ``decode`` for tables of group size ``gs``, made on first use: item descriptors, the counters of the one-launch
         form (status, then an arrival count a descriptor, then one a (token, 64 columns) cell) and the output."""
 
         if gs not in self._fused:
@@ -87,8 +87,6 @@ class MoEBuffers:
             self._fused[gs] = dict(
                 items=items * DONE_STRIDE,          # ints the descriptors' arrival counters take
                 desc=torch.zeros((1 + items, DESC_INTS), dtype=torch.int32, device=dev),
-                xs_x=torch.empty((self.rows, cfg.hidden_size // gs), dtype=torch.float32, device=dev),
-                xs_act=torch.empty((pairs, cfg.moe_intermediate_size // gs), dtype=torch.float32, device=dev),
                 counters=torch.zeros((1 + items * DONE_STRIDE + cells,), dtype=torch.int32, device=dev),
                 out=torch.empty((self.rows, cfg.hidden_size), dtype=torch.bfloat16, device=dev))
         return self._fused[gs]
@@ -156,7 +154,6 @@ def decode(x: torch.Tensor, logits: torch.Tensor, ex: grouped.Experts, buf: MoEB
     if logits.dtype != torch.float32 or logits.stride(1) != 1:
         raise ValueError("select: logits must be fp32 with unit-stride rows")
     f = buf.fused(ex.gs)
-    grouped.wrote(buf.act)          # the launches below rewrite the pair activations: sums a plan kept of them are void
     if out is None:
         out = f["out"][:n]
     plan = buf.plan
@@ -166,12 +163,11 @@ def decode(x: torch.Tensor, logits: torch.Tensor, ex: grouped.Experts, buf: MoEB
     ctr = f["counters"]
     if FUSED_DECODE:
         _lib.call("tf_moe_route_decode", _lib.ptr(logits), logits.stride(0), n, experts, top_k, int(buf.shared),
-                  _lib.ptr(x), x.stride(0), ex.dims, ex.gs, _lib.ptr(buf.pick), _lib.ptr(buf.wts), _lib.ptr(plan.members),
-                  _lib.ptr(plan.items), _lib.ptr(plan.counts), _lib.ptr(f["desc"]), _lib.ptr(f["xs_x"]), _lib.ptr(ctr),
-                  1 + f["items"] + cells)
+                  _lib.ptr(buf.pick), _lib.ptr(buf.wts), _lib.ptr(plan.members), _lib.ptr(plan.items),
+                  _lib.ptr(plan.counts), _lib.ptr(f["desc"]), _lib.ptr(ctr), 1 + f["items"] + cells)
         _lib.call("tf_moe_decode_experts", ex.gs, int(ex.swiglu), _lib.ptr(x), x.stride(0), n, buf.slots,
                   _lib.ptr(ex.up), _lib.ptr(ex.down), ex.dims, ex.width, _lib.ptr(f["desc"]), _lib.ptr(plan.counts),
-                  _lib.ptr(buf.wts), _lib.ptr(f["xs_x"]), _lib.ptr(buf.act), _lib.ptr(f["xs_act"]), _lib.ptr(buf.y),
+                  _lib.ptr(buf.wts), _lib.ptr(buf.act), _lib.ptr(buf.y),
                   _lib.ptr(out), ctr.data_ptr() + 4, ctr.data_ptr() + 4 * (1 + f["items"]), _lib.ptr(ctr), ex.limit,
                   items)
         return out
@@ -180,12 +176,11 @@ def decode(x: torch.Tensor, logits: torch.Tensor, ex: grouped.Experts, buf: MoEB
     if ROUTING_LAUNCH:
         # the routing in a launch of its own, then up, down and combine from its item descriptors
         _lib.call("tf_moe_route_decode", _lib.ptr(logits), logits.stride(0), n, experts, top_k, int(buf.shared),
-                  _lib.ptr(x), x.stride(0), ex.dims, ex.gs, _lib.ptr(buf.pick), _lib.ptr(buf.wts), _lib.ptr(plan.members),
-                  _lib.ptr(plan.items), _lib.ptr(plan.counts), _lib.ptr(f["desc"]), _lib.ptr(f["xs_x"]), arrive, cells)
+                  _lib.ptr(buf.pick), _lib.ptr(buf.wts), _lib.ptr(plan.members), _lib.ptr(plan.items),
+                  _lib.ptr(plan.counts), _lib.ptr(f["desc"]), arrive, cells)
         _lib.call("tf_experts_run_desc", ex.gs, 2 if ex.swiglu else 1, _lib.ptr(x), x.stride(0), buf.slots,
                   _lib.ptr(ex.up), ex.dims // ex.gs, ex.width // grouped.COLS, _lib.ptr(f["desc"]),
-                  _lib.ptr(plan.counts), _lib.ptr(act), ex.width, ex.limit, items, _lib.ptr(f["xs_x"]),
-                  _lib.ptr(f["xs_act"]))
+                  _lib.ptr(plan.counts), _lib.ptr(act), ex.width, ex.limit, items)
     else:
         # few logits: every workgroup of the up projection routes for itself; many: the top-k runs once, in a launch
         # before, and the workgroups only rebuild the plan from its picks
@@ -196,10 +191,10 @@ def decode(x: torch.Tensor, logits: torch.Tensor, ex: grouped.Experts, buf: MoEB
                   int(buf.shared), ex.gs,
                   int(ex.swiglu), _lib.ptr(x), x.stride(0), _lib.ptr(ex.up), ex.dims, ex.width, _lib.ptr(buf.pick),
                   _lib.ptr(buf.wts), _lib.ptr(plan.members), _lib.ptr(plan.items), _lib.ptr(plan.counts),
-                  _lib.ptr(f["desc"]), _lib.ptr(act), _lib.ptr(f["xs_act"]), ex.limit, items, arrive, cells)
+                  _lib.ptr(f["desc"]), _lib.ptr(act), ex.limit, items, arrive, cells)
     # the down projection; the workgroup that completes a (token, 64 columns) cell writes the combined output
     _lib.call("tf_moe_down_combine", ex.gs, _lib.ptr(act), n, buf.slots, _lib.ptr(ex.down), ex.dims, ex.width,
-              _lib.ptr(f["desc"]), _lib.ptr(buf.wts), _lib.ptr(f["xs_act"]), _lib.ptr(buf.y), _lib.ptr(out), arrive, items)
+              _lib.ptr(f["desc"]), _lib.ptr(buf.wts), _lib.ptr(buf.y), _lib.ptr(out), arrive, items)
     return out
 
 

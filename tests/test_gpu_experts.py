@@ -86,26 +86,36 @@ def test_plan_groups_pairs_by_expert(rows, prefill, tile):
     assert np.array_equal(plan.members.cpu().numpy(), members)
 
 
-@pytest.mark.parametrize("case", CASES)
-def test_group_sums_made_by_the_kernel_equal_those_passed_in(case):
-    """tf_experts_run without ``xs`` sums each group of its rows itself: same bits as with tf_group_sums' sums."""
+@pytest.mark.parametrize("gs", [32, 64])
+def test_the_sums_a_wave_takes_from_its_inputs(gs):
+    """The affine form needs the sum of every group of inputs; each wave takes it from the inputs it streams.  A table
+    whose codes and scales are zero and whose bias is 1 in one group a column and 0 elsewhere makes every output
+    that group's sum itself: out[p, n] = sum of x[p, group n % KG], which pins the sums (a dropped chunk, a lane
+    left out of the row's tree or a wrong group would each show) for one and for two rows a pass."""
 
-    from tensorfold_amd import _lib, qmm
-    ex, _, _ = build(case, 44)
-    for rows in (1, 9):
-        x = synthetic.activations(rows, ex.dims, 45, 0.5).to(DEV)
-        picks = picks_for(rows, case, 46, hot=True if rows > 1 else None)
-        act, y, plan = run(ex, x, picks)
-        slots = picks.shape[1]
-        bound = experts.max_items(rows * slots, ex.count, experts.TILE)
-        act2, y2 = torch.empty_like(act), torch.empty_like(y)
-        _lib.call("tf_experts_run", ex.gs, 2 if ex.swiglu else 1, _lib.ptr(x), x.stride(0), slots, _lib.ptr(ex.up),
-                  ex.dims // ex.gs, ex.width // 32, _lib.ptr(plan.items), _lib.ptr(plan.counts), _lib.ptr(plan.members),
-                  _lib.ptr(act2), ex.width, ex.limit, bound * (ex.width // 32), None, None)
-        _lib.call("tf_experts_run", ex.gs, 0, _lib.ptr(act2), ex.width, 0, _lib.ptr(ex.down), ex.width // ex.gs,
-                  ex.dims // 32, _lib.ptr(plan.items), _lib.ptr(plan.counts), _lib.ptr(plan.members), _lib.ptr(y2),
-                  ex.dims, 0.0, bound * (ex.dims // 32), None, None)
-        assert torch.equal(act2, act) and torch.equal(y2, y), rows
+    d, k, e = 7 * gs, 6 * 64, 3                      # 7 or 14 column blocks (7: a half-empty pair), K of 12 or 6 groups
+    kg = k // gs
+    words = torch.zeros((e, d, k // 8), dtype=torch.int32)
+    scales = torch.zeros((e, d, kg), dtype=torch.bfloat16)
+    biases = torch.zeros((e, d, kg), dtype=torch.bfloat16)
+    cols = torch.arange(d)
+    biases[:, cols, cols % kg] = 1.0
+    down = tuple(t.to(DEV) for t in (words, scales, biases))
+    ex = experts.make([tuple(t.to(DEV) for t in synthetic.affine_general(k, d, gs, 3, (e,)))], down, gs)
+    assert ex.width == k and ex.dims == d
+    for rows, picks in ((1, [[2]]), (5, [[0], [0], [1], [0], [1]])):          # items of 1, of 3 (passes of 2 + 1), of 2
+        picks = torch.tensor(picks, dtype=torch.int32, device=DEV)
+        act = synthetic.activations(rows, k, 91 + rows, 1.0).to(DEV)
+        plan = experts.Plan(rows, 1, e, DEV)
+        experts.route(picks, plan)
+        y = torch.empty((rows, d), dtype=torch.float32, device=DEV)
+        experts.down(act, ex, plan, y, rows)
+        want = act.float().view(rows, kg, gs).double().sum(-1)[:, cols % kg]
+        assert (y.double().cpu() - want.cpu()).abs().max() <= 1e-5 * float(act.float().abs().sum(-1).max())
+        # every output of a group's columns holds the same bits: the sum does not depend on the lane or the wave
+        for g in range(kg):
+            same = y[:, g::kg]
+            assert torch.equal(same, same[:, :1].expand_as(same)), g
 
 
 def test_an_expert_shared_by_many_rows_makes_items_of_16():
@@ -310,27 +320,3 @@ def test_prompt_experts_beyond_the_range_of_fp16():
     assert rel_l2(f32(y), y_ref) <= 2e-3
     print(f"bf16 prompt form: act rel-L2 {rel_l2(f32(act), ora.bf16_from_bits(act_ref)):.2e}, "
           f"y rel-L2 {rel_l2(f32(y), y_ref):.2e}, max-abs {max_abs(f32(y), y_ref):.3e}")
-
-
-def test_group_sums_kept_by_a_plan_are_dropped_when_the_activations_are_rewritten():
-    """``down`` reuses the group sums ``gate_up`` left in its plan only while that call is still the last one to have
-    written the activation buffer: a second ``gate_up`` into the same buffer under another plan voids them."""
-
-    case = CASES[2]
-    ex, _, _ = build(case, 53)
-    rows = 6
-    picks = picks_for(rows, case, 54).to(DEV).contiguous()
-    slots = picks.shape[1]
-    x1 = synthetic.activations(rows, ex.dims, 55, 0.5).to(DEV)
-    x2 = synthetic.activations(rows, ex.dims, 56, 2.0).to(DEV)
-    a, b = experts.Plan(rows, slots, ex.count, DEV), experts.Plan(rows, slots, ex.count, DEV)
-    experts.route(picks, a)
-    experts.route(picks, b)
-    act = torch.empty((rows * slots, ex.width), dtype=torch.bfloat16, device=DEV)
-    experts.gate_up(x1, ex, a, act, rows)
-    experts.gate_up(x2, ex, b, act, rows)             # the buffer now holds x2's activations; a's sums are x1's
-    ya = torch.empty((rows * slots, ex.dims), dtype=torch.float32, device=DEV)
-    yb = torch.empty_like(ya)
-    experts.down(act, ex, a, ya, rows)
-    experts.down(act, ex, b, yb, rows)
-    assert torch.equal(ya, yb)
