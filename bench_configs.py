@@ -1,7 +1,7 @@
 """Kernel timings of the benchmark configurations that are not bench.py's headline: 0 (dense 4-bit projection),
 2 (verify-window MoE layer), 3 (prompt chunk, grouped MFMA) and 4 (EXL3 projections).
 
-    python bench_configs.py [c0] [c2] [c3] [c4] [c4p] [glue] [c4x] [mfma] [floor]
+    python bench_configs.py [c0] [c2] [c3] [c4] [c4p] [glue] [c4x] [mfma] [floor] [timeline]
 
 One JSON line a configuration: time of one pass (hipGraph of back-to-back passes cycling over enough weight copies to
 miss the 256 MB Infinity Cache, HIP events around the replay), algorithmic bytes or flops, and the fraction of the
@@ -359,11 +359,77 @@ def floor() -> dict:
     return out
 
 
+def timeline() -> dict:
+    """Where a decode launch of configuration 1 spends its time, workgroup by workgroup: the two launches of the
+    layer (routing + up projection; down projection + combine) run through the timeline build of the library, whose
+    kernels note when each workgroup passes six marks.  Ten launches back to back in a graph, cycling the layers'
+    tables; the marks kept are the last launch's, in microseconds from its first workgroup's start."""
+
+    import ctypes
+
+    import numpy as np
+
+    import bench as b
+    from tensorfold_amd import _lib, build
+
+    marks = ("entry", "item_known", "first_loads_out", "wave0_streamed", "all_waves_streamed", "unit_done")
+    tables, keep = b.device_tables(b.SHAPE, b.LAYERS, DEV)
+    del keep
+    out = {"config": "timeline: per-workgroup marks of the decode layer's two launches (configuration 1)",
+           "marks": list(marks), "unit": "us from the launch's first workgroup", "launches": {}}
+    for tokens in (1, 4, 8):
+        layer = b.Layer(tokens, tables, DEV)
+        layer.route_plans()
+        plan = layer.plans[2]
+        with _lib.through(build.TIMELINE_LIB) as tl:
+            for name, fn in (("route_up", lambda i: layer.up(i, plan)), ("down_combine", lambda i: layer.down(i, plan))):
+                fn(0)
+                torch.cuda.synchronize()
+                if tl.tf_timeline_clear():
+                    raise RuntimeError(tl.tf_last_error().decode())
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    for i in range(10):
+                        fn(i)
+                g.replay()
+                g.replay()
+                torch.cuda.synchronize()
+                h = np.zeros((len(marks) + 1, 4096), dtype=np.uint64)
+                if tl.tf_timeline_read(h.ctypes.data_as(ctypes.c_void_p), h.shape[0], h.shape[1]):
+                    raise RuntimeError(tl.tf_last_error().decode())
+                where = h[len(marks)]
+                h = h[:len(marks)].astype(np.int64)
+                started, live = h[0] > 0, h[3] > 0
+                t0 = h[0][started].min()
+                row = {"workgroups": int(started.sum()), "streaming": int(live.sum())}
+                for k, mark in enumerate(marks):
+                    sel = (started if k == 0 else live) & (h[k] > 0)
+                    if not sel.any():
+                        continue
+                    v = (h[k][sel] - t0) / 100.0
+                    row[mark] = {"min": float(v.min()), "median": float(np.median(v)),
+                                 "p90": float(np.percentile(v, 90)), "max": float(v.max())}
+                d = (h[3] - h[2])[live] / 100.0
+                row["wave0_stream_us"] = {"min": float(d.min()), "median": float(np.median(d)), "max": float(d.max())}
+                # the compute unit of a workgroup: (XCC, engine, shader array, unit); how many streaming workgroups
+                # each unit ran, and when the last of them finished
+                hw = where[live]
+                cu = ((hw >> np.uint64(32)) << np.uint64(8)) | ((hw >> np.uint64(8)) & np.uint64(0xFF))
+                ids, count = np.unique(cu, return_counts=True)
+                end = (h[5][live] - t0) / 100.0
+                last = {int(n): [float(np.max(end[cu == u])) for u in ids[count == n]] for n in np.unique(count)}
+                row["units_used"] = int(len(ids))
+                row["by_workgroups_a_unit"] = {str(n): {"units": len(v), "mean_last_done_us": float(np.mean(v))}
+                                               for n, v in last.items()}
+                out["launches"][f"{tokens}_tokens_{name}"] = row
+    return out
+
+
 def main() -> int:
     torch.cuda.set_device(0)
     which = sys.argv[1:] or ["c0", "c2", "c3", "c4"]
     for name in which:
-        res = {"mfma": mfma, "c0": c0, "c2": c2, "c3": c3, "c4": c4, "c4p": c4p, "glue": glue_, "c4x": c4x, "floor": floor}[name]()
+        res = {"mfma": mfma, "c0": c0, "c2": c2, "c3": c3, "c4": c4, "c4p": c4p, "glue": glue_, "c4x": c4x, "floor": floor, "timeline": timeline}[name]()
         torch.cuda.empty_cache()
         print(json.dumps(res, default=lambda v: round(v, 4)), flush=True)
     return 0

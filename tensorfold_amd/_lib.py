@@ -2,9 +2,11 @@
 
 from __future__ import annotations
 
+import contextlib
 import ctypes
 from ctypes import c_float, c_int, c_int64, c_void_p
 from functools import lru_cache
+from pathlib import Path
 
 import torch
 
@@ -47,9 +49,7 @@ PROTOTYPES = {
 }
 
 
-@lru_cache(maxsize=1)
-def lib() -> ctypes.CDLL:
-    so = build.load()
+def _declare(so: ctypes.CDLL) -> ctypes.CDLL:
     so.tf_last_error.restype = ctypes.c_char_p
     so.tf_last_error.argtypes = []
     so.tf_version.restype = c_int
@@ -59,6 +59,28 @@ def lib() -> ctypes.CDLL:
         fn.argtypes = args
         fn.restype = c_int
     return so
+
+
+@lru_cache(maxsize=1)
+def lib() -> ctypes.CDLL:
+    return _declare(build.load())
+
+
+_other: ctypes.CDLL | None = None
+
+
+@contextlib.contextmanager
+def through(path):
+    """Route ``call`` through another build of the library (the timeline build) inside the block; yields it."""
+
+    global _other
+    if not Path(path).exists():
+        raise RuntimeError(f"tensorfold-amd: {path} is missing: run `python -c 'import __graft_entry__ as g; g.build()'`")
+    _other = _declare(ctypes.CDLL(str(path)))
+    try:
+        yield _other
+    finally:
+        _other = None
 
 
 @lru_cache(maxsize=1)
@@ -86,7 +108,7 @@ def call(name: str, *args) -> None:
     """Run entry point ``name`` on the current stream; a non-zero status raises with the library's sentence."""
 
     _ready()
-    so = lib()
+    so = _other or lib()
     if getattr(so, name)(*args, stream()):
         raise RuntimeError(so.tf_last_error().decode())
 

@@ -18,6 +18,7 @@ ARCH = "gfx950"
 HERE = Path(__file__).resolve().parent
 CSRC = HERE / "csrc"
 LIB = HERE / "libtfmi.so"
+TIMELINE_LIB = HERE / "libtfmi_timeline.so"      # the same kernels with per-workgroup timestamps (see compile)
 PROBE = HERE / "probe_mfma"          # stand-alone measurement of the matrix instructions' issue rates (csrc/probe_mfma.hip)
 SOURCES = ("api.hip", "pack.hip", "decode.hip", "fused.hip", "route.hip", "norm.hip", "prefill.hip", "exl3.hip", "exl3_experts.hip")
 # packed-fp32 VALU forms are switched off for the device pass (the host pass warns that it does not know the feature)
@@ -63,9 +64,10 @@ def stale() -> bool:
     return built_id() != source_id()
 
 
-def compile(verbose: bool = False) -> Path:
+def compile(verbose: bool = False, timeline: bool = False) -> Path:
     """Compile every kernel for gfx950 into ``libtfmi.so`` (cross-compiles without a GPU): one hipcc per source,
-    side by side, then a link."""
+    side by side, then a link.  ``timeline``: the same sources with -DTF_TIMELINE into ``libtfmi_timeline.so``, whose
+    decode expert kernels note per-workgroup timestamps (``bench_configs.py timeline`` reads them)."""
 
     import tempfile
     from concurrent.futures import ThreadPoolExecutor
@@ -73,7 +75,8 @@ def compile(verbose: bool = False) -> Path:
     cc = hipcc()
     if cc is None:
         raise RuntimeError("tensorfold-amd: hipcc was not found; ROCm's compiler is needed to build libtfmi.so")
-    say(f"building {LIB.name} for {ARCH} (about half a minute)")
+    target = TIMELINE_LIB if timeline else LIB
+    say(f"building {target.name} for {ARCH} (about half a minute)")
     noise = "packed-fp32-ops"
 
     def run(cmd: list[str]) -> str:
@@ -84,18 +87,21 @@ def compile(verbose: bool = False) -> Path:
         return err
 
     compile_flags = [f for f in FLAGS if f != "-shared"] + [f'-DTF_BUILD_ID="{source_id()}"']
+    if timeline:
+        compile_flags.append("-DTF_TIMELINE")
     with tempfile.TemporaryDirectory(prefix="tfmi-build-") as tmp:
         objects = [str(Path(tmp) / (Path(s).stem + ".o")) for s in SOURCES]
         with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
             logs = list(pool.map(lambda so: run([cc, *compile_flags, "-c", str(CSRC / so[0]), "-o", so[1]]),
                                  zip(SOURCES, objects)))
-        logs.append(run([cc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", str(LIB), *objects]))
-        logs.append(run([cc, "-O3", f"--offload-arch={ARCH}", "-o", str(PROBE), str(CSRC / "probe_mfma.hip")]))
+        logs.append(run([cc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", str(target), *objects]))
+        if not timeline:
+            logs.append(run([cc, "-O3", f"--offload-arch={ARCH}", "-o", str(PROBE), str(CSRC / "probe_mfma.hip")]))
     if verbose:
         for text in logs:
             if text:
                 say(text)
-    return LIB
+    return target
 
 
 @lru_cache(maxsize=1)

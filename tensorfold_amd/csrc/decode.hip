@@ -130,9 +130,9 @@ __device__ __forceinline__ void qmm_block(const uint16_t* __restrict__ X, int64_
   const uint32_t* wbase = W + ((size_t)tile * KG) * (size_t)(CH * 256) + lane * 4;
   const int col = tile * 64 + lane;
   auto wq = [&](int g, int m, int i) { return ldg16(wbase + ((size_t)g * CH + i) * 256); };
-  auto sb = [&](int g, int m, float& s, float& b) {
-    s = bf16_f32(S[(size_t)g * sb_stride + col]);
-    b = bf16_f32(B[(size_t)g * sb_stride + col]);
+  auto sb = [&](int g, int m, uint32_t& s, uint32_t& b) {
+    s = S[(size_t)g * sb_stride + col];
+    b = B[(size_t)g * sb_stride + col];
   };
   const int g0 = gs0 + (int)((long long)wave * per / WAVES), g1 = gs0 + (int)((long long)(wave + 1) * per / WAVES);
   float* xs = nullptr;
@@ -243,9 +243,9 @@ __device__ __forceinline__ void qmm_fat_block(const uint16_t* __restrict__ X, in
   const uint32_t* wbase = W + ((size_t)tile * KG) * (size_t)(CH * 256) + lane * 4;
   const int col = tile * 64 + lane;
   auto wq = [&](int g, int m, int i) { return ldg16(wbase + ((size_t)g * CH + i) * 256); };
-  auto sb = [&](int g, int m, float& s, float& b) {
-    s = bf16_f32(S[(size_t)g * sb_stride + col]);
-    b = bf16_f32(B[(size_t)g * sb_stride + col]);
+  auto sb = [&](int g, int m, uint32_t& s, uint32_t& b) {
+    s = S[(size_t)g * sb_stride + col];
+    b = B[(size_t)g * sb_stride + col];
   };
   auto sub_begin = [&](int u) { return (u >> 2) * per + (int)((long long)(u & 3) * per / 4); };
   const int SPW = 4 * SK / FW;

@@ -101,6 +101,7 @@ __global__ void __launch_bounds__(WAVES * 64)
                         const int* __restrict__ desc, const float* __restrict__ wts, float* __restrict__ y, uint16_t* __restrict__ out, int* __restrict__ arrive, int astride) {
   extern __shared__ float lds[];
   __shared__ int pairs[16];
+  TF_MARK(0);
   __builtin_amdgcn_s_setprio(3);       // the descriptor and the first requests issue ahead of the workgroups that already stream
   const int NB = D / 32, NB2d = (NB + 1) >> 1;
   const int it = blockIdx.x / NB2d, cb2 = blockIdx.x - it * NB2d;
@@ -113,6 +114,7 @@ __global__ void __launch_bounds__(WAVES * 64)
   NoHook none;
   expert_unit<GS, 1, 0, WAVES, COH_OUT>(act, NI, 0, Wdown, NI / GS, NB, e, cnt, pairs, cb2, y, D, 0.f, lds, none);
   combine_cells<WAVES>(pairs, cnt, slots, cb2, NB2d, D, astride, wts, y, out, arrive);
+  TF_MARK(5);
 }
 
 template <int GS, int NM, int EPI_UP, int WAVES>
@@ -171,6 +173,7 @@ __global__ void __launch_bounds__(WAVES * 64)
   extern __shared__ float lds[];
   __shared__ int pk[PLAN_THREADS];
   __shared__ ItemLds item;
+  TF_MARK(0);
   __builtin_amdgcn_s_setprio(3);       // the lookup issues ahead of the workgroups that already stream
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, threads = WAVES * 64;
   const int slots = TOPK + (shared ? 1 : 0), P = R * slots, E = NE + (shared ? 1 : 0);
@@ -420,6 +423,27 @@ int launch_fused(const uint16_t* x, int64_t x_stride, int slots, const uint32_t*
 }  // namespace tf
 
 using namespace tf;
+
+#ifdef TF_TIMELINE
+// The timeline build's two extra entry points: the marks of the last tf_moe_route_up / tf_moe_down_combine /
+// tf_moe_decode_experts launches, [TIMELINE_ROWS][TIMELINE_GROUPS]: six rows of 64-bit ticks of 10 ns (0: never
+// passed), then the row of hardware ids.
+extern "C" int tf_timeline_read(unsigned long long* host, int rows, int groups) {
+  clear_error();
+  TF_REQUIRE(host && rows == TIMELINE_ROWS && groups == TIMELINE_GROUPS, "timeline: the table is %d x %d",
+             TIMELINE_ROWS, TIMELINE_GROUPS);
+  TF_REQUIRE(hipMemcpyFromSymbol(host, HIP_SYMBOL(tf_timeline_marks), sizeof(tf_timeline_marks)) == hipSuccess,
+             "timeline: the copy failed");
+  return 0;
+}
+extern "C" int tf_timeline_clear(void) {
+  clear_error();
+  static const unsigned long long zeros[TIMELINE_ROWS][TIMELINE_GROUPS] = {};
+  TF_REQUIRE(hipMemcpyToSymbol(HIP_SYMBOL(tf_timeline_marks), zeros, sizeof(zeros)) == hipSuccess,
+             "timeline: the clear failed");
+  return 0;
+}
+#endif
 
 extern "C" int tf_moe_decode_experts(int gs, int swiglu, const uint16_t* x, int64_t x_stride, int rows, int slots,
                                      const uint32_t* up, const uint32_t* down, int d, int ni, const int32_t* desc,

@@ -79,11 +79,13 @@ __device__ __forceinline__ float dot2_bcast(float acc, uint32_t x, uint32_t q) {
 }
 
 // A group in registers: the weights of NM matrices (GS/32 16-byte chunks, scale and bias) and, of each of RB rows,
-// the lane's dword of each chunk of the group's inputs.
+// the lane's dword of each chunk of the group's inputs.  Scale and bias stay as they were loaded (bf16 bits: the
+// scale in the low half of `s`, the bias in the low half of `b`, or with BHI in its high half) until the group is
+// added: turning them into floats where they are loaded would make the wave wait for every load it has just issued.
 template <int GS, int NM>
 struct Stage {
   uint4 w[NM][GS / 32];
-  float s[NM], b[NM];
+  uint32_t s[NM], b[NM];
   uint32_t x[RBMAX][GS / 32];
 };
 
@@ -168,12 +170,12 @@ __device__ __forceinline__ void chunk_dot(float (&p)[NM][RB], const Stage<GS, NM
 
 // One wave's share of a GEMV: groups [gA, gB) of NM matrices against RB rows.
 //   wq(g, m, i)     -> the lane's 16 bytes of chunk i of group g of matrix m
-//   sb(g, m, s, b)  -> the lane's column's scale and bias of that group
+//   sb(g, m, s, b)  -> the lane's column's scale and bias of that group, as loaded (see Stage)
 //   xl[r]           -> row r's inputs as dwords, offset by lane % 16
 //   xsum(r, g)      -> row r's sum over group g (wave-uniform); with XIN the sums are taken from the staged inputs
 //   flush(g, acc)   -> called after group g has been added (wave-uniform); may park and clear acc
 // `st` holds the weights of groups gA .. gA + DEPTH - 1 on entry when `loaded`.
-template <int GS, int NM, int RB, int COH, bool XIN = false, class WQ, class SB, class XS, class FLUSH>
+template <int GS, int NM, int RB, int COH, bool XIN = false, bool BHI = false, class WQ, class SB, class XS, class FLUSH>
 __device__ __forceinline__ void gemv_stream(float (&acc)[NM][RB], Stage<GS, NM> (&st)[DEPTH], bool loaded,
                                             const WQ& wq, const SB& sb, const uint32_t* const (&xl)[RB],
                                             const XS& xsum, int gA, int gB, FLUSH& flush) {
@@ -213,7 +215,9 @@ __device__ __forceinline__ void gemv_stream(float (&acc)[NM][RB], Stage<GS, NM> 
 #pragma unroll
           for (int m = 0; m < NM; ++m) {
             const float pq = fmaf(-128.f, sc, p[m][r]);
-            acc[m][r] = fmaf(sc, st[d].b[m], fmaf(pq, st[d].s[m], acc[m][r]));
+            const float scale = __uint_as_float(st[d].s[m] << 16);
+            const float bias = __uint_as_float(BHI ? st[d].b[m] & 0xFFFF0000u : st[d].b[m] << 16);
+            acc[m][r] = fmaf(sc, bias, fmaf(pq, scale, acc[m][r]));
           }
         }
         flush(g, acc);
@@ -283,8 +287,11 @@ __device__ __forceinline__ void expert_pass(const uint16_t* __restrict__ X, int6
   };
   const int gA = slice_begin(wave * SPW, KG), gB = slice_begin((wave + 1) * SPW, KG);
   auto no_sums = [](int, int) { return 0.f; };
-  gemv_stream<GS, NM, RB, COH, true>(acc, st, loaded, wq, sb, xl, no_sums, gA, gB, flush);
+  if (first_pass) TF_MARK(2);
+  gemv_stream<GS, NM, RB, COH, true, true>(acc, st, loaded, wq, sb, xl, no_sums, gA, gB, flush);
+  TF_MARK(3);
   __syncthreads();
+  TF_MARK(4);
   // a wave a row, a lane a column: the slices' sums in slice order, then the epilogue
   for (int r = wave; r < RB; r += WAVES) {
     const int l = lane;
@@ -345,11 +352,10 @@ __device__ __forceinline__ bool expert_unit(const uint16_t* __restrict__ X, int6
       W + (((size_t)e * NB + (col_ok ? nb : NB - 1)) * KG) * (size_t)(NM * BW) + c * 4;
   const uint32_t* sbase = wbase - c * 4 + 32 * GS / 8 + c;
   auto wq = [&](int g, int m, int i) { return ldg16(wbase + ((size_t)g * NM + m) * BW + i * 128); };
-  auto sb = [&](int g, int m, float& s, float& b) {
-    const uint32_t v = __builtin_nontemporal_load(sbase + ((size_t)g * NM + m) * BW);
-    s = bf16_lo(v);
-    b = bf16_hi(v);
+  auto sb = [&](int g, int m, uint32_t& s, uint32_t& b) {
+    s = b = __builtin_nontemporal_load(sbase + ((size_t)g * NM + m) * BW);      // (scale | bias << 16)
   };
+  TF_MARK(1);
   const int gA = slice_begin(wave * SPW, KG), gB = slice_begin((wave + 1) * SPW, KG);
   float* part = lds;
   // the wave's first groups are on their way before anything else is read
@@ -372,6 +378,7 @@ __device__ __forceinline__ bool expert_unit(const uint16_t* __restrict__ X, int6
     TF_PASS(1);
   }
 #undef TF_PASS
+  TF_MARK(5);
   return true;
 }
 

@@ -94,6 +94,42 @@ __device__ __forceinline__ void prio_by_progress(int left, int n) {
   }
 }
 
+// ---- timeline build -----------------------------------------------------------------------------------------------
+//
+// Compiled with -DTF_TIMELINE (libtfmi_timeline.so) the decode expert kernels note when thread 0 of each workgroup
+// passes a few marks, on the 100 MHz clock every compute unit reads alike: 0 kernel entry, 1 the workgroup knows its
+// item, 2 its first weights and inputs are requested, 3 wave 0 has streamed its share, 4 every wave has, 5 the unit
+// has stored its output (and combined what it completed); a seventh row says which compute unit ran the workgroup.
+// The marks are kept in LDS and written out once, at mark
+// 5 (a store to memory at each mark would put its round trip into the waits that follow it).  The ordinary build
+// compiles the marks away.
+#ifdef TF_TIMELINE
+constexpr int TIMELINE_MARKS = 6, TIMELINE_ROWS = TIMELINE_MARKS + 1, TIMELINE_GROUPS = 4096;
+static __device__ unsigned long long tf_timeline_marks[TIMELINE_ROWS][TIMELINE_GROUPS];
+__device__ __forceinline__ unsigned long long* timeline_lds() {
+  __shared__ unsigned long long t[TIMELINE_MARKS];
+  return t;
+}
+__device__ __forceinline__ void timeline_mark(int k) {
+  if (threadIdx.x != 0) return;
+  unsigned long long* t = timeline_lds();
+  if (k == 0)
+    for (int i = 1; i < TIMELINE_MARKS; ++i) t[i] = 0;
+  t[k] = wall_clock64();
+  if (k == TIMELINE_MARKS - 1 && blockIdx.x < TIMELINE_GROUPS) {
+    for (int i = 0; i < TIMELINE_MARKS; ++i) tf_timeline_marks[i][blockIdx.x] = t[i];
+    // where it ran: the XCC id above the hardware id word (compute unit in bits 8-11, shader array 12, engine 13-15)
+    tf_timeline_marks[TIMELINE_MARKS][blockIdx.x] =
+        ((unsigned long long)__builtin_amdgcn_s_getreg((31 << 11) | 20) << 32) | __builtin_amdgcn_s_getreg((31 << 11) | 4);
+  }
+}
+#define TF_MARK(K_) timeline_mark(K_)
+#else
+#define TF_MARK(K_) \
+  do {              \
+  } while (0)
+#endif
+
 // ---- 4-bit blocks -------------------------------------------------------------------------------------------------
 
 constexpr uint32_t NIB_MASK = 0x000F000Fu;
