@@ -334,7 +334,12 @@ def mfma() -> dict:
 
 def floor() -> dict:
     """What a launch costs and how fast a short stream runs: a graph of one-workgroup kernels (the gap a launch adds
-    to a layer of two launches), and plain streaming reads of the sizes a decode launch moves (17, 34, 113 MB)."""
+    to a layer of two launches), and the stand-alone probe that streams configuration 1's expert units with the
+    decode kernels' access pattern and nothing else (csrc/probe_stream.hip; its table as text)."""
+
+    import subprocess
+
+    from tensorfold_amd import build
 
     from tensorfold_amd import _lib
 
@@ -348,15 +353,14 @@ def floor() -> dict:
         tiny(i)
         tiny(i)
 
-    out = {"config": "floor: launch gap in a graph and the streaming rate of short reads",
-           "one_tiny_kernel_us": graph_us(tiny, 200), "two_tiny_kernels_us": graph_us(pair, 100), "reads": {}}
-    for mb in (17, 34, 113):
-        ts = [torch.empty(mb * 1024 * 1024 // 4, dtype=torch.float32, device=DEV).normal_() for _ in range(4)]
-        o = torch.empty((), device=DEV)
-        us = graph_us(lambda i: torch.sum(ts[i % 4], dim=0, out=o), 40)
-        out["reads"][f"{mb}MB"] = {"us": us, "gbs": mb * 1.048576 / us * 1e3}
-        del ts
-    return out
+    if not build.PROBE_STREAM.exists():
+        raise RuntimeError(f"{build.PROBE_STREAM} is missing: run `python -c 'import __graft_entry__ as g; g.build()'`")
+    done = subprocess.run([str(build.PROBE_STREAM)], capture_output=True, text=True, timeout=120)
+    if done.returncode:
+        raise RuntimeError(f"probe_stream failed: {done.stdout} {done.stderr}")
+    return {"config": "floor: launch gap in a graph, and what a launch streams with the decode units' access pattern",
+            "one_tiny_kernel_us": graph_us(tiny, 200), "two_tiny_kernels_us": graph_us(pair, 100),
+            "probe_stream": done.stdout.splitlines()}
 
 
 def timeline() -> dict:

@@ -20,6 +20,7 @@ CSRC = HERE / "csrc"
 LIB = HERE / "libtfmi.so"
 TIMELINE_LIB = HERE / "libtfmi_timeline.so"      # the same kernels with per-workgroup timestamps (see compile)
 PROBE = HERE / "probe_mfma"          # stand-alone measurement of the matrix instructions' issue rates (csrc/probe_mfma.hip)
+PROBE_STREAM = HERE / "probe_stream"  # what a launch streams with the decode units' access pattern (csrc/probe_stream.hip)
 SOURCES = ("api.hip", "pack.hip", "decode.hip", "fused.hip", "route.hip", "norm.hip", "prefill.hip", "exl3.hip", "exl3_experts.hip")
 # packed-fp32 VALU forms are switched off for the device pass (the host pass warns that it does not know the feature)
 FLAGS = ("-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",
@@ -97,6 +98,8 @@ def compile(verbose: bool = False, timeline: bool = False) -> Path:
         logs.append(run([cc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", str(target), *objects]))
         if not timeline:
             logs.append(run([cc, "-O3", f"--offload-arch={ARCH}", "-o", str(PROBE), str(CSRC / "probe_mfma.hip")]))
+            logs.append(run([cc, "-O3", f"--offload-arch={ARCH}", "-o", str(PROBE_STREAM),
+                             str(CSRC / "probe_stream.hip")]))
     if verbose:
         for text in logs:
             if text:
