@@ -1,5 +1,10 @@
-"""EXL3 on the GPU: the device decoder against the oracle bit for bit (every codebook and width), the layer against
-the float64 forward, row invariance, dtypes, layouts (properties after tests/cuda/test_exl3_linear.py)."""
+"""The EXL3 linear on the GPU.  Bit-exact: the device decoder against the oracle's bit-by-bit decoder for every codebook
+at every width the linear takes, and at benchmark configuration 4's full size against the C decoder.  Within 2e-3: the layer
+against the float64 forward that rounds the rotated input to fp16 as the rotation kernel does.  Bit-equal among
+themselves: a row alone, in any window of rows, under any split of K, in either stored layout.  (The properties the
+reference's tests/cuda/test_exl3_linear.py asks of its kernels.)"""
+
+import dataclasses
 
 import numpy as np
 import pytest
@@ -10,40 +15,57 @@ from oracle import native
 from tensorfold_amd import synthetic
 from tensorfold_amd.exl3 import format as fmt
 from tensorfold_amd.exl3 import linear
-from tests.helpers import rel_l2, max_abs
+from tests.helpers import max_abs, rel_l2
 
 pytestmark = pytest.mark.gpu
-COMBOS = [("3inst", b) for b in (1, 2, 3, 4, 5, 6, 7, 8)] + [("mcg", b) for b in (1, 2, 3, 4, 5, 6, 7, 8)] \
-    + [("mul1", b) for b in (1, 1.5, 2, 2.5, 3, 3.5, 4, 5, 6, 7, 8)]
-ROWS = (1, 2, 3, 16, 17, 64, 128)
+WINDOWS = (1, 2, 3, 16, 17, 64, 128)
 
 
-def tensors(codebook, bits, kt=16, nt=8, seed=0):
-    rng = np.random.default_rng(seed)
-    trellis = torch.from_numpy(rng.integers(-2 ** 15, 2 ** 15, size=(kt, nt, fmt.tile_words(bits))).astype(np.int16))
-    k, n = 16 * kt, 16 * nt
-    suh = torch.from_numpy((rng.standard_normal(k) * 0.05).astype(np.float16))
-    svh = torch.from_numpy((rng.standard_normal(n) * 0.05).astype(np.float16))
-    return trellis, suh, svh
+@dataclasses.dataclass
+class Group:
+    """A synthetic quantized group: random trellis words, small signed input and output scales."""
+
+    codebook: str
+    bits: float
+    trellis: torch.Tensor
+    suh: torch.Tensor
+    svh: torch.Tensor
+
+    @classmethod
+    def draw(cls, codebook, bits, k=256, n=128, seed=0):
+        rng = np.random.default_rng(seed)
+        words = rng.integers(-2 ** 15, 2 ** 15, size=(k // 16, n // 16, fmt.tile_words(bits))).astype(np.int16)
+        scale = lambda size: torch.from_numpy((rng.standard_normal(size) * 0.05).astype(np.float16))
+        return cls(codebook, bits, torch.from_numpy(words), scale(k), scale(n))
+
+    def layer(self, **kw):
+        return linear.Exl3Linear.from_tensors(self.trellis, self.suh, self.svh, self.codebook, **kw)
+
+    def float64(self, x):
+        return ore.forward(x.numpy(), self.trellis.numpy(), self.suh.numpy(), self.svh.numpy(), self.bits,
+                           self.codebook, half_input=True)
 
 
-@pytest.mark.parametrize("codebook,bits", COMBOS)
-def test_decode_is_bit_exact(codebook, bits):
-    trellis, _, _ = tensors(codebook, bits)
-    w = linear.unpack_gpu(trellis, codebook)
-    ref = ore.unpack(trellis.numpy(), bits, codebook)
-    assert np.array_equal(w.cpu().numpy().view(np.uint16), ref.view(np.uint16))
+@pytest.mark.parametrize("codebook", list(ore.CODEBOOK_IDS))
+def test_every_width_decodes_bit_exactly(codebook):
+    """Every width the linear takes: whole bits with any codebook, 1.5 / 2.5 / 3.5 bits with mul1.  (The routed experts
+    take every half-bit width with every codebook; tests/test_gpu_exl3_experts.py decodes those.)"""
+
+    for bits in fmt.BITS:
+        if codebook != "mul1" and not float(bits).is_integer():
+            continue
+        g = Group.draw(codebook, bits, seed=int(2 * bits))
+        got = linear.unpack_gpu(g.trellis, codebook).cpu().numpy().view(np.uint16)
+        assert np.array_equal(got, ore.unpack(g.trellis.numpy(), bits, codebook).view(np.uint16)), bits
 
 
 def test_config4_decode_is_bit_exact_at_full_size():
     """benchmark configuration 4's gate/up trellis [320, 1088, 48] at 3 bits, all three codebooks, against the C decoder."""
 
     trellis, suh, svh = synthetic.exl3_layer(5120, 17408, 3, 4000)
-    for cb in ("3inst", "mcg", "mul1"):
-        layer = linear.Exl3Linear.from_tensors(trellis, suh, svh, cb)
-        got = layer.unpack().cpu().numpy().view(np.uint16)
-        want = native.exl3_unpack(trellis.numpy(), 6, ore.CODEBOOK_IDS[cb]).view(np.uint16)
-        assert np.array_equal(got, want), cb
+    for cb, cb_id in ore.CODEBOOK_IDS.items():
+        got = linear.Exl3Linear.from_tensors(trellis, suh, svh, cb).unpack().cpu().numpy().view(np.uint16)
+        assert np.array_equal(got, native.exl3_unpack(trellis.numpy(), 6, cb_id).view(np.uint16)), cb
 
 
 @pytest.mark.parametrize("m", [1, 8])
@@ -54,98 +76,87 @@ def test_config4_projections(k, n, m):
 
     trellis, suh, svh = synthetic.exl3_layer(k, n, 3, 4100 + k // 1000)
     x = synthetic.activations(m, k, 4200 + m, dtype=torch.float16)
-    layer = linear.Exl3Linear.from_tensors(trellis, suh, svh, "3inst")
-    y = layer(x.cuda())
+    y = linear.Exl3Linear.from_tensors(trellis, suh, svh, "3inst")(x.cuda())
     assert y.dtype == torch.float16 and y.shape == (m, n)
-    cols = slice(0, 1024)
-    want = native.exl3_linear(x.numpy(), trellis.numpy()[:, :64], suh.numpy(), svh.numpy()[cols], 6, 0)
-    got = y[:, cols].float().cpu().numpy()
+    want = native.exl3_linear(x.numpy(), trellis.numpy()[:, :64], suh.numpy(), svh.numpy()[:1024], 6, 0)
+    got = y[:, :1024].float().cpu().numpy()
     err = rel_l2(got, want)
     print(f"config 4 K={k} N={n} M={m}: rel-L2 {err:.2e}, max-abs {max_abs(got, want):.3e}")
     assert err <= 2e-3
 
 
-@pytest.mark.parametrize("codebook,bits", [("mul1", 2), ("mul1", 3), ("mul1", 6), ("3inst", 4), ("mcg", 8),
-                                           ("mul1", 2.5)])
 @pytest.mark.parametrize("split", [(1, 4), (2, 4), (8, 4), (2, 8), (1, 2)])
-def test_row_invariance(codebook, bits, split):
-    """Rows 1..128 identical in every window and under every split of K."""
-
-    trellis, suh, svh = tensors(codebook, bits, kt=64)          # K = 1024
-    layer = linear.Exl3Linear.from_tensors(trellis, suh, svh, codebook)
+@pytest.mark.parametrize("codebook,bits", [("mul1", 2), ("mul1", 3), ("mul1", 6), ("3inst", 4), ("mcg", 8), ("mul1", 2.5)])
+def test_a_rows_bits_do_not_depend_on_its_window_or_the_split(codebook, bits, split):
+    layer = Group.draw(codebook, bits, k=1024).layer()
     layer.split = split
-    x = synthetic.activations(128, layer.k, 3, dtype=torch.float16).cuda()
+    x = synthetic.activations(max(WINDOWS), layer.k, 3, dtype=torch.float16).cuda()
     whole = layer(x)
-    for m in ROWS:
-        assert torch.equal(layer(x[:m]), whole[:m]), f"rows 1..{m}"
-        for r in sorted({0, m // 2, m - 1}):
-            assert torch.equal(layer(x[r:r + 1])[0], whole[r]), f"row {r} alone vs {m}-row window"
-    assert int(layer.counters.abs().sum()) == 0                 # the arrival counters are left zero
+    for m in WINDOWS:
+        assert torch.equal(layer(x[:m]), whole[:m]), f"the first {m} rows as a window"
+        for r in {0, m // 2, m - 1}:
+            assert torch.equal(layer(x[r:r + 1])[0], whole[r]), f"row {r} by itself"
+    assert not layer.counters.any()                 # the arrival counters of the K splits are left at zero
 
 
 @pytest.mark.parametrize("codebook,bits", [("mul1", 2), ("mul1", 4), ("mul1", 6), ("3inst", 8), ("mcg", 4),
                                            ("3inst", 3), ("mul1", 3.5)])
-def test_matches_the_float64_reference(codebook, bits):
-    trellis, suh, svh = tensors(codebook, bits)
-    layer = linear.Exl3Linear.from_tensors(trellis, suh, svh, codebook)
-    x = synthetic.activations(17, layer.k, 5, dtype=torch.float16)
-    got = layer(x.cuda(), out_dtype=torch.float32).cpu().numpy()
-    want = ore.forward(x.numpy(), trellis.numpy(), suh.numpy(), svh.numpy(), bits, codebook, half_input=True)
-    assert rel_l2(got, want) < 2e-3
-    # the C statement of the same forward agrees
-    c = native.exl3_linear(x.numpy(), trellis.numpy(), suh.numpy(), svh.numpy(), int(2 * bits),
+def test_the_layer_against_the_float64_forward(codebook, bits):
+    g = Group.draw(codebook, bits)
+    x = synthetic.activations(17, 256, 5, dtype=torch.float16)
+    want = g.float64(x)
+    assert rel_l2(g.layer()(x.cuda(), out_dtype=torch.float32).cpu().numpy(), want) < 2e-3
+    # the C statement of the same forward agrees with the numpy one
+    c = native.exl3_linear(x.numpy(), g.trellis.numpy(), g.suh.numpy(), g.svh.numpy(), int(2 * bits),
                            ore.CODEBOOK_IDS[codebook])
     assert rel_l2(c, want) < 1e-5
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
-def test_input_and_output_dtypes(dtype):
-    trellis, suh, svh = tensors("mul1", 4)
-    layer = linear.Exl3Linear.from_tensors(trellis, suh, svh, "mul1")
+def test_activations_of_any_float_type(dtype):
+    layer = Group.draw("mul1", 4).layer()
     x = synthetic.activations(8, layer.k, 6, dtype=torch.float32).to(dtype).cuda()
-    half = layer(x.half(), out_dtype=torch.float32)
-    got = layer(x, out_dtype=torch.float32)
-    assert torch.allclose(got, half, rtol=2e-3, atol=2e-3)
-    assert layer(x).dtype == dtype and layer(x, out_dtype=torch.bfloat16).dtype == torch.bfloat16
+    as_half = layer(x.half(), out_dtype=torch.float32)
+    assert torch.allclose(layer(x, out_dtype=torch.float32), as_half, rtol=2e-3, atol=2e-3)
+    assert layer(x).dtype == dtype                                  # the output follows the input unless told
+    assert layer(x, out_dtype=torch.bfloat16).dtype == torch.bfloat16
 
 
-def test_bias_and_the_sign_words_of_older_checkpoints():
-    trellis, suh, svh = tensors("mcg", 4)
-    bias = torch.from_numpy((np.random.default_rng(2).standard_normal(svh.numel()) * 0.05).astype(np.float16))
-    plain = linear.Exl3Linear.from_tensors(trellis, suh, svh, "mcg")
-    with_bias = linear.Exl3Linear.from_tensors(trellis, suh, svh, "mcg", bias=bias)
-    x = synthetic.activations(3, plain.k, 7, dtype=torch.float16).cuda()
-    assert torch.allclose((with_bias(x, out_dtype=torch.float32) - plain(x, out_dtype=torch.float32)).cpu(),
-                          bias.float(), rtol=2e-2, atol=2e-2)
-
-    def pack(scales):
-        neg = (scales.numpy() < 0).reshape(-1, 16).astype(np.uint16)
-        words = (neg * (1 << np.arange(16, dtype=np.uint16))).sum(1).astype(np.uint16)
-        return torch.from_numpy(words.view(np.int16).copy())
-
-    signs = linear.Exl3Linear.from_tensors(trellis, pack(suh), pack(svh), "mcg")
-    assert torch.equal(signs.suh.cpu(), torch.from_numpy(ore.unpack_signs(pack(suh).numpy())))
-    assert torch.equal(signs.svh.cpu(), torch.where(svh < 0, -1.0, 1.0).half())
+def test_a_bias_is_added_after_the_output_scales():
+    g = Group.draw("mcg", 4)
+    bias = torch.from_numpy((np.random.default_rng(2).standard_normal(g.svh.numel()) * 0.05).astype(np.float16))
+    x = synthetic.activations(3, 256, 7, dtype=torch.float16).cuda()
+    delta = g.layer(bias=bias)(x, out_dtype=torch.float32) - g.layer()(x, out_dtype=torch.float32)
+    assert torch.allclose(delta.cpu(), bias.float().expand_as(delta), rtol=2e-2, atol=2e-2)
 
 
-def test_stored_layout_gives_the_same_bits():
-    trellis, suh, svh = tensors("mul1", 3)
-    a = linear.Exl3Linear.from_tensors(trellis, suh, svh, "mul1", layout="strips")
-    b = linear.Exl3Linear.from_tensors(trellis, suh, svh, "mul1", layout="stored")
-    assert a.words.shape != b.words.shape
-    x = synthetic.activations(5, a.k, 8, dtype=torch.float16).cuda()
-    assert torch.equal(a(x), b(x))
-    assert torch.equal(a.unpack(), b.unpack())
+def test_older_checkpoints_store_only_the_signs():
+    """int16 words, bit b of word w set when element 16 w + b is negative: they load as vectors of +-1."""
+
+    g = Group.draw("mcg", 4)
+    words = lambda v: torch.from_numpy(np.packbits((v.numpy() < 0).reshape(-1, 16), axis=1, bitorder="little")
+                                       .view(np.int16).reshape(-1).copy())
+    layer = linear.Exl3Linear.from_tensors(g.trellis, words(g.suh), words(g.svh), "mcg")
+    for got, scales in ((layer.suh, g.suh), (layer.svh, g.svh)):
+        assert torch.equal(got.cpu(), torch.where(scales < 0, -1.0, 1.0).half())
+    assert torch.equal(layer.suh.cpu(), torch.from_numpy(ore.unpack_signs(words(g.suh).numpy())))
 
 
-def test_bad_arguments_raise():
-    trellis, suh, svh = tensors("3inst", 3)
-    with pytest.raises(ValueError):
-        linear.Exl3Linear.from_tensors(trellis, suh, svh, "2mad")
-    with pytest.raises(ValueError):
-        linear.Exl3Linear.from_tensors(tensors("mul1", 2.5)[0], suh, svh, "3inst")
-    layer = linear.Exl3Linear.from_tensors(trellis, suh, svh, "3inst")
-    with pytest.raises(ValueError):
-        layer(torch.zeros((129, layer.k), dtype=torch.float16, device="cuda"))
-    with pytest.raises(ValueError):
-        layer(torch.zeros((1, layer.k + 128), dtype=torch.float16, device="cuda"))
+def test_both_stored_layouts_give_the_same_bits():
+    g = Group.draw("mul1", 3)
+    strips, stored = g.layer(layout="strips"), g.layer(layout="stored")
+    assert strips.words.shape != stored.words.shape
+    x = synthetic.activations(5, 256, 8, dtype=torch.float16).cuda()
+    assert torch.equal(strips(x), stored(x)) and torch.equal(strips.unpack(), stored.unpack())
+
+
+def test_what_the_layer_refuses():
+    g = Group.draw("3inst", 3)
+    with pytest.raises(ValueError):                                  # no such codebook
+        linear.Exl3Linear.from_tensors(g.trellis, g.suh, g.svh, "2mad")
+    with pytest.raises(ValueError):                                  # the linear kernel has half-bit widths for mul1 only
+        linear.Exl3Linear.from_tensors(Group.draw("mul1", 2.5).trellis, g.suh, g.svh, "3inst")
+    layer = g.layer()
+    for shape in ((129, layer.k), (1, layer.k + 128)):               # more rows than a decode call takes; a wrong K
+        with pytest.raises(ValueError):
+            layer(torch.zeros(shape, dtype=torch.float16, device="cuda"))
