@@ -264,7 +264,8 @@ def other_configs() -> dict:
     r = bc.c0()
     out["c0"] = {"workload": r["config"],
                  "rows": {str(m): {k: rnd(v) for k, v in d.items()} for m, d in r["rows"].items()},
-                 "prompt_form": {k: rnd(v) for k, v in r["prompt_form"].items()}}
+                 "prompt_form": {k: rnd(v) for k, v in r["prompt_form"].items()},
+                 "prompt_form_fp8": rnd(r["prompt_form_fp8"])}
     torch.cuda.empty_cache()
     r = bc.c2()
     out["c2"] = {k: rnd(v) for k, v in r.items() if k != "config"} | {"workload": r["config"]}

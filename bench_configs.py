@@ -78,8 +78,22 @@ def c0() -> dict:
     us = graph_us(lambda i: qmm.prefill_matmul(x, copies[i % len(copies)], out=y), 12)
     flop = 2.0 * m * n * k
     prompt = {"rows": m, "us": us, "tflops": flop / us * 1e-6, "frac_mfma": flop / us * 1e-6 / MFMA}
+    # the FP8 prompt path on the same weight: the rows quantized to e4m3 (a launch of its own), then the matmul; and
+    # at groups of 32, where the per-group fma weighs twice as much
+    xq = qmm.quantize_rows(x, 64)
+    q_us = graph_us(lambda i: qmm.quantize_rows(x, 64), 12)
+    m_us = graph_us(lambda i: qmm.prefill_matmul8(xq, copies[i % len(copies)], out=y), 12)
+    fp8 = {"rows": m, "quantize_us": q_us, "matmul_us": m_us, "tflops": flop / m_us * 1e-6,
+           "tflops_with_quantize": flop / (m_us + q_us) * 1e-6}
+    del copies
+    torch.cuda.empty_cache()
+    g32 = [qmm.pack(*rand_affine(n, k, 32, gen), 32) for _ in range(24)]
+    xq32 = qmm.quantize_rows(x, 32)
+    us16 = graph_us(lambda i: qmm.prefill_matmul(x, g32[i % len(g32)], out=y), 12)
+    us8 = graph_us(lambda i: qmm.prefill_matmul8(xq32, g32[i % len(g32)], out=y), 12)
+    fp8["g32"] = {"f16_tflops": flop / us16 * 1e-6, "fp8_tflops": flop / us8 * 1e-6}
     return {"config": "c0: dense 4-bit/g64 projection, N = K = 4096 (qmm kernel + slice reduce; group sums given)",
-            "bound": "hbm", "rows": out, "prompt_form": prompt}
+            "bound": "hbm", "rows": out, "prompt_form": prompt, "prompt_form_fp8": fp8}
 
 
 def moe_tables(shape, layers: int, gen):

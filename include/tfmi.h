@@ -100,6 +100,20 @@ int tf_qmm_prefill(const uint16_t* x, int64_t ldx, const uint32_t* weight, const
                    const uint16_t* biases, void* out, int m, int n, int k, int gs, int f32, int tile, int arith,
                    tf_stream_t stream);
 
+/* The FP8 prompt path.  tf_quantize_rows: a row's scale a = max|x| / 448 (1 for a row of zeros), x8 = OCP e4m3 of
+ * x / a (round to nearest even), xs[g] = bf16(sum of group g's inputs / a); x8 uint8 [m, k] with every octet of
+ * inputs stored in the matrix operand's order (0, 4, 1, 5, 2, 6, 3, 7), xs bf16 [m, k / gs], a fp32 [m]; k a multiple
+ * of gs and of 32.  Replaces kernels/qmm.py:222-255 `quantize_rows` (Triton).
+ * tf_qmm_prefill8: out = (sum over groups, in order, of fma(P, scale, .) with P = the group's sum of x8 * code, exact
+ * e4m3 operands; + xs . bias over the groups) * a, on tf_quantize_rows' output and a packed weight; out fp32 (f32) or
+ * bf16 [m, n]; k in whole steps of 64; a row's bits depend on that row alone; `tile` (0-11) is accepted and changes
+ * nothing.  Replaces kernels/qmm.cpp:151-157 `qmm_prefill8` (kernels/qmm_prefill8.cu). */
+int tf_quantize_rows(const uint16_t* x, int64_t ldx, int m, int k, int gs, uint8_t* x8, uint16_t* xs, float* a,
+                     tf_stream_t stream);
+int tf_qmm_prefill8(const uint8_t* x8, const uint16_t* xs, const float* a, const uint32_t* weight,
+                    const uint16_t* scales, const uint16_t* biases, void* out, int m, int n, int k, int gs, int f32,
+                    int tile, tf_stream_t stream);
+
 /* ---- routed experts (experts.cpp:77-82, module tensorfold_experts_v7) ---------------------------------------------- */
 
 /* MLX words [E, N, K/8], scales/biases [E, N, K/gs] -> blocks [E, N/32, K/gs, 32*gs/8 + 32].

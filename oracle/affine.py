@@ -183,3 +183,69 @@ def add_moe_norm(h: np.ndarray, y: np.ndarray, wts: np.ndarray, w: np.ndarray, e
     (families/nemotron_h/cuda/glue.py:103-141)."""
 
     return add_rmsnorm(h, moe_delta(y, wts, top_k), w, eps, gs)
+
+
+# -- the FP8 prompt path (cuda/kernels/qmm.py:222-268, qmm_prefill8.cu:1-2,186-188) --------------------------------
+
+def e4m3_bits(x: np.ndarray) -> np.ndarray:
+    """float32 -> OCP e4m3 (e4m3fn: bias 7, no infinities, largest 448) bit patterns, round to nearest even.  Values
+    are taken within +-464 (nothing larger is asked of it: ``quantize_rows`` divides by the row's max / 448)."""
+
+    v = np.ascontiguousarray(x, dtype=np.float32)
+    a = np.abs(v).astype(np.float64)
+    e = np.floor(np.log2(np.maximum(a, 2.0 ** -20)))
+    e = np.clip(e, -6, 8)                                  # below 2^-6 the step stays 2^-9 (subnormals)
+    step = 2.0 ** (e - 3)
+    q = np.rint(a / step)                                  # ties to even; 16 steps of a binade carry into the next
+    mag = q * step
+    e2 = np.floor(np.log2(np.maximum(mag, 2.0 ** -20)))
+    code = np.where(mag < 2.0 ** -6, np.rint(mag * 512.0),
+                    (e2 + 7) * 8 + np.rint(mag / 2.0 ** (e2 - 3)) - 8).astype(np.int64)
+    code = np.minimum(code, 0x7E)
+    return (code | ((np.signbit(v)).astype(np.int64) << 7)).astype(np.uint8)
+
+
+def e4m3_values(b: np.ndarray) -> np.ndarray:
+    """e4m3 bit patterns -> float32 values."""
+
+    b = np.ascontiguousarray(b).astype(np.int64)
+    ex, man = (b >> 3) & 15, b & 7
+    mag = np.where(ex == 0, man * 2.0 ** -9, (8 + man) * 2.0 ** (ex - 10))
+    return np.where(b & 0x80, -mag, mag).astype(np.float32)
+
+
+def quantize_rows(x: np.ndarray, gs: int):
+    """``quantize_rows`` (kernels/qmm.py:222-255).  x float32 [M, K] of bf16 values -> (x8 uint8 [M, K] e4m3 bits in
+    input order, xs float32 [M, K / gs] of bf16 values, a float32 [M]).  a = max|x| / 448 (1 for a row of zeros),
+    x8 = e4m3(x / a), xs = bf16(sum of the group's inputs / a); the sum is taken an octet of inputs at a time, in order,
+    and the octets' sums in order (the order the kernel fixes; the reference's Triton sum leaves it open)."""
+
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    m, k = x.shape
+    top = np.abs(x).max(axis=1)
+    a = np.where(top > 0, top / np.float32(448), np.float32(1)).astype(np.float32)
+    x8 = e4m3_bits(x / a[:, None])
+    octets = np.cumsum(x.reshape(m, k // 8, 8), axis=2, dtype=np.float32)[:, :, -1]
+    sums = np.cumsum(octets.reshape(m, k // gs, gs // 8), axis=2, dtype=np.float32)[:, :, -1]
+    return x8, bf16(sums / a[:, None]), a
+
+
+def prefill8(x8: np.ndarray, xs: np.ndarray, a: np.ndarray, words: np.ndarray, scales: np.ndarray,
+             biases: np.ndarray, gs: int) -> np.ndarray:
+    """``prefill_matmul8`` on ``quantize_rows`` output (qmm_prefill8.cu:1-2): per group, in order,
+    acc = fma(P, s, acc) with P the group's sum of x8 * q (exact operands; taken in float64 here, the matrix unit's
+    fp32 sum of the same exact products can differ in its last bit), then acc += xs . bias over the groups, then
+    out = acc * a.  float32 [M, N]."""
+
+    xv = e4m3_values(x8).astype(np.float64)
+    q = nibbles(words).astype(np.float64)                               # [N, K]
+    m, k = xv.shape
+    s = np.asarray(scales, dtype=np.float32)
+    b = np.asarray(biases, dtype=np.float32)
+    acc = np.zeros((m, q.shape[0]), dtype=np.float32)
+    for g in range(k // gs):
+        part = (xv[:, g * gs:(g + 1) * gs] @ q[:, g * gs:(g + 1) * gs].T).astype(np.float32)
+        acc = (part.astype(np.float64) * s[:, g].astype(np.float64)[None, :] + acc.astype(np.float64)).astype(np.float32)
+    acc = (acc.astype(np.float64) + np.asarray(xs, dtype=np.float64) @ b.astype(np.float64).T).astype(np.float32)
+    return acc * np.asarray(a, dtype=np.float32)[:, None]
+

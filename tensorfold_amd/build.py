@@ -21,7 +21,7 @@ LIB = HERE / "libtfmi.so"
 TIMELINE_LIB = HERE / "libtfmi_timeline.so"      # the same kernels with per-workgroup timestamps (see compile)
 PROBE = HERE / "probe_mfma"          # stand-alone measurement of the matrix instructions' issue rates (csrc/probe_mfma.hip)
 PROBE_STREAM = HERE / "probe_stream"  # what a launch streams with the decode units' access pattern (csrc/probe_stream.hip)
-SOURCES = ("api.hip", "pack.hip", "decode.hip", "fused.hip", "route.hip", "norm.hip", "prefill.hip", "exl3.hip", "exl3_experts.hip")
+SOURCES = ("api.hip", "pack.hip", "decode.hip", "fused.hip", "route.hip", "norm.hip", "prefill.hip", "prefill8.hip", "exl3.hip", "exl3_experts.hip")
 # packed-fp32 VALU forms are switched off for the device pass (the host pass warns that it does not know the feature)
 FLAGS = ("-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops")

@@ -241,3 +241,51 @@ def prefill_matmul(x: torch.Tensor, q: Q4, *, f32: bool = False, tile: int = 0,
               _lib.ptr(q.biases.contiguous()), _lib.ptr(out), m, q.n, q.k, q.gs, int(f32), tile,
               q.arith if arith is None else int(arith))
     return out
+
+
+def quantize_rows(x: torch.Tensor, gs: int = 64) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Inputs for ``prefill_matmul8`` (cuda/kernels/qmm.py:245-255): e4m3 bytes [M, K] with every octet of inputs in
+    the matrix operand's order, each group's input sum over the row scale (bf16 [M, K / gs]), the row scales (fp32
+    [M]: max|x| / 448)."""
+
+    _lib.on_gpu(x)
+    if x.dim() != 2 or x.dtype != torch.bfloat16:
+        raise ValueError("quantize_rows: x must be bf16 (M, K)")
+    m, k = (int(v) for v in x.shape)
+    if k % gs or k % 32:
+        raise ValueError("quantize_rows takes K a multiple of the group and of 32")
+    if x.stride(1) != 1 or (m > 1 and x.stride(0) % 8) or x.data_ptr() % 16:
+        x = x.clone(memory_format=torch.contiguous_format)
+    x8 = torch.empty((m, k), dtype=torch.uint8, device=x.device)
+    xs = torch.empty((m, k // gs), dtype=torch.bfloat16, device=x.device)
+    a = torch.empty((m,), dtype=torch.float32, device=x.device)
+    _lib.call("tf_quantize_rows", _lib.ptr(x), x.stride(0), m, k, gs, _lib.ptr(x8), _lib.ptr(xs), _lib.ptr(a))
+    return x8, xs, a
+
+
+def prefill_matmul8(xq: tuple[torch.Tensor, torch.Tensor, torch.Tensor], q: Q4, *, f32: bool = False, tile: int = 0,
+                    out: torch.Tensor | None = None) -> torch.Tensor:
+    """FP8 prompt matmul on ``quantize_rows`` output, the 4-bit codes as exact e4m3 operands
+    (cuda/kernels/qmm.py:258-268); a row's bits depend only on that row.  K in whole steps of 64."""
+
+    x8, xs, a = xq
+    _lib.on_gpu(x8, xs, a)
+    if x8.dim() != 2 or x8.shape[1] != q.k:
+        raise ValueError(f"prefill_matmul8: inputs must be (M, {q.k})")
+    m = int(x8.shape[0])
+    if x8.dtype != torch.uint8 or not x8.is_contiguous() or xs.dtype != torch.bfloat16 or not xs.is_contiguous() \
+            or tuple(xs.shape) != (m, q.k // q.gs) or a.dtype != torch.float32 or tuple(a.shape) != (m,) \
+            or not a.is_contiguous():
+        raise ValueError("prefill_matmul8: takes what quantize_rows returned for this weight's group size")
+    if q.k % 64:
+        raise ValueError("prefill_matmul8 takes K in whole steps of 64 inputs")
+    if out is None:
+        out = torch.empty((m, q.n), dtype=torch.float32 if f32 else torch.bfloat16, device=x8.device)
+    elif tuple(out.shape) != (m, q.n) or out.dtype != (torch.float32 if f32 else torch.bfloat16) \
+            or not out.is_contiguous() or out.device != x8.device:
+        raise ValueError(f"prefill_matmul8: out must be contiguous ({m}, {q.n}) {'fp32' if f32 else 'bf16'}")
+    _lib.call("tf_qmm_prefill8", _lib.ptr(x8), _lib.ptr(xs), _lib.ptr(a), _lib.ptr(q.weight),
+              _lib.ptr(q.scales.contiguous()), _lib.ptr(q.biases.contiguous()), _lib.ptr(out), m, q.n, q.k, q.gs,
+              int(f32), tile)
+    return out
+

@@ -178,3 +178,67 @@ def test_moe_delta_weights_the_routed_slots_only():
     assert np.array_equal(hn, ora.bf16(h + got))
     h2, out2, xs2 = ora.add_rmsnorm(h, got, w, 1e-5)
     assert np.array_equal(out, out2) and np.array_equal(xs, xs2) and np.array_equal(hn, h2)
+
+
+# -- the FP8 prompt path's oracle -----------------------------------------------------------------------------------
+
+def test_e4m3_against_an_independent_conversion_and_known_codes():
+    """The numpy e4m3 rounding against torch's float8_e4m3fn (another implementation of the OCP format) over the whole
+    range that quantize_rows produces, ties and subnormals included; the value table of all 256 codes; known codes."""
+
+    import torch
+
+    rng = np.random.default_rng(0)
+    v = np.concatenate([rng.uniform(-448, 448, 20000), rng.uniform(-1, 1, 20000), rng.uniform(-2 ** -5, 2 ** -5, 20000),
+                        [0, 448, -448, 2 ** -9, 2 ** -10, 3 * 2 ** -10, 15.5, 16.5, 17, 18, 232, 240, 248, 463.9]]
+                       ).astype(np.float32)
+    want = torch.from_numpy(v).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(ora.e4m3_bits(v), want)
+    table = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).float().numpy()
+    mine = ora.e4m3_values(np.arange(256, dtype=np.uint8))
+    assert np.array_equal(mine[~np.isnan(table)], table[~np.isnan(table)])
+    assert ora.e4m3_bits(np.float32([1.0, 448.0, -0.5, 2 ** -9])).tolist() == [0x38, 0x7E, 0xB0, 0x01]
+    # a 4-bit code in a byte is the e4m3 number code * 2^-9: what lets the packed nibbles be the matrix operand
+    assert np.array_equal(ora.e4m3_values(np.arange(16, dtype=np.uint8)), np.arange(16, dtype=np.float32) * 2.0 ** -9)
+
+
+def test_quantize_rows_closed_forms():
+    """The largest magnitude of a row lands on +-448; a row of zeros keeps scale 1; the group sums are the inputs'
+    sums over the scale; dequantizing x8 * a gives x back within e4m3's half step (2^-4 relative)."""
+
+    rng = np.random.default_rng(1)
+    x = ora.bf16(rng.standard_normal((5, 256)).astype(np.float32))
+    x[3] = 0
+    x[4, 7] = 50.0
+    x8, xs, a = ora.quantize_rows(x, 64)
+    v = ora.e4m3_values(x8)
+    assert np.array_equal(np.abs(v).max(1)[[0, 1, 2, 4]], np.float32([448] * 4)) and not v[3].any() and a[3] == 1
+    assert a[4] == np.float32(50.0) / np.float32(448)
+    back = v * a[:, None]
+    assert np.all(np.abs(back - x) <= np.abs(x) * 2.0 ** -4 + a[:, None] * 2.0 ** -10)
+    want = x.reshape(5, 4, 64).astype(np.float64).sum(-1) / a[:, None]
+    assert np.all(np.abs(xs - want) <= np.abs(want) * 2.0 ** -8 + 1e-3)
+
+
+def test_prefill8_is_the_dequantized_product_of_the_quantized_rows():
+    """prefill8 on exact inputs: with x already on the e4m3 grid times a power-of-two row scale the quantization is
+    lossless, and the result must be the float64 dequant-then-matmul to fp32 rounding."""
+
+    rng = np.random.default_rng(2)
+    n, k, gs = 40, 128, 32
+    words, scales, biases = rng_tables(n, k, gs, 3)
+    grid = ora.e4m3_values(rng.integers(0, 0x7F, (6, k)).astype(np.uint8)) * np.where(rng.random((6, k)) < 0.5, -1, 1)
+    grid[:, 0] = 448.0                                              # every row's scale is then 2^-3 exactly
+    x = (grid * 0.125).astype(np.float32)
+    assert np.array_equal(ora.bf16(x), x)
+    x8, xs, a = ora.quantize_rows(x, gs)
+    assert np.array_equal(ora.e4m3_values(x8), grid.astype(np.float32)) and np.all(a == 0.125)
+    got = ora.prefill8(x8, xs, a, words, scales, biases, gs)
+    dense = ora.dequantize(words, scales, biases, gs).astype(np.float64)
+    # xs is rounded to bf16 (8 bits): the bias term carries that, so compare the scale term tightly and the whole loosely
+    q = ora.nibbles(words).astype(np.float64)
+    scale_term = (x.astype(np.float64)[:, None, :] * q[None] * np.repeat(scales.astype(np.float64), gs, 1)[None]).sum(-1)
+    bias_term = (xs.astype(np.float64) * a[:, None]) @ biases.astype(np.float64).T
+    assert np.allclose(got, scale_term + bias_term, rtol=1e-5, atol=1e-5)
+    want = x.astype(np.float64) @ dense.T
+    assert np.linalg.norm(got - want) / np.linalg.norm(want) < 5e-3
