@@ -403,7 +403,7 @@ def timeline() -> dict:
             for name, fn in (("route_up", lambda i: layer.up(i, plan)), ("down_combine", lambda i: layer.down(i, plan))):
                 fn(0)
                 torch.cuda.synchronize()
-                if tl.tf_timeline_clear():
+                if tl.tf_timeline_clear_moe():
                     raise RuntimeError(tl.tf_last_error().decode())
                 g = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(g):
@@ -413,7 +413,7 @@ def timeline() -> dict:
                 g.replay()
                 torch.cuda.synchronize()
                 h = np.zeros((len(marks) + 1, 4096), dtype=np.uint64)
-                if tl.tf_timeline_read(h.ctypes.data_as(ctypes.c_void_p), h.shape[0], h.shape[1]):
+                if tl.tf_timeline_read_moe(h.ctypes.data_as(ctypes.c_void_p), h.shape[0], h.shape[1]):
                     raise RuntimeError(tl.tf_last_error().decode())
                 where = h[len(marks)]
                 h = h[:len(marks)].astype(np.int64)
@@ -440,6 +440,60 @@ def timeline() -> dict:
                 row["by_workgroups_a_unit"] = {str(n): {"units": len(v), "mean_last_done_us": float(np.mean(v))}
                                                for n, v in last.items()}
                 out["launches"][f"{tokens}_tokens_{name}"] = row
+    del tables
+    torch.cuda.empty_cache()
+    # the EXL3 linear kernel of configuration 4 at one row: marks 0 entry, 1 the wave's walk over its k-tile pairs
+    # begins, 2 wave 0 has walked, 3 every wave has, 4 the K split's partial sums are out and acknowledged, 5 done
+    # (the last workgroup of a column block has added the splits and stored the rows)
+    gen = torch.Generator(device=DEV).manual_seed(4)
+    names = ("entry", "walk_begins", "wave0_walked", "all_waves_walked", "partials_out", "done")
+    for label, (k, n) in (("gate_5120x17408", (5120, 17408)), ("down_17408x5120", (17408, 5120))):
+        layers = []
+        for _ in range(4):
+            trellis = torch.randint(-2 ** 15, 2 ** 15, (k // 16, n // 16, 48), generator=gen, device=DEV,
+                                    dtype=torch.int32).to(torch.int16)
+            sc = lambda size: (torch.rand(size, generator=gen, device=DEV) * 1.5 + 0.5).half()
+            layers.append(exl3.Exl3Linear.from_tensors(trellis, sc(k), sc(n), "3inst", device=DEV))
+        x = synthetic.activations(1, k, 4201, dtype=torch.float16).to(DEV)
+        y, xh = torch.empty((1, n), dtype=torch.float16, device=DEV), torch.empty_like(x)
+        z = torch.empty((16 * n,), dtype=torch.float32, device=DEV)
+        with _lib.through(build.TIMELINE_LIB) as tl:
+            layers[0](x, y, xh=xh, z=z)
+            torch.cuda.synchronize()
+            if tl.tf_timeline_clear_exl3():
+                raise RuntimeError(tl.tf_last_error().decode())
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                for i in range(12):
+                    layers[i % 4](x, y, xh=xh, z=z)
+            g.replay()
+            g.replay()
+            torch.cuda.synchronize()
+            h = np.zeros((len(names) + 1, 4096), dtype=np.uint64)
+            if tl.tf_timeline_read_exl3(h.ctypes.data_as(ctypes.c_void_p), h.shape[0], h.shape[1]):
+                raise RuntimeError(tl.tf_last_error().decode())
+        where = h[len(names)]
+        h = h[:len(names)].astype(np.int64)
+        live = h[5] > 0
+        t0 = h[0][live].min()
+        row = {"workgroups": int(live.sum())}
+        hw = where[live]
+        cu = ((hw >> np.uint64(32)) << np.uint64(8)) | ((hw >> np.uint64(8)) & np.uint64(0xFF))
+        ids, count = np.unique(cu, return_counts=True)
+        end = (h[5][live] - t0) / 100.0
+        row["units_used"] = int(len(ids))
+        row["by_workgroups_a_unit"] = {
+            str(int(c)): {"units": int((count == c).sum()),
+                          "mean_last_done_us": float(np.mean([end[cu == u].max() for u in ids[count == c]]))}
+            for c in np.unique(count)}
+        for i, mark in enumerate(names):
+            sel = live & (h[i] > 0)
+            v = (h[i][sel] - t0) / 100.0
+            row[mark] = {"min": float(v.min()), "median": float(np.median(v)), "p90": float(np.percentile(v, 90)),
+                         "max": float(v.max())}
+        out["launches"][f"exl3_linear_1_row_{label}"] = row
+        del layers
+        torch.cuda.empty_cache()
     return out
 
 

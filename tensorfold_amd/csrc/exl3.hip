@@ -53,6 +53,7 @@ __global__ void __launch_bounds__(WK * 64)
   const int pr0 = (int)((long long)slot * pairs / nslots), pr1 = (int)((long long)(slot + 1) * pairs / nslots);
   const uint32_t* tiles = T + (size_t)nb * stride_nb;
   const int col0 = nb * 128;
+  TF_MARK(0);
 
   for (int m0 = 0, pass = 0; m0 < M; m0 += 16, ++pass) {
     const int R = min(16, M - m0);
@@ -63,9 +64,12 @@ __global__ void __launch_bounds__(WK * 64)
     const uint16_t* xr = xh + (size_t)(m0 + (c < R ? c : R - 1)) * K + 2 * kq;
     uint32_t* stage = reinterpret_cast<uint32_t*>(red) + wave * (16 * 128);       // 16 tiles of TW + 2 words
     if (pass) __syncthreads();                 // the previous pass is done with red
+    TF_MARK(1);
     wave_block<K2, CB>(xr, tiles, stride_k, pr0, pr1, stage, lane, L, h, acc);
+    TF_MARK(2);
     // D[row 4 kq + i][column c] of column tile j -> red[wave][row][16 j + c]
     __syncthreads();
+    TF_MARK(3);
 #pragma unroll
     for (int j = 0; j < 8; ++j)
 #pragma unroll
@@ -92,6 +96,7 @@ __global__ void __launch_bounds__(WK * 64)
     if (SK > 1) {
       __builtin_amdgcn_s_waitcnt(0);        // this wave's stores are acknowledged ...
       __syncthreads();                      // ... every wave's are ...
+      TF_MARK(4);
       if (threadIdx.x == 0)                 // ... then the block counts itself in
         last = __hip_atomic_fetch_add(counters + (size_t)(pass * NB + nb) * TF_EXL3_COUNTER_STRIDE, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == SK - 1;
       __syncthreads();
@@ -121,6 +126,7 @@ __global__ void __launch_bounds__(WK * 64)
       }
     }
   }
+  TF_MARK(5);
 }
 
 // W_q [K, N] fp16: a wave a tile
@@ -326,6 +332,8 @@ extern "C" int tf_exl3_rot_in(const void* x, int x_dtype, const uint16_t* suh, u
   TF_LAUNCH_OK("tf_exl3_rot_in");
   return 0;
 }
+
+TF_TIMELINE_EXPORT(exl3)
 
 extern "C" int tf_exl3_linear(const uint16_t* xh, const uint32_t* T, int64_t stride_k, int64_t stride_nb,
                               const uint16_t* svh, const uint16_t* bias, void* y, int y_dtype, float* Z,

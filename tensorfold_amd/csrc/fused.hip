@@ -424,26 +424,7 @@ int launch_fused(const uint16_t* x, int64_t x_stride, int slots, const uint32_t*
 
 using namespace tf;
 
-#ifdef TF_TIMELINE
-// The timeline build's two extra entry points: the marks of the last tf_moe_route_up / tf_moe_down_combine /
-// tf_moe_decode_experts launches, [TIMELINE_ROWS][TIMELINE_GROUPS]: six rows of 64-bit ticks of 10 ns (0: never
-// passed), then the row of hardware ids.
-extern "C" int tf_timeline_read(unsigned long long* host, int rows, int groups) {
-  clear_error();
-  TF_REQUIRE(host && rows == TIMELINE_ROWS && groups == TIMELINE_GROUPS, "timeline: the table is %d x %d",
-             TIMELINE_ROWS, TIMELINE_GROUPS);
-  TF_REQUIRE(hipMemcpyFromSymbol(host, HIP_SYMBOL(tf_timeline_marks), sizeof(tf_timeline_marks)) == hipSuccess,
-             "timeline: the copy failed");
-  return 0;
-}
-extern "C" int tf_timeline_clear(void) {
-  clear_error();
-  static const unsigned long long zeros[TIMELINE_ROWS][TIMELINE_GROUPS] = {};
-  TF_REQUIRE(hipMemcpyToSymbol(HIP_SYMBOL(tf_timeline_marks), zeros, sizeof(zeros)) == hipSuccess,
-             "timeline: the clear failed");
-  return 0;
-}
-#endif
+TF_TIMELINE_EXPORT(moe)
 
 extern "C" int tf_moe_decode_experts(int gs, int swiglu, const uint16_t* x, int64_t x_stride, int rows, int slots,
                                      const uint32_t* up, const uint32_t* down, int d, int ni, const int32_t* desc,

@@ -116,18 +116,40 @@ __device__ __forceinline__ void timeline_mark(int k) {
   if (k == 0)
     for (int i = 1; i < TIMELINE_MARKS; ++i) t[i] = 0;
   t[k] = wall_clock64();
-  if (k == TIMELINE_MARKS - 1 && blockIdx.x < TIMELINE_GROUPS) {
-    for (int i = 0; i < TIMELINE_MARKS; ++i) tf_timeline_marks[i][blockIdx.x] = t[i];
+  const unsigned group = blockIdx.x + blockIdx.y * gridDim.x;
+  if (k == TIMELINE_MARKS - 1 && group < TIMELINE_GROUPS) {
+    for (int i = 0; i < TIMELINE_MARKS; ++i) tf_timeline_marks[i][group] = t[i];
     // where it ran: the XCC id above the hardware id word (compute unit in bits 8-11, shader array 12, engine 13-15)
-    tf_timeline_marks[TIMELINE_MARKS][blockIdx.x] =
+    tf_timeline_marks[TIMELINE_MARKS][group] =
         ((unsigned long long)__builtin_amdgcn_s_getreg((31 << 11) | 20) << 32) | __builtin_amdgcn_s_getreg((31 << 11) | 4);
   }
 }
+// The timeline build's two extra entry points of a source file that places marks: the marks of that file's last
+// launches, [TIMELINE_ROWS][TIMELINE_GROUPS]: six rows of 64-bit ticks of 10 ns (0: never passed), then the row of
+// hardware ids (each source file has its own table).
+#define TF_TIMELINE_EXPORT(NAME_)                                                                                   \
+  extern "C" int tf_timeline_read_##NAME_(unsigned long long* host, int rows, int groups) {                         \
+    ::tf::clear_error();                                                                                            \
+    TF_REQUIRE(host && rows == ::tf::TIMELINE_ROWS && groups == ::tf::TIMELINE_GROUPS, "timeline: the table is %d x %d", \
+               ::tf::TIMELINE_ROWS, ::tf::TIMELINE_GROUPS);                                                          \
+    TF_REQUIRE(hipMemcpyFromSymbol(host, HIP_SYMBOL(::tf::tf_timeline_marks), sizeof(::tf::tf_timeline_marks)) ==    \
+                   hipSuccess,                                                                                      \
+               "timeline: the copy failed");                                                                        \
+    return 0;                                                                                                       \
+  }                                                                                                                 \
+  extern "C" int tf_timeline_clear_##NAME_(void) {                                                                  \
+    ::tf::clear_error();                                                                                            \
+    static const unsigned long long zeros[::tf::TIMELINE_ROWS][::tf::TIMELINE_GROUPS] = {};                          \
+    TF_REQUIRE(hipMemcpyToSymbol(HIP_SYMBOL(::tf::tf_timeline_marks), zeros, sizeof(zeros)) == hipSuccess,           \
+               "timeline: the clear failed");                                                                       \
+    return 0;                                                                                                       \
+  }
 #define TF_MARK(K_) timeline_mark(K_)
 #else
 #define TF_MARK(K_) \
   do {              \
   } while (0)
+#define TF_TIMELINE_EXPORT(NAME_)
 #endif
 
 // ---- 4-bit blocks -------------------------------------------------------------------------------------------------
