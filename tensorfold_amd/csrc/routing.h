@@ -280,30 +280,6 @@ __device__ __forceinline__ void topk_lane(const float* __restrict__ row, int NE,
   else topk_lane_n<TOPK_VPL>(row, NE, TOPK, shared, lane, id, w);
 }
 
-// fp32 sums of every group of GS inputs of R rows into xs[r * KG + g]: the arithmetic of tf_group_sums (eight
-// inputs a lane in order, then a fixed xor tree over the group's lanes)
-template <int GS>
-__device__ __forceinline__ void group_sums_rows(const uint16_t* __restrict__ X, int64_t ldx, int R, int KG, float* xs,
-                                                int tid, int threads) {
-  constexpr int LPG = GS / 8;
-  const int part = tid % LPG;
-  for (int o = tid / LPG; o < R * KG; o += threads / LPG) {
-    const int r = o / KG, g = o - r * KG;
-    const uint4 v = *reinterpret_cast<const uint4*>(X + (size_t)r * ldx + (size_t)g * GS + part * 8);
-    float s = bf16_lo(v.x);
-    s += bf16_hi(v.x);
-    s += bf16_lo(v.y);
-    s += bf16_hi(v.y);
-    s += bf16_lo(v.z);
-    s += bf16_hi(v.z);
-    s += bf16_lo(v.w);
-    s += bf16_hi(v.w);
-#pragma unroll
-    for (int m = 1; m < LPG; m <<= 1) s += __shfl_xor(s, m);
-    if (part == 0) xs[o] = s;
-  }
-}
-
 __device__ __forceinline__ void topk_row(const float* __restrict__ row, int NE, int TOPK, int shared, int lane,
                                          int* __restrict__ pick, float* __restrict__ wts) {
   int id;

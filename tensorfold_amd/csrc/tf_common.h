@@ -158,11 +158,6 @@ constexpr uint32_t NIB_MASK = 0x000F000Fu;
 constexpr uint32_t BF16_ONES = 0x3F803F80u;  // the bf16 pair (1, 1)
 constexpr uint32_t BF16_128 = 0x43004300u;   // the bf16 pair (128, 128): OR-ing a nibble into the mantissa gives 128 + q
 
-// (word >> 4 i) & mask | 128.0: the bf16 pair (128 + q[2 i], 128 + q[2 i + 1]) of a packed word
-__device__ __forceinline__ uint32_t nib_pair(uint32_t word, int i) {
-  return ((word >> (4 * i)) & NIB_MASK) | BF16_128;
-}
-
 // int32 words of an experts block: 32 columns x gs inputs of codes, then 32 (scale | bias << 16) words
 __host__ __device__ constexpr int block_words(int gs) { return 32 * gs / 8 + 32; }
 
