@@ -58,8 +58,10 @@ def pack(words: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, gs: in
         raise ValueError(f"experts: shape {tuple(words.shape)} with scales {tuple(scales.shape)} does not pack")
     _lib.on_gpu(words, scales, biases)
     blocks = words.new_empty((e, n // COLS, k // gs, block_words(gs)), dtype=torch.int32)
-    _lib.call("tf_experts_pack", _lib.ptr(words.contiguous()), _lib.ptr(scales.contiguous()),
-              _lib.ptr(biases.contiguous()), e, n, k, gs, _lib.ptr(blocks))
+    # converted or re-laid copies are held by name until the launch is queued: a temporary freed between two
+    # arguments would hand its memory to the next one
+    words, scales, biases = words.contiguous(), scales.to(torch.bfloat16).contiguous(), biases.to(torch.bfloat16).contiguous()
+    _lib.call("tf_experts_pack", _lib.ptr(words), _lib.ptr(scales), _lib.ptr(biases), e, n, k, gs, _lib.ptr(blocks))
     return blocks
 
 

@@ -50,9 +50,11 @@ def pack(weight: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, gs: i
     q = Q4(words.new_empty((npad // 64, kg, gs // 32, 64, 4)),
            words.new_empty((kg, npad), dtype=torch.bfloat16), words.new_empty((kg, npad), dtype=torch.bfloat16),
            n, k, gs)
-    _lib.call("tf_qmm_pack", _lib.ptr(words.contiguous()), _lib.ptr(scales.to(torch.bfloat16).contiguous()),
-              _lib.ptr(biases.to(torch.bfloat16).contiguous()), n, k, gs, _lib.ptr(q.weight), _lib.ptr(q.scales),
-              _lib.ptr(q.biases))
+    # converted or re-laid copies are held by name until the launch is queued: a temporary freed between two
+    # arguments would hand its memory to the next one
+    words, s16, b16 = words.contiguous(), scales.to(torch.bfloat16).contiguous(), biases.to(torch.bfloat16).contiguous()
+    _lib.call("tf_qmm_pack", _lib.ptr(words), _lib.ptr(s16), _lib.ptr(b16), n, k, gs, _lib.ptr(q.weight),
+              _lib.ptr(q.scales), _lib.ptr(q.biases))
     from .experts import ARITH_BF16, ARITH_F16, fits_f16
 
     q.arith = ARITH_F16 if fits_f16(scales, biases) else ARITH_BF16
@@ -66,9 +68,41 @@ def unpack(q: Q4) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     words = q.weight.new_empty((q.n, q.k // 8))
     scales = q.scales.new_empty((q.n, kg))
     biases = q.scales.new_empty((q.n, kg))
-    _lib.call("tf_qmm_unpack", _lib.ptr(q.weight), _lib.ptr(q.scales.contiguous()), _lib.ptr(q.biases.contiguous()),
-              q.n, q.k, q.gs, _lib.ptr(words), _lib.ptr(scales), _lib.ptr(biases))
+    weight, s16, b16 = q.weight.contiguous(), q.scales.contiguous(), q.biases.contiguous()      # views of ``rows``
+    _lib.call("tf_qmm_unpack", _lib.ptr(weight), _lib.ptr(s16), _lib.ptr(b16), q.n, q.k, q.gs, _lib.ptr(words),
+              _lib.ptr(scales), _lib.ptr(biases))
     return words, scales, biases
+
+
+def rows(q: Q4, a: int, b: int) -> Q4:
+    """Output rows [a, b) of a packed weight (families/qwen3_5/cuda/qmm_fast.py:28-38).  From a 64-row tile edge and in
+    whole blocks of 128 rows it is a view of ``q``; any other range unpacks the tiles it touches and packs the rows
+    again (a small copy).  ``matmul`` on the part gives the whole weight's bits when it is told the whole weight's
+    ``sk`` (``matmul_rows`` does)."""
+
+    if not 0 <= a < b <= q.n:
+        raise ValueError(f"rows [{a}, {b}) of a weight of {q.n}")
+    if a % 64 == 0 and (b - a) % 128 == 0:
+        return Q4(q.weight[a // 64:b // 64], q.scales[:, a:b], q.biases[:, a:b], b - a, q.k, q.gs, q.arith)
+    t0, t1 = a // 64, -(-b // 64)
+    span = 128 * -(-(t1 - t0) // 2)                 # tiles come in pairs: a packed weight's rows are padded to 128
+    first = min(t0, q.weight.shape[0] - span // 64)
+    tiles = Q4(q.weight[first:first + span // 64], q.scales[:, 64 * first:64 * first + span],
+               q.biases[:, 64 * first:64 * first + span], span, q.k, q.gs, q.arith)
+    words, scales, biases = unpack(tiles)
+    lo, hi = a - 64 * first, b - 64 * first
+    part = pack(words[lo:hi].contiguous(), scales[lo:hi].contiguous(), biases[lo:hi].contiguous(), q.gs)
+    part.arith = q.arith
+    return part
+
+
+def matmul_rows(x: torch.Tensor, parts: list[Q4]) -> torch.Tensor:
+    """x against row blocks of one weight, side by side, with the bits of the stacked weight's ``matmul``: the K
+    split is the stacked weight's (families/qwen3_5/cuda/qmm_fast.py:41-46)."""
+
+    sk = split_k(sum(p.n for p in parts), parts[0].k, parts[0].gs)
+    xs = group_sums(x, parts[0].gs)
+    return torch.cat([matmul(x, p, xs, sk=sk) for p in parts], dim=1)
 
 
 def split_k(n: int, k: int, gs: int = 64, target: int = 1024) -> int:
@@ -237,8 +271,9 @@ def prefill_matmul(x: torch.Tensor, q: Q4, *, f32: bool = False, tile: int = 0,
     elif tuple(out.shape) != (m, q.n) or out.dtype != (torch.float32 if f32 else torch.bfloat16) \
             or not out.is_contiguous() or out.device != x.device:
         raise ValueError(f"prefill_matmul: out must be contiguous ({m}, {q.n}) {'fp32' if f32 else 'bf16'}")
-    _lib.call("tf_qmm_prefill", _lib.ptr(x), x.stride(0), _lib.ptr(q.weight), _lib.ptr(q.scales.contiguous()),
-              _lib.ptr(q.biases.contiguous()), _lib.ptr(out), m, q.n, q.k, q.gs, int(f32), tile,
+    s16, b16 = q.scales.contiguous(), q.biases.contiguous()
+    _lib.call("tf_qmm_prefill", _lib.ptr(x), x.stride(0), _lib.ptr(q.weight), _lib.ptr(s16), _lib.ptr(b16),
+              _lib.ptr(out), m, q.n, q.k, q.gs, int(f32), tile,
               q.arith if arith is None else int(arith))
     return out
 
@@ -284,8 +319,9 @@ def prefill_matmul8(xq: tuple[torch.Tensor, torch.Tensor, torch.Tensor], q: Q4, 
     elif tuple(out.shape) != (m, q.n) or out.dtype != (torch.float32 if f32 else torch.bfloat16) \
             or not out.is_contiguous() or out.device != x8.device:
         raise ValueError(f"prefill_matmul8: out must be contiguous ({m}, {q.n}) {'fp32' if f32 else 'bf16'}")
-    _lib.call("tf_qmm_prefill8", _lib.ptr(x8), _lib.ptr(xs), _lib.ptr(a), _lib.ptr(q.weight),
-              _lib.ptr(q.scales.contiguous()), _lib.ptr(q.biases.contiguous()), _lib.ptr(out), m, q.n, q.k, q.gs,
+    s16, b16 = q.scales.contiguous(), q.biases.contiguous()
+    _lib.call("tf_qmm_prefill8", _lib.ptr(x8), _lib.ptr(xs), _lib.ptr(a), _lib.ptr(q.weight), _lib.ptr(s16),
+              _lib.ptr(b16), _lib.ptr(out), m, q.n, q.k, q.gs,
               int(f32), tile)
     return out
 
