@@ -209,6 +209,7 @@ def c4() -> dict:
         return exl3.Exl3Linear.from_tensors(trellis, sc(k), sc(n), "3inst", device=DEV)
 
     mlps = [(layer(5120, 17408), layer(5120, 17408), layer(17408, 5120)) for _ in range(4)]     # 4 x 100 MB
+    stacks = [exl3.Exl3Stack.of([g, u]) for g, u, _ in mlps]          # gate and up side by side: one launch for both
     out = {}
     for m in (1, 8):
         x = synthetic.activations(m, 5120, 4200 + m, dtype=torch.float16).to(DEV)
@@ -224,19 +225,29 @@ def c4() -> dict:
             u(x, ys[1], xh=xh, z=z)
             d(h, yd, xh=hh, z=z)
 
-        us = graph_us(step, 48)
+        separate_us = graph_us(step, 48)
+        y2 = torch.empty((2, m, 17408), dtype=torch.float16, device=DEV)
+        xh2 = torch.empty((2, m, 5120), dtype=torch.float16, device=DEV)
+        z2 = torch.empty((2 * 16 * m * 17408,), dtype=torch.float32, device=DEV)
+
+        def step_stacked(i):
+            stacks[i % len(stacks)](x, y2, xh=xh2, z=z2)
+            mlps[i % len(mlps)][2](h, yd, xh=hh, z=z)
+
+        us = graph_us(step_stacked, 48)
         gate_us = graph_us(lambda i: mlps[i % 4][0](x, ys[0], xh=xh, z=z), 48)
         down_us = graph_us(lambda i: mlps[i % 4][2](h, yd, xh=hh, z=z), 48)
         per = 5120 * 17408 * 3 // 8
         nbytes = 3 * per + 3 * 2 * (5120 + 17408) + m * (2 * 5120 + 17408 + 17408 * 2 + 5120) * 2
         ops = 3 * 5120 * 17408 * EXL3_VALU_PER_WEIGHT          # lane-operations of one MLP's decode
-        out[m] = {"mlp_us": us, "bytes": nbytes, "gbs": nbytes / us * 1e-3, "frac": nbytes / us * 1e-3 / HBM,
+        out[m] = {"mlp_us": us, "mlp_separate_calls_us": separate_us, "bytes": nbytes, "gbs": nbytes / us * 1e-3, "frac": nbytes / us * 1e-3 / HBM,
                   "gate_us": gate_us, "gate_gbs": per / gate_us * 1e-3, "down_us": down_us,
                   "down_gbs": per / down_us * 1e-3,
                   "valu": {"bound": "valu", "achieved": ops / us * 1e-6, "peak": VALU * 1e-12, "unit": "Tlane-op/s",
                            "frac": ops / us * 1e6 / VALU, "ops_per_weight": EXL3_VALU_PER_WEIGHT,
                            "floor_us": ops / VALU * 1e6}}
-    return {"config": "c4: EXL3 3.0 bpw MLP, gate/up 5120 -> 17408, down 17408 -> 5120 (input rotation + linear kernel each)",
+    return {"config": "c4: EXL3 3.0 bpw MLP, gate/up 5120 -> 17408 as a stack of two (one rotation and one linear launch "
+                      "for both), down 17408 -> 5120 (rotation + linear); mlp_separate_calls_us: three separate layers",
             "bound": "hbm", "rows": out}
 
 
@@ -447,16 +458,22 @@ def timeline() -> dict:
     # (the last workgroup of a column block has added the splits and stored the rows)
     gen = torch.Generator(device=DEV).manual_seed(4)
     names = ("entry", "walk_begins", "wave0_walked", "all_waves_walked", "partials_out", "done")
-    for label, (k, n) in (("gate_5120x17408", (5120, 17408)), ("down_17408x5120", (17408, 5120))):
+    for label, (k, n), stacked in (("gate_5120x17408", (5120, 17408), 1), ("gate_and_up_stacked_2x5120x17408", (5120, 17408), 2),
+                                  ("down_17408x5120", (17408, 5120), 1)):
         layers = []
         for _ in range(4):
-            trellis = torch.randint(-2 ** 15, 2 ** 15, (k // 16, n // 16, 48), generator=gen, device=DEV,
-                                    dtype=torch.int32).to(torch.int16)
-            sc = lambda size: (torch.rand(size, generator=gen, device=DEV) * 1.5 + 0.5).half()
-            layers.append(exl3.Exl3Linear.from_tensors(trellis, sc(k), sc(n), "3inst", device=DEV))
+            made = []
+            for _ in range(stacked):
+                trellis = torch.randint(-2 ** 15, 2 ** 15, (k // 16, n // 16, 48), generator=gen, device=DEV,
+                                        dtype=torch.int32).to(torch.int16)
+                sc = lambda size: (torch.rand(size, generator=gen, device=DEV) * 1.5 + 0.5).half()
+                made.append(exl3.Exl3Linear.from_tensors(trellis, sc(k), sc(n), "3inst", device=DEV))
+            layers.append(made[0] if stacked == 1 else exl3.Exl3Stack.of(made))
         x = synthetic.activations(1, k, 4201, dtype=torch.float16).to(DEV)
-        y, xh = torch.empty((1, n), dtype=torch.float16, device=DEV), torch.empty_like(x)
-        z = torch.empty((16 * n,), dtype=torch.float32, device=DEV)
+        lead = () if stacked == 1 else (stacked,)
+        y = torch.empty((*lead, 1, n), dtype=torch.float16, device=DEV)
+        xh = torch.empty((*lead, 1, k), dtype=torch.float16, device=DEV)
+        z = torch.empty((stacked * 16 * n,), dtype=torch.float32, device=DEV)
         with _lib.through(build.TIMELINE_LIB) as tl:
             layers[0](x, y, xh=xh, z=z)
             torch.cuda.synchronize()

@@ -246,6 +246,17 @@ int tf_exl3_rot_in(const void* x, int x_dtype, const uint16_t* suh, uint16_t* xh
 int tf_exl3_linear(const uint16_t* xh, const uint32_t* T, int64_t stride_k, int64_t stride_nb, const uint16_t* svh,
                    const uint16_t* bias, void* y, int y_dtype, float* Z, int32_t* counters, int m, int k, int n,
                    int k2, int cb, int sk, int wk, tf_stream_t stream);
+/* The same two calls over a stack of 1 to 64 layers of one shape, width and codebook that read the same x (an MLP's
+ * gate and up projections): one launch each instead of one a layer, every layer's bits those of its own call.
+ * suh [layers, k]; xh [layers, m, k]; layer z's trellis stride_layer words past layer 0's; svh, bias [layers, n];
+ * y [layers, m, n]; Z [layers, sk, m, n]; counters [layers, 8 * n/128 * TF_EXL3_COUNTER_STRIDE].  The reference's
+ * linear module has no such call; its affine path groups launches the same way (kernels/qmm.cpp:51-54 `qmm_group`). */
+int tf_exl3_rot_in_stacked(const void* x, int x_dtype, const uint16_t* suh, uint16_t* xh, int layers, int m, int k,
+                           tf_stream_t stream);
+int tf_exl3_linear_stacked(const uint16_t* xh, const uint32_t* T, int64_t stride_k, int64_t stride_nb,
+                           int64_t stride_layer, const uint16_t* svh, const uint16_t* bias, void* y, int y_dtype,
+                           float* Z, int32_t* counters, int layers, int m, int k, int n, int k2, int cb, int sk, int wk,
+                           tf_stream_t stream);
 /* W[k, n] fp16 = the decoded trellis (bit-exact codebook values).  Replaces exl3/linear.cpp:61-68 `unpack`. */
 int tf_exl3_unpack(const uint32_t* T, uint16_t* W, int k, int n, int64_t stride_k, int64_t stride_nb, int k2, int cb,
                    tf_stream_t stream);

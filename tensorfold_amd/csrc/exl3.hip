@@ -8,11 +8,14 @@ namespace tf {
 namespace {
 
 // xh = fp16(((x * suh) H) / sqrt(128)), a wave a (row, block of 128); a workgroup walks rows blockIdx.y, + gridDim.y, ...
+// blockIdx.z is the layer of a stack: its own suh [K] and xh [M, K] over the one x.
 __global__ void __launch_bounds__(256)
     rot_in_kernel(const void* __restrict__ x, int x_dtype, const uint16_t* __restrict__ suh, uint16_t* __restrict__ xh,
                   int M, int K) {
   const int blk = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (blk * 128 >= K) return;
+  suh += (size_t)blockIdx.z * K;
+  xh += (size_t)blockIdx.z * M * K;
   const int k = blk * 128 + 2 * lane;
   float sa, sb;
   load2(suh, TF_F16, k, sa, sb);
@@ -37,16 +40,28 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-// grid (N / 128, SK); WK waves a block; each wave walks its range of k-tile pairs over the block's eight column tiles
+// grid (N / 128, SK, layers); WK waves a block; each wave walks its range of k-tile pairs over the block's eight column
+// tiles.  The layers of a stack share K, N, width and codebook; layer z has its own xh [M, K], trellis (stride_layer
+// words on), svh and bias [N], y [M, N], Z [SK, M, N] and counters.
 template <int K2, int CB, int WK>
 __global__ void __launch_bounds__(WK * 64)
     linear_kernel(const uint16_t* __restrict__ xh, const uint32_t* __restrict__ T, int64_t stride_k, int64_t stride_nb,
-                  const uint16_t* __restrict__ svh, const uint16_t* __restrict__ bias, void* __restrict__ y, int y_dtype,
-                  float* __restrict__ Z, int* __restrict__ counters, int M, int K, int N, int SK) {
+                  int64_t stride_layer, const uint16_t* __restrict__ svh, const uint16_t* __restrict__ bias,
+                  void* __restrict__ y, int y_dtype, float* __restrict__ Z, int* __restrict__ counters, int M, int K,
+                  int N, int SK) {
   constexpr int TW = tile_words<K2>();
   extern __shared__ __align__(16) float red[];              // [WK][16][128]
   __shared__ int last;
   const int nb = blockIdx.x, split = blockIdx.y, NB = gridDim.x;
+  if (const size_t z = blockIdx.z) {
+    xh += z * M * K;
+    T += z * stride_layer;
+    svh += z * N;
+    if (bias) bias += z * N;
+    y = static_cast<char*>(y) + z * M * N * (y_dtype == TF_F32 ? 4 : 2);
+    if (Z) Z += z * SK * M * N;
+    if (counters) counters += z * 8 * NB * TF_EXL3_COUNTER_STRIDE;
+  }
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c = lane & 15, kq = lane >> 4;
   const int L = 4 * (c & 7) + kq, h = c >> 3;
   const int pairs = K >> 5, slot = split * WK + wave, nslots = SK * WK;
@@ -321,49 +336,79 @@ __global__ void __launch_bounds__(64 * WAVES, 8 / WAVES)
 
 using namespace tf;
 
-extern "C" int tf_exl3_rot_in(const void* x, int x_dtype, const uint16_t* suh, uint16_t* xh, int m, int k,
-                              tf_stream_t stream) {
+static int rot_in_launch(const char* who, const void* x, int x_dtype, const uint16_t* suh, uint16_t* xh, int layers,
+                         int m, int k, tf_stream_t stream) {
   clear_error();
-  TF_REQUIRE(x && suh && xh, "rot_in: null pointer argument");
+  TF_REQUIRE(x && suh && xh, "%s: null pointer argument", who);
   TF_REQUIRE(x_dtype == TF_F16 || x_dtype == TF_BF16 || x_dtype == TF_F32, "x: expected fp16, bf16 or fp32");
   TF_REQUIRE(m >= 1 && k >= 128 && k % 128 == 0, "x and xh must be [M, K], K a multiple of 128, suh [K]");
+  TF_REQUIRE(layers >= 1 && layers <= 64, "%s: 1 to 64 layers a stack", who);
   TF_REQUIRE(aligned16(x) && aligned16(xh), "x: must be 16-byte aligned");
-  rot_in_kernel<<<dim3((k / 128 + 3) / 4, m < 1024 ? m : 1024), 256, 0, as_stream(stream)>>>(x, x_dtype, suh, xh, m, k);
-  TF_LAUNCH_OK("tf_exl3_rot_in");
+  rot_in_kernel<<<dim3((k / 128 + 3) / 4, m < 1024 ? m : 1024, layers), 256, 0, as_stream(stream)>>>(x, x_dtype, suh, xh, m, k);
+  TF_LAUNCH_OK(who);
   return 0;
+}
+
+extern "C" int tf_exl3_rot_in(const void* x, int x_dtype, const uint16_t* suh, uint16_t* xh, int m, int k,
+                              tf_stream_t stream) {
+  return rot_in_launch("tf_exl3_rot_in", x, x_dtype, suh, xh, 1, m, k, stream);
+}
+
+extern "C" int tf_exl3_rot_in_stacked(const void* x, int x_dtype, const uint16_t* suh, uint16_t* xh, int layers, int m,
+                                      int k, tf_stream_t stream) {
+  return rot_in_launch("tf_exl3_rot_in_stacked", x, x_dtype, suh, xh, layers, m, k, stream);
 }
 
 TF_TIMELINE_EXPORT(exl3)
 
-extern "C" int tf_exl3_linear(const uint16_t* xh, const uint32_t* T, int64_t stride_k, int64_t stride_nb,
-                              const uint16_t* svh, const uint16_t* bias, void* y, int y_dtype, float* Z,
-                              int32_t* counters, int m, int k, int n, int k2, int cb, int sk, int wk,
-                              tf_stream_t stream) {
+static int linear_launch(const char* who, const uint16_t* xh, const uint32_t* T, int64_t stride_k, int64_t stride_nb,
+                         int64_t stride_layer, const uint16_t* svh, const uint16_t* bias, void* y, int y_dtype, float* Z,
+                         int32_t* counters, int layers, int m, int k, int n, int k2, int cb, int sk, int wk,
+                         tf_stream_t stream) {
   clear_error();
-  TF_REQUIRE(xh && T && svh && y, "linear: null pointer argument");
+  TF_REQUIRE(xh && T && svh && y, "%s: null pointer argument", who);
   TF_REQUIRE(y_dtype == TF_F16 || y_dtype == TF_BF16 || y_dtype == TF_F32, "y: expected fp16, bf16 or fp32");
   TF_REQUIRE(m >= 1 && m <= 128, "xh and y must have the same 1 to 128 rows");
   TF_REQUIRE(k >= 128 && n >= 128 && k % 128 == 0 && n % 128 == 0, "K and N must be multiples of 128");
   TF_REQUIRE(aligned16(T) && aligned16(xh) && aligned16(y), "T must be 16-byte aligned");
+  TF_REQUIRE(layers >= 1 && layers <= 64 && (layers == 1 || (stride_layer > 0 && stride_layer % 4 == 0)),
+             "%s: 1 to 64 layers, a whole number of 16-byte pieces apart", who);
+  TF_REQUIRE(layers == 1 || ((int64_t)m * k % 8 == 0 && (int64_t)m * n % 8 == 0), "%s: layers' xh and y must stay 16-byte aligned", who);
   TF_REQUIRE(wk == 2 || wk == 4 || wk == 8, "WK must be 2, 4 or 8");
   TF_REQUIRE(sk >= 1 && sk <= 64 && (int64_t)sk * wk <= k / 32, "K / 32 = %d tile pairs do not split over %d x %d waves",
              k / 32, sk, wk);
   TF_REQUIRE(sk == 1 || (Z && counters), "Z and counters are needed with more than one split");
-  const dim3 grid((unsigned)(n / 128), (unsigned)sk);
+  const dim3 grid((unsigned)(n / 128), (unsigned)sk, (unsigned)layers);
   hipStream_t s = as_stream(stream);
   const size_t smem = (size_t)wk * 16 * 128 * sizeof(float);
 #define TF_LAUNCH(K2_, CB_)                                                                                             \
   if (k2 == K2_ && cb == CB_) {                                                                                         \
-    if (wk == 2) linear_kernel<K2_, CB_, 2><<<grid, 128, smem, s>>>(xh, T, stride_k, stride_nb, svh, bias, y, y_dtype, Z, counters, m, k, n, sk); \
-    else if (wk == 4) linear_kernel<K2_, CB_, 4><<<grid, 256, smem, s>>>(xh, T, stride_k, stride_nb, svh, bias, y, y_dtype, Z, counters, m, k, n, sk); \
-    else linear_kernel<K2_, CB_, 8><<<grid, 512, smem, s>>>(xh, T, stride_k, stride_nb, svh, bias, y, y_dtype, Z, counters, m, k, n, sk); \
-    TF_LAUNCH_OK("tf_exl3_linear");                                                                                     \
+    if (wk == 2) linear_kernel<K2_, CB_, 2><<<grid, 128, smem, s>>>(xh, T, stride_k, stride_nb, stride_layer, svh, bias, y, y_dtype, Z, counters, m, k, n, sk); \
+    else if (wk == 4) linear_kernel<K2_, CB_, 4><<<grid, 256, smem, s>>>(xh, T, stride_k, stride_nb, stride_layer, svh, bias, y, y_dtype, Z, counters, m, k, n, sk); \
+    else linear_kernel<K2_, CB_, 8><<<grid, 512, smem, s>>>(xh, T, stride_k, stride_nb, stride_layer, svh, bias, y, y_dtype, Z, counters, m, k, n, sk); \
+    TF_LAUNCH_OK(who);                                                                                                  \
     return 0;                                                                                                           \
   }
   TF_EXL3_ALL(TF_LAUNCH)
 #undef TF_LAUNCH
   set_error("unsupported EXL3 width/codebook: K2=%d codebook=%d", k2, cb);
   return 1;
+}
+
+extern "C" int tf_exl3_linear(const uint16_t* xh, const uint32_t* T, int64_t stride_k, int64_t stride_nb,
+                              const uint16_t* svh, const uint16_t* bias, void* y, int y_dtype, float* Z,
+                              int32_t* counters, int m, int k, int n, int k2, int cb, int sk, int wk,
+                              tf_stream_t stream) {
+  return linear_launch("tf_exl3_linear", xh, T, stride_k, stride_nb, 0, svh, bias, y, y_dtype, Z, counters, 1, m, k, n,
+                       k2, cb, sk, wk, stream);
+}
+
+extern "C" int tf_exl3_linear_stacked(const uint16_t* xh, const uint32_t* T, int64_t stride_k, int64_t stride_nb,
+                                      int64_t stride_layer, const uint16_t* svh, const uint16_t* bias, void* y,
+                                      int y_dtype, float* Z, int32_t* counters, int layers, int m, int k, int n, int k2,
+                                      int cb, int sk, int wk, tf_stream_t stream) {
+  return linear_launch("tf_exl3_linear_stacked", xh, T, stride_k, stride_nb, stride_layer, svh, bias, y, y_dtype, Z,
+                       counters, layers, m, k, n, k2, cb, sk, wk, stream);
 }
 
 extern "C" int tf_exl3_unpack(const uint32_t* T, uint16_t* W, int k, int n, int64_t stride_k, int64_t stride_nb, int k2,

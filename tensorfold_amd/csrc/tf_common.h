@@ -116,7 +116,7 @@ __device__ __forceinline__ void timeline_mark(int k) {
   if (k == 0)
     for (int i = 1; i < TIMELINE_MARKS; ++i) t[i] = 0;
   t[k] = wall_clock64();
-  const unsigned group = blockIdx.x + blockIdx.y * gridDim.x;
+  const unsigned group = blockIdx.x + (blockIdx.y + blockIdx.z * gridDim.y) * gridDim.x;
   if (k == TIMELINE_MARKS - 1 && group < TIMELINE_GROUPS) {
     for (int i = 0; i < TIMELINE_MARKS; ++i) tf_timeline_marks[i][group] = t[i];
     // where it ran: the XCC id above the hardware id word (compute unit in bits 8-11, shader array 12, engine 13-15)

@@ -174,6 +174,87 @@ class Exl3Linear:
         return _decode(self.words, self.k, self.n, self.strides, self.k2, self.codebook, out)
 
 
+@dataclasses.dataclass
+class Exl3Stack:
+    """Layers of one shape, width, codebook and layout that read the same input (an MLP's gate and up projections),
+    laid side by side so that a call is one rotation launch and one linear launch for all of them.  Every layer's
+    output has the bits of its own ``Exl3Linear`` call."""
+
+    words: torch.Tensor           # int32 [L, ...one layer's words...]
+    suh: torch.Tensor             # fp16 [L, K]
+    svh: torch.Tensor             # fp16 [L, N]
+    bias: torch.Tensor | None     # fp16 [L, N] (layers without one add zero)
+    bits: float
+    codebook: str
+    k: int
+    n: int
+    layout: str
+    split: tuple[int, int]
+
+    @classmethod
+    def of(cls, layers: list[Exl3Linear]) -> "Exl3Stack":
+        """A copy of the layers' tensors in one piece (drop the layers afterwards to give their memory back)."""
+
+        first = layers[0]
+        same = lambda l: (l.k, l.n, l.bits, l.codebook, l.layout, l.words.shape) == \
+            (first.k, first.n, first.bits, first.codebook, first.layout, first.words.shape)
+        if not 1 <= len(layers) <= 64 or not all(same(l) for l in layers):
+            raise ValueError("a stack takes 1 to 64 layers of one shape, width, codebook and layout")
+        bias = None
+        if any(l.bias is not None for l in layers):
+            bias = torch.stack([l.bias if l.bias is not None else torch.zeros_like(first.svh) for l in layers])
+        return cls(torch.stack([l.words for l in layers]), torch.stack([l.suh for l in layers]),
+                   torch.stack([l.svh for l in layers]), bias, first.bits, first.codebook, first.k, first.n, first.layout,
+                   first.split)
+
+    def __post_init__(self) -> None:
+        self.counters = torch.zeros((len(self), 8 * (self.n // 128) * COUNTER_STRIDE), dtype=torch.int32,
+                                    device=self.words.device)
+
+    def __len__(self) -> int:
+        return int(self.words.shape[0])
+
+    def layer(self, i: int) -> Exl3Linear:
+        """Layer ``i`` as an ``Exl3Linear`` over the stack's memory."""
+
+        return Exl3Linear(self.words[i], self.suh[i], self.svh[i], None if self.bias is None else self.bias[i],
+                          self.bits, self.codebook, self.k, self.n, self.layout, self.split)
+
+    def __call__(self, x: torch.Tensor, out: torch.Tensor | None = None, out_dtype: torch.dtype | None = None,
+                 xh: torch.Tensor | None = None, z: torch.Tensor | None = None) -> torch.Tensor:
+        """y [L, M, N] for x [M, K], M = 1..128.  ``xh`` (fp16, L * M * K values) and ``z`` (fp32, L * splits * M * N)
+        are scratch, allocated here when not passed."""
+
+        if x.dim() != 2 or x.shape[1] != self.k or not 1 <= x.shape[0] <= 128 or x.dtype not in _DTYPES:
+            raise ValueError(f"x must be [1..128, {self.k}] fp16, bf16 or fp32, got {tuple(x.shape)} {x.dtype}")
+        _lib.on_gpu(x)
+        x = x.contiguous()
+        count, m = len(self), int(x.shape[0])
+        if out is None:
+            out = x.new_empty((count, m, self.n), dtype=out_dtype or x.dtype)
+        elif tuple(out.shape) != (count, m, self.n) or out.dtype not in _DTYPES or not out.is_contiguous() \
+                or out.device != x.device:
+            raise ValueError(f"out must be contiguous ({count}, {m}, {self.n}) fp16, bf16 or fp32 on x's device")
+        sk, wk = self.split
+        if xh is None:
+            xh = x.new_empty((count, m, self.k), dtype=torch.float16)
+        elif xh.dtype != torch.float16 or xh.numel() < count * m * self.k or not xh.is_contiguous() or xh.device != x.device:
+            raise ValueError(f"xh must hold {count} x {m} x {self.k} fp16 values on x's device")
+        if sk > 1 and z is None:
+            z = x.new_empty((count * sk * m * self.n,), dtype=torch.float32)
+        elif sk > 1 and (z.dtype != torch.float32 or z.numel() < count * sk * m * self.n or not z.is_contiguous()
+                         or z.device != x.device):
+            raise ValueError(f"z must hold {count} x {sk} x {m} x {self.n} fp32 values on x's device")
+        stride_k, stride_nb = self.layer(0).strides
+        _lib.call("tf_exl3_rot_in_stacked", _lib.ptr(x), _DTYPES[x.dtype], _lib.ptr(self.suh), _lib.ptr(xh), count, m,
+                  self.k)
+        _lib.call("tf_exl3_linear_stacked", _lib.ptr(xh), _lib.ptr(self.words), stride_k, stride_nb,
+                  self.words.stride(0), _lib.ptr(self.svh), _lib.ptr(self.bias), _lib.ptr(out), _DTYPES[out.dtype],
+                  _lib.ptr(z) if sk > 1 else None, _lib.ptr(self.counters), count, m, self.k, self.n, k2_of(self.bits),
+                  CODEBOOK_IDS[self.codebook], sk, wk)
+        return out
+
+
 def unpack_gpu(trellis: torch.Tensor, codebook: str) -> torch.Tensor:
     """W_q [K, N] fp16 from trellis int16 [K/16, N/16, 16 * bits], decoded on the GPU from the stored order."""
 

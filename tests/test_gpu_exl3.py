@@ -150,6 +150,33 @@ def test_both_stored_layouts_give_the_same_bits():
     assert torch.equal(strips(x), stored(x)) and torch.equal(strips.unpack(), stored.unpack())
 
 
+@pytest.mark.parametrize("codebook,bits,split", [("3inst", 3, (7, 4)), ("mul1", 2.5, (1, 2)), ("mcg", 4, (3, 8)), ("mul1", 6, (2, 2))])
+def test_a_stack_of_layers_gives_each_layer_its_own_bits(codebook, bits, split):
+    """Gate and up of an MLP read the same input: stacked, they take one rotation launch and one linear launch, and
+    every layer's rows are those of its own call, at any row count."""
+
+    groups = [Group.draw(codebook, bits, k=1024, n=256, seed=40 + i) for i in range(3)]
+    bias = torch.from_numpy((np.random.default_rng(3).standard_normal(256) * 0.05).astype(np.float16))
+    layers = [groups[0].layer(), groups[1].layer(bias=bias), groups[2].layer()]
+    for layer in layers:
+        layer.split = split
+    stack = linear.Exl3Stack.of(layers)
+    assert len(stack) == 3 and stack.split == split and stack.bias is not None
+    for m in (1, 8, 17, 128):
+        x = synthetic.activations(m, 1024, 50 + m, dtype=torch.float16).cuda()
+        got = stack(x)
+        assert got.shape == (3, m, 256) and got.dtype == torch.float16
+        for i, layer in enumerate(layers):
+            assert torch.equal(got[i], layer(x)), (m, i)
+            assert torch.equal(stack.layer(i)(x), got[i]), (m, i)
+        assert torch.equal(stack(x, out_dtype=torch.float32)[1], layers[1](x, out_dtype=torch.float32))
+    assert not stack.counters.any()
+    with pytest.raises(ValueError):
+        linear.Exl3Stack.of([layers[0], Group.draw(codebook, bits, k=1024, n=128).layer()])
+    with pytest.raises(ValueError):
+        stack(x, out=torch.empty((2, 128, 256), dtype=torch.float16, device="cuda"))
+
+
 def test_what_the_layer_refuses():
     g = Group.draw("3inst", 3)
     with pytest.raises(ValueError):                                  # no such codebook
