@@ -92,7 +92,7 @@ def c0() -> dict:
     us16 = graph_us(lambda i: qmm.prefill_matmul(x, g32[i % len(g32)], out=y), 12)
     us8 = graph_us(lambda i: qmm.prefill_matmul8(xq32, g32[i % len(g32)], out=y), 12)
     fp8["g32"] = {"f16_tflops": flop / us16 * 1e-6, "fp8_tflops": flop / us8 * 1e-6}
-    return {"config": "c0: dense 4-bit/g64 projection, N = K = 4096 (qmm kernel + slice reduce; group sums given)",
+    return {"config": "c0: dense 4-bit/g64 projection, N = K = 4096 (the K slices added up in the matmul's launch; group sums given)",
             "bound": "hbm", "rows": out, "prompt_form": prompt, "prompt_form_fp8": fp8}
 
 

@@ -58,10 +58,14 @@ int tf_group_sums(const uint16_t* x, int64_t ldx, int m, int k, int gs, float* x
  * slices summed in slice order; one rounding to bf16 (or fp32 with f32).  `part` fp32 [sk, m, n] is required when
  * sk > 1 (with reduce == 0 the slices are left there unadded; with few rows and reduce != 0 the slices are added
  * inside the one launch, in the same order, and `part` goes unused).  sb_stride = elements between scale rows
- * (>= npad).  Replaces kernels/qmm.cpp:18-48 `qmm`. */
+ * (>= npad).  `counters` (may be NULL): n_counters arrival counters of the weight, TF_QMM_COUNTER_STRIDE ints apart,
+ * zero on entry and left zero; with one for every column tile of 64, one or two rows' slices are added up in the
+ * matmul's own launch by the last workgroup of a tile to finish (same order, same bits);
+ * calls on one weight's counters must not overlap.  Replaces kernels/qmm.cpp:18-48 `qmm`. */
+#define TF_QMM_COUNTER_STRIDE 16
 int tf_qmm(const uint16_t* x, int64_t ldx, const float* xs, const uint32_t* weight, const uint16_t* scales,
-           const uint16_t* biases, int64_t sb_stride, void* out, float* part, int m, int n, int k, int sk, int gs,
-           int bm, int f32, int reduce, tf_stream_t stream);
+           const uint16_t* biases, int64_t sb_stride, void* out, float* part, int32_t* counters, int n_counters, int m,
+           int n, int k, int sk, int gs, int bm, int f32, int reduce, tf_stream_t stream);
 /* tf_qmm (reduce != 0) for callers that cannot allocate or pass a workspace: code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc.  The K slices that tf_qmm keeps in `part` live in a fixed array
  * inside the library's device image (TF_QMM_STATIC_FLOATS fp32 = 16 MiB, held by every GPU the library runs on

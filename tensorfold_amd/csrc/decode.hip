@@ -78,7 +78,7 @@ struct NoFlush {
 };
 
 // One pass of a row tile: RB rows r0 .. r0 + RB - 1 against the workgroup's 64 columns and K slice.
-template <int GS, int WAVES, int RB, class WQ, class SB>
+template <int GS, int WAVES, int RB, bool COH, class WQ, class SB>
 __device__ __forceinline__ void qmm_pass(const uint16_t* __restrict__ X, int64_t ldx, const float* __restrict__ XS,
                                          const WQ& wq, const SB& sb, int r0, int tile, int slice, int gs0, int per,
                                          int g0, int g1, void* __restrict__ out, float* __restrict__ part_out, int M,
@@ -108,15 +108,18 @@ __device__ __forceinline__ void qmm_pass(const uint16_t* __restrict__ X, int64_t
     float s = part[r * 64 + l];
     for (int w = 1; w < WAVES; ++w) s += part[(w * RB + r) * 64 + l];
     const size_t at = (size_t)(r0 + r) * N + cc;
-    if (SK > 1) part_out[(size_t)slice * M * N + at] = s;
-    else if (f32) reinterpret_cast<float*>(out)[at] = s;
+    if (SK > 1) {
+      // COH: another workgroup adds the slices up in this launch: the store goes through to where it can read it
+      if (COH) __hip_atomic_store(part_out + (size_t)slice * M * N + at, s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      else part_out[(size_t)slice * M * N + at] = s;
+    } else if (f32) reinterpret_cast<float*>(out)[at] = s;
     else reinterpret_cast<uint16_t*>(out)[at] = (uint16_t)f32_bf16_bits(s);
   }
 }
 
 // grid (column tiles of 64 x row tiles of BM, 1, SK).  Slice z takes groups [z * per, (z + 1) * per), its waves
 // split them again (added in wave order); SK > 1 leaves the slice's fp32 sums in part[z].  Rows go in passes of 2 or 1.
-template <int GS, int WAVES>
+template <int GS, int WAVES, bool COH = false>
 __device__ __forceinline__ void qmm_block(const uint16_t* __restrict__ X, int64_t ldx, const float* __restrict__ XS,
                                           const uint32_t* __restrict__ W, const uint16_t* __restrict__ S,
                                           const uint16_t* __restrict__ B, int64_t sb_stride, void* __restrict__ out,
@@ -145,8 +148,8 @@ __device__ __forceinline__ void qmm_block(const uint16_t* __restrict__ X, int64_
     if (g0 + d < g1) load_weights<GS, 1>(st[d], wq, sb, g0 + d);
   bool loaded = true;
 #define TF_QMM_PASS(RB_)                                                                                             \
-  qmm_pass<GS, WAVES, RB_>(X, ldx, XS, wq, sb, r0, tile, slice, gs0, per, g0, g1, out, part_out, M, N, KG, SK, f32, xs, \
-                           part, st, loaded);                                                                        \
+  qmm_pass<GS, WAVES, RB_, COH>(X, ldx, XS, wq, sb, r0, tile, slice, gs0, per, g0, g1, out, part_out, M, N, KG, SK, f32, \
+                                xs, part, st, loaded);                                                                      \
   loaded = g1 - g0 <= DEPTH
   for (; r0 + 2 <= m_end; r0 += 2) {
     TF_QMM_PASS(2);
@@ -165,6 +168,52 @@ __global__ void __launch_bounds__(WAVES * 64)
                int BM, int f32) {
   extern __shared__ float lds[];            // partials [WAVES][RBMAX][64]
   qmm_block<GS, WAVES>(X, ldx, XS, W, S, B, sb_stride, out, part_out, M, N, KG, SK, BM, f32, blockIdx.x, blockIdx.z, lds);
+}
+
+// The split matmul with its reduce in the same launch: a slice's workgroup leaves its sums in part[z] with stores
+// that go through to memory, waits for them to be acknowledged and counts itself in at the (column tile, row tile)'s
+// counter; the workgroup that finds the others there adds the slices in slice order (qmm_reduce_kernel's arithmetic)
+// and puts the counter back to zero.  A thousand short workgroups fill the chip where the one-launch form above has
+// one workgroup a column tile.
+template <int GS, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64)
+    qmm_arrive_kernel(const uint16_t* __restrict__ X, int64_t ldx, const float* __restrict__ XS,
+                      const uint32_t* __restrict__ W, const uint16_t* __restrict__ S, const uint16_t* __restrict__ B,
+                      int64_t sb_stride, void* __restrict__ out, float* __restrict__ part_out, int* __restrict__ counters,
+                      int M, int N, int KG, int SK, int BM, int f32) {
+  extern __shared__ float lds[];
+  __shared__ int last;
+  qmm_block<GS, WAVES, true>(X, ldx, XS, W, S, B, sb_stride, out, part_out, M, N, KG, SK, BM, f32, blockIdx.x, blockIdx.z, lds);
+  __builtin_amdgcn_s_waitcnt(0);        // this wave's stores are acknowledged ...
+  __syncthreads();                      // ... every wave's are ...
+  int* counter = counters + (size_t)blockIdx.x * TF_QMM_COUNTER_STRIDE;
+  if (threadIdx.x == 0)                 // ... then the workgroup counts itself in
+    last = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == SK - 1;
+  __syncthreads();
+  if (!last) return;
+  const int tiles = (N + 63) >> 6, tile = blockIdx.x % tiles, rt = blockIdx.x / tiles;
+  const int r_first = rt * BM, rows = min(M, r_first + BM) - r_first;
+  const long long total = (long long)M * N;
+  for (int o = threadIdx.x; o < rows * 64; o += WAVES * 64) {
+    const int cc = tile * 64 + (o & 63);
+    if (cc >= N) continue;
+    const size_t at = (size_t)(r_first + (o >> 6)) * N + cc;
+    // eight slices' loads go out together, then the sums in slice order
+    float acc = 0.f;
+    for (int z0 = 0; z0 < SK; z0 += 8) {
+      float v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        v[j] = __hip_atomic_load(part_out + (long long)(z0 + j < SK ? z0 + j : SK - 1) * total + at, __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (z0 + j < SK) acc = z0 + j ? acc + v[j] : v[j];
+    }
+    if (f32) reinterpret_cast<float*>(out)[at] = acc;
+    else reinterpret_cast<uint16_t*>(out)[at] = (uint16_t)f32_bf16_bits(acc);
+  }
+  if (threadIdx.x == 0) *counter = 0;   // every slice of the tile has arrived: ready for the next call
 }
 
 // The split matmul and its reduce in ONE launch, with no traffic between workgroups: a workgroup of FW waves takes a
@@ -477,8 +526,9 @@ extern "C" int tf_group_sums(const uint16_t* x, int64_t ldx, int m, int k, int g
 
 // tf_qmm and tf_qmm_static: the checks and launches of the decode-form matmul; `part` holds the K slices.
 static int qmm_launch(const uint16_t* x, int64_t ldx, const float* xs, const uint32_t* weight, const uint16_t* scales,
-                      const uint16_t* biases, int64_t sb_stride, void* out, float* part, int m, int n, int k, int sk,
-                      int gs, int bm, int f32, int reduce, tf_stream_t stream) {
+                      const uint16_t* biases, int64_t sb_stride, void* out, float* part, int32_t* counters,
+                      int n_counters, int m, int n, int k, int sk, int gs, int bm, int f32, int reduce,
+                      tf_stream_t stream) {
   TF_REQUIRE(gs == 32 || gs == 64, "groups of 32 or 64");
   TF_REQUIRE(bm == 16 || bm == 32 || bm == 64, "row tile 16, 32 or 64");
   TF_REQUIRE(x && xs && weight && scales && biases && out && m >= 1 && n >= 1, "qmm: null pointer or empty shape");
@@ -494,6 +544,20 @@ static int qmm_launch(const uint16_t* x, int64_t ldx, const float* xs, const uin
   const size_t smem = sizeof(float) * ((size_t)QMM_WAVES * RBMAX * 64);
   TF_REQUIRE((int64_t)tiles * rts <= 0x7FFFFFFF && sk <= 65535, "qmm: grid too large");
   const int64_t fat_blocks = (int64_t)((n + 63) / 64) * ((m + RBMAX - 1) / RBMAX);
+  const dim3 grid((unsigned)(tiles * rts), 1, (unsigned)sk);
+  if (reduce && sk > 1 && counters && m <= RBMAX && (int64_t)tiles * rts <= n_counters) {
+    // one pass of rows and arrival counters: the slices are added up by the last workgroup of a tile to finish.  A
+    // thousand four-wave workgroups beat the one-launch form's workgroup a column tile (4096 x 4096 at one row: 6.2-6.8
+    // against 7.4 us); with more rows the stores that go through to memory cost more than a reduce launch
+    if (gs == 64)
+      qmm_arrive_kernel<64, QMM_WAVES><<<grid, QMM_WAVES * 64, smem, s>>>(x, ldx, xs, weight, scales, biases, sb_stride,
+                                                                           out, part, counters, m, n, kg, sk, bm, f32);
+    else
+      qmm_arrive_kernel<32, QMM_WAVES><<<grid, QMM_WAVES * 64, smem, s>>>(x, ldx, xs, weight, scales, biases, sb_stride,
+                                                                           out, part, counters, m, n, kg, sk, bm, f32);
+    TF_LAUNCH_OK("tf_qmm");
+    return 0;
+  }
   if (reduce && (m <= RBMAX || (m <= FAT_ROWS && fat_blocks <= 512)) && (sk == 2 || sk == 4 || sk == 8 || sk == 16)) {
     // few rows: split and reduce in one launch, a workgroup of 8 or 16 waves taking every slice of a tile for RBMAX
     // rows in one pass (same bits), while those workgroups fit the chip at once (512 of 16 waves).  Past that, and
@@ -515,7 +579,6 @@ static int qmm_launch(const uint16_t* x, int64_t ldx, const float* xs, const uin
     TF_LAUNCH_OK("tf_qmm");
     return 0;
   }
-  const dim3 grid((unsigned)(tiles * rts), 1, (unsigned)sk);
   if (gs == 64)
     qmm_kernel<64, QMM_WAVES><<<grid, QMM_WAVES * 64, smem, s>>>(x, ldx, xs, weight, scales, biases, sb_stride, out,
                                                                 part, m, n, kg, sk, bm, f32);
@@ -532,10 +595,13 @@ static int qmm_launch(const uint16_t* x, int64_t ldx, const float* xs, const uin
 }
 
 extern "C" int tf_qmm(const uint16_t* x, int64_t ldx, const float* xs, const uint32_t* weight, const uint16_t* scales,
-                      const uint16_t* biases, int64_t sb_stride, void* out, float* part, int m, int n, int k, int sk,
-                      int gs, int bm, int f32, int reduce, tf_stream_t stream) {
+                      const uint16_t* biases, int64_t sb_stride, void* out, float* part, int32_t* counters,
+                      int n_counters, int m, int n, int k, int sk, int gs, int bm, int f32, int reduce,
+                      tf_stream_t stream) {
   clear_error();
-  return qmm_launch(x, ldx, xs, weight, scales, biases, sb_stride, out, part, m, n, k, sk, gs, bm, f32, reduce, stream);
+  TF_REQUIRE(!counters || n_counters >= 0, "qmm: a negative number of counters");
+  return qmm_launch(x, ldx, xs, weight, scales, biases, sb_stride, out, part, counters, n_counters, m, n, k, sk, gs, bm,
+                    f32, reduce, stream);
 }
 
 // The K slices of tf_qmm_static: one array a GPU, part of the loaded code object, so no call ever allocates it.
@@ -575,7 +641,8 @@ extern "C" int tf_qmm_static(const uint16_t* x, int64_t ldx, const float* xs, co
              "tf_qmm with a part buffer", sk, m, n, (long long)sk * m * n, (long long)TF_QMM_STATIC_FLOATS);
   float* part = nullptr;
   if (sk > 1 && !(part = static_part())) return 1;
-  return qmm_launch(x, ldx, xs, weight, scales, biases, sb_stride, out, part, m, n, k, sk, gs, bm, f32, 1, stream);
+  return qmm_launch(x, ldx, xs, weight, scales, biases, sb_stride, out, part, nullptr, 0, m, n, k, sk, gs, bm, f32, 1,
+                    stream);
 }
 
 extern "C" int tf_qmm_group(const uint16_t* x, int64_t ldx, const float* xs, int count, const uint32_t* const* weights,

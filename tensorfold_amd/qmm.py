@@ -15,6 +15,9 @@ import torch
 from . import _lib
 
 
+COUNTER_STRIDE = 16          # TF_QMM_COUNTER_STRIDE of include/tfmi.h
+
+
 @dataclasses.dataclass
 class Q4:
     """A packed (n, k) weight.
@@ -30,9 +33,21 @@ class Q4:
     k: int
     gs: int
     arith: int = 0       # the prompt form's arithmetic (TF_ARITH_*): 1 when a scale or bias does not fit the fp16 form
+    _counters: torch.Tensor | None = dataclasses.field(default=None, init=False, repr=False, compare=False)
 
     def nbytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in (self.weight, self.scales, self.biases))
+
+    @property
+    def counters(self) -> torch.Tensor:
+        """Arrival counters of the K slices, one a column tile of 64, each alone in 64 bytes; zero between calls.
+        With them ``matmul`` on one or two rows adds the slices up in its own launch.  Calls on one weight that
+        overlap in time (two streams) need a ``Q4`` of their own each (``dataclasses.replace`` shares the packed
+        tensors and starts with fresh counters)."""
+
+        if self._counters is None:
+            self._counters = torch.zeros((-(-self.n // 64) * COUNTER_STRIDE,), dtype=torch.int32, device=self.weight.device)
+        return self._counters
 
 
 def pack(weight: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, gs: int) -> Q4:
@@ -175,8 +190,10 @@ def matmul(x: torch.Tensor, q: Q4, xs: torch.Tensor | None = None, *, sk: int | 
     if xs.dtype != torch.float32 or tuple(xs.shape) != (m, q.k // q.gs) or not xs.is_contiguous() \
             or xs.device != x.device:
         raise ValueError(f"matmul: xs must be contiguous fp32 ({m}, {q.k // q.gs}), the group sums of x")
+    counters = q.counters if reduce and sk > 1 and m <= 2 else None
     _lib.call("tf_qmm", _lib.ptr(x), x.stride(0), _lib.ptr(xs), _lib.ptr(q.weight), _lib.ptr(q.scales),
-              _lib.ptr(q.biases), q.scales.stride(0), _lib.ptr(out), _lib.ptr(part), m, q.n, q.k, sk, q.gs, bucket(m),
+              _lib.ptr(q.biases), q.scales.stride(0), _lib.ptr(out), _lib.ptr(part), _lib.ptr(counters),
+              0 if counters is None else counters.numel() // COUNTER_STRIDE, m, q.n, q.k, sk, q.gs, bucket(m),
               int(f32), int(reduce))
     if reduce or sk == 1:
         return out

@@ -98,6 +98,48 @@ def test_rows_do_not_depend_on_row_count(n, k, gs):
     assert torch.equal(torch.cat([qmm.matmul(x[r:r + 1], q, f32=True) for r in range(40)]), f32_)
 
 
+@pytest.mark.parametrize("n,k,gs", [(4096, 4096, 64), (200, 1024, 32), (1536, 2048, 32)])
+def test_the_slices_added_in_the_matmuls_own_launch(n, k, gs):
+    """One or two rows with a weight's arrival counters: the last workgroup of a tile adds the K slices up; without
+    them a second launch does (or, to eight rows, the one-launch form).  The same bits, the counters zero again
+    afterwards, also on replays of a graph; more rows take the other forms whatever is passed."""
+
+    from tensorfold_amd import _lib
+
+    q = qmm.pack(*gpu(*synthetic.affine_general(n, k, gs, n + k)), gs)
+    sk = qmm.split_k(n, k, gs)
+    assert sk > 1
+    x = synthetic.activations(65, k, 12).to(DEV)
+
+    def two_launches(rows, f32=False):
+        xs, m = qmm.group_sums(rows, gs), int(rows.shape[0])
+        out = torch.empty((m, n), device=DEV, dtype=torch.float32 if f32 else torch.bfloat16)
+        part = torch.empty((sk, m, n), device=DEV, dtype=torch.float32)
+        _lib.call("tf_qmm", _lib.ptr(rows), rows.stride(0), _lib.ptr(xs), _lib.ptr(q.weight), _lib.ptr(q.scales),
+                  _lib.ptr(q.biases), q.scales.stride(0), _lib.ptr(out), _lib.ptr(part), None, 0, m, n, k, sk, gs,
+                  qmm.bucket(m), int(f32), 1)
+        return out
+
+    for m in (1, 2, 3, 8, 9, 17, 65):
+        assert torch.equal(qmm.matmul(x[:m], q), two_launches(x[:m])), m
+        assert not q.counters.any(), m
+    for r in (5, 64):
+        assert torch.equal(qmm.matmul(x[r:r + 1], q)[0], two_launches(x[:65])[r]), r
+    assert torch.equal(qmm.matmul(x[:2], q, f32=True), two_launches(x[:2], f32=True))
+    out, part = torch.empty((2, n), device=DEV, dtype=torch.bfloat16), torch.empty((sk, 2, n), device=DEV)
+    xs = qmm.group_sums(x[:2], gs)
+    qmm.matmul(x[:2], q, xs, out=out, part=part)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(3):
+            qmm.matmul(x[:2], q, xs, out=out, part=part)
+    want = two_launches(x[:2])
+    for _ in range(3):
+        out.zero_()
+        graph.replay()
+        assert torch.equal(out, want) and not q.counters.any()
+
+
 def test_split_depends_only_on_shape():
     for n, k in [(48, 5120), (1024, 5120), (5120, 6144), (17408, 5120), (5120, 17408), (248320, 5120), (4096, 4096)]:
         sk = qmm.split_k(n, k)

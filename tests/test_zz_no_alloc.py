@@ -22,7 +22,7 @@ def both(x, q, sk, f32):
     common = (_lib.ptr(x), x.stride(0), _lib.ptr(xs), _lib.ptr(q.weight), _lib.ptr(q.scales), _lib.ptr(q.biases),
               q.scales.stride(0))
     shape = (m, q.n, q.k, sk, q.gs, qmm.bucket(m), int(f32))
-    _lib.call("tf_qmm", *common, _lib.ptr(want), _lib.ptr(part), *shape, 1)
+    _lib.call("tf_qmm", *common, _lib.ptr(want), _lib.ptr(part), None, 0, *shape, 1)      # no arrival counters
     _lib.call("tf_qmm_static", *common, _lib.ptr(got), *shape)
     torch.cuda.synchronize()
     return want, got
