@@ -72,6 +72,8 @@ __global__ void __launch_bounds__(WAVES * 64)
 
 // ---- dense lane matmul ---------------------------------------------------------------------------------------------
 
+constexpr int QRB = 8;          // rows a pass of the dense split kernels (the one-launch form keeps pairs)
+
 struct NoFlush {
   template <class A>
   __device__ __forceinline__ void operator()(int, A&) const {}
@@ -83,7 +85,7 @@ __device__ __forceinline__ void qmm_pass(const uint16_t* __restrict__ X, int64_t
                                          const WQ& wq, const SB& sb, int r0, int tile, int slice, int gs0, int per,
                                          int g0, int g1, void* __restrict__ out, float* __restrict__ part_out, int M,
                                          int N, int KG, int SK, int f32, float* xs, float* part,
-                                         Stage<GS, 1> (&st)[DEPTH], bool loaded) {
+                                         Stage<GS, 1, QRB> (&st)[DEPTH], bool loaded) {
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t* xl[RB];
   const_u32_ptr xsr[RB];
@@ -118,7 +120,8 @@ __device__ __forceinline__ void qmm_pass(const uint16_t* __restrict__ X, int64_t
 }
 
 // grid (column tiles of 64 x row tiles of BM, 1, SK).  Slice z takes groups [z * per, (z + 1) * per), its waves
-// split them again (added in wave order); SK > 1 leaves the slice's fp32 sums in part[z].  Rows go in passes of 2 or 1.
+// split them again (added in wave order); SK > 1 leaves the slice's fp32 sums in part[z].  Rows go in passes of 8, 4,
+// 2 or 1 (a row's arithmetic is the same in each: what a pass shares is the unpacked weights).
 template <int GS, int WAVES, bool COH = false>
 __device__ __forceinline__ void qmm_block(const uint16_t* __restrict__ X, int64_t ldx, const float* __restrict__ XS,
                                           const uint32_t* __restrict__ W, const uint16_t* __restrict__ S,
@@ -142,7 +145,7 @@ __device__ __forceinline__ void qmm_block(const uint16_t* __restrict__ X, int64_
   float* part = lds;
   const int m_end = min(M, (rt + 1) * BM);
   int r0 = rt * BM;
-  Stage<GS, 1> st[DEPTH];
+  Stage<GS, 1, QRB> st[DEPTH];
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d)
     if (g0 + d < g1) load_weights<GS, 1>(st[d], wq, sb, g0 + d);
@@ -150,8 +153,15 @@ __device__ __forceinline__ void qmm_block(const uint16_t* __restrict__ X, int64_
 #define TF_QMM_PASS(RB_)                                                                                             \
   qmm_pass<GS, WAVES, RB_, COH>(X, ldx, XS, wq, sb, r0, tile, slice, gs0, per, g0, g1, out, part_out, M, N, KG, SK, f32, \
                                 xs, part, st, loaded);                                                                      \
-  loaded = g1 - g0 <= DEPTH
-  for (; r0 + 2 <= m_end; r0 += 2) {
+  loaded = g1 - g0 <= DEPTH;                                                                                          \
+  r0 += RB_
+  while (r0 + 8 <= m_end) {
+    TF_QMM_PASS(8);
+  }
+  if (r0 + 4 <= m_end) {
+    TF_QMM_PASS(4);
+  }
+  if (r0 + 2 <= m_end) {
     TF_QMM_PASS(2);
   }
   if (r0 < m_end) {
@@ -166,7 +176,7 @@ __global__ void __launch_bounds__(WAVES * 64)
                const uint32_t* __restrict__ W, const uint16_t* __restrict__ S, const uint16_t* __restrict__ B,
                int64_t sb_stride, void* __restrict__ out, float* __restrict__ part_out, int M, int N, int KG, int SK,
                int BM, int f32) {
-  extern __shared__ float lds[];            // partials [WAVES][RBMAX][64]
+  extern __shared__ float lds[];            // partials [WAVES][QRB][64]
   qmm_block<GS, WAVES>(X, ldx, XS, W, S, B, sb_stride, out, part_out, M, N, KG, SK, BM, f32, blockIdx.x, blockIdx.z, lds);
 }
 
@@ -414,6 +424,7 @@ __global__ void __launch_bounds__(256)
 
 constexpr int QMM_WAVES = 4;
 constexpr int FAT_ROWS = 8;          // rows up to which tf_qmm runs the one-launch form
+constexpr int ARRIVE_ROWS = 4;       // rows up to which, given arrival counters, the split launch adds its own slices
 
 // Waves a workgroup of the expert GEMV: few workgroups (a small batch) spread each one's K over 16 waves, many
 // workgroups keep 4 longer-running waves each so that more of them are resident.  Scheduling only: bits do not move.
@@ -541,14 +552,14 @@ static int qmm_launch(const uint16_t* x, int64_t ldx, const float* xs, const uin
   TF_REQUIRE(sk == 1 || part, "part: at least (SK, M, n) fp32 is needed when K is split");
   hipStream_t s = as_stream(stream);
   const int tiles = (n + 63) / 64, rts = (m + bm - 1) / bm, per = kg / sk;
-  const size_t smem = sizeof(float) * ((size_t)QMM_WAVES * RBMAX * 64);
+  const size_t smem = sizeof(float) * ((size_t)QMM_WAVES * QRB * 64);
   TF_REQUIRE((int64_t)tiles * rts <= 0x7FFFFFFF && sk <= 65535, "qmm: grid too large");
   const int64_t fat_blocks = (int64_t)((n + 63) / 64) * ((m + RBMAX - 1) / RBMAX);
   const dim3 grid((unsigned)(tiles * rts), 1, (unsigned)sk);
-  if (reduce && sk > 1 && counters && m <= RBMAX && (int64_t)tiles * rts <= n_counters) {
-    // one pass of rows and arrival counters: the slices are added up by the last workgroup of a tile to finish.  A
-    // thousand four-wave workgroups beat the one-launch form's workgroup a column tile (4096 x 4096 at one row: 6.2-6.8
-    // against 7.4 us); with more rows the stores that go through to memory cost more than a reduce launch
+  if (reduce && sk > 1 && counters && m <= ARRIVE_ROWS && (int64_t)tiles * rts <= n_counters) {
+    // a few rows in one pass, and arrival counters: the slices are added up by the last workgroup of a tile to finish.
+    // A thousand four-wave workgroups beat the one-launch form's workgroup a column tile (4096 x 4096: 6.6-6.8 us at
+    // 1 or 2 rows, 7.2 at 4, against 7.5-8.5); from 5 rows on the one-launch form is ahead again (8.5 against 9.4)
     if (gs == 64)
       qmm_arrive_kernel<64, QMM_WAVES><<<grid, QMM_WAVES * 64, smem, s>>>(x, ldx, xs, weight, scales, biases, sb_stride,
                                                                            out, part, counters, m, n, kg, sk, bm, f32);
@@ -706,7 +717,7 @@ extern "C" int tf_qmm_group(const uint16_t* x, int64_t ldx, const float* xs, int
     TF_LAUNCH_OK("tf_qmm_group");
     return 0;
   }
-  const size_t smem = sizeof(float) * ((size_t)QMM_WAVES * RBMAX * 64);
+  const size_t smem = sizeof(float) * ((size_t)QMM_WAVES * QRB * 64);
   const dim3 grid((unsigned)blocks, 1, (unsigned)max_sk);
   if (gs == 64) qmm_group_kernel<64, QMM_WAVES><<<grid, QMM_WAVES * 64, smem, s>>>(x, ldx, xs, a, m, kg, bm, f32);
   else qmm_group_kernel<32, QMM_WAVES><<<grid, QMM_WAVES * 64, smem, s>>>(x, ldx, xs, a, m, kg, bm, f32);

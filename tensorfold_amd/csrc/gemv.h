@@ -82,15 +82,16 @@ __device__ __forceinline__ float dot2_bcast(float acc, uint32_t x, uint32_t q) {
 // the lane's dword of each chunk of the group's inputs.  Scale and bias stay as they were loaded (bf16 bits: the
 // scale in the low half of `s`, the bias in the low half of `b`, or with BHI in its high half) until the group is
 // added: turning them into floats where they are loaded would make the wave wait for every load it has just issued.
-template <int GS, int NM>
+// RBM: the most rows a pass of the kernel holding the stage takes.
+template <int GS, int NM, int RBM = RBMAX>
 struct Stage {
   uint4 w[NM][GS / 32];
   uint32_t s[NM], b[NM];
-  uint32_t x[RBMAX][GS / 32];
+  uint32_t x[RBM][GS / 32];
 };
 
-template <int GS, int NM, class WQ, class SB>
-__device__ __forceinline__ void load_weights(Stage<GS, NM>& st, const WQ& wq, const SB& sb, int g) {
+template <int GS, int NM, int RBM, class WQ, class SB>
+__device__ __forceinline__ void load_weights(Stage<GS, NM, RBM>& st, const WQ& wq, const SB& sb, int g) {
 #pragma unroll
   for (int m = 0; m < NM; ++m) {
 #pragma unroll
@@ -114,8 +115,8 @@ __device__ __forceinline__ float row16_sum(float s) {
 
 // Row r's sum over the staged group, from the dwords the dot products read anyway: a lane adds its two inputs of
 // each chunk in chunk order (a dot product against ones), then the sixteen lanes that share the row add up.
-template <int GS, int NM>
-__device__ __forceinline__ float stage_row_sum(const Stage<GS, NM>& st, int r) {
+template <int GS, int NM, int RBM>
+__device__ __forceinline__ float stage_row_sum(const Stage<GS, NM, RBM>& st, int r) {
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < GS / 32; ++i) s = dot2(st.x[r][i], BF16_ONES, s);
@@ -123,8 +124,8 @@ __device__ __forceinline__ float stage_row_sum(const Stage<GS, NM>& st, int r) {
 }
 
 // xl[r]: row r's inputs as dwords, already offset by (lane % 16)
-template <int GS, int NM, int RB, int COH>
-__device__ __forceinline__ void load_inputs(Stage<GS, NM>& st, const uint32_t* const (&xl)[RB], int g) {
+template <int GS, int NM, int RB, int COH, int RBM>
+__device__ __forceinline__ void load_inputs(Stage<GS, NM, RBM>& st, const uint32_t* const (&xl)[RB], int g) {
 #pragma unroll
   for (int r = 0; r < RB; ++r)
 #pragma unroll
@@ -149,8 +150,8 @@ __device__ __forceinline__ void word_dot(float (&p)[NM][RB], const uint32_t (&wo
 }
 
 // p += sum over chunk i of x * (128 + q)
-template <int GS, int NM, int RB>
-__device__ __forceinline__ void chunk_dot(float (&p)[NM][RB], const Stage<GS, NM>& st, int i) {
+template <int GS, int NM, int RB, int RBM>
+__device__ __forceinline__ void chunk_dot(float (&p)[NM][RB], const Stage<GS, NM, RBM>& st, int i) {
   const uint32_t magic = BF16_128;
   uint32_t x[RB];
 #pragma unroll
@@ -175,8 +176,9 @@ __device__ __forceinline__ void chunk_dot(float (&p)[NM][RB], const Stage<GS, NM
 //   xsum(r, g)      -> row r's sum over group g (wave-uniform); with XIN the sums are taken from the staged inputs
 //   flush(g, acc)   -> called after group g has been added (wave-uniform); may park and clear acc
 // `st` holds the weights of groups gA .. gA + DEPTH - 1 on entry when `loaded`.
-template <int GS, int NM, int RB, int COH, bool XIN = false, bool BHI = false, class WQ, class SB, class XS, class FLUSH>
-__device__ __forceinline__ void gemv_stream(float (&acc)[NM][RB], Stage<GS, NM> (&st)[DEPTH], bool loaded,
+template <int GS, int NM, int RB, int COH, bool XIN = false, bool BHI = false, int RBM, class WQ, class SB, class XS,
+          class FLUSH>
+__device__ __forceinline__ void gemv_stream(float (&acc)[NM][RB], Stage<GS, NM, RBM> (&st)[DEPTH], bool loaded,
                                             const WQ& wq, const SB& sb, const uint32_t* const (&xl)[RB],
                                             const XS& xsum, int gA, int gB, FLUSH& flush) {
   constexpr int CH = GS / 32;

@@ -41,7 +41,7 @@ class Q4:
     @property
     def counters(self) -> torch.Tensor:
         """Arrival counters of the K slices, one a column tile of 64, each alone in 64 bytes; zero between calls.
-        With them ``matmul`` on one or two rows adds the slices up in its own launch.  Calls on one weight that
+        With them ``matmul`` on up to four rows adds the slices up in its own launch.  Calls on one weight that
         overlap in time (two streams) need a ``Q4`` of their own each (``dataclasses.replace`` shares the packed
         tensors and starts with fresh counters)."""
 
@@ -190,7 +190,7 @@ def matmul(x: torch.Tensor, q: Q4, xs: torch.Tensor | None = None, *, sk: int | 
     if xs.dtype != torch.float32 or tuple(xs.shape) != (m, q.k // q.gs) or not xs.is_contiguous() \
             or xs.device != x.device:
         raise ValueError(f"matmul: xs must be contiguous fp32 ({m}, {q.k // q.gs}), the group sums of x")
-    counters = q.counters if reduce and sk > 1 and m <= 2 else None
+    counters = q.counters if reduce and sk > 1 and m <= 4 else None
     _lib.call("tf_qmm", _lib.ptr(x), x.stride(0), _lib.ptr(xs), _lib.ptr(q.weight), _lib.ptr(q.scales),
               _lib.ptr(q.biases), q.scales.stride(0), _lib.ptr(out), _lib.ptr(part), _lib.ptr(counters),
               0 if counters is None else counters.numel() // COUNTER_STRIDE, m, q.n, q.k, sk, q.gs, bucket(m),

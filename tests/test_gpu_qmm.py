@@ -100,7 +100,7 @@ def test_rows_do_not_depend_on_row_count(n, k, gs):
 
 @pytest.mark.parametrize("n,k,gs", [(4096, 4096, 64), (200, 1024, 32), (1536, 2048, 32)])
 def test_the_slices_added_in_the_matmuls_own_launch(n, k, gs):
-    """One or two rows with a weight's arrival counters: the last workgroup of a tile adds the K slices up; without
+    """Up to four rows with a weight's arrival counters: the last workgroup of a tile adds the K slices up; without
     them a second launch does (or, to eight rows, the one-launch form).  The same bits, the counters zero again
     afterwards, also on replays of a graph; more rows take the other forms whatever is passed."""
 
@@ -120,20 +120,20 @@ def test_the_slices_added_in_the_matmuls_own_launch(n, k, gs):
                   qmm.bucket(m), int(f32), 1)
         return out
 
-    for m in (1, 2, 3, 8, 9, 17, 65):
+    for m in (1, 2, 3, 4, 5, 8, 9, 17, 65):
         assert torch.equal(qmm.matmul(x[:m], q), two_launches(x[:m])), m
         assert not q.counters.any(), m
     for r in (5, 64):
         assert torch.equal(qmm.matmul(x[r:r + 1], q)[0], two_launches(x[:65])[r]), r
-    assert torch.equal(qmm.matmul(x[:2], q, f32=True), two_launches(x[:2], f32=True))
-    out, part = torch.empty((2, n), device=DEV, dtype=torch.bfloat16), torch.empty((sk, 2, n), device=DEV)
-    xs = qmm.group_sums(x[:2], gs)
-    qmm.matmul(x[:2], q, xs, out=out, part=part)
+    assert torch.equal(qmm.matmul(x[:3], q, f32=True), two_launches(x[:3], f32=True))
+    out, part = torch.empty((3, n), device=DEV, dtype=torch.bfloat16), torch.empty((sk, 3, n), device=DEV)
+    xs = qmm.group_sums(x[:3], gs)
+    qmm.matmul(x[:3], q, xs, out=out, part=part)
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         for _ in range(3):
-            qmm.matmul(x[:2], q, xs, out=out, part=part)
-    want = two_launches(x[:2])
+            qmm.matmul(x[:3], q, xs, out=out, part=part)
+    want = two_launches(x[:3])
     for _ in range(3):
         out.zero_()
         graph.replay()
