@@ -59,7 +59,7 @@ int tf_group_sums(const uint16_t* x, int64_t ldx, int m, int k, int gs, float* x
  * sk > 1 (with reduce == 0 the slices are left there unadded; with few rows and reduce != 0 the slices are added
  * inside the one launch, in the same order, and `part` goes unused).  sb_stride = elements between scale rows
  * (>= npad).  `counters` (may be NULL): n_counters arrival counters of the weight, TF_QMM_COUNTER_STRIDE ints apart,
- * zero on entry and left zero; with one for every column tile of 64, the slices of up to four rows are added up in the
+ * zero on entry and left zero; with one for every column tile of 64, the slices of up to eight rows are added up in the
  * matmul's own launch by the last workgroup of a tile to finish (same order, same bits);
  * calls on one weight's counters must not overlap.  Replaces kernels/qmm.cpp:18-48 `qmm`. */
 #define TF_QMM_COUNTER_STRIDE 16

@@ -85,14 +85,15 @@ __device__ __forceinline__ void qmm_pass(const uint16_t* __restrict__ X, int64_t
                                          const WQ& wq, const SB& sb, int r0, int tile, int slice, int gs0, int per,
                                          int g0, int g1, void* __restrict__ out, float* __restrict__ part_out, int M,
                                          int N, int KG, int SK, int f32, float* xs, float* part,
-                                         Stage<GS, 1, QRB> (&st)[DEPTH], bool loaded) {
+                                         Stage<GS, 1, QRB> (&st)[DEPTH], bool loaded, int valid) {
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t* xl[RB];
   const_u32_ptr xsr[RB];
 #pragma unroll
   for (int r = 0; r < RB; ++r) {
-    xl[r] = reinterpret_cast<const uint32_t*>(X + (size_t)(r0 + r) * ldx) + (lane & 15);
-    xsr[r] = as_const(XS + (size_t)(r0 + r) * KG);
+    const int row = r0 + (r < valid ? r : valid - 1);          // a pass past the last row walks that row again, unstored
+    xl[r] = reinterpret_cast<const uint32_t*>(X + (size_t)row * ldx) + (lane & 15);
+    xsr[r] = as_const(XS + (size_t)row * KG);
   }
   __syncthreads();                                  // the previous pass is done with part
   float acc[1][RB];
@@ -104,7 +105,7 @@ __device__ __forceinline__ void qmm_pass(const uint16_t* __restrict__ X, int64_t
 #pragma unroll
   for (int r = 0; r < RB; ++r) part[(wave * RB + r) * 64 + lane] = acc[0][r];
   __syncthreads();
-  for (int o = tid; o < RB * 64; o += WAVES * 64) {
+  for (int o = tid; o < valid * 64; o += WAVES * 64) {
     const int r = o >> 6, l = o & 63, cc = tile * 64 + l;
     if (cc >= N) continue;
     float s = part[r * 64 + l];
@@ -121,7 +122,8 @@ __device__ __forceinline__ void qmm_pass(const uint16_t* __restrict__ X, int64_t
 
 // grid (column tiles of 64 x row tiles of BM, 1, SK).  Slice z takes groups [z * per, (z + 1) * per), its waves
 // split them again (added in wave order); SK > 1 leaves the slice's fp32 sums in part[z].  Rows go in passes of 8, 4,
-// 2 or 1 (a row's arithmetic is the same in each: what a pass shares is the unpacked weights).
+// 2 or 1 (a row's arithmetic is the same in each: what a pass shares is the unpacked weights); 5 to 7 rows take the
+// pass of 8 and 3 rows the pass of 4, rather than two passes over the weights.
 template <int GS, int WAVES, bool COH = false>
 __device__ __forceinline__ void qmm_block(const uint16_t* __restrict__ X, int64_t ldx, const float* __restrict__ XS,
                                           const uint32_t* __restrict__ W, const uint16_t* __restrict__ S,
@@ -151,22 +153,17 @@ __device__ __forceinline__ void qmm_block(const uint16_t* __restrict__ X, int64_
     if (g0 + d < g1) load_weights<GS, 1>(st[d], wq, sb, g0 + d);
   bool loaded = true;
 #define TF_QMM_PASS(RB_)                                                                                             \
-  qmm_pass<GS, WAVES, RB_, COH>(X, ldx, XS, wq, sb, r0, tile, slice, gs0, per, g0, g1, out, part_out, M, N, KG, SK, f32, \
-                                xs, part, st, loaded);                                                                      \
-  loaded = g1 - g0 <= DEPTH;                                                                                          \
-  r0 += RB_
-  while (r0 + 8 <= m_end) {
-    TF_QMM_PASS(8);
+  {                                                                                                                  \
+    const int valid = min(RB_, m_end - r0);                                                                          \
+    qmm_pass<GS, WAVES, RB_, COH>(X, ldx, XS, wq, sb, r0, tile, slice, gs0, per, g0, g1, out, part_out, M, N, KG, SK, \
+                                  f32, xs, part, st, loaded, valid);                                                 \
+    loaded = g1 - g0 <= DEPTH;                                                                                       \
+    r0 += valid;                                                                                                     \
   }
-  if (r0 + 4 <= m_end) {
-    TF_QMM_PASS(4);
-  }
-  if (r0 + 2 <= m_end) {
-    TF_QMM_PASS(2);
-  }
-  if (r0 < m_end) {
-    TF_QMM_PASS(1);
-  }
+  while (m_end - r0 >= 5) TF_QMM_PASS(8)
+  if (m_end - r0 >= 3) TF_QMM_PASS(4)
+  if (m_end - r0 == 2) TF_QMM_PASS(2)
+  if (m_end - r0 == 1) TF_QMM_PASS(1)
 #undef TF_QMM_PASS
 }
 
@@ -424,7 +421,7 @@ __global__ void __launch_bounds__(256)
 
 constexpr int QMM_WAVES = 4;
 constexpr int FAT_ROWS = 8;          // rows up to which tf_qmm runs the one-launch form
-constexpr int ARRIVE_ROWS = 4;       // rows up to which, given arrival counters, the split launch adds its own slices
+constexpr int ARRIVE_ROWS = QRB;      // rows up to which, given arrival counters, the split launch adds its own slices
 
 // Waves a workgroup of the expert GEMV: few workgroups (a small batch) spread each one's K over 16 waves, many
 // workgroups keep 4 longer-running waves each so that more of them are resident.  Scheduling only: bits do not move.
@@ -557,9 +554,10 @@ static int qmm_launch(const uint16_t* x, int64_t ldx, const float* xs, const uin
   const int64_t fat_blocks = (int64_t)((n + 63) / 64) * ((m + RBMAX - 1) / RBMAX);
   const dim3 grid((unsigned)(tiles * rts), 1, (unsigned)sk);
   if (reduce && sk > 1 && counters && m <= ARRIVE_ROWS && (int64_t)tiles * rts <= n_counters) {
-    // a few rows in one pass, and arrival counters: the slices are added up by the last workgroup of a tile to finish.
-    // A thousand four-wave workgroups beat the one-launch form's workgroup a column tile (4096 x 4096: 6.6-6.8 us at
-    // 1 or 2 rows, 7.2 at 4, against 7.5-8.5); from 5 rows on the one-launch form is ahead again (8.5 against 9.4)
+    // one pass of rows, and arrival counters: the slices are added up by the last workgroup of a tile to finish.
+    // Hundreds of four-wave workgroups beat the one-launch form's workgroup a column tile and row pair: 4096 x 4096
+    // 6.0 us at 1 row against 7.5, 7.1 at 4 against 8.5 (9.1 against 8.3 at 8, the one shape where that form wins);
+    // 5120 x 17408 at 8 rows 24 against 40
     if (gs == 64)
       qmm_arrive_kernel<64, QMM_WAVES><<<grid, QMM_WAVES * 64, smem, s>>>(x, ldx, xs, weight, scales, biases, sb_stride,
                                                                            out, part, counters, m, n, kg, sk, bm, f32);

@@ -41,7 +41,7 @@ class Q4:
     @property
     def counters(self) -> torch.Tensor:
         """Arrival counters of the K slices, one a column tile of 64, each alone in 64 bytes; zero between calls.
-        With them ``matmul`` on up to four rows adds the slices up in its own launch.  Calls on one weight that
+        With them ``matmul`` on up to eight rows adds the slices up in its own launch.  Calls on one weight that
         overlap in time (two streams) need a ``Q4`` of their own each (``dataclasses.replace`` shares the packed
         tensors and starts with fresh counters)."""
 
@@ -120,15 +120,17 @@ def matmul_rows(x: torch.Tensor, parts: list[Q4]) -> torch.Tensor:
     return torch.cat([matmul(x, p, xs, sk=sk) for p in parts], dim=1)
 
 
-def split_k(n: int, k: int, gs: int = 64, target: int = 1024) -> int:
+def split_k(n: int, k: int, gs: int = 64, target: int = 768) -> int:
     """Number of K slices of an (n, k) weight - from the shape alone, never the row count.
 
-    Doubles while there are fewer than ``target`` workgroups (64-column tiles x slices; an MI355X has 256 CUs and
-    wants a few workgroups on each), the groups still divide evenly and a slice keeps at least 4 groups."""
+    Doubles while that keeps the workgroups (64-column tiles x slices) within ``target`` (an MI355X has 256 CUs and
+    the launch is fastest with two or three four-wave workgroups on each: 4096 x 4096 at one row takes 6.0 us with 8
+    slices, 6.1 with 16; 6144 x 5120 7.1 against 9.1; 5120 x 17408 12.3 against 15.4), the groups still divide evenly
+    and a slice keeps at least 4 groups."""
 
     tiles, groups = -(-n // 64), k // gs
     sk = 1
-    while sk < 16 and tiles * sk < target and groups % (2 * sk) == 0 and groups // (2 * sk) >= 4:
+    while sk < 16 and 2 * tiles * sk <= target and groups % (2 * sk) == 0 and groups // (2 * sk) >= 4:
         sk *= 2
     return sk
 
@@ -190,7 +192,7 @@ def matmul(x: torch.Tensor, q: Q4, xs: torch.Tensor | None = None, *, sk: int | 
     if xs.dtype != torch.float32 or tuple(xs.shape) != (m, q.k // q.gs) or not xs.is_contiguous() \
             or xs.device != x.device:
         raise ValueError(f"matmul: xs must be contiguous fp32 ({m}, {q.k // q.gs}), the group sums of x")
-    counters = q.counters if reduce and sk > 1 and m <= 4 else None
+    counters = q.counters if reduce and sk > 1 and m <= 8 else None
     _lib.call("tf_qmm", _lib.ptr(x), x.stride(0), _lib.ptr(xs), _lib.ptr(q.weight), _lib.ptr(q.scales),
               _lib.ptr(q.biases), q.scales.stride(0), _lib.ptr(out), _lib.ptr(part), _lib.ptr(counters),
               0 if counters is None else counters.numel() // COUNTER_STRIDE, m, q.n, q.k, sk, q.gs, bucket(m),

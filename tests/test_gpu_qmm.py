@@ -100,8 +100,8 @@ def test_rows_do_not_depend_on_row_count(n, k, gs):
 
 @pytest.mark.parametrize("n,k,gs", [(4096, 4096, 64), (200, 1024, 32), (1536, 2048, 32)])
 def test_the_slices_added_in_the_matmuls_own_launch(n, k, gs):
-    """Up to four rows with a weight's arrival counters: the last workgroup of a tile adds the K slices up; without
-    them a second launch does (or, to eight rows, the one-launch form).  The same bits, the counters zero again
+    """Up to eight rows with a weight's arrival counters: the last workgroup of a tile adds the K slices up; without
+    them the one-launch form runs (or, past eight rows, a second launch).  The same bits, the counters zero again
     afterwards, also on replays of a graph; more rows take the other forms whatever is passed."""
 
     from tensorfold_amd import _lib
@@ -120,7 +120,7 @@ def test_the_slices_added_in_the_matmuls_own_launch(n, k, gs):
                   qmm.bucket(m), int(f32), 1)
         return out
 
-    for m in (1, 2, 3, 4, 5, 8, 9, 17, 65):
+    for m in (1, 2, 3, 4, 5, 6, 7, 8, 9, 11, 13, 17, 65):
         assert torch.equal(qmm.matmul(x[:m], q), two_launches(x[:m])), m
         assert not q.counters.any(), m
     for r in (5, 64):
