@@ -64,6 +64,28 @@ def opened(path, way: str) -> dr.SafeTensors:
     return files
 
 
+@pytest.mark.parametrize("way", WAYS)
+def test_any_range_of_a_file_reads_back(tmp_path, monkeypatch, way):
+    """Drawn (offset, length) pairs against the file's own bytes, pieces of one, two and sixteen blocks."""
+
+    rng = np.random.default_rng(3)
+    blob = rng.integers(0, 256, 150_003, dtype=np.uint8)
+    path = tmp_path / "blob.bin"
+    path.write_bytes(blob.tobytes())
+    for blocks in (1, 2, 16):
+        monkeypatch.setattr(dr, "PIECE", blocks * dr.ALIGN)
+        reader = dr.Reader()
+        reader.direct = reader.direct and way == "o_direct"
+        edges = [0, 1, 4095, 4096, 4097, 8192, 150_002, 150_003]
+        starts = list(rng.integers(0, blob.size, 20)) + edges[:-1]
+        for first in starts:
+            for n in (int(rng.integers(0, blob.size - first + 1)), min(4096, blob.size - first), blob.size - first):
+                got = reader.read(path, int(first), n)
+                assert got.dtype == torch.uint8 and np.array_equal(got.numpy(), blob[first:first + n]), (blocks, first, n)
+        with pytest.raises(IOError, match="short read"):
+            reader.read(path, blob.size - 10, 11)
+
+
 def test_pieces_cover_a_range_once_in_whole_blocks(monkeypatch):
     monkeypatch.setattr(dr, "PIECE", 2 * dr.ALIGN)
     for offset, n, size in ((0, 1, 1), (13, 30_000, 40_000), (8192, 8192, 16384), (4095, 2, 9000), (20_000, 5, 20_005)):
