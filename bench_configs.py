@@ -158,7 +158,7 @@ def c2() -> dict:
             "down_gbs": uniq[0] * per_expert / 3 / down_us * 1e-3}
 
 
-def c3(tiles=((64, torch.float32), (128, torch.float32), ("128_y_bf16", torch.bfloat16))) -> dict:
+def c3(tiles=((64, torch.float32), (128, torch.float32), ("128_y_bf16", torch.bfloat16), ("128_y_f16", torch.float16))) -> dict:
     s, rows = synthetic.C2, 4096
     gen = torch.Generator(device=DEV).manual_seed(3)
     ex = moe_tables(s, 1, gen)[0]
@@ -170,7 +170,8 @@ def c3(tiles=((64, torch.float32), (128, torch.float32), ("128_y_bf16", torch.bf
     slots = s.top_k + 1
     out = {}
     # items of 64 and of 128 with fp32 pair outputs (this build's default), then items of 128 with the reference's
-    # bf16 pair outputs (cuda/moe.py:99), which halve the traffic between the down projection and the combine
+    # bf16 pair outputs (cuda/moe.py:99), which halve the traffic between the down projection and the combine, and
+    # with fp16 ones: the same bytes at an eighth of the rounding
     for tile, ydt in tiles:
         key, tile = tile, 128 if isinstance(tile, str) else tile
         plan = experts.Plan(rows, slots, s.experts + 1, DEV, prefill=True)

@@ -159,7 +159,7 @@ int tf_experts_run(int gs, int epi, const uint16_t* x, int64_t x_stride, int slo
 int tf_experts_run_desc(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg,
                         int nb, const int32_t* desc, const int32_t* counts, void* out, int n, float limit,
                         int64_t max_items, tf_stream_t stream);
-/* Prompt form on MFMA, each weight rounded once as in tf_qmm_prefill (arith: TF_ARITH_*); epi 3: bf16 out.  `tile` is
+/* Prompt form on MFMA, each weight rounded once as in tf_qmm_prefill (arith: TF_ARITH_*); epi 3: bf16 out; epi 4: fp16 out, values beyond fp16's range stored as +-65504.  `tile` is
  * the plan's item size (16, 64 or 128).  Replaces experts.cpp:50-55 `prefill`. */
 int tf_experts_prefill(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg,
                        int nb, const int32_t* items, const int32_t* counts, const int32_t* members, void* out, int n,
@@ -175,7 +175,7 @@ int tf_moe_router(const uint16_t* x, int64_t ldx, const uint16_t* rows, float* l
  * pick int32 and wts fp32 are [rows, top_k + (shared ? 1 : 0)].  Replaces moe.py:58-108 `_topk_rows` / `select_rows`. */
 int tf_moe_topk(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared, int32_t* pick,
                 float* wts, tf_stream_t stream);
-/* out[r] = bf16(sum_k wts[r, k] * y[r, k]) in slot order, fp32; y is fp32 (y_bf16 == 0) or bf16.
+/* out[r] = bf16(sum_k wts[r, k] * y[r, k]) in slot order, fp32; y is fp32 (y_bf16 == 0), bf16 (1) or fp16 (2).
  * Replaces moe.py:131-151 `_combine` / `combine`. */
 int tf_moe_combine(const void* y, int y_bf16, const float* wts, uint16_t* out, int rows, int slots, int d,
                    tf_stream_t stream);

@@ -111,12 +111,14 @@ __device__ __forceinline__ bf16x8_t dequant8b(uint32_t w, uint32_t sb) {
   return __builtin_bit_cast(bf16x8_t, r);
 }
 
-// EPI 0: fp32; 1: bf16 relu(bf16 a)^2; 2: bf16 SwiGLU(matrix 0, matrix 1); 3: bf16
+// EPI 0: fp32; 1: bf16 relu(bf16 a)^2; 2: bf16 SwiGLU(matrix 0, matrix 1); 3: bf16; 4: fp16, values beyond its
+// range stored as +-65504 (pair outputs at half the bytes of fp32 and an eighth of bf16's rounding)
 template <int EPI>
 __device__ __forceinline__ void store_out(void* out, size_t at, float a, float u, float limit) {
   if constexpr (EPI == 0) reinterpret_cast<float*>(out)[at] = a;
   else if constexpr (EPI == 1) reinterpret_cast<uint16_t*>(out)[at] = (uint16_t)f32_bf16_bits(relu2(a));
   else if constexpr (EPI == 2) reinterpret_cast<uint16_t*>(out)[at] = (uint16_t)f32_bf16_bits(swiglu(a, u, limit));
+  else if constexpr (EPI == 4) reinterpret_cast<_Float16*>(out)[at] = (_Float16)fminf(fmaxf(a, -65504.f), 65504.f);
   else reinterpret_cast<uint16_t*>(out)[at] = (uint16_t)f32_bf16_bits(a);
 }
 
@@ -719,8 +721,8 @@ extern "C" int tf_experts_prefill(int gs, int epi, const uint16_t* x, int64_t x_
 #define TF_PRE(GS_, NM_, EPI_) \
   if (gs == GS_ && epi == EPI_) \
     return launch_experts_prefill<GS_, NM_, EPI_>(tile, arith, x, x_stride, slots, w, kg, nb, items, counts, members, out, n, limit, max_items, s);
-  TF_PRE(32, 1, 0) TF_PRE(32, 1, 1) TF_PRE(32, 1, 3) TF_PRE(32, 2, 2)
-  TF_PRE(64, 1, 0) TF_PRE(64, 1, 1) TF_PRE(64, 1, 3) TF_PRE(64, 2, 2)
+  TF_PRE(32, 1, 0) TF_PRE(32, 1, 1) TF_PRE(32, 1, 3) TF_PRE(32, 1, 4) TF_PRE(32, 2, 2)
+  TF_PRE(64, 1, 0) TF_PRE(64, 1, 1) TF_PRE(64, 1, 3) TF_PRE(64, 1, 4) TF_PRE(64, 2, 2)
 #undef TF_PRE
   set_error("experts: no prefill kernel for group %d and epilogue %d", gs, epi);
   return 1;

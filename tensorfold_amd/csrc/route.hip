@@ -198,7 +198,8 @@ __global__ void plan_scatter_kernel(const int* __restrict__ picks, int P, int E,
 
 // ---- combine ---------------------------------------------------------------------------------------------------------
 
-template <bool YBF16>
+// YKIND: what the pair outputs are stored as: 0 fp32, 1 bf16, 2 fp16
+template <int YKIND>
 __global__ void __launch_bounds__(256)
     combine_kernel(const void* __restrict__ Y, const float* __restrict__ Wt, uint16_t* __restrict__ out, int S, int D) {
   const int r = blockIdx.x;
@@ -213,10 +214,15 @@ __global__ void __launch_bounds__(256)
       const int k = k0 + j < S ? k0 + j : S - 1;
       w[j] = Wt[(size_t)r * S + k];
       const size_t at = ((size_t)r * S + k) * D + d;
-      if (YBF16) {
+      if (YKIND == 1) {
         const uint32_t v = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(Y) + at);
         v0[j] = bf16_lo(v);
         v1[j] = bf16_hi(v);
+      } else if (YKIND == 2) {
+        typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+        const half2_t v = *reinterpret_cast<const half2_t*>(reinterpret_cast<const _Float16*>(Y) + at);
+        v0[j] = (float)v[0];
+        v1[j] = (float)v[1];
       } else {
         const float2 v = *reinterpret_cast<const float2*>(reinterpret_cast<const float*>(Y) + at);
         v0[j] = v.x;
@@ -347,8 +353,9 @@ extern "C" int tf_moe_combine(const void* y, int y_bf16, const float* wts, uint1
     return 0;
   }
   const dim3 grid(rows, (d / 2 + 255) / 256);
-  if (y_bf16) combine_kernel<true><<<grid, 256, 0, as_stream(stream)>>>(y, wts, out, slots, d);
-  else combine_kernel<false><<<grid, 256, 0, as_stream(stream)>>>(y, wts, out, slots, d);
+  if (y_bf16 == 1) combine_kernel<1><<<grid, 256, 0, as_stream(stream)>>>(y, wts, out, slots, d);
+  else if (y_bf16 == 2) combine_kernel<2><<<grid, 256, 0, as_stream(stream)>>>(y, wts, out, slots, d);
+  else combine_kernel<0><<<grid, 256, 0, as_stream(stream)>>>(y, wts, out, slots, d);
   TF_LAUNCH_OK("tf_moe_combine");
   return 0;
 }

@@ -183,7 +183,7 @@ def _check(x: torch.Tensor, k: int, out: torch.Tensor, n: int, epi: int) -> None
         raise RuntimeError("x: rows of K = groups * group size inputs, 16-byte aligned")
     if not out.is_contiguous() or out.dim() != 2 or out.shape[1] != n:
         raise RuntimeError("out: contiguous rows of n columns")
-    if out.dtype != (torch.float32 if epi == 0 else torch.bfloat16):
+    if out.dtype != {0: torch.float32, 4: torch.float16}.get(epi, torch.bfloat16):
         raise RuntimeError("out has the wrong dtype")
     _lib.on_gpu(x, out)
 
@@ -218,10 +218,13 @@ def gate_up(x: torch.Tensor, ex: Experts, plan: Plan, out: torch.Tensor, rows: i
 
 
 def down(act: torch.Tensor, ex: Experts, plan: Plan, out: torch.Tensor, rows: int) -> None:
-    """Pair activations bf16 [R * slots, NI] -> every pair's output [R * slots, D]: fp32, or bf16 when a prompt plan
-    is given a bf16 ``out``."""
+    """Pair activations bf16 [R * slots, NI] -> every pair's output [R * slots, D]: fp32; a prompt plan also takes a
+    bf16 ``out`` (the reference's choice, cuda/moe.py:99: half the bytes, a rounding of 2^-9) or an fp16 one (half the
+    bytes, a rounding of 2^-12; a value beyond +-65504 is stored as +-65504)."""
 
-    epi = 3 if (plan.prefill and out.dtype == torch.bfloat16) else 0
+    epi = 0
+    if plan.prefill and out.dtype in (torch.bfloat16, torch.float16):
+        epi = 3 if out.dtype == torch.bfloat16 else 4
     _check(act, ex.width, out, ex.dims, epi)
     _fits(plan, rows, None, min(act.shape[0], out.shape[0]))
     _launch(act, 0, ex.down, ex.gs, ex.width, ex.dims, epi, plan, out, 0.0, rows, ex.arith)

@@ -57,10 +57,13 @@ class MoEBuffers:
     """Preallocated scratch of a layer for at most ``rows`` rows, so that a captured graph can replay it.
 
     ``prefill`` selects the prompt arithmetic of the experts; ``shared=False`` is for layers
-    without a shared expert: no extra logit column, no extra slot."""
+    without a shared expert: no extra logit column, no extra slot.  ``y_dtype``: what the pair outputs are kept as
+    between the down projection and the combine: fp32, or with ``prefill`` fp16 or bf16 (half the bytes)."""
 
     def __init__(self, rows: int, cfg, device: torch.device | str, *, prefill: bool = False,
-                 shared: bool = True) -> None:
+                 shared: bool = True, y_dtype: torch.dtype = torch.float32) -> None:
+        if y_dtype != torch.float32 and not (prefill and y_dtype in (torch.float16, torch.bfloat16)):
+            raise ValueError("pair outputs are fp32; a prompt plan also takes fp16 or bf16")
         extra = int(shared)
         self.rows, self.shared = rows, shared
         self.slots = cfg.num_experts_per_tok + extra
@@ -70,10 +73,10 @@ class MoEBuffers:
         self.wts = torch.empty((rows, self.slots), **f32)
         self.plan = grouped.Plan(rows, self.slots, cfg.num_experts + extra, device, prefill=prefill)
         self.act = torch.empty((rows, self.slots, cfg.moe_intermediate_size), dtype=torch.bfloat16, device=device)
-        # Pair outputs stay fp32 in both forms.  (The reference keeps bf16 pair outputs in its prompt form; that
-        # rounding alone costs 1.1e-3 relative L2 at the combine, most of a 2e-3 budget.  ``experts.down`` still
-        # writes bf16 into a bf16 ``out`` on a prompt plan for callers that want the smaller buffer.)
-        self.y = torch.empty((rows, self.slots, cfg.hidden_size), device=device, dtype=torch.float32)
+        # Pair outputs are fp32 unless told.  (The reference keeps bf16 pair outputs in its prompt form,
+        # cuda/moe.py:99; that rounding alone puts the layer 2.7e-3 relative L2 from the dequant-then-matmul result,
+        # past a 2e-3 bound.  fp16 takes the same bytes and leaves it at 9e-4: ``run`` uses it for prompts.)
+        self.y = torch.empty((rows, self.slots, cfg.hidden_size), device=device, dtype=y_dtype)
         self.cfg, self.device, self._fused = cfg, device, {}
 
     def fused(self, gs: int) -> dict:
@@ -199,7 +202,8 @@ def decode(x: torch.Tensor, logits: torch.Tensor, ex: grouped.Experts, buf: MoEB
 
 
 def combine(y: torch.Tensor, wts: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
-    """bf16 [R, D] = sum over slots, in slot order and in fp32, of wts[r, k] * y[r, k]; y is fp32 or bf16 [R, S, D]."""
+    """bf16 [R, D] = sum over slots, in slot order and in fp32, of wts[r, k] * y[r, k]; y is fp32, bf16 or fp16
+    [R, S, D]."""
 
     _lib.on_gpu(y, wts)
     if not y.is_contiguous() or not wts.is_contiguous() or wts.dtype != torch.float32:
@@ -207,7 +211,10 @@ def combine(y: torch.Tensor, wts: torch.Tensor, out: torch.Tensor | None = None)
     r, s, d = y.shape
     if out is None:
         out = y.new_empty((r, d), dtype=torch.bfloat16)
-    _lib.call("tf_moe_combine", _lib.ptr(y), int(y.dtype == torch.bfloat16), _lib.ptr(wts), _lib.ptr(out), r, s, d)
+    kind = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}.get(y.dtype)
+    if kind is None:
+        raise ValueError("combine: y must be fp32, bf16 or fp16")
+    _lib.call("tf_moe_combine", _lib.ptr(y), kind, _lib.ptr(wts), _lib.ptr(out), r, s, d)
     return out
 
 
@@ -238,13 +245,17 @@ _pool: dict[tuple, MoEBuffers] = {}
 
 def run(x: torch.Tensor, m: Routed, *, prefill: bool = False) -> torch.Tensor:
     """The whole layer: bf16 [R, D] in, bf16 [R, D] out.  Scratch is pooled by the row count rounded up to a power
-    of two (16 at least), so every layer of a model shares it."""
+    of two (16 at least), so every layer of a model shares it.  A prompt's pair outputs are kept in fp16 between the
+    down projection and the combine (half the traffic of fp32; a pair output beyond +-65504 is stored as +-65504)
+    when the layer runs the fp16 prompt arithmetic, which makes the same assumption of its activations; a layer
+    made with ``ARITH_BF16`` keeps them in fp32."""
 
     n = int(x.shape[0])
     cap = max(16, 1 << (n - 1).bit_length())
-    key = (cap, m.count, m.top_k, m.experts.width, m.experts.dims, m.experts.gs, prefill, x.device)
+    y_dtype = torch.float16 if prefill and m.experts.arith == grouped.ARITH_F16 else torch.float32
+    key = (cap, m.count, m.top_k, m.experts.width, m.experts.dims, m.experts.gs, prefill, y_dtype, x.device)
     if key not in _pool:
-        _pool[key] = MoEBuffers(cap, _Dims(m), x.device, prefill=prefill)
+        _pool[key] = MoEBuffers(cap, _Dims(m), x.device, prefill=prefill, y_dtype=y_dtype)
     buf, x = _pool[key], x.contiguous()
     if fusable(x, m.experts, buf):
         router(x, m.router, buf.logits[:n])

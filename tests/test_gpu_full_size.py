@@ -161,3 +161,11 @@ def test_config3_at_full_size():
     idx = torch.from_numpy(sample[:40]).to(DEV)
     small, _ = run_chunk(ex, xd[idx].contiguous(), pd[idx].contiguous(), wd[idx].contiguous(), 64)
     assert torch.equal(small, outs[128][idx])
+    # pair outputs kept in fp16 between the down projection and the combine, as moe.run keeps a prompt's
+    half, _ = run_chunk(ex, xd, pd, wd, 128, torch.float16)
+    got16 = f32(half[torch.from_numpy(sample).to(DEV)])
+    err16 = rel_l2(got16, want)
+    print(f"config 3 at full size, fp16 pair outputs: rel-L2 {err16:.2e}, max-abs {max_abs(got16, want):.3e}")
+    assert err16 <= TOL
+    small16, _ = run_chunk(ex, xd[idx].contiguous(), pd[idx].contiguous(), wd[idx].contiguous(), 64, torch.float16)
+    assert torch.equal(small16, half[idx])

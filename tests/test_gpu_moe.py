@@ -183,6 +183,11 @@ def test_config3_prefill_chunk_small():
     experts.down(act, ex, plan, y16, rows)
     assert torch.equal(y16, y.bfloat16())
     outs["y_bf16"] = moe.combine(y16.view(rows, -1, shape.hidden), wts.to(DEV))
+    # fp16 pair outputs: half the bytes as well, three more bits than bf16
+    yh = torch.empty((rows * picks.shape[1], shape.hidden), dtype=torch.float16, device=DEV)
+    experts.down(act, ex, plan, yh, rows)
+    assert torch.equal(yh, y.half())
+    outs["y_f16"] = moe.combine(yh.view(rows, -1, shape.hidden), wts.to(DEV))
     sample = list(range(0, rows, 37))
     want_bits = native.moe_layer(bits16(x[sample]), picks[sample].numpy(), wts[sample].numpy(),
                                  (u32(up[0][0]), bits16(up[0][1]), bits16(up[0][2])),
@@ -195,6 +200,9 @@ def test_config3_prefill_chunk_small():
     err16 = rel_l2(f32(outs["y_bf16"][sample]), want)
     print(f"config 3 (small, bf16 pair outputs): rel-L2 {err16:.2e}, max-abs {max_abs(f32(outs['y_bf16'][sample]), want):.3e}")
     assert err16 <= 2 * TOL          # measured 2.7e-3: over the bound, which is why fp32 pair outputs are this build's default
+    errh = rel_l2(f32(outs["y_f16"][sample]), want)
+    print(f"config 3 (small, fp16 pair outputs): rel-L2 {errh:.2e}, max-abs {max_abs(f32(outs['y_f16'][sample]), want):.3e}")
+    assert errh <= TOL
 
 
 def test_moe_run_rows_do_not_depend_on_the_window():
@@ -214,6 +222,41 @@ def test_moe_run_rows_do_not_depend_on_the_window():
     for r in (0, 7):
         assert torch.equal(moe.run(x[r:r + 1], layer, prefill=True)[0], whole_p[r]), r
     assert rel_l2(f32(whole_p), f32(whole)) < 1e-2
+
+
+def test_a_prompts_pair_outputs_in_fp16():
+    """``run`` keeps a prompt's pair outputs in fp16 for a layer on the fp16 prompt arithmetic and in fp32 for one
+    made with ARITH_BF16; fp16 pair outputs are the fp32 ones rounded once, those beyond fp16's range stored as
+    +-65504; decode buffers take fp32 only."""
+
+    shape = synthetic.MoEShape("small", 512, 16, 128, 4, 32, True, True)
+    up, down = layer_tables(shape, 7, 16)
+    tables = [tuple(t.to(DEV) for t in m) for m in up], tuple(t.to(DEV) for t in down)
+    rr = (torch.randn((17, 512), generator=torch.Generator().manual_seed(3)) * 0.05).bfloat16().to(DEV)
+    x = synthetic.activations(40, 512, 9).to(DEV)
+    kept = {}
+    for arith in (experts.ARITH_F16, experts.ARITH_BF16):
+        layer = moe.Routed(rr, experts.make(*tables, 32, arith=arith), 4)
+        out = moe.run(x, layer, prefill=True)
+        kept[arith] = {b.y.dtype for key, b in moe._pool.items() if key[6] and key[0] == 64 and key[3] == 128}
+        buf = moe.MoEBuffers(40, moe._Dims(layer), DEV, prefill=True)            # fp32 pair outputs, by hand
+        moe.moe(x, layer.router, layer.experts, buf, 4, 16)
+        assert rel_l2(f32(out), f32(moe.combine(buf.y, buf.wts))) < 1.5e-3
+    assert torch.float16 in kept[experts.ARITH_F16] and torch.float32 in kept[experts.ARITH_BF16]
+    with pytest.raises(ValueError):
+        moe.MoEBuffers(8, moe._Dims(layer), DEV, y_dtype=torch.float16)
+
+    # 64 inputs of 1e4 against weights of 1.5 (code 15, scale 0.1, bias 0): 9.6e5 a pair output
+    ones = lambda n, k: (torch.full((1, n, k // 8), -1, dtype=torch.int32), torch.full((1, n, k // 32), 0.1).bfloat16(),
+                         torch.zeros((1, n, k // 32)).bfloat16())
+    ex = experts.make([tuple(t.to(DEV) for t in ones(64, 64))], tuple(t.to(DEV) for t in ones(64, 64)), 32)
+    plan = experts.Plan(2, 1, 1, DEV, prefill=True)
+    experts.route(torch.zeros((2, 1), dtype=torch.int32, device=DEV), plan, 64)
+    act = torch.tensor([[1e4] * 64, [-2.0] * 64], device=DEV).bfloat16()
+    y32, y16 = torch.empty((2, 64), device=DEV), torch.empty((2, 64), device=DEV, dtype=torch.float16)
+    experts.down(act, ex, plan, y32, 2)
+    experts.down(act, ex, plan, y16, 2)
+    assert float(y32[0, 0]) > 9e5 and torch.all(y16[0] == 65504) and torch.equal(y16[1], y32[1].half())
 
 
 @pytest.mark.parametrize("shape,ne,rows", [(synthetic.C1, 24, 1), (synthetic.C1, 24, 8), (synthetic.C2, 48, 32),
