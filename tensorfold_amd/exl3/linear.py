@@ -196,10 +196,10 @@ class Exl3Stack:
         """A copy of the layers' tensors in one piece (drop the layers afterwards to give their memory back)."""
 
         first = layers[0]
-        same = lambda l: (l.k, l.n, l.bits, l.codebook, l.layout, l.words.shape) == \
-            (first.k, first.n, first.bits, first.codebook, first.layout, first.words.shape)
+        same = lambda l: (l.k, l.n, l.bits, l.codebook, l.layout, l.words.shape, tuple(l.split)) == \
+            (first.k, first.n, first.bits, first.codebook, first.layout, first.words.shape, tuple(first.split))
         if not 1 <= len(layers) <= 64 or not all(same(l) for l in layers):
-            raise ValueError("a stack takes 1 to 64 layers of one shape, width, codebook and layout")
+            raise ValueError("a stack takes 1 to 64 layers of one shape, width, codebook, layout and K split")
         bias = None
         if any(l.bias is not None for l in layers):
             bias = torch.stack([l.bias if l.bias is not None else torch.zeros_like(first.svh) for l in layers])
