@@ -81,11 +81,13 @@ int tf_qmm_static(const uint16_t* x, int64_t ldx, const float* xs, const uint32_
 /* `count` (1 to 4) weights against one x in one launch (plus one reduce launch when any K is split and the rows are
  * many): the bits of tf_qmm on each.  The arrays are host arrays of `count` entries, read during the call: packed weights, transposed
  * scales and biases with their row strides, outputs, parts (fp32 [sks[i], m, ns[i]], may be NULL where sks[i] == 1),
- * column counts and slice counts.  Replaces kernels/qmm.cpp:51-80 `qmm_group`. */
+ * column counts and slice counts; `counters` (may be NULL) the weights' arrival counters with their counts, as in
+ * tf_qmm: with them up to eight rows take one launch in which every weight's slices are added up by the last
+ * workgroup of a tile.  Replaces kernels/qmm.cpp:51-80 `qmm_group`. */
 int tf_qmm_group(const uint16_t* x, int64_t ldx, const float* xs, int count, const uint32_t* const* weights,
                  const uint16_t* const* scales, const uint16_t* const* biases, const int64_t* sb_strides,
-                 void* const* outs, float* const* parts, const int* ns, const int* sks, int m, int k, int gs, int bm,
-                 int f32, tf_stream_t stream);
+                 void* const* outs, float* const* parts, int32_t* const* counters, const int* n_counters, const int* ns,
+                 const int* sks, int m, int k, int gs, int bm, int f32, tf_stream_t stream);
 /* The arithmetic of the prompt-form (MFMA) matmuls.
  *   TF_ARITH_F16: operands in fp16 - each weight rounded once as fp16(256 w), activations converted to fp16 (exact for a
  *     bf16 value between 2^-14 and 65504 in magnitude; larger ones are clamped to +-65504, smaller ones keep 2^-24

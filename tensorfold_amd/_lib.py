@@ -21,7 +21,7 @@ PROTOTYPES = {
     "tf_group_sums": [P, L, I, I, I, P, P],
     "tf_qmm": [P, L, P, P, P, P, L, P, P, P, I, I, I, I, I, I, I, I, I, P],
     "tf_qmm_static": [P, L, P, P, P, P, L, P, I, I, I, I, I, I, I, P],
-    "tf_qmm_group": [P, L, P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, P],
+    "tf_qmm_group": [P, L, P, I, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, P],
     "tf_qmm_prefill": [P, L, P, P, P, P, I, I, I, I, I, I, I, P],
     "tf_quantize_rows": [P, L, I, I, I, P, P, P, P],
     "tf_qmm_prefill8": [P, P, P, P, P, P, P, I, I, I, I, I, I, P],

@@ -182,23 +182,19 @@ __global__ void __launch_bounds__(WAVES * 64)
 // counter; the workgroup that finds the others there adds the slices in slice order (qmm_reduce_kernel's arithmetic)
 // and puts the counter back to zero.  A thousand short workgroups fill the chip where the one-launch form above has
 // one workgroup a column tile.
-template <int GS, int WAVES>
-__global__ void __launch_bounds__(WAVES * 64)
-    qmm_arrive_kernel(const uint16_t* __restrict__ X, int64_t ldx, const float* __restrict__ XS,
-                      const uint32_t* __restrict__ W, const uint16_t* __restrict__ S, const uint16_t* __restrict__ B,
-                      int64_t sb_stride, void* __restrict__ out, float* __restrict__ part_out, int* __restrict__ counters,
-                      int M, int N, int KG, int SK, int BM, int f32) {
-  extern __shared__ float lds[];
-  __shared__ int last;
-  qmm_block<GS, WAVES, true>(X, ldx, XS, W, S, B, sb_stride, out, part_out, M, N, KG, SK, BM, f32, blockIdx.x, blockIdx.z, lds);
+// What a slice's workgroup does once its sums are in part[z] (stored through to memory): wait for the stores'
+// acknowledgement, count itself in at the tile's counter, and if every other slice is there already add them up.
+template <int WAVES>
+__device__ __forceinline__ void qmm_arrive_tail(int* __restrict__ counter, const float* __restrict__ part_out,
+                                                void* __restrict__ out, int M, int N, int SK, int BM, int f32, int block,
+                                                int* last) {
   __builtin_amdgcn_s_waitcnt(0);        // this wave's stores are acknowledged ...
   __syncthreads();                      // ... every wave's are ...
-  int* counter = counters + (size_t)blockIdx.x * TF_QMM_COUNTER_STRIDE;
   if (threadIdx.x == 0)                 // ... then the workgroup counts itself in
-    last = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == SK - 1;
+    *last = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == SK - 1;
   __syncthreads();
-  if (!last) return;
-  const int tiles = (N + 63) >> 6, tile = blockIdx.x % tiles, rt = blockIdx.x / tiles;
+  if (!*last) return;
+  const int tiles = (N + 63) >> 6, tile = block % tiles, rt = block / tiles;
   const int r_first = rt * BM, rows = min(M, r_first + BM) - r_first;
   const long long total = (long long)M * N;
   for (int o = threadIdx.x; o < rows * 64; o += WAVES * 64) {
@@ -221,6 +217,19 @@ __global__ void __launch_bounds__(WAVES * 64)
     else reinterpret_cast<uint16_t*>(out)[at] = (uint16_t)f32_bf16_bits(acc);
   }
   if (threadIdx.x == 0) *counter = 0;   // every slice of the tile has arrived: ready for the next call
+}
+
+template <int GS, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64)
+    qmm_arrive_kernel(const uint16_t* __restrict__ X, int64_t ldx, const float* __restrict__ XS,
+                      const uint32_t* __restrict__ W, const uint16_t* __restrict__ S, const uint16_t* __restrict__ B,
+                      int64_t sb_stride, void* __restrict__ out, float* __restrict__ part_out, int* __restrict__ counters,
+                      int M, int N, int KG, int SK, int BM, int f32) {
+  extern __shared__ float lds[];
+  __shared__ int last;
+  qmm_block<GS, WAVES, true>(X, ldx, XS, W, S, B, sb_stride, out, part_out, M, N, KG, SK, BM, f32, blockIdx.x, blockIdx.z, lds);
+  qmm_arrive_tail<WAVES>(counters + (size_t)blockIdx.x * TF_QMM_COUNTER_STRIDE, part_out, out, M, N, SK, BM, f32,
+                         blockIdx.x, &last);
 }
 
 // The split matmul and its reduce in ONE launch, with no traffic between workgroups: a workgroup of FW waves takes a
@@ -338,6 +347,7 @@ struct GroupArgs {
   const uint16_t* b[GROUP_MAX];
   void* out[GROUP_MAX];
   float* part[GROUP_MAX];
+  int* counters[GROUP_MAX];      // arrival counters of a weight (the arriving form), else unused
   int64_t sb_stride[GROUP_MAX];
   int n[GROUP_MAX], sk[GROUP_MAX];
   int first[GROUP_MAX + 1];      // workgroups (matmul) or 256-element chunks (reduce) before weight w
@@ -359,6 +369,27 @@ __global__ void __launch_bounds__(WAVES * 64)
 }
 
 // The grouped launch in the one-launch form (see qmm_fat_block): every weight's K split is 4, 8 or 16.
+// the grouped launch whose slices are added up by the last workgroup of a tile to finish (qmm_arrive_kernel's way);
+// a weight whose K is not split stores its rows itself
+template <int GS, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64)
+    qmm_group_arrive_kernel(const uint16_t* __restrict__ X, int64_t ldx, const float* __restrict__ XS, GroupArgs a, int M,
+                            int KG, int BM, int f32) {
+  extern __shared__ float lds[];
+  __shared__ int last;
+  int w = 0;
+#pragma unroll
+  for (int i = 1; i < GROUP_MAX; ++i)
+    if (i < a.count && (int)blockIdx.x >= a.first[i]) w = i;
+  if ((int)blockIdx.z >= a.sk[w]) return;
+  const int block = blockIdx.x - a.first[w];
+  qmm_block<GS, WAVES, true>(X, ldx, XS, a.w[w], a.s[w], a.b[w], a.sb_stride[w], a.out[w], a.part[w], M, a.n[w], KG,
+                             a.sk[w], BM, f32, block, blockIdx.z, lds);
+  if (a.sk[w] > 1)
+    qmm_arrive_tail<WAVES>(a.counters[w] + (size_t)block * TF_QMM_COUNTER_STRIDE, a.part[w], a.out[w], M, a.n[w],
+                           a.sk[w], BM, f32, block, &last);
+}
+
 template <int GS>
 __global__ void __launch_bounds__(1024)
     qmm_group_fat_kernel(const uint16_t* __restrict__ X, int64_t ldx, const float* __restrict__ XS, GroupArgs a, int M,
@@ -656,20 +687,25 @@ extern "C" int tf_qmm_static(const uint16_t* x, int64_t ldx, const float* xs, co
 
 extern "C" int tf_qmm_group(const uint16_t* x, int64_t ldx, const float* xs, int count, const uint32_t* const* weights,
                             const uint16_t* const* scales, const uint16_t* const* biases, const int64_t* sb_strides,
-                            void* const* outs, float* const* parts, const int* ns, const int* sks, int m, int k, int gs,
-                            int bm, int f32, tf_stream_t stream) {
+                            void* const* outs, float* const* parts, int32_t* const* counters, const int* n_counters,
+                            const int* ns, const int* sks, int m, int k, int gs, int bm, int f32, tf_stream_t stream) {
   clear_error();
   TF_REQUIRE(gs == 32 || gs == 64, "groups of 32 or 64");
   TF_REQUIRE(bm == 16 || bm == 32 || bm == 64, "row tile 16, 32 or 64");
   TF_REQUIRE(count >= 1 && count <= GROUP_MAX, "qmm_group: 1 to %d weights, not %d", GROUP_MAX, count);
+  TF_REQUIRE(!counters || n_counters, "qmm_group: counters come with their counts");
   TF_REQUIRE(x && xs && weights && scales && biases && sb_strides && outs && parts && ns && sks && m >= 1,
              "qmm_group: null pointer or empty shape");
   TF_REQUIRE(aligned16(x) && (m == 1 || ldx % 8 == 0), "x rows must start on 16-byte boundaries");
   TF_REQUIRE(ldx >= k || m == 1, "x: (M, K) bf16 with contiguous rows");
   TF_REQUIRE(k % gs == 0, "K splits into whole groups a slice");
   const int kg = k / gs;
+  // one pass of rows and every split weight's arrival counters: the arriving form, as tf_qmm
+  bool arrive = counters && m <= ARRIVE_ROWS;
+  for (int i = 0; i < count && arrive; ++i)
+    arrive = ns && sks && (sks[i] == 1 || (counters[i] && (ns[i] + 63) / 64 * ((m + bm - 1) / bm) <= n_counters[i]));
   // few rows and every K split 4, 8 or 16: the one-launch form (two rows a workgroup), as tf_qmm
-  bool fat = m <= FAT_ROWS;
+  bool fat = !arrive && m <= FAT_ROWS;
   int64_t fat_blocks = 0;
   for (int i = 0; i < count && fat; ++i) {
     fat = ns && sks && ns[i] >= 1 && (sks[i] == 4 || sks[i] == 8 || sks[i] == 16);
@@ -694,6 +730,7 @@ extern "C" int tf_qmm_group(const uint16_t* x, int64_t ldx, const float* xs, int
     a.b[i] = biases[i];
     a.out[i] = outs[i];
     a.part[i] = parts[i];
+    a.counters[i] = arrive ? counters[i] : nullptr;
     a.sb_stride[i] = sb_strides[i];
     a.n[i] = n;
     a.sk[i] = sk;
@@ -717,6 +754,12 @@ extern "C" int tf_qmm_group(const uint16_t* x, int64_t ldx, const float* xs, int
   }
   const size_t smem = sizeof(float) * ((size_t)QMM_WAVES * QRB * 64);
   const dim3 grid((unsigned)blocks, 1, (unsigned)max_sk);
+  if (arrive) {
+    if (gs == 64) qmm_group_arrive_kernel<64, QMM_WAVES><<<grid, QMM_WAVES * 64, smem, s>>>(x, ldx, xs, a, m, kg, bm, f32);
+    else qmm_group_arrive_kernel<32, QMM_WAVES><<<grid, QMM_WAVES * 64, smem, s>>>(x, ldx, xs, a, m, kg, bm, f32);
+    TF_LAUNCH_OK("tf_qmm_group");
+    return 0;
+  }
   if (gs == 64) qmm_group_kernel<64, QMM_WAVES><<<grid, QMM_WAVES * 64, smem, s>>>(x, ldx, xs, a, m, kg, bm, f32);
   else qmm_group_kernel<32, QMM_WAVES><<<grid, QMM_WAVES * 64, smem, s>>>(x, ldx, xs, a, m, kg, bm, f32);
   TF_LAUNCH_OK("tf_qmm_group");

@@ -269,9 +269,11 @@ def matmul_group(x: torch.Tensor, qs: list[Q4], xs: torch.Tensor | None = None, 
             raise ValueError(f"matmul_group: parts[{i}] must hold {sk} x {m} x {q.n} fp32 values")
     n = len(qs)
     ptrs = lambda ts: (ctypes.c_void_p * n)(*[None if t is None else t.data_ptr() for t in ts])
+    counters = [q.counters if sk > 1 and m <= 8 else None for q, sk in zip(qs, sks)]
     _lib.call("tf_qmm_group", _lib.ptr(x), x.stride(0), _lib.ptr(xs), n, ptrs([q.weight for q in qs]),
               ptrs([q.scales for q in qs]), ptrs([q.biases for q in qs]),
-              (ctypes.c_int64 * n)(*[q.scales.stride(0) for q in qs]), ptrs(outs), ptrs(parts),
+              (ctypes.c_int64 * n)(*[q.scales.stride(0) for q in qs]), ptrs(outs), ptrs(parts), ptrs(counters),
+              (ctypes.c_int * n)(*[0 if c is None else c.numel() // COUNTER_STRIDE for c in counters]),
               (ctypes.c_int * n)(*[q.n for q in qs]), (ctypes.c_int * n)(*sks), m, k, gs, bucket(m), int(f32))
     return outs
 
