@@ -72,9 +72,13 @@ int tf_qmm(const uint16_t* x, int64_t ldx, const float* xs, const uint32_t* weig
  * until the process ends); sk * m * n beyond that is refused with a message.  Nothing is allocated or freed by the
  * call.  Same kernels and bits as tf_qmm.  Every call on a GPU shares that GPU's array: calls that overlap on one
  * GPU (two streams, two threads) race; calls on one stream are ordered.  Nothing in the array needs to start at
- * zero (each slice is written in full before the reduce reads it).  No counterpart in the reference, whose `qmm`
- * allocates `part` itself when none is given (kernels/qmm.cpp:40-45). */
+ * zero (each slice is written in full before it is read).  The arrival counters that let up to eight rows finish in
+ * one launch live in the device image too (TF_QMM_STATIC_COUNTERS of them, 256 KiB; zero when the image is loaded,
+ * put back to zero by every launch; a weight of more column tiles of 64 than that takes tf_qmm's counter-less
+ * forms).  No counterpart in the reference, whose `qmm` allocates `part` itself when none is given
+ * (kernels/qmm.cpp:40-45). */
 #define TF_QMM_STATIC_FLOATS (4u << 20)
+#define TF_QMM_STATIC_COUNTERS 4096
 int tf_qmm_static(const uint16_t* x, int64_t ldx, const float* xs, const uint32_t* weight, const uint16_t* scales,
                   const uint16_t* biases, int64_t sb_stride, void* out, int m, int n, int k, int sk, int gs, int bm,
                   int f32, tf_stream_t stream);

@@ -648,27 +648,35 @@ extern "C" int tf_qmm(const uint16_t* x, int64_t ldx, const float* xs, const uin
 // Host code may not use the array's name as an address; it asks the runtime once a device for where that device
 // holds its copy and passes that pointer to the kernels like any other buffer.
 static __device__ __align__(256) float scratch[TF_QMM_STATIC_FLOATS];
+// the arrival counters of the column tiles, zero when the image is loaded and put back to zero by every launch
+static __device__ __align__(256) int scratch_counters[TF_QMM_STATIC_COUNTERS * TF_QMM_COUNTER_STRIDE];
 
-static float* static_part() {
+// where the current device holds the two arrays (asked once a device)
+static bool static_scratch(float** part, int32_t** counters) {
   constexpr int MAX_DEVICES = 64;
   static float* where[MAX_DEVICES];
+  static int32_t* where_counters[MAX_DEVICES];
   static std::mutex guard;
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
     set_error("tf_qmm_static: no current HIP device (or its index is %d or more)", MAX_DEVICES);
-    return nullptr;
+    return false;
   }
   std::lock_guard<std::mutex> lock(guard);
   if (!where[dev]) {
-    void* p = nullptr;
-    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-    if (e != hipSuccess || !p) {
+    void *p = nullptr, *c = nullptr;
+    hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e == hipSuccess) e = hipGetSymbolAddress(&c, HIP_SYMBOL(scratch_counters));
+    if (e != hipSuccess || !p || !c) {
       set_error("tf_qmm_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
-      return nullptr;
+      return false;
     }
     where[dev] = static_cast<float*>(p);
+    where_counters[dev] = static_cast<int32_t*>(c);
   }
-  return where[dev];
+  *part = where[dev];
+  *counters = where_counters[dev];
+  return true;
 }
 
 extern "C" int tf_qmm_static(const uint16_t* x, int64_t ldx, const float* xs, const uint32_t* weight,
@@ -680,9 +688,10 @@ extern "C" int tf_qmm_static(const uint16_t* x, int64_t ldx, const float* xs, co
              "tf_qmm_static: %d slices x %d rows x %d columns = %lld fp32 partial sums exceed the built-in %lld; use "
              "tf_qmm with a part buffer", sk, m, n, (long long)sk * m * n, (long long)TF_QMM_STATIC_FLOATS);
   float* part = nullptr;
-  if (sk > 1 && !(part = static_part())) return 1;
-  return qmm_launch(x, ldx, xs, weight, scales, biases, sb_stride, out, part, nullptr, 0, m, n, k, sk, gs, bm, f32, 1,
-                    stream);
+  int32_t* counters = nullptr;
+  if (sk > 1 && !static_scratch(&part, &counters)) return 1;
+  return qmm_launch(x, ldx, xs, weight, scales, biases, sb_stride, out, part, counters, TF_QMM_STATIC_COUNTERS, m, n, k,
+                    sk, gs, bm, f32, 1, stream);
 }
 
 extern "C" int tf_qmm_group(const uint16_t* x, int64_t ldx, const float* xs, int count, const uint32_t* const* weights,
