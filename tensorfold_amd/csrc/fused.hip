@@ -503,7 +503,7 @@ extern "C" int tf_moe_down_combine(int gs, const uint16_t* act, int rows, int sl
   down_combine_kernel<GS_, W_><<<g, W_ * 64, smem, s>>>(act, slots, down, d, ni, desc, wts, y, out, arrive, \
                                                         arrive_stride(rows))
 #define TF_GS(GS_)                      \
-  switch (fused_waves(grid + grid / 2)) {      \
+  switch (fused_waves(grid)) {                 \
     case 16: TF_GO(GS_, 16); break;     \
     case 8: TF_GO(GS_, 8); break;       \
     default: TF_GO(GS_, 4);             \
