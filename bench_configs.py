@@ -337,8 +337,8 @@ def c4x() -> dict:
         nbytes = distinct * (3 * d * width // 2 + 2 * (3 * d + 3 * width)) + rows * d * 6
         out[rows] = {"layer_us": us, "distinct_experts": distinct, "bytes": nbytes, "gbs": nbytes / us * 1e-3,
                      "frac": nbytes / us * 1e-3 / HBM}
-    return {"config": "c4x: EXL3 routed experts at decode, 288 experts 4096 -> 2048 -> 4096, 4.0 bpw mcg, top-8 (group, "
-                      "rotation, gate/up, SwiGLU epilogue, down, rotation + combine: six launches)",
+    return {"config": "c4x: EXL3 routed experts at decode, 288 experts 4096 -> 2048 -> 4096, 4.0 bpw mcg, top-8 (grouping + "
+                      "rotation, gate/up, SwiGLU epilogue, down, rotation + combine: five launches)",
             "bound": "hbm", "rows": out}
 
 
@@ -424,7 +424,7 @@ def timeline() -> dict:
                 g.replay()
                 g.replay()
                 torch.cuda.synchronize()
-                h = np.zeros((len(marks) + 1, 4096), dtype=np.uint64)
+                h = np.zeros((len(marks) + 1, 16384), dtype=np.uint64)
                 if tl.tf_timeline_read_moe(h.ctypes.data_as(ctypes.c_void_p), h.shape[0], h.shape[1]):
                     raise RuntimeError(tl.tf_last_error().decode())
                 where = h[len(marks)]
@@ -487,7 +487,7 @@ def timeline() -> dict:
             g.replay()
             g.replay()
             torch.cuda.synchronize()
-            h = np.zeros((len(names) + 1, 4096), dtype=np.uint64)
+            h = np.zeros((len(names) + 1, 16384), dtype=np.uint64)
             if tl.tf_timeline_read_exl3(h.ctypes.data_as(ctypes.c_void_p), h.shape[0], h.shape[1]):
                 raise RuntimeError(tl.tf_last_error().decode())
         where = h[len(names)]

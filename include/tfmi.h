@@ -313,6 +313,13 @@ int tf_exl3x_gateup_epilogue(const float* z, const int32_t* pick, const uint16_t
 int tf_exl3x_down_combine(const float* z, const int32_t* pick, const uint16_t* svh_d, float* y, const float* wts,
                           float* out, int rows, int slots, int d, int sk, int experts, tf_stream_t stream);
 
+/* tf_experts_plan (tile 16, at most 1,024 pairs) and tf_exl3x_rot_in in one launch: workgroup 0 groups the pairs,
+ * the others rotate them (neither needs the other's result).  Replaces experts.py:173-185 (the pair sort and
+ * experts.cpp `rot_in`). */
+int tf_exl3x_plan_rot_in(const void* x, int x_dtype, int64_t x_stride, const int32_t* pick, const uint16_t* suh0,
+                         const uint16_t* suh1, uint16_t* out0, uint16_t* out1, int rows, int slots, int k, int experts,
+                         int tile, int32_t* members, int32_t* items, int32_t* counts, tf_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -42,6 +42,7 @@ PROTOTYPES = {
     "tf_exl3x_grouped": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
     "tf_exl3x_gateup_epilogue": [P, P, P, P, P, P, I, I, I, I, F, I, P],
     "tf_exl3x_down_combine": [P, P, P, P, P, P, I, I, I, I, I, P],
+    "tf_exl3x_plan_rot_in": [P, I, L, P, P, P, P, P, I, I, I, I, I, P, P, P, P],
     "tf_add_norm": [P, P, I, P, I, I, P, F, P, P, P, I, I, I, P],
     "tf_exl3_rot_in": [P, I, P, P, I, I, P],
     "tf_exl3_linear": [P, P, L, L, P, P, P, I, P, P, I, I, I, I, I, I, I, P],

@@ -7,8 +7,12 @@
 // trellis at the expert's own width, its rows gathered through `members`.  K splits write fp32 partials that the
 // epilogues add in split order; every butterfly and sum runs in a fixed order and no row reads another row, so a
 // row's bits do not depend on the window it arrives in.
+//
+// tf_exl3x_plan_rot_in puts the grouping and the input rotation into one launch (workgroup 0 groups, the others
+// rotate; neither needs the other's result).
 
 #include "exl3_decode.h"
+#include "routing.h"
 
 namespace tf {
 namespace {
@@ -34,6 +38,36 @@ __global__ void __launch_bounds__(256)
   store2(mat ? out1 : out0, TF_F16, (size_t)p * K + k, a * HAD_SCALE, b * HAD_SCALE);
 }
 
+// The grouping and the input rotation in one launch: workgroup 0 makes the plan (tf_experts_plan's, up to 1,024
+// pairs), every other workgroup rotates sixteen (matrix, pair, block of 128) units as x_rot_in_kernel does.
+__global__ void __launch_bounds__(PLAN_THREADS)
+    plan_rot_in_kernel(const void* __restrict__ x, int x_dtype, int64_t x_stride, const int* __restrict__ pick,
+                       const uint16_t* __restrict__ suh0, const uint16_t* __restrict__ suh1,
+                       uint16_t* __restrict__ out0, uint16_t* __restrict__ out1, int K, int slots, int E, int P, int T,
+                       int* __restrict__ members, int* __restrict__ items, int* __restrict__ counts) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (blockIdx.x == 0) {
+    __shared__ int pk[PLAN_THREADS];
+    __shared__ PlanLds plan;
+    plan_small(pick, P, E, T, members, items, counts, pk, plan);
+    return;
+  }
+  const int KB = K / 128, unit = (blockIdx.x - 1) * (PLAN_THREADS / 64) + wave;
+  const int mats = suh1 ? 2 : 1;
+  if (unit >= P * KB * mats) return;
+  const int mat = unit / (P * KB), rest = unit - mat * (P * KB), p = rest / KB, blk = rest - p * KB;
+  const int e = pick[p];
+  if (e < 0 || e >= E) return;
+  const int k = blk * 128 + 2 * lane;
+  float a, b, sa, sb;
+  load2(x, x_dtype, (size_t)(p / slots) * x_stride + k, a, b);
+  load2(mat ? suh1 : suh0, TF_F16, (size_t)e * K + k, sa, sb);
+  a *= sa;
+  b *= sb;
+  fwht128(a, b, lane);
+  store2(mat ? out1 : out0, TF_F16, (size_t)p * K + k, a * HAD_SCALE, b * HAD_SCALE);
+}
+
 struct GroupedArgs {
   const uint16_t* x[2];        // rotated inputs fp16 [P, K] of matrix 0 and 1
   const int64_t* tp[2];        // each expert's trellis address
@@ -44,6 +78,69 @@ struct GroupedArgs {
   float* Z;                    // [mats * SK, P, N] partial sums
   int mats, K, N, P, SK, E;
 };
+
+// the sum over K splits, in split order, of the two columns of pair p that lane holds
+__device__ __forceinline__ float2 split_sum(const float* z, size_t split_stride, int SK) {
+  float2 s = {0.f, 0.f};
+  for (int q0 = 0; q0 < SK; q0 += 8) {
+    float2 v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = *reinterpret_cast<const float2*>(z + (size_t)(q0 + j < SK ? q0 + j : SK - 1) * split_stride);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (q0 + j < SK) {
+        s.x += v[j].x;
+        s.y += v[j].y;
+      }
+  }
+  return s;
+}
+
+__device__ __forceinline__ float half_f32(uint16_t v) { return __half2float(__ushort_as_half(v)); }
+
+// Pair p's block of 128 of the width after gate and up (a wave; n = the lane's first column): splits summed, rotated,
+// * svh, SwiGLU (act_mode 0: bf16 roundings; 1: fp32), then xd = fp16(((act * suh_d) H) / sqrt(128))
+__device__ __forceinline__ void gateup_row(const float* __restrict__ Z, int p, int e, int n, int lane,
+                                           const uint16_t* __restrict__ svh_g, const uint16_t* __restrict__ svh_u,
+                                           const uint16_t* __restrict__ suh_d, uint16_t* __restrict__ xd, int P, int N,
+                                           int SK, float limit, int act_mode) {
+  const size_t ss = (size_t)P * N;
+  float2 gv = split_sum(Z + (size_t)p * N + n, ss, SK);
+  float2 uv = split_sum(Z + (size_t)SK * ss + (size_t)p * N + n, ss, SK);
+  fwht128(gv.x, gv.y, lane);
+  fwht128(uv.x, uv.y, lane);
+  const uint32_t sg = *reinterpret_cast<const uint32_t*>(svh_g + (size_t)e * N + n);
+  const uint32_t su = *reinterpret_cast<const uint32_t*>(svh_u + (size_t)e * N + n);
+  const uint32_t sd = *reinterpret_cast<const uint32_t*>(suh_d + (size_t)e * N + n);
+  const float g2[2] = {gv.x, gv.y}, u2[2] = {uv.x, uv.y};
+  float v[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const float wg = half_f32((uint16_t)(sg >> (16 * j))), wu = half_f32((uint16_t)(su >> (16 * j)));
+    float act;
+    if (act_mode == 0) {
+      const float gg = fminf(round_bf16(g2[j] * HAD_SCALE * wg), limit);
+      const float uu = fminf(fmaxf(round_bf16(u2[j] * HAD_SCALE * wu), -limit), limit);
+      act = round_bf16(round_bf16(gg / (1.f + expf(-gg))) * uu);
+    } else {
+      const float gg = fminf(g2[j] * HAD_SCALE * wg, limit);
+      const float uu = fminf(fmaxf(u2[j] * HAD_SCALE * wu, -limit), limit);
+      act = gg / (1.f + expf(-gg)) * uu;
+    }
+    v[j] = act * half_f32((uint16_t)(sd >> (16 * j)));
+  }
+  fwht128(v[0], v[1], lane);
+  store2(xd, TF_F16, (size_t)p * N + n, v[0] * HAD_SCALE, v[1] * HAD_SCALE);
+}
+
+// Pair p's block of 128 of the output after down (a wave): ((splits summed) H / sqrt(128)) * svh_d
+__device__ __forceinline__ float2 down_row(const float* __restrict__ Z, int p, int e, int n, int lane,
+                                           const uint16_t* __restrict__ svh_d, int P, int D, int SK) {
+  float2 v = split_sum(Z + (size_t)p * D + n, (size_t)P * D, SK);
+  fwht128(v.x, v.y, lane);
+  const uint32_t sv = *reinterpret_cast<const uint32_t*>(svh_d + (size_t)e * D + n);
+  return make_float2(v.x * HAD_SCALE * half_f32((uint16_t)sv), v.y * HAD_SCALE * half_f32((uint16_t)(sv >> 16)));
+}
 
 // One item, one 128-column block, one K split, one matrix: the dense linear's pass with gathered rows.
 template <int K2, int CB>
@@ -108,24 +205,6 @@ __global__ void __launch_bounds__(XWK * 64) grouped_kernel(const GroupedArgs g) 
   }
 }
 
-// the sum over K splits, in split order, of the two columns of pair p that lane holds
-__device__ __forceinline__ float2 split_sum(const float* z, size_t split_stride, int SK) {
-  float2 s = {0.f, 0.f};
-  for (int q0 = 0; q0 < SK; q0 += 8) {
-    float2 v[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = *reinterpret_cast<const float2*>(z + (size_t)(q0 + j < SK ? q0 + j : SK - 1) * split_stride);
-#pragma unroll
-    for (int j = 0; j < 8; ++j)
-      if (q0 + j < SK) {
-        s.x += v[j].x;
-        s.y += v[j].y;
-      }
-  }
-  return s;
-}
-
-__device__ __forceinline__ float half_f32(uint16_t v) { return __half2float(__ushort_as_half(v)); }
 
 // a wave a (pair, block of 128 of the width): splits summed, rotated, * svh, SwiGLU (act_mode 0: bf16 roundings;
 // 1: fp32), then xd = fp16(((act * suh_d) H) / sqrt(128))
@@ -137,34 +216,7 @@ __global__ void __launch_bounds__(256)
   if (blk * 128 >= N) return;
   const int e = pick[p];
   if (e < 0 || e >= E) return;
-  const int n = blk * 128 + 2 * lane;
-  const size_t ss = (size_t)P * N;
-  float2 gv = split_sum(Z + (size_t)p * N + n, ss, SK);
-  float2 uv = split_sum(Z + (size_t)SK * ss + (size_t)p * N + n, ss, SK);
-  fwht128(gv.x, gv.y, lane);
-  fwht128(uv.x, uv.y, lane);
-  const uint32_t sg = *reinterpret_cast<const uint32_t*>(svh_g + (size_t)e * N + n);
-  const uint32_t su = *reinterpret_cast<const uint32_t*>(svh_u + (size_t)e * N + n);
-  const uint32_t sd = *reinterpret_cast<const uint32_t*>(suh_d + (size_t)e * N + n);
-  const float g2[2] = {gv.x, gv.y}, u2[2] = {uv.x, uv.y};
-  float v[2];
-#pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const float wg = half_f32((uint16_t)(sg >> (16 * j))), wu = half_f32((uint16_t)(su >> (16 * j)));
-    float act;
-    if (act_mode == 0) {
-      const float gg = fminf(round_bf16(g2[j] * HAD_SCALE * wg), limit);
-      const float uu = fminf(fmaxf(round_bf16(u2[j] * HAD_SCALE * wu), -limit), limit);
-      act = round_bf16(round_bf16(gg / (1.f + expf(-gg))) * uu);
-    } else {
-      const float gg = fminf(g2[j] * HAD_SCALE * wg, limit);
-      const float uu = fminf(fmaxf(u2[j] * HAD_SCALE * wu, -limit), limit);
-      act = gg / (1.f + expf(-gg)) * uu;
-    }
-    v[j] = act * half_f32((uint16_t)(sd >> (16 * j)));
-  }
-  fwht128(v[0], v[1], lane);
-  store2(xd, TF_F16, (size_t)p * N + n, v[0] * HAD_SCALE, v[1] * HAD_SCALE);
+  gateup_row(Z, p, e, blk * 128 + 2 * lane, lane, svh_g, svh_u, suh_d, xd, P, N, SK, limit, act_mode);
 }
 
 // grid (D / 128, rows): y[p] = ((splits summed) H / sqrt(128)) * svh_d for the routed slots (the others keep what
@@ -181,11 +233,7 @@ __global__ void __launch_bounds__(256)
     const int e = pick[p];
     float2 o;
     if (e >= 0 && e < E) {
-      float2 v = split_sum(Z + (size_t)p * D + n, (size_t)P * D, SK);
-      fwht128(v.x, v.y, lane);
-      const uint32_t sv = *reinterpret_cast<const uint32_t*>(svh_d + (size_t)e * D + n);
-      o.x = v.x * HAD_SCALE * half_f32((uint16_t)sv);
-      o.y = v.y * HAD_SCALE * half_f32((uint16_t)(sv >> 16));
+      o = down_row(Z, p, e, n, lane, svh_d, P, D, SK);
       *reinterpret_cast<float2*>(y + (size_t)p * D + n) = o;
     } else if (wts) {
       o = *reinterpret_cast<const float2*>(y + (size_t)p * D + n);
@@ -255,6 +303,28 @@ extern "C" int tf_exl3x_grouped(const uint16_t* x0, const uint16_t* x1, const in
     return 1;
   }
   TF_LAUNCH_OK("tf_exl3x_grouped");
+  return 0;
+}
+
+extern "C" int tf_exl3x_plan_rot_in(const void* x, int x_dtype, int64_t x_stride, const int32_t* pick,
+                                    const uint16_t* suh0, const uint16_t* suh1, uint16_t* out0, uint16_t* out1, int rows,
+                                    int slots, int k, int experts, int tile, int32_t* members, int32_t* items,
+                                    int32_t* counts, tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(x && pick && suh0 && out0 && (!suh1 == !out1) && members && items && counts,
+             "exl3x plan_rot_in: null pointer argument");
+  TF_REQUIRE(x_dtype == TF_F16 || x_dtype == TF_BF16 || x_dtype == TF_F32, "x: expected fp16, bf16 or fp32");
+  TF_REQUIRE(rows >= 1 && slots >= 1 && (int64_t)rows * slots <= PLAN_THREADS, "exl3x plan_rot_in: at most %d pairs",
+             PLAN_THREADS);
+  TF_REQUIRE(experts >= 1 && experts <= EMAX, "experts: at most %d experts", EMAX);
+  TF_REQUIRE(tile == 16, "exl3x plan_rot_in: items hold 16 pairs");
+  TF_REQUIRE(k >= 128 && k % 128 == 0 && x_stride >= k && x_stride % 2 == 0, "x rows of K values, K a multiple of 128");
+  TF_REQUIRE(((uintptr_t)x & 7) == 0 && aligned16(out0) && aligned16(out1), "x 8-byte, outputs 16-byte aligned");
+  const int64_t units = (int64_t)rows * slots * (k / 128) * (suh1 ? 2 : 1);
+  const int per = PLAN_THREADS / 64;
+  plan_rot_in_kernel<<<dim3((unsigned)(1 + (units + per - 1) / per)), PLAN_THREADS, 0, as_stream(stream)>>>(
+      x, x_dtype, x_stride, pick, suh0, suh1, out0, out1, k, slots, experts, rows * slots, tile, members, items, counts);
+  TF_LAUNCH_OK("tf_exl3x_plan_rot_in");
   return 0;
 }
 

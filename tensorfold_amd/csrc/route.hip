@@ -45,19 +45,7 @@ __global__ void __launch_bounds__(PLAN_THREADS)
                       int* __restrict__ items, int* __restrict__ counts) {
   __shared__ int pk[PLAN_THREADS];
   __shared__ PlanLds plan;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  plan.cnt[tid] = 0;
-  __syncthreads();
-  int e = tid < P ? picks[tid] : -1;
-  if ((unsigned)e >= (unsigned)E) e = -1;            // an id outside the table joins no expert (and faults nothing)
-  pk[tid] = e;
-  if (e >= 0) atomicAdd(&plan.cnt[e], 1);
-  __syncthreads();
-  place_items(plan, tid < E ? plan.cnt[tid] : 0, E, T, items, counts);
-  for (int x = wave; x < E; x += PLAN_THREADS / 64) {
-    const int c = plan.cnt[x], at = plan.first[x];
-    if (c) expert_pairs(pk, P, x, c, lane, [&](int rank, int p) { members[at + rank] = p; });
-  }
+  plan_small(picks, P, E, T, members, items, counts, pk, plan);
 }
 
 // The decode layer's whole routing in one workgroup (rows * slots <= 1024): top-k of every row, the pair sort, one

@@ -395,6 +395,25 @@ __device__ __forceinline__ int wave_scan(int x) {
 
 // ---- item descriptors ---------------------------------------------------------------------------------------------------
 //
+// The plan of up to PLAN_THREADS pairs by one workgroup of PLAN_THREADS threads: count, scan and place; then a wave
+// an expert that has pairs collects them in pair order (ballots over the pairs, 64 a step).  pk: PLAN_THREADS ints.
+__device__ __forceinline__ void plan_small(const int* __restrict__ picks, int P, int E, int T, int* __restrict__ members,
+                                           int* __restrict__ items, int* __restrict__ counts, int* pk, PlanLds& plan) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  plan.cnt[tid] = 0;
+  __syncthreads();
+  int e = tid < P ? picks[tid] : -1;
+  if ((unsigned)e >= (unsigned)E) e = -1;            // an id outside the table joins no expert (and faults nothing)
+  pk[tid] = e;
+  if (e >= 0) atomicAdd(&plan.cnt[e], 1);
+  __syncthreads();
+  place_items(plan, tid < E ? plan.cnt[tid] : 0, E, T, items, counts);
+  for (int x = wave; x < E; x += PLAN_THREADS / 64) {
+    const int c = plan.cnt[x], at = plan.first[x];
+    if (c) expert_pairs(pk, P, x, c, lane, [&](int rank, int p) { members[at + rank] = p; });
+  }
+}
+
 // What the routing kernels leave for the decode expert kernels: the plan cut again into items of at most DTILE pairs
 // (a workgroup walks its rows two at a time, so short items keep every workgroup to two passes over its weights and
 // spread an expert that many rows share over more workgroups).  int32 rows of DESC: row 0 holds the number of

@@ -104,7 +104,7 @@ __device__ __forceinline__ void prio_by_progress(int left, int n) {
 // 5 (a store to memory at each mark would put its round trip into the waits that follow it).  The ordinary build
 // compiles the marks away.
 #ifdef TF_TIMELINE
-constexpr int TIMELINE_MARKS = 6, TIMELINE_ROWS = TIMELINE_MARKS + 1, TIMELINE_GROUPS = 4096;
+constexpr int TIMELINE_MARKS = 6, TIMELINE_ROWS = TIMELINE_MARKS + 1, TIMELINE_GROUPS = 16384;
 static __device__ unsigned long long tf_timeline_marks[TIMELINE_ROWS][TIMELINE_GROUPS];
 __device__ __forceinline__ unsigned long long* timeline_lds() {
   __shared__ unsigned long long t[TIMELINE_MARKS];

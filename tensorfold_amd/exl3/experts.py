@@ -197,7 +197,7 @@ def routed(x: torch.Tensor, pick: torch.Tensor, wts: torch.Tensor | None, ex: Ex
            group: bool = True) -> torch.Tensor:
     """Routed experts of R rows (picks outside [0, E) skipped): Y fp32 per pair, or ``out`` fp32 [R, D] = the
     wts-weighted sum over the slots when ``wts`` is given; no host sync.  ``group=False`` reuses the grouping of the
-    last call on the same picks."""
+    last call on the same picks.  Five launches up to 1,024 pairs (the grouping shares the rotation's), else six."""
 
     d, width, n_exp, slots = ex.dims, ex.width, ex.count, s.slots
     p = R * slots
@@ -215,12 +215,19 @@ def routed(x: torch.Tensor, pick: torch.Tensor, wts: torch.Tensor | None, ex: Ex
         raise ValueError("act_mode is ACT_BF16 or ACT_F32")
     _lib.on_gpu(x, pick, wts)
     plan = s.plan
-    if group:
-        grouped.route(pick, plan)                         # the pair sort drops ids outside [0, E)
     items = grouped.max_items(p, n_exp, grouped.TILE)
     plan_args = (_lib.ptr(plan.items), _lib.ptr(plan.counts), _lib.ptr(plan.members))
-    _lib.call("tf_exl3x_rot_in", _lib.ptr(x), _DTYPES[x.dtype], x.stride(0), _lib.ptr(pick), _lib.ptr(ex.suh[GATE]),
-              _lib.ptr(ex.suh[UP]), _lib.ptr(s.xg), _lib.ptr(s.xu), R, slots, d, n_exp)
+    rot_args = (_lib.ptr(x), _DTYPES[x.dtype], x.stride(0), _lib.ptr(pick), _lib.ptr(ex.suh[GATE]), _lib.ptr(ex.suh[UP]),
+                _lib.ptr(s.xg), _lib.ptr(s.xu), R, slots, d, n_exp)
+    if group and p <= grouped.SMALL:
+        # one launch for the pair sort (it drops ids outside [0, E)) and the rotation: neither needs the other
+        plan.tile = grouped.TILE
+        _lib.call("tf_exl3x_plan_rot_in", *rot_args, grouped.TILE, _lib.ptr(plan.members), _lib.ptr(plan.items),
+                  _lib.ptr(plan.counts))
+    else:
+        if group:
+            grouped.route(pick, plan)
+        _lib.call("tf_exl3x_rot_in", *rot_args)
     _lib.call("tf_exl3x_grouped", _lib.ptr(s.xg), _lib.ptr(s.xu), _lib.ptr(ex.ptr[GATE]), _lib.ptr(ex.ptr[UP]),
               _lib.ptr(ex.k2[GATE]), _lib.ptr(ex.k2[UP]), *plan_args, _lib.ptr(s.z), 2, d, width, p, s.sk_gu, ex.cb,
               n_exp, items)

@@ -7,6 +7,7 @@ import pytest
 import torch
 
 from oracle import exl3 as ore
+from tensorfold_amd import experts as grouped
 from tensorfold_amd.exl3 import experts
 from tests.helpers import rel_l2
 
@@ -135,6 +136,35 @@ def test_fused_down_and_combine_equal_the_separate_steps(slots):
     scratch.y.fill_(7.0)
     out = experts.routed(x, sel, w, ex, scratch, None, rows, group=False)
     assert np.array_equal(out.cpu().numpy(), acc)
+
+
+@pytest.mark.parametrize("cb,rows,slots", [("mcg", 1, 9), ("3inst", 8, 9), ("mul1", 37, 5), ("mcg", 16, 64)])
+def test_grouping_in_the_rotations_launch(cb, rows, slots):
+    """The launch that groups and rotates at once leaves the plan and the rotated inputs of the two separate launches
+    (``group=False`` after a ``route`` of one's own takes those), and so the same outputs; with slots that are not
+    routed and a row that has none."""
+
+    n_exp, d, width = 70, 384, 256
+    ex, _ = make_layer(n_exp, d, width, cb, lambda e: ((2, 3.5, 4, 5)[e % 4],) * 2 + ((3, 4)[e % 2],), 91)
+    gen = torch.Generator().manual_seed(rows)
+    x = torch.randn((rows, d), generator=gen).to(torch.bfloat16).to(DEV)
+    sel, w = picks(n_exp, rows, slots - 1, 17 + rows, shared=True)
+    sel[rows // 2, 0] = -3
+    if rows > 2:
+        sel[rows - 2] = n_exp + 1
+    mine = torch.randn((rows * slots, d), generator=gen).to(DEV)
+    one, two = experts.Scratch(ex, rows, slots), experts.Scratch(ex, rows, slots)
+    for n in (rows, max(1, rows - 3)):
+        one.y.copy_(mine), two.y.copy_(mine)
+        a = experts.routed(x[:n], sel[:n].contiguous(), w[:n].contiguous(), ex, one, None, n, limit=1.5).clone()
+        grouped.route(sel[:n].contiguous(), two.plan)
+        b = experts.routed(x[:n], sel[:n].contiguous(), w[:n].contiguous(), ex, two, None, n, limit=1.5, group=False)
+        torch.cuda.synchronize()
+        k = int(two.plan.counts[0])
+        assert torch.equal(one.plan.counts, two.plan.counts) and torch.equal(one.plan.items[:k], two.plan.items[:k])
+        assert torch.equal(one.plan.members, two.plan.members)
+        assert torch.equal(one.xg, two.xg) and torch.equal(one.xu, two.xu) and torch.equal(one.y, two.y)
+        assert torch.equal(a, b), n
 
 
 def test_graph_replay_equals_eager():

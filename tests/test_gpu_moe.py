@@ -261,7 +261,11 @@ def test_a_prompts_pair_outputs_in_fp16():
 
 @pytest.mark.parametrize("shape,ne,rows", [(synthetic.C1, 24, 1), (synthetic.C1, 24, 8), (synthetic.C2, 48, 32),
                                            (synthetic.MoEShape("small", 512, 16, 128, 4, 32, True, True), 16, 5),
-                                           (synthetic.MoEShape("small64", 384, 12, 192, 3, 64, False, False), 12, 19)])
+                                           (synthetic.MoEShape("small64", 384, 12, 192, 3, 64, False, False), 12, 19),
+                                           # short K under a full down launch: 6 groups for 16 slices and an odd
+                                           # number of column pairs; 8 groups of 64
+                                           (synthetic.MoEShape("short32", 448, 16, 192, 6, 32, True, True), 16, 64),
+                                           (synthetic.MoEShape("short64", 1024, 40, 512, 8, 64, False, False), 40, 24)])
 @pytest.mark.parametrize("path", ["route_up", "topk_then_up", "route_then_up", "one_launch"])
 def test_the_fused_decode_layer_equals_the_separate_kernels(shape, ne, rows, path, monkeypatch):
     """The forms of ``decode`` (routing inside the up launch; a top-k launch, then the plan inside the up launch; a
