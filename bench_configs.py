@@ -1,7 +1,7 @@
 """Kernel timings of the benchmark configurations that are not bench.py's headline: 0 (dense 4-bit projection),
 2 (verify-window MoE layer), 3 (prompt chunk, grouped MFMA) and 4 (EXL3 projections).
 
-    python bench_configs.py [c0] [c2] [c3] [c4] [c4p] [glue] [c4x] [mfma] [floor] [timeline]
+    python bench_configs.py [c0] [c2] [c3] [c4] [c4p] [glue] [c4x] [mfma] [floor] [timeline] [timeline_c2]
 
 One JSON line a configuration: time of one pass (hipGraph of back-to-back passes cycling over enough weight copies to
 miss the 256 MB Infinity Cache, HIP events around the replay), algorithmic bytes or flops, and the fraction of the
@@ -515,11 +515,93 @@ def timeline() -> dict:
     return out
 
 
+def timeline_c2() -> dict:
+    """The same marks for the two expert launches of configuration 2's layer (32 rows, 513 experts: the top-k runs in
+    a launch before them, so the up launch finds its items from the picks), with each launch's own time beside them:
+    how long a workgroup lives, how many are alive at once, how many a compute unit ran."""
+
+    import ctypes
+
+    import numpy as np
+
+    from tensorfold_amd import _lib, build
+
+    s, rows = synthetic.C2, 32
+    gen = torch.Generator(device=DEV).manual_seed(2)
+    tabs = moe_tables(s, 2, gen)
+    x = synthetic.activations(rows, s.hidden, 1201).to(DEV)
+    logits = [synthetic.logits(rows, s.experts + 1, 3000 + i).to(DEV) for i in range(4)]
+    bufs = [moe.MoEBuffers(rows, cfg_of(s), DEV, shared=True) for _ in range(4)]
+    out = torch.empty((rows, s.hidden), dtype=torch.bfloat16, device=DEV)
+    for j, b in enumerate(bufs):          # routes each buffer's plan and fills its descriptors and activations
+        moe.decode(x, logits[j], tabs[j % 2], b, s.top_k, s.experts, out)
+    torch.cuda.synchronize()
+    items = experts.max_items(rows * bufs[0].slots, s.experts + 1, moe.DESC_TILE)
+
+    def up(i):
+        b, ex = bufs[i % 4], tabs[i % 2]
+        f, plan = b.fused(ex.gs), b.plan
+        _lib.call("tf_moe_route_up", None, logits[0].stride(0), rows, s.experts, s.top_k, 1, ex.gs, int(ex.swiglu),
+                  _lib.ptr(x), x.stride(0), _lib.ptr(ex.up), ex.dims, ex.width, _lib.ptr(b.pick), _lib.ptr(b.wts),
+                  _lib.ptr(plan.members), _lib.ptr(plan.items), _lib.ptr(plan.counts), _lib.ptr(f["desc"]),
+                  _lib.ptr(b.act.view(-1, ex.width)), ex.limit, items, None, 0)
+
+    def down(i):
+        b, ex = bufs[i % 4], tabs[i % 2]
+        f = b.fused(ex.gs)
+        _lib.call("tf_moe_down_combine", ex.gs, _lib.ptr(b.act.view(-1, ex.width)), rows, b.slots, _lib.ptr(ex.down),
+                  ex.dims, ex.width, _lib.ptr(f["desc"]), _lib.ptr(b.wts), _lib.ptr(b.y), _lib.ptr(out),
+                  f["counters"].data_ptr() + 4 * (1 + f["items"]), items)
+
+    res = {"config": "timeline_c2: the decode layer's launches on configuration 2 (32 rows), each alone",
+           "items": [int(b.fused(s.gs)["desc"].view(-1)[0]) for b in bufs],
+           "topk_us": graph_us(lambda i: moe.select_rows(logits[i % 4], bufs[i % 4], s.top_k, s.experts), 32),
+           "up_us": graph_us(up, 32), "down_us": graph_us(down, 32), "launches": {}}
+    marks = 6
+    with _lib.through(build.TIMELINE_LIB) as tl:
+        for name, fn in (("up", up), ("down", down)):
+            fn(0)
+            torch.cuda.synchronize()
+            if tl.tf_timeline_clear_moe():
+                raise RuntimeError(tl.tf_last_error().decode())
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                for i in range(10):
+                    fn(i)
+            g.replay()
+            g.replay()
+            torch.cuda.synchronize()
+            h = np.zeros((marks + 1, 16384), dtype=np.uint64)
+            if tl.tf_timeline_read_moe(h.ctypes.data_as(ctypes.c_void_p), h.shape[0], h.shape[1]):
+                raise RuntimeError(tl.tf_last_error().decode())
+            where, h = h[marks], h[:marks].astype(np.int64)
+            # a launch's workgroups differ from draw to draw: keep the marks of the last launch alone
+            end = h[5].max()
+            live = (h[5] > 0) & (h[0] > end - int(115 * res[name + "_us"]))
+            t0 = h[0][live].min()
+            quart = lambda v: [round(float(q), 2) for q in (v.min(), np.median(v), np.percentile(v, 90), v.max())]
+            row = {"workgroups": int(live.sum()), "launch_us": float((end - t0) / 100.0)}
+            for k, mark in enumerate(("entry", "item_known", "first_loads_out", "wave0_streamed", "all_waves_streamed",
+                                      "unit_done")):
+                sel = live & (h[k] > 0)
+                if sel.any():
+                    row[mark] = quart((h[k][sel] - t0) / 100.0)
+            row["life_us"] = quart((h[5] - h[0])[live] / 100.0)
+            hw = where[live]
+            cu = ((hw >> np.uint64(32)) << np.uint64(8)) | ((hw >> np.uint64(8)) & np.uint64(0xFF))
+            count = np.unique(cu, return_counts=True)[1]
+            row["a_compute_unit"] = [int(count.min()), round(float(count.mean()), 2), int(count.max())]
+            begin, done = (h[0][live] - t0) / 100.0, (h[5][live] - t0) / 100.0
+            row["alive_at_us"] = {str(t): int((begin <= t).sum() - (done <= t).sum()) for t in (5, 15, 25, 35, 45, 55)}
+            res["launches"][name] = row
+    return res
+
+
 def main() -> int:
     torch.cuda.set_device(0)
     which = sys.argv[1:] or ["c0", "c2", "c3", "c4"]
     for name in which:
-        res = {"mfma": mfma, "c0": c0, "c2": c2, "c3": c3, "c4": c4, "c4p": c4p, "glue": glue_, "c4x": c4x, "floor": floor, "timeline": timeline}[name]()
+        res = {"mfma": mfma, "c0": c0, "c2": c2, "c3": c3, "c4": c4, "c4p": c4p, "glue": glue_, "c4x": c4x, "floor": floor, "timeline": timeline, "timeline_c2": timeline_c2}[name]()
         torch.cuda.empty_cache()
         print(json.dumps(res, default=lambda v: round(v, 4)), flush=True)
     return 0
