@@ -235,20 +235,25 @@ def c4() -> dict:
             stacks[i % len(stacks)](x, y2, xh=xh2, z=z2)
             mlps[i % len(mlps)][2](h, yd, xh=hh, z=z)
 
-        us = graph_us(step_stacked, 48)
+        stacked_us = graph_us(step_stacked, 48)
+        # the whole MLP, SwiGLU included: the gate and up launch's workgroups apply it and the down projection's rotation
+        whole = [exl3.Exl3MLP(stacks[i], mlps[i][2]) for i in range(len(mlps))]
+        scratch = whole[0].scratch(m)
+        us = graph_us(lambda i: whole[i % len(whole)](x, yd, scratch=scratch), 48)
         gate_us = graph_us(lambda i: mlps[i % 4][0](x, ys[0], xh=xh, z=z), 48)
         down_us = graph_us(lambda i: mlps[i % 4][2](h, yd, xh=hh, z=z), 48)
         per = 5120 * 17408 * 3 // 8
         nbytes = 3 * per + 3 * 2 * (5120 + 17408) + m * (2 * 5120 + 17408 + 17408 * 2 + 5120) * 2
         ops = 3 * 5120 * 17408 * EXL3_VALU_PER_WEIGHT          # lane-operations of one MLP's decode
-        out[m] = {"mlp_us": us, "mlp_separate_calls_us": separate_us, "bytes": nbytes, "gbs": nbytes / us * 1e-3, "frac": nbytes / us * 1e-3 / HBM,
+        out[m] = {"mlp_us": us, "mlp_linears_only_us": stacked_us, "mlp_separate_calls_us": separate_us, "bytes": nbytes, "gbs": nbytes / us * 1e-3, "frac": nbytes / us * 1e-3 / HBM,
                   "gate_us": gate_us, "gate_gbs": per / gate_us * 1e-3, "down_us": down_us,
                   "down_gbs": per / down_us * 1e-3,
                   "valu": {"bound": "valu", "achieved": ops / us * 1e-6, "peak": VALU * 1e-12, "unit": "Tlane-op/s",
                            "frac": ops / us * 1e6 / VALU, "ops_per_weight": EXL3_VALU_PER_WEIGHT,
                            "floor_us": ops / VALU * 1e6}}
-    return {"config": "c4: EXL3 3.0 bpw MLP, gate/up 5120 -> 17408 as a stack of two (one rotation and one linear launch "
-                      "for both), down 17408 -> 5120 (rotation + linear); mlp_separate_calls_us: three separate layers",
+    return {"config": "c4: EXL3 3.0 bpw MLP down(silu(gate(x)) * up(x)), 5120 -> 17408 -> 5120, three launches (rotation; gate "
+                      "and up with the SwiGLU and down's rotation; down); mlp_linears_only_us: the stack and the down layer "
+                      "as two calls on independent inputs, no SwiGLU; mlp_separate_calls_us: three separate layers, no SwiGLU",
             "bound": "hbm", "rows": out}
 
 

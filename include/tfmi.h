@@ -267,6 +267,21 @@ int tf_exl3_linear_stacked(const uint16_t* xh, const uint32_t* T, int64_t stride
                            int64_t stride_layer, const uint16_t* svh, const uint16_t* bias, void* y, int y_dtype,
                            float* Z, int32_t* counters, int layers, int m, int k, int n, int k2, int cb, int sk, int wk,
                            tf_stream_t stream);
+/* An MLP's gate and up projections with the SwiGLU and the down projection's input rotation in the same launch:
+ * tf_exl3_linear_stacked over two layers (gate first), in which the workgroup that completes a column block over both
+ * layers' K splits also writes xh_next[m, n] = fp16(((act * suh_next) H) / sqrt(128)), act = r(r(g / (1 + exp(-g))) * u)
+ * with g, u the two outputs as y_dtype holds them and r the rounding to y_dtype: the input tf_exl3_linear takes for
+ * the down projection.  y [2, m, n] may be null; Z [2, sk, m, n] and counters [8 * n/128 * TF_EXL3_COUNTER_STRIDE]
+ * (zero before, left zero) are needed at every sk.  tf_exl3_swiglu_rot_in is the same producer as a launch of its own
+ * over a stored y [2, m, n] (same bits).  The reference's linear module has neither: its callers run the elementwise
+ * steps in torch between two `linear` calls (exl3/linear.py:165-186 `__call__`); the roundings are those of its
+ * other SwiGLU epilogues (kernels/qwen/flash_next/v1/base.py:35, experts.py:122). */
+int tf_exl3_gate_up(const uint16_t* xh, const uint32_t* T, int64_t stride_k, int64_t stride_nb, int64_t stride_layer,
+                    const uint16_t* svh, const uint16_t* bias, void* y, int y_dtype, float* Z, int32_t* counters,
+                    const uint16_t* suh_next, uint16_t* xh_next, int m, int k, int n, int k2, int cb, int sk, int wk,
+                    tf_stream_t stream);
+int tf_exl3_swiglu_rot_in(const void* y, int y_dtype, const uint16_t* suh, uint16_t* xh, int m, int n,
+                          tf_stream_t stream);
 /* W[k, n] fp16 = the decoded trellis (bit-exact codebook values).  Replaces exl3/linear.cpp:61-68 `unpack`. */
 int tf_exl3_unpack(const uint32_t* T, uint16_t* W, int k, int n, int64_t stride_k, int64_t stride_nb, int k2, int cb,
                    tf_stream_t stream);

@@ -48,6 +48,8 @@ PROTOTYPES = {
     "tf_exl3_linear": [P, P, L, L, P, P, P, I, P, P, I, I, I, I, I, I, I, P],
     "tf_exl3_rot_in_stacked": [P, I, P, P, I, I, I, P],
     "tf_exl3_linear_stacked": [P, P, L, L, L, P, P, P, I, P, P, I, I, I, I, I, I, I, I, P],
+    "tf_exl3_gate_up": [P, P, L, L, L, P, P, P, I, P, P, P, P, I, I, I, I, I, I, I, P],
+    "tf_exl3_swiglu_rot_in": [P, I, P, P, I, I, P],
     "tf_exl3_unpack": [P, P, I, I, L, L, I, I, P],
     "tf_exl3_unpack_k8": [P, P, I, I, L, L, I, I, P],
     "tf_exl3_gemm": [P, P, P, P, P, I, L, I, I, I, P],

@@ -40,28 +40,58 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// The SwiGLU of a stack's two outputs (gate y[0], up y[1], each [M, N]) and the next layer's input rotation in a
+// launch of its own: what the linear kernel's workgroups do themselves when they are given xh_next.  A wave a
+// (row, block of 128).
+__global__ void __launch_bounds__(256)
+    swiglu_rot_in_kernel(const void* __restrict__ y, int y_dtype, const uint16_t* __restrict__ suh,
+                         uint16_t* __restrict__ xh, int M, int N) {
+  const int blk = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (blk * 128 >= N) return;
+  const int col = blk * 128 + 2 * lane;
+  float sa, sb;
+  load2(suh, TF_F16, col, sa, sb);
+  for (int row = blockIdx.y; row < M; row += gridDim.y) {
+    const size_t at = (size_t)row * N + col;
+    float g0, g1, u0, u1;
+    load2(y, y_dtype, at, g0, g1);
+    load2(y, y_dtype, (size_t)M * N + at, u0, u1);
+    swiglu_rot(g0, g1, u0, u1, y_dtype, lane, sa, sb, xh, at);
+  }
+}
+
 // grid (N / 128, SK, layers); WK waves a block; each wave walks its range of k-tile pairs over the block's eight column
 // tiles.  The layers of a stack share K, N, width and codebook; layer z has its own xh [M, K], trellis (stride_layer
 // words on), svh and bias [N], y [M, N], Z [SK, M, N] and counters.
+// (The second launch bound, waves a SIMD, keeps the kernel within 128 registers at the widths where that costs no
+// spill; the widest decodes need a few more and run three waves a SIMD.)
 template <int K2, int CB, int WK>
-__global__ void __launch_bounds__(WK * 64)
+__global__ void __launch_bounds__(WK * 64, K2 <= 12 ? 4 : 1)
     linear_kernel(const uint16_t* __restrict__ xh, const uint32_t* __restrict__ T, int64_t stride_k, int64_t stride_nb,
                   int64_t stride_layer, const uint16_t* __restrict__ svh, const uint16_t* __restrict__ bias,
                   void* __restrict__ y, int y_dtype, float* __restrict__ Z, int* __restrict__ counters, int M, int K,
-                  int N, int SK) {
+                  int N, int SK, const uint16_t* __restrict__ suh_next, uint16_t* __restrict__ xh_next) {
   constexpr int TW = tile_words<K2>();
   extern __shared__ __align__(16) float red[];              // [WK][16][128]
   __shared__ int last;
   const int nb = blockIdx.x, split = blockIdx.y, NB = gridDim.x;
+  // With xh_next the two layers are an MLP's gate and up: the workgroup that completes a column block over BOTH
+  // layers' K splits (one counter for the two, the first layer's) finishes both layers' rows, and writes the next
+  // layer's rotated input from their SwiGLU.  y may then be null.
+  const bool mlp = xh_next != nullptr;
+  const uint16_t *svh0 = svh, *bias0 = bias;
+  void* y0 = y;
+  float* Z0 = Z;
   if (const size_t z = blockIdx.z) {
     xh += z * M * K;
     T += z * stride_layer;
     svh += z * N;
     if (bias) bias += z * N;
-    y = static_cast<char*>(y) + z * M * N * (y_dtype == TF_F32 ? 4 : 2);
+    if (y) y = static_cast<char*>(y) + z * M * N * (y_dtype == TF_F32 ? 4 : 2);
     if (Z) Z += z * SK * M * N;
-    if (counters) counters += z * 8 * NB * TF_EXL3_COUNTER_STRIDE;
+    if (counters && !mlp) counters += z * 8 * NB * TF_EXL3_COUNTER_STRIDE;
   }
+  const int arrivals = mlp ? 2 * SK : SK;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c = lane & 15, kq = lane >> 4;
   const int L = 4 * (c & 7) + kq, h = c >> 3;
   const int pairs = K >> 5, slot = split * WK + wave, nslots = SK * WK;
@@ -99,7 +129,7 @@ __global__ void __launch_bounds__(WK * 64)
         s.y += q.y;
       }
       const size_t at = (size_t)(m0 + r) * N + col0 + 2 * lane;
-      if (SK == 1) finish_row(s.x, s.y, lane, svh, bias, col0 + 2 * lane, y, y_dtype, at);
+      if (arrivals == 1) finish_row(s.x, s.y, lane, svh, bias, col0 + 2 * lane, y, y_dtype, at);
       else {
         // partial sums cross to another XCD's workgroup: agent-scope stores and loads are coherent by themselves
         // (a cache-wide write-back or invalidate, which __threadfence would issue, costs far more than the sums)
@@ -108,23 +138,23 @@ __global__ void __launch_bounds__(WK * 64)
         __hip_atomic_store(zp + 1, s.y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
-    if (SK > 1) {
+    if (arrivals > 1) {
       __builtin_amdgcn_s_waitcnt(0);        // this wave's stores are acknowledged ...
       __syncthreads();                      // ... every wave's are ...
       TF_MARK(4);
       if (threadIdx.x == 0)                 // ... then the block counts itself in
-        last = __hip_atomic_fetch_add(counters + (size_t)(pass * NB + nb) * TF_EXL3_COUNTER_STRIDE, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == SK - 1;
+        last = __hip_atomic_fetch_add(counters + (size_t)(pass * NB + nb) * TF_EXL3_COUNTER_STRIDE, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == arrivals - 1;
       __syncthreads();
       if (last) {
-        for (int r = wave; r < R; r += WK) {
-          const size_t at = (size_t)(m0 + r) * N + col0 + 2 * lane;
-          // eight splits' loads go out together (one trip to memory, not eight), then the sums in split order
-          float sx = 0.f, sy = 0.f;
+        // a row's sum over the K splits of the layer whose partial sums start at Zl: eight splits' loads go out
+        // together (one trip to memory, not eight), then the sums in split order
+        auto split_sums = [&](const float* Zl, size_t at, float& sx, float& sy) {
+          sx = sy = 0.f;
           for (int q0 = 0; q0 < SK; q0 += 8) {
             float vx[8], vy[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-              const float* zq = Z + (size_t)(q0 + j < SK ? q0 + j : SK - 1) * M * N + at;
+              const float* zq = Zl + (size_t)(q0 + j < SK ? q0 + j : SK - 1) * M * N + at;
               vx[j] = __hip_atomic_load(zq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
               vy[j] = __hip_atomic_load(zq + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
@@ -135,7 +165,31 @@ __global__ void __launch_bounds__(WK * 64)
                 sy = q0 + j ? sy + vy[j] : vy[j];
               }
           }
-          finish_row(sx, sy, lane, svh, bias, col0 + 2 * lane, y, y_dtype, at);
+        };
+        // the columns' scales are requested once, ahead of the rows' sums
+        const int col = col0 + 2 * lane;
+        const OutScale own(mlp ? svh0 : svh, mlp ? bias0 : bias, col);
+        const OutScale other(svh0 + (mlp ? N : 0), mlp && bias0 ? bias0 + N : nullptr, col);       // up's, for an MLP
+        float na = 0.f, nb2 = 0.f;
+        if (mlp) load2(suh_next, TF_F16, col, na, nb2);
+        for (int r = wave; r < R; r += WK) {
+          const size_t at = (size_t)(m0 + r) * N + col;
+          if (!mlp) {
+            float sx, sy;
+            split_sums(Z, at, sx, sy);
+            finish_row(sx, sy, lane, own, y, y_dtype, at);
+            continue;
+          }
+          float g0, g1, u0, u1;
+          split_sums(Z0, at, g0, g1);
+          split_sums(Z0 + (size_t)SK * M * N, at, u0, u1);
+          finish_values(g0, g1, lane, own);
+          finish_values(u0, u1, lane, other);
+          if (y0) {
+            store2(y0, y_dtype, at, g0, g1);
+            store2(y0, y_dtype, (size_t)M * N + at, u0, u1);
+          }
+          swiglu_rot(g0, g1, u0, u1, y_dtype, lane, na, nb2, xh_next, at);
         }
         if (threadIdx.x == 0) counters[(size_t)(pass * NB + nb) * TF_EXL3_COUNTER_STRIDE] = 0;     // every block of the column has arrived
       }
@@ -364,13 +418,15 @@ TF_TIMELINE_EXPORT(exl3)
 static int linear_launch(const char* who, const uint16_t* xh, const uint32_t* T, int64_t stride_k, int64_t stride_nb,
                          int64_t stride_layer, const uint16_t* svh, const uint16_t* bias, void* y, int y_dtype, float* Z,
                          int32_t* counters, int layers, int m, int k, int n, int k2, int cb, int sk, int wk,
-                         tf_stream_t stream) {
+                         tf_stream_t stream, const uint16_t* suh_next = nullptr, uint16_t* xh_next = nullptr) {
   clear_error();
-  TF_REQUIRE(xh && T && svh && y, "%s: null pointer argument", who);
+  TF_REQUIRE(xh && T && svh && (y || xh_next), "%s: null pointer argument", who);
+  TF_REQUIRE(!xh_next || (layers == 2 && suh_next && Z && counters && aligned16(xh_next)),
+             "%s: the SwiGLU needs two layers (gate, up), the next layer's suh, Z and counters", who);
   TF_REQUIRE(y_dtype == TF_F16 || y_dtype == TF_BF16 || y_dtype == TF_F32, "y: expected fp16, bf16 or fp32");
   TF_REQUIRE(m >= 1 && m <= 128, "xh and y must have the same 1 to 128 rows");
   TF_REQUIRE(k >= 128 && n >= 128 && k % 128 == 0 && n % 128 == 0, "K and N must be multiples of 128");
-  TF_REQUIRE(aligned16(T) && aligned16(xh) && aligned16(y), "T must be 16-byte aligned");
+  TF_REQUIRE(aligned16(T) && aligned16(xh) && aligned16(y), "T must be 16-byte aligned");          // (a null y is aligned)
   TF_REQUIRE(layers >= 1 && layers <= 64 && (layers == 1 || (stride_layer > 0 && stride_layer % 4 == 0)),
              "%s: 1 to 64 layers, a whole number of 16-byte pieces apart", who);
   TF_REQUIRE(layers == 1 || ((int64_t)m * k % 8 == 0 && (int64_t)m * n % 8 == 0), "%s: layers' xh and y must stay 16-byte aligned", who);
@@ -383,9 +439,9 @@ static int linear_launch(const char* who, const uint16_t* xh, const uint32_t* T,
   const size_t smem = (size_t)wk * 16 * 128 * sizeof(float);
 #define TF_LAUNCH(K2_, CB_)                                                                                             \
   if (k2 == K2_ && cb == CB_) {                                                                                         \
-    if (wk == 2) linear_kernel<K2_, CB_, 2><<<grid, 128, smem, s>>>(xh, T, stride_k, stride_nb, stride_layer, svh, bias, y, y_dtype, Z, counters, m, k, n, sk); \
-    else if (wk == 4) linear_kernel<K2_, CB_, 4><<<grid, 256, smem, s>>>(xh, T, stride_k, stride_nb, stride_layer, svh, bias, y, y_dtype, Z, counters, m, k, n, sk); \
-    else linear_kernel<K2_, CB_, 8><<<grid, 512, smem, s>>>(xh, T, stride_k, stride_nb, stride_layer, svh, bias, y, y_dtype, Z, counters, m, k, n, sk); \
+    if (wk == 2) linear_kernel<K2_, CB_, 2><<<grid, 128, smem, s>>>(xh, T, stride_k, stride_nb, stride_layer, svh, bias, y, y_dtype, Z, counters, m, k, n, sk, suh_next, xh_next); \
+    else if (wk == 4) linear_kernel<K2_, CB_, 4><<<grid, 256, smem, s>>>(xh, T, stride_k, stride_nb, stride_layer, svh, bias, y, y_dtype, Z, counters, m, k, n, sk, suh_next, xh_next); \
+    else linear_kernel<K2_, CB_, 8><<<grid, 512, smem, s>>>(xh, T, stride_k, stride_nb, stride_layer, svh, bias, y, y_dtype, Z, counters, m, k, n, sk, suh_next, xh_next); \
     TF_LAUNCH_OK(who);                                                                                                  \
     return 0;                                                                                                           \
   }
@@ -409,6 +465,28 @@ extern "C" int tf_exl3_linear_stacked(const uint16_t* xh, const uint32_t* T, int
                                       int cb, int sk, int wk, tf_stream_t stream) {
   return linear_launch("tf_exl3_linear_stacked", xh, T, stride_k, stride_nb, stride_layer, svh, bias, y, y_dtype, Z,
                        counters, layers, m, k, n, k2, cb, sk, wk, stream);
+}
+
+extern "C" int tf_exl3_gate_up(const uint16_t* xh, const uint32_t* T, int64_t stride_k, int64_t stride_nb,
+                               int64_t stride_layer, const uint16_t* svh, const uint16_t* bias, void* y, int y_dtype,
+                               float* Z, int32_t* counters, const uint16_t* suh_next, uint16_t* xh_next, int m, int k,
+                               int n, int k2, int cb, int sk, int wk, tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(suh_next && xh_next, "tf_exl3_gate_up: null pointer argument");
+  return linear_launch("tf_exl3_gate_up", xh, T, stride_k, stride_nb, stride_layer, svh, bias, y, y_dtype, Z, counters, 2, m,
+                       k, n, k2, cb, sk, wk, stream, suh_next, xh_next);
+}
+
+extern "C" int tf_exl3_swiglu_rot_in(const void* y, int y_dtype, const uint16_t* suh, uint16_t* xh, int m, int n,
+                                     tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(y && suh && xh, "tf_exl3_swiglu_rot_in: null pointer argument");
+  TF_REQUIRE(y_dtype == TF_F16 || y_dtype == TF_BF16 || y_dtype == TF_F32, "y: expected fp16, bf16 or fp32");
+  TF_REQUIRE(m >= 1 && n >= 128 && n % 128 == 0, "y must be [2, M, N], N a multiple of 128, suh [N]");
+  TF_REQUIRE(aligned16(y) && aligned16(xh) && (int64_t)m * n % 8 == 0, "y and xh must be 16-byte aligned");
+  swiglu_rot_in_kernel<<<dim3((n / 128 + 3) / 4, m < 1024 ? m : 1024), 256, 0, as_stream(stream)>>>(y, y_dtype, suh, xh, m, n);
+  TF_LAUNCH_OK("tf_exl3_swiglu_rot_in");
+  return 0;
 }
 
 extern "C" int tf_exl3_unpack(const uint32_t* T, uint16_t* W, int k, int n, int64_t stride_k, int64_t stride_nb, int k2,

@@ -183,21 +183,60 @@ __device__ __forceinline__ void store2(void* p, int dtype, size_t i, float a, fl
 }
 
 
+// The lane's two columns' output scales and bias of a layer, loaded once for all the rows a wave finishes.
+struct OutScale {
+  float sa, sb, ba, bb;
+  __device__ __forceinline__ OutScale(const uint16_t* svh, const uint16_t* bias, int col) {
+    load2(svh, TF_F16, col, sa, sb);
+    ba = bb = 0.f;
+    has_bias = bias != nullptr;
+    if (bias) load2(bias, TF_F16, col, ba, bb);
+  }
+  bool has_bias;
+};
+
 // the finished outputs of one row's 128 columns from their fp32 sums: H / sqrt(128), * svh, + bias
+__device__ __forceinline__ void finish_values(float& a, float& b, int lane, const OutScale& s) {
+  fwht128(a, b, lane);
+  a = a * HAD_SCALE * s.sa;
+  b = b * HAD_SCALE * s.sb;
+  if (s.has_bias) {
+    a += s.ba;
+    b += s.bb;
+  }
+}
+
+__device__ __forceinline__ void finish_row(float a, float b, int lane, const OutScale& s, void* y, int y_dtype,
+                                           size_t at) {
+  finish_values(a, b, lane, s);
+  store2(y, y_dtype, at, a, b);
+}
+
 __device__ __forceinline__ void finish_row(float a, float b, int lane, const uint16_t* svh, const uint16_t* bias,
                                            int col, void* y, int y_dtype, size_t at) {
+  finish_row(a, b, lane, OutScale(svh, bias, col), y, y_dtype, at);
+}
+
+// a value as a store to `dtype` and a load back leave it
+__device__ __forceinline__ float rounded(float v, int dtype) {
+  if (dtype == TF_F32) return v;
+  if (dtype == TF_BF16) return round_bf16(v);
+  return __half2float(__float2half_rn(v));
+}
+
+// SwiGLU of one row's 128 columns of gate (g) and up (u), two a lane, then the next layer's input rotation with its
+// input scales (sa, sb): xh[at ..] = fp16(((act * suh) H) / sqrt(128)).  g and u are rounded to `dtype` first (what a
+// y of that type holds), act = rounded(rounded(g / (1 + exp(-g))) * u): the roundings of the two elementwise steps
+// on tensors of that type.
+__device__ __forceinline__ void swiglu_rot(float g0, float g1, float u0, float u1, int dtype, int lane, float sa,
+                                           float sb, uint16_t* xh, size_t at) {
+  g0 = rounded(g0, dtype), g1 = rounded(g1, dtype), u0 = rounded(u0, dtype), u1 = rounded(u1, dtype);
+  float a = rounded(rounded(g0 / (1.f + expf(-g0)), dtype) * u0, dtype);
+  float b = rounded(rounded(g1 / (1.f + expf(-g1)), dtype) * u1, dtype);
+  a *= sa;
+  b *= sb;
   fwht128(a, b, lane);
-  float sa, sb;
-  load2(svh, TF_F16, col, sa, sb);
-  a = a * HAD_SCALE * sa;
-  b = b * HAD_SCALE * sb;
-  if (bias) {
-    float ba, bb;
-    load2(bias, TF_F16, col, ba, bb);
-    a += ba;
-    b += bb;
-  }
-  store2(y, y_dtype, at, a, b);
+  store2(xh, TF_F16, at, a * HAD_SCALE, b * HAD_SCALE);
 }
 
 // One wave's sums of up to 16 rows over the k-tile pairs [pr0, pr1) of a 128-column block: acc[j] is the 16 x 16

@@ -255,6 +255,89 @@ class Exl3Stack:
         return out
 
 
+@dataclasses.dataclass
+class Exl3MLP:
+    """down(silu(gate(x)) * up(x)) in three launches: the input rotation for gate and up, their linear launch — whose
+    workgroups also apply the SwiGLU and the down projection's input rotation to every column block they complete —
+    and the down projection's linear launch.  The elementwise steps round as they would on tensors of ``mid_dtype``
+    (gate and up's outputs, silu, the product); the bits are those of ``Exl3Stack`` + ``swiglu_rot_in`` + the down
+    layer's linear launch."""
+
+    gate_up: Exl3Stack            # gate first
+    down: Exl3Linear
+
+    @classmethod
+    def of(cls, gate: Exl3Linear, up: Exl3Linear, down: Exl3Linear) -> "Exl3MLP":
+        if down.k != gate.n or down.n != gate.k:
+            raise ValueError(f"down must be {gate.n} -> {gate.k}, got {down.k} -> {down.n}")
+        return cls(Exl3Stack.of([gate, up]), down)
+
+    def scratch(self, m: int, device=None) -> dict[str, torch.Tensor]:
+        """Buffers of a call on up to ``m`` rows: rotated inputs of both stages and the K splits' partial sums."""
+
+        g, d = self.gate_up, self.down
+        device = device or g.words.device
+        floats = max(2 * g.split[0] * m * g.n, d.split[0] * m * d.n)
+        return {"xh": torch.empty((2, m, g.k), dtype=torch.float16, device=device),
+                "hh": torch.empty((m, g.n), dtype=torch.float16, device=device),
+                "z": torch.empty((floats,), dtype=torch.float32, device=device)}
+
+    def __call__(self, x: torch.Tensor, out: torch.Tensor | None = None, mid_dtype: torch.dtype = torch.float16,
+                 scratch: dict[str, torch.Tensor] | None = None, mid: torch.Tensor | None = None) -> torch.Tensor:
+        """y [M, D] for x [M, D], M = 1..128.  ``mid`` ([2, M, I] of ``mid_dtype``), when given, receives gate's and
+        up's outputs as well."""
+
+        g, d = self.gate_up, self.down
+        if x.dim() != 2 or x.shape[1] != g.k or not 1 <= x.shape[0] <= 128 or x.dtype not in _DTYPES:
+            raise ValueError(f"x must be [1..128, {g.k}] fp16, bf16 or fp32, got {tuple(x.shape)} {x.dtype}")
+        if mid_dtype not in _DTYPES:
+            raise ValueError("mid_dtype: fp16, bf16 or fp32")
+        _lib.on_gpu(x)
+        x = x.contiguous()
+        m = int(x.shape[0])
+        s = scratch or self.scratch(m, x.device)
+        if s["xh"].numel() < 2 * m * g.k or s["hh"].numel() < m * g.n or \
+                s["z"].numel() < max(2 * g.split[0] * m * g.n, d.split[0] * m * d.n):
+            raise ValueError(f"the scratch does not hold {m} rows")
+        if out is None:
+            out = x.new_empty((m, d.n))
+        elif tuple(out.shape) != (m, d.n) or out.dtype not in _DTYPES or not out.is_contiguous() or out.device != x.device:
+            raise ValueError(f"out must be contiguous ({m}, {d.n}) fp16, bf16 or fp32 on x's device")
+        if mid is not None and (tuple(mid.shape) != (2, m, g.n) or mid.dtype != mid_dtype or not mid.is_contiguous()
+                                or mid.device != x.device):
+            raise ValueError(f"mid must be contiguous (2, {m}, {g.n}) {mid_dtype} on x's device")
+        (sk, wk), (dsk, dwk) = g.split, d.split
+        stride_k, stride_nb = g.layer(0).strides
+        _lib.call("tf_exl3_rot_in_stacked", _lib.ptr(x), _DTYPES[x.dtype], _lib.ptr(g.suh), _lib.ptr(s["xh"]), 2, m, g.k)
+        _lib.call("tf_exl3_gate_up", _lib.ptr(s["xh"]), _lib.ptr(g.words), stride_k, stride_nb, g.words.stride(0),
+                  _lib.ptr(g.svh), _lib.ptr(g.bias), _lib.ptr(mid), _DTYPES[mid_dtype], _lib.ptr(s["z"]),
+                  _lib.ptr(g.counters), _lib.ptr(d.suh), _lib.ptr(s["hh"]), m, g.k, g.n, k2_of(g.bits),
+                  CODEBOOK_IDS[g.codebook], sk, wk)
+        stride_k, stride_nb = d.strides
+        _lib.call("tf_exl3_linear", _lib.ptr(s["hh"]), _lib.ptr(d.words), stride_k, stride_nb, _lib.ptr(d.svh),
+                  _lib.ptr(d.bias), _lib.ptr(out), _DTYPES[out.dtype], _lib.ptr(s["z"]) if dsk > 1 else None,
+                  _lib.ptr(d.counters), m, d.k, d.n, d.k2, CODEBOOK_IDS[d.codebook], dsk, dwk)
+        return out
+
+
+def swiglu_rot_in(y: torch.Tensor, suh: torch.Tensor, xh: torch.Tensor | None = None) -> torch.Tensor:
+    """The rotated input of a down projection from a stack's gate and up outputs ``y`` [2, M, I] (a launch of its own;
+    ``Exl3MLP`` folds it into the stack's): fp16 [M, I]."""
+
+    _lib.on_gpu(y, suh)
+    if y.dim() != 3 or y.shape[0] != 2 or y.dtype not in _DTYPES or not y.is_contiguous() or y.shape[2] % 128:
+        raise ValueError("y must be a contiguous [2, M, I] fp16, bf16 or fp32, I a multiple of 128")
+    if suh.dtype != torch.float16 or tuple(suh.shape) != (y.shape[2],) or not suh.is_contiguous():
+        raise ValueError(f"suh must be fp16 [{y.shape[2]}]")
+    m, n = int(y.shape[1]), int(y.shape[2])
+    if xh is None:
+        xh = torch.empty((m, n), dtype=torch.float16, device=y.device)
+    elif xh.dtype != torch.float16 or tuple(xh.shape) != (m, n) or not xh.is_contiguous() or xh.device != y.device:
+        raise ValueError(f"xh must be a contiguous fp16 ({m}, {n}) on y's device")
+    _lib.call("tf_exl3_swiglu_rot_in", _lib.ptr(y), _DTYPES[y.dtype], _lib.ptr(suh), _lib.ptr(xh), m, n)
+    return xh
+
+
 def unpack_gpu(trellis: torch.Tensor, codebook: str) -> torch.Tensor:
     """W_q [K, N] fp16 from trellis int16 [K/16, N/16, 16 * bits], decoded on the GPU from the stored order."""
 

@@ -177,6 +177,48 @@ def test_a_stack_of_layers_gives_each_layer_its_own_bits(codebook, bits, split):
         stack(x, out=torch.empty((2, 128, 256), dtype=torch.float16, device="cuda"))
 
 
+@pytest.mark.parametrize("codebook,bits,split,mid", [("3inst", 3, (7, 4), torch.float16), ("mul1", 2.5, (1, 2), torch.bfloat16),
+                                                     ("mcg", 4, (3, 8), torch.float16), ("mul1", 6, (2, 2), torch.float32)])
+def test_an_mlp_in_three_launches(codebook, bits, split, mid):
+    """``Exl3MLP``: the workgroups of the gate and up launch apply the SwiGLU and the down projection's rotation
+    themselves.  Gate's and up's outputs, the rotated activations and the result have the bits of the stack, the
+    producer run as a launch of its own, and the down layer's linear launch; against torch's silu and product on the
+    same outputs the result stays within 2e-3; twice in a row on one scratch, rows 1 to 33."""
+
+    from tensorfold_amd import _lib
+
+    k, n = 1024, 768
+    gate, up, down = Group.draw(codebook, bits, k=k, n=n, seed=71), Group.draw(codebook, bits, k=k, n=n, seed=72), \
+        Group.draw(codebook, bits, k=n, n=k, seed=73)
+    bias = torch.from_numpy((np.random.default_rng(5).standard_normal(n) * 0.05).astype(np.float16))
+    layers = [gate.layer(), up.layer(bias=bias), down.layer()]
+    layers[0].split = layers[1].split = split
+    mlp = linear.Exl3MLP.of(*layers)
+    stack, dl = linear.Exl3Stack.of(layers[:2]), layers[2]
+    for m in (1, 5, 16, 33):
+        x = synthetic.activations(m, k, 80 + m, dtype=torch.float16).cuda()
+        scratch = mlp.scratch(m)
+        y2 = stack(x, out_dtype=mid)
+        hh = linear.swiglu_rot_in(y2, dl.suh)
+        want = torch.empty((m, k), dtype=torch.float16, device="cuda")
+        dsk, dwk = dl.split
+        z = torch.empty((dsk * m * k,), dtype=torch.float32, device="cuda")
+        _lib.call("tf_exl3_linear", _lib.ptr(hh), _lib.ptr(dl.words), *dl.strides, _lib.ptr(dl.svh), _lib.ptr(dl.bias),
+                  _lib.ptr(want), linear._DTYPES[want.dtype], _lib.ptr(z), _lib.ptr(dl.counters), m, dl.k, dl.n, dl.k2,
+                  linear.CODEBOOK_IDS[dl.codebook], dsk, dwk)
+        for _ in range(2):
+            kept = torch.empty((2, m, n), dtype=mid, device="cuda")
+            got = mlp(x, mid_dtype=mid, scratch=scratch, mid=kept)
+            assert torch.equal(kept, y2) and torch.equal(scratch["hh"][:m], hh) and torch.equal(got, want), m
+            assert torch.equal(mlp(x, mid_dtype=mid, scratch=scratch), want), m            # without keeping gate and up
+        act = (torch.nn.functional.silu(y2[0].float()).to(mid).float() * y2[1].float()).to(mid)
+        ref = dl(act)
+        assert rel_l2(got.float().cpu().numpy(), ref.float().cpu().numpy()) <= 2e-3, m
+    assert not mlp.gate_up.counters.any() and not dl.counters.any()
+    with pytest.raises(ValueError):
+        linear.Exl3MLP.of(layers[0], layers[1], layers[0])
+
+
 def test_what_the_layer_refuses():
     g = Group.draw("3inst", 3)
     with pytest.raises(ValueError):                                  # no such codebook
