@@ -1,4 +1,5 @@
-// EXL3 trellis-coded linear layers: tf_exl3_rot_in, tf_exl3_linear, tf_exl3_unpack.
+// EXL3 trellis-coded linear layers: tf_exl3_rot_in, tf_exl3_linear (and their stacked forms), tf_exl3_gate_up,
+// tf_exl3_swiglu_rot_in, tf_exl3_unpack, tf_exl3_unpack_k8, tf_exl3_gemm.
 //
 // The decode primitives are in exl3_decode.h.
 
