@@ -1,7 +1,7 @@
 """Kernel timings of the benchmark configurations that are not bench.py's headline: 0 (dense 4-bit projection),
 2 (verify-window MoE layer), 3 (prompt chunk, grouped MFMA) and 4 (EXL3 projections).
 
-    python bench_configs.py [c0] [c2] [c3] [c4] [c4p] [glue] [c4x] [mfma] [floor] [timeline] [timeline_c2]
+    python bench_configs.py [c0] [c2] [c3] [c4] [c4p] [glue] [c4x] [cal] [timeline] [timeline_c2]
 
 One JSON line a configuration: time of one pass (hipGraph of back-to-back passes cycling over enough weight copies to
 miss the 256 MB Infinity Cache, HIP events around the replay), algorithmic bytes or flops, and the fraction of the
@@ -347,51 +347,30 @@ def c4x() -> dict:
             "bound": "hbm", "rows": out}
 
 
-def mfma() -> dict:
-    """Issue rates of the candidate matrix instructions (f16, fp8, block-scaled fp8), bare and with the per-group fma
-    of an 8-bit prompt path: the stand-alone probe built beside the library (csrc/probe_mfma.hip), its table as text."""
+def cal() -> dict:
+    """What a tuned library GEMM gets from this chip at this clock, by the same graph method as the other legs:
+    ``torch.matmul`` (hipBLASLt / rocBLAS) on fp16 and bf16 operands already in HBM, fp32 accumulation, at the dense
+    prompt form's size (4096 cubed) and at configuration 4's gate projection (4096 x 5120 -> 17408).  No
+    dequantization, no epilogue: the ceiling the 4-bit and EXL3 prompt kernels are judged against beside the
+    2.5 PFLOP/s of the data sheet."""
 
-    import subprocess
-
-    from tensorfold_amd import build
-
-    if not build.PROBE.exists():
-        raise RuntimeError(f"{build.PROBE} is missing: run `python -c 'import __graft_entry__ as g; g.build()'`")
-    done = subprocess.run([str(build.PROBE)], capture_output=True, text=True, timeout=120)
-    if done.returncode:
-        raise RuntimeError(f"probe_mfma failed: {done.stderr}")
-    return {"config": "mfma: issue rates of the matrix instructions (probe_mfma)", "lines": done.stdout.splitlines()}
-
-
-def floor() -> dict:
-    """What a launch costs and how fast a short stream runs: a graph of one-workgroup kernels (the gap a launch adds
-    to a layer of two launches), and the stand-alone probe that streams configuration 1's expert units with the
-    decode kernels' access pattern and nothing else (csrc/probe_stream.hip; its table as text)."""
-
-    import subprocess
-
-    from tensorfold_amd import build
-
-    from tensorfold_amd import _lib
-
-    x = synthetic.activations(1, 64, 1).to(DEV)
-    xs = torch.empty((1, 1), dtype=torch.float32, device=DEV)
-
-    def tiny(i):
-        _lib.call("tf_group_sums", _lib.ptr(x), x.stride(0), 1, 64, 64, _lib.ptr(xs))
-
-    def pair(i):
-        tiny(i)
-        tiny(i)
-
-    if not build.PROBE_STREAM.exists():
-        raise RuntimeError(f"{build.PROBE_STREAM} is missing: run `python -c 'import __graft_entry__ as g; g.build()'`")
-    done = subprocess.run([str(build.PROBE_STREAM)], capture_output=True, text=True, timeout=120)
-    if done.returncode:
-        raise RuntimeError(f"probe_stream failed: {done.stdout} {done.stderr}")
-    return {"config": "floor: launch gap in a graph, and what a launch streams with the decode units' access pattern",
-            "one_tiny_kernel_us": graph_us(tiny, 200), "two_tiny_kernels_us": graph_us(pair, 100),
-            "probe_stream": done.stdout.splitlines()}
+    out = {}
+    for name, (m, k, n) in {"4096x4096x4096": (4096, 4096, 4096), "4096x5120x17408": (4096, 5120, 17408)}.items():
+        row = {}
+        for dtype in (torch.float16, torch.bfloat16):
+            gen = torch.Generator(device=DEV).manual_seed(3)
+            a = torch.randn((m, k), generator=gen, device=DEV).to(dtype)
+            # weight copies cycled as in the other legs ([N, K] each, used transposed, as a linear layer holds them)
+            ws = [(torch.randn((n, k), generator=gen, device=DEV) * 0.05).to(dtype) for _ in range(6)]
+            y = torch.empty((m, n), dtype=dtype, device=DEV)
+            us = graph_us(lambda i: torch.matmul(a, ws[i % len(ws)].t(), out=y), 12)
+            flop = 2.0 * m * n * k
+            row[str(dtype).split(".")[-1]] = {"us": us, "tflops": flop / us * 1e-6, "frac_mfma": flop / us * 1e-6 / MFMA}
+            del ws
+            torch.cuda.empty_cache()
+        out[name] = row
+    return {"config": "cal: torch.matmul (the vendor's tuned GEMM) at the prompt kernels' sizes, same timing method",
+            "bound": "mfma", "sizes": out}
 
 
 def timeline() -> dict:
@@ -416,7 +395,7 @@ def timeline() -> dict:
         layer = b.Layer(tokens, tables, DEV)
         layer.route_plans()
         plan = layer.plans[2]
-        with _lib.through(build.TIMELINE_LIB) as tl:
+        with _lib.through(build.timeline_lib()) as tl:
             for name, fn in (("route_up", lambda i: layer.up(i, plan)), ("down_combine", lambda i: layer.down(i, plan))):
                 fn(0)
                 torch.cuda.synchronize()
@@ -480,7 +459,7 @@ def timeline() -> dict:
         y = torch.empty((*lead, 1, n), dtype=torch.float16, device=DEV)
         xh = torch.empty((*lead, 1, k), dtype=torch.float16, device=DEV)
         z = torch.empty((stacked * 16 * n,), dtype=torch.float32, device=DEV)
-        with _lib.through(build.TIMELINE_LIB) as tl:
+        with _lib.through(build.timeline_lib()) as tl:
             layers[0](x, y, xh=xh, z=z)
             torch.cuda.synchronize()
             if tl.tf_timeline_clear_exl3():
@@ -563,7 +542,7 @@ def timeline_c2() -> dict:
            "topk_us": graph_us(lambda i: moe.select_rows(logits[i % 4], bufs[i % 4], s.top_k, s.experts), 32),
            "up_us": graph_us(up, 32), "down_us": graph_us(down, 32), "launches": {}}
     marks = 6
-    with _lib.through(build.TIMELINE_LIB) as tl:
+    with _lib.through(build.timeline_lib()) as tl:
         for name, fn in (("up", up), ("down", down)):
             fn(0)
             torch.cuda.synchronize()
@@ -606,7 +585,7 @@ def main() -> int:
     torch.cuda.set_device(0)
     which = sys.argv[1:] or ["c0", "c2", "c3", "c4"]
     for name in which:
-        res = {"mfma": mfma, "c0": c0, "c2": c2, "c3": c3, "c4": c4, "c4p": c4p, "glue": glue_, "c4x": c4x, "floor": floor, "timeline": timeline, "timeline_c2": timeline_c2}[name]()
+        res = {"c0": c0, "c2": c2, "c3": c3, "c4": c4, "c4p": c4p, "glue": glue_, "c4x": c4x, "cal": cal, "timeline": timeline, "timeline_c2": timeline_c2}[name]()
         torch.cuda.empty_cache()
         print(json.dumps(res, default=lambda v: round(v, 4)), flush=True)
     return 0

@@ -105,6 +105,9 @@ int tf_qmm_group(const uint16_t* x, int64_t ldx, const float* xs, int count, con
 enum { TF_ARITH_F16 = 0, TF_ARITH_BF16 = 1 };
 
 /* Prompt-form matmul on MFMA: each weight rounded once (see TF_ARITH_*), one fp32 chain over K.
+ * tile: 0 = chosen from the row count (what kernels/qmm.py:202-205 `prompt_tile` stands for); 1, 4, 8 = the four-wave
+ * kernel on 16, 64 or 128 rows a workgroup; 9 = the eight-wave kernel (128 rows x 512 columns; fp16 arithmetic and K
+ * in whole steps of 64 only).  A row's bits are the same whatever the tile.
  * Replaces kernels/qmm.cpp:83-102 `qmm_prefill`. */
 int tf_qmm_prefill(const uint16_t* x, int64_t ldx, const uint32_t* weight, const uint16_t* scales,
                    const uint16_t* biases, void* out, int m, int n, int k, int gs, int f32, int tile, int arith,

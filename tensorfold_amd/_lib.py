@@ -78,11 +78,15 @@ _other: ctypes.CDLL | None = None
 
 @contextlib.contextmanager
 def through(path):
-    """Route ``call`` through another build of the library (the timeline build) inside the block; yields it."""
+    """Route ``call`` through another build of the library (the timeline build) inside the block; yields it.  The
+    other build must carry the digest of the sources beside it: one built before an entry point changed its
+    arguments would be called with shifted pointers."""
 
     global _other
     if not Path(path).exists():
-        raise RuntimeError(f"tensorfold-amd: {path} is missing: run `python -c 'import __graft_entry__ as g; g.build()'`")
+        raise RuntimeError(f"tensorfold-amd: {path} is missing (build.timeline_lib() builds the timeline library)")
+    if build.built_id(Path(path)) != build.source_id():
+        raise RuntimeError(f"tensorfold-amd: {path} was built from other sources than the ones beside it")
     _other = _declare(ctypes.CDLL(str(path)))
     try:
         yield _other

@@ -19,8 +19,6 @@ HERE = Path(__file__).resolve().parent
 CSRC = HERE / "csrc"
 LIB = HERE / "libtfmi.so"
 TIMELINE_LIB = HERE / "libtfmi_timeline.so"      # the same kernels with per-workgroup timestamps (see compile)
-PROBE = HERE / "probe_mfma"          # stand-alone measurement of the matrix instructions' issue rates (csrc/probe_mfma.hip)
-PROBE_STREAM = HERE / "probe_stream"  # what a launch streams with the decode units' access pattern (csrc/probe_stream.hip)
 SOURCES = ("api.hip", "pack.hip", "decode.hip", "fused.hip", "route.hip", "norm.hip", "prefill.hip", "prefill8.hip", "exl3.hip", "exl3_experts.hip")
 # packed-fp32 VALU forms are switched off for the device pass (the host pass warns that it does not know the feature)
 FLAGS = ("-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",
@@ -47,12 +45,12 @@ def source_id() -> str:
     return h.hexdigest()[:16]
 
 
-def built_id() -> str | None:
-    """The digest the library file carries (``tf_build_id``), read from the file without loading it."""
+def built_id(path: Path = LIB) -> str | None:
+    """The digest a library file carries (``tf_build_id``), read from the file without loading it."""
 
-    if not LIB.exists():
+    if not path.exists():
         return None
-    blob, mark = LIB.read_bytes(), b"TFMI_BUILD_ID="
+    blob, mark = path.read_bytes(), b"TFMI_BUILD_ID="
     at = blob.find(mark)
     return None if at < 0 else blob[at + len(mark):at + len(mark) + 16].decode(errors="replace")
 
@@ -65,10 +63,23 @@ def stale() -> bool:
     return built_id() != source_id()
 
 
+def timeline_lib() -> Path:
+    """``libtfmi_timeline.so`` for the sources beside it: built on request only (``bench_configs.py timeline*`` asks),
+    and again whenever its digest is not the sources'.  A timeline build of other sources is never loaded: its entry
+    points may take other arguments than the prototypes of this tree."""
+
+    if built_id(TIMELINE_LIB) != source_id():
+        if hipcc() is None:
+            raise RuntimeError(f"tensorfold-amd: {TIMELINE_LIB} is missing or was built from other sources, and there "
+                               "is no hipcc to build it")
+        compile(timeline=True)
+    return TIMELINE_LIB
+
+
 def compile(verbose: bool = False, timeline: bool = False) -> Path:
     """Compile every kernel for gfx950 into ``libtfmi.so`` (cross-compiles without a GPU): one hipcc per source,
     side by side, then a link.  ``timeline``: the same sources with -DTF_TIMELINE into ``libtfmi_timeline.so``, whose
-    decode expert kernels note per-workgroup timestamps (``bench_configs.py timeline`` reads them)."""
+    decode expert kernels note per-workgroup timestamps (an instrument: only ``timeline_lib`` builds it)."""
 
     import tempfile
     from concurrent.futures import ThreadPoolExecutor
@@ -96,10 +107,6 @@ def compile(verbose: bool = False, timeline: bool = False) -> Path:
             logs = list(pool.map(lambda so: run([cc, *compile_flags, "-c", str(CSRC / so[0]), "-o", so[1]]),
                                  zip(SOURCES, objects)))
         logs.append(run([cc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", str(target), *objects]))
-        if not timeline:
-            logs.append(run([cc, "-O3", f"--offload-arch={ARCH}", "-o", str(PROBE), str(CSRC / "probe_mfma.hip")]))
-            logs.append(run([cc, "-O3", f"--offload-arch={ARCH}", "-o", str(PROBE_STREAM),
-                             str(CSRC / "probe_stream.hip")]))
     if verbose:
         for text in logs:
             if text:

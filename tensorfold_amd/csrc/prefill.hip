@@ -671,8 +671,10 @@ int launch_experts_prefill(int tile, int arith, const uint16_t* x, int64_t x_str
   return 0;
 }
 
+// tile: 0 = chosen from the row count; 1, 4, 8 = the four-wave kernel on 16, 64 or 128 rows a workgroup; 9 = the
+// eight-wave kernel (128 rows x 512 columns; K in whole steps of 64).  The same bits whatever the tile.
 template <int GS, int EPI>
-int launch_qmm_prefill(int arith, const uint16_t* x, int64_t ldx, const uint32_t* w, const uint16_t* s,
+int launch_qmm_prefill(int arith, int tile, const uint16_t* x, int64_t ldx, const uint32_t* w, const uint16_t* s,
                        const uint16_t* b, void* out, int m, int n, int kg, hipStream_t st) {
   const int npad = (n + 127) / 128 * 128;
   const int ct = (n + 127) / 128;
@@ -680,15 +682,18 @@ int launch_qmm_prefill(int arith, const uint16_t* x, int64_t ldx, const uint32_t
   qmm_prefill_kernel<GS, EPI, RT_, AR_><<<(unsigned)(((m + 16 * RT_ - 1) / (16 * RT_)) * ct), 256, stage_bytes<RT_>(), \
                                           st>>>(x, ldx, w, s, b, out, m, n, kg, npad)
   TF_REQUIRE((int64_t)((m + 15) / 16) * ct <= 0x7FFFFFFF, "qmm_prefill: grid too large");
+  const bool big_ok = !arith && (kg * GS) % KSTEP == 0 && (int64_t)npad * kg * GS / 2 < (1ll << 32);
+  TF_REQUIRE(tile != 9 || big_ok, "qmm_prefill: tile 9 (the eight-wave kernel) takes the fp16 arithmetic and K in whole steps of 64");
+  const int rows = tile == 1 ? 16 : tile == 4 ? 64 : tile == 8 ? 128 : tile == 9 ? 129 : m;     // as if this many rows
   if (arith) {
-    if (m <= 16) TF_SMALL(1, 1);
-    else if (m <= 64) TF_SMALL(4, 1);
+    if (rows <= 16) TF_SMALL(1, 1);
+    else if (rows <= 64) TF_SMALL(4, 1);
     else TF_SMALL(8, 1);
-  } else if (m <= 16) {
+  } else if (rows <= 16) {
     TF_SMALL(1, 0);
-  } else if (m <= 64) {
+  } else if (rows <= 64) {
     TF_SMALL(4, 0);
-  } else if ((kg * GS) % KSTEP == 0 && (int64_t)npad * kg * GS / 2 < (1ll << 32)) {
+  } else if (big_ok && tile != 8) {
     const int64_t grid = (int64_t)((m + BIG_ROWS - 1) / BIG_ROWS) * ((n + 511) / 512);
     qmm_prefill_big_kernel<GS, EPI><<<(unsigned)grid, BIG_THREADS, 2 * BIG_ROWS * AROW, st>>>(x, ldx, w, s, b, out, m, n,
                                                                                             kg, npad);
@@ -734,14 +739,14 @@ extern "C" int tf_qmm_prefill(const uint16_t* x, int64_t ldx, const uint32_t* we
   clear_error();
   TF_REQUIRE(arith == TF_ARITH_F16 || arith == TF_ARITH_BF16, "prefill arithmetic %d: TF_ARITH_F16 or TF_ARITH_BF16", arith);
   TF_REQUIRE(gs == 32 || gs == 64, "groups of 32 or 64");
-  TF_REQUIRE(tile >= 0 && tile <= 11, "tile 0-11");
+  TF_REQUIRE(tile == 0 || tile == 1 || tile == 4 || tile == 8 || tile == 9, "qmm_prefill: tile 0 (chosen from the row count), 1, 4, 8 or 9, not %d", tile);
   TF_REQUIRE(x && weight && scales && biases && out && m >= 1 && n >= 1, "qmm_prefill: null pointer or empty shape");
   TF_REQUIRE(aligned16(x) && (m == 1 || ldx % 8 == 0), "x rows must start on 16-byte boundaries");
   TF_REQUIRE(k >= gs && k % gs == 0, "K splits into whole groups");
   hipStream_t s = as_stream(stream);
   const int kg = k / gs;
-  if (gs == 64) return f32 ? launch_qmm_prefill<64, 0>(arith, x, ldx, weight, scales, biases, out, m, n, kg, s)
-                           : launch_qmm_prefill<64, 3>(arith, x, ldx, weight, scales, biases, out, m, n, kg, s);
-  return f32 ? launch_qmm_prefill<32, 0>(arith, x, ldx, weight, scales, biases, out, m, n, kg, s)
-             : launch_qmm_prefill<32, 3>(arith, x, ldx, weight, scales, biases, out, m, n, kg, s);
+  if (gs == 64) return f32 ? launch_qmm_prefill<64, 0>(arith, tile, x, ldx, weight, scales, biases, out, m, n, kg, s)
+                           : launch_qmm_prefill<64, 3>(arith, tile, x, ldx, weight, scales, biases, out, m, n, kg, s);
+  return f32 ? launch_qmm_prefill<32, 0>(arith, tile, x, ldx, weight, scales, biases, out, m, n, kg, s)
+             : launch_qmm_prefill<32, 3>(arith, tile, x, ldx, weight, scales, biases, out, m, n, kg, s);
 }

@@ -22,14 +22,27 @@ PREFILL_TILE = 128    # default prompt item; the MFMA kernels also take 16 and 6
 SMALL = 1024          # a plan up to this many pairs is sorted by one workgroup
 _GROUPS = (32, 64)
 ARITH_F16, ARITH_BF16 = 0, 1      # TF_ARITH_* of the C header: the prompt form's operand arithmetic
-F16_TABLE_LIMIT = 255.9           # |scale| and |bias| below this ride the fp16 form (256 x stays finite in fp16)
+F16_TABLE_LIMIT = 255.9           # the fp16 form holds 256 w, so |w| below this stays finite in fp16
 
 
 def fits_f16(*tensors: torch.Tensor) -> bool:
-    """Whether every scale and bias given is finite and small enough for the prompt form's fp16 arithmetic (one
-    reduction and a host read: for load time)."""
+    """Whether the tables given as (scales, biases, scales, biases, ...) fit the prompt form's fp16 arithmetic, which
+    holds fp16(fma(q, 256 s, 256 b)) for every code q of 0..15: every scale finite and below the limit, and both ends
+    of every group's range of weights, b and 15 s + b, below it too (a few reductions and a host read: for load
+    time)."""
 
-    return all(bool(torch.isfinite(t).all()) and float(t.abs().max()) < F16_TABLE_LIMIT for t in tensors if t.numel())
+    if len(tensors) % 2:
+        raise ValueError("fits_f16 takes scales and biases in pairs")
+    for s, b in zip(tensors[::2], tensors[1::2]):
+        if not s.numel():
+            continue
+        s, b = s.float(), b.float()
+        top = 15.0 * s + b
+        if not bool(torch.isfinite(top).all()):
+            return False
+        if max(float(s.abs().max()), float(b.abs().max()), float(top.abs().max())) >= F16_TABLE_LIMIT:
+            return False
+    return True
 
 
 def block_words(gs: int) -> int:
@@ -119,10 +132,11 @@ class Experts:
 def make(up: list[tuple], down: tuple, gs: int, *, limit: float = 0.0, arith: int | None = None) -> Experts:
     """Pack a layer.  ``up`` = [(words, scales, biases)] for relu^2 or [gate, up] for SwiGLU; ``down`` one triple.
 
-    ``arith`` fixes the prompt form's arithmetic; left None it is the fp16 form unless a scale or bias of the layer
-    is too large for it (``fits_f16``), in which case the layer takes the reference's bf16 form.  The fp16 form also
-    clamps activations beyond +-65504: a layer whose prompt activations can exceed that (a wide relu^2) should be made
-    with ``arith=ARITH_BF16``."""
+    ``arith`` fixes the prompt form's arithmetic.  Left None, a gated (SwiGLU) layer takes the fp16 form unless a
+    group of one of its tables holds a weight too large for it (``fits_f16``); then, and for every relu^2 layer, it
+    is the reference's bf16 form.  The fp16 form clamps activations (and ``moe.run`` a prompt's pair outputs) beyond
+    +-65504, and a relu^2 activation passes that as soon as an up output passes 256, which no look at the tables
+    rules out; a caller who knows the activations of such a layer stay below may ask for ``arith=ARITH_F16``."""
 
     if len(up) not in (1, 2):
         raise ValueError("experts take a gate and an up projection, or an up projection alone")
@@ -130,7 +144,8 @@ def make(up: list[tuple], down: tuple, gs: int, *, limit: float = 0.0, arith: in
     table_up = torch.stack([pack(w, s, b, gs) for (w, s, b) in up], dim=3)
     table_down = pack(*down, gs).unsqueeze(3)
     if arith is None:
-        arith = ARITH_F16 if fits_f16(*[t for m in (*up, down) for t in m[1:]]) else ARITH_BF16
+        small = len(up) == 2 and fits_f16(*[t for m in (*up, down) for t in m[1:]])
+        arith = ARITH_F16 if small else ARITH_BF16
     return Experts(table_up, table_down, gs, ni, d, float(limit), int(arith))
 
 

@@ -35,6 +35,12 @@ class Q4:
     arith: int = 0       # the prompt form's arithmetic (TF_ARITH_*): 1 when a scale or bias does not fit the fp16 form
     _counters: torch.Tensor | None = dataclasses.field(default=None, init=False, repr=False, compare=False)
 
+    def __post_init__(self) -> None:
+        # made with the weight, never inside a matmul call (which may run under graph capture)
+        if self.weight.is_cuda:
+            self._counters = torch.zeros((-(-self.n // 64) * COUNTER_STRIDE,), dtype=torch.int32,
+                                         device=self.weight.device)
+
     def nbytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in (self.weight, self.scales, self.biases))
 
@@ -42,8 +48,8 @@ class Q4:
     def counters(self) -> torch.Tensor:
         """Arrival counters of the K slices, one a column tile of 64, each alone in 64 bytes; zero between calls.
         With them ``matmul`` on up to eight rows adds the slices up in its own launch.  Calls on one weight that
-        overlap in time (two streams) need a ``Q4`` of their own each (``dataclasses.replace`` shares the packed
-        tensors and starts with fresh counters)."""
+        overlap in time (two streams), or one weight given twice to ``matmul_group``, need a ``Q4`` of their own each
+        (``dataclasses.replace`` shares the packed tensors and starts with fresh counters)."""
 
         if self._counters is None:
             self._counters = torch.zeros((-(-self.n // 64) * COUNTER_STRIDE,), dtype=torch.int32, device=self.weight.device)
@@ -247,6 +253,9 @@ def matmul_group(x: torch.Tensor, qs: list[Q4], xs: torch.Tensor | None = None, 
         raise ValueError("matmul_group: x must be (M, K) bf16 with every weight's K")
     if any(q.gs != qs[0].gs for q in qs):
         raise ValueError("matmul_group: the weights must share a group size")
+    if len({id(q.counters) for q in qs}) != len(qs):
+        raise ValueError("matmul_group: a weight given twice would share its arrival counters with itself; "
+                         "give the second one as dataclasses.replace(q)")
     x = _check_x(x, qs[0], "matmul_group")
     m, gs, k = int(x.shape[0]), qs[0].gs, qs[0].k
     xs = group_sums(x, gs) if xs is None else xs
@@ -278,13 +287,28 @@ def matmul_group(x: torch.Tensor, qs: list[Q4], xs: torch.Tensor | None = None, 
     return outs
 
 
+def prompt_tile(m: int, n: int, k: int = 64, arith: int = 0) -> int:
+    """The prompt matmul's tile for ``m`` rows (cuda/kernels/qmm.py:202-205 names the reference's one tile, tuned for
+    its chip): 1, 4 or 8 = a four-wave workgroup on 16, 64 or 128 rows x 128 columns; 9 = eight waves on 128 rows x
+    512 columns, from 65 rows on, for the fp16 arithmetic and K in whole steps of 64.  What ``tile=0`` picks."""
+
+    if m <= 16:
+        return 1
+    if m <= 64:
+        return 4
+    return 9 if not arith and k % 64 == 0 else 8
+
+
 def prefill_matmul(x: torch.Tensor, q: Q4, *, f32: bool = False, tile: int = 0,
                    out: torch.Tensor | None = None, arith: int | None = None) -> torch.Tensor:
     """Prompt-form x @ W.T on MFMA: every weight is rounded once and K is one fp32 chain, so chunking a prompt never
     changes a row's bits (they differ from ``matmul``'s).  ``arith`` 0: fp16 operands (256 w rounded to fp16;
     activations beyond +-65504 are clamped); 1: the reference's bf16 operands (w rounded to bf16), slower, with
-    bf16's range; None: what ``pack`` found the weight's scales and biases to need."""
+    bf16's range; None: what ``pack`` found the weight's scales and biases to need.  ``tile``: 0 or a ``prompt_tile``
+    code; the bits are the same whatever the tile."""
 
+    if tile not in (0, 1, 4, 8, 9):
+        raise ValueError("prefill_matmul: tile 0, 1, 4, 8 or 9 (see prompt_tile)")
     x = _check_x(x, q, "prefill_matmul")
     m = int(x.shape[0])
     if out is None:

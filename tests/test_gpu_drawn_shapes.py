@@ -85,11 +85,15 @@ def test_routed_experts_both_forms(seed):
     assert torch.equal(outs[(64, "prompt")], outs[(128, "prompt")])
     sample = sorted(rnd.sample(range(rows), min(rows, 6)))
     t = lambda m: (u32(m[0]), bits16(m[1]), bits16(m[2]))
-    want = ora.bf16_from_bits(native.moe_layer(bits16(x[sample]), picks[sample].numpy(), wts[sample].numpy(),
-                                               t(up[0]) if swiglu else None, t(up[1]) if swiglu else t(up[0]),
-                                               t(down), gs))
+    def want(form):
+        return ora.bf16_from_bits(native.moe_layer(bits16(x[sample]), picks[sample].numpy(), wts[sample].numpy(),
+                                                   t(up[0]) if swiglu else None, t(up[1]) if swiglu else t(up[0]),
+                                                   t(down), gs, prefill=form))
+    # a relu^2 layer's prompt form is the reference's bf16 arithmetic (weights rounded to bf16 once, the oracle's
+    # form 2), which by itself sits past the bound from the unrounded weights; everything else against those
     for key, o in outs.items():
-        assert rel_l2(f32(o[sample]), want) <= TOL, key
+        bf16_form = key[1] == "prompt" and ex.arith == experts.ARITH_BF16
+        assert rel_l2(f32(o[sample]), want(2 if bf16_form else 0)) <= TOL, key
 
 
 @pytest.mark.parametrize("seed", range(10))

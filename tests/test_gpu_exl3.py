@@ -219,6 +219,40 @@ def test_an_mlp_in_three_launches(codebook, bits, split, mid):
         linear.Exl3MLP.of(layers[0], layers[1], layers[0])
 
 
+@pytest.mark.parametrize("m", [1, 8])
+def test_config4_mlp_at_full_size(m):
+    """benchmark configuration 4's whole MLP (5120 -> 17408 -> 5120, 3.0 bpw, default codebook, the splits the layers
+    choose for themselves) through ``Exl3MLP``, the three launches the benchmark times, straight against the oracle:
+    gate and up in full on the CPU, SwiGLU with the roundings of fp16 tensors, then a 1,024-column slice of the down
+    projection; rel-L2 <= 2e-3.  ``Exl3Stack`` on the same layers has gate's and up's bits (checked too)."""
+
+    d, width = 5120, 17408
+    tg, sug, svg = synthetic.exl3_layer(d, width, 3, 4301)
+    tu, suu, svu = synthetic.exl3_layer(d, width, 3, 4302)
+    td, sud, svd = synthetic.exl3_layer(width, d, 3, 4303)
+    layers = [linear.Exl3Linear.from_tensors(tg, sug, svg, "3inst"), linear.Exl3Linear.from_tensors(tu, suu, svu, "3inst"),
+              linear.Exl3Linear.from_tensors(td, sud, svd, "3inst")]
+    mlp = linear.Exl3MLP.of(*layers)
+    assert mlp.gate_up.split == (7, 4) and mlp.down.split == linear.Exl3Linear.from_tensors(td, sud, svd, "3inst").split
+    x = synthetic.activations(m, d, 4310 + m, 0.02, dtype=torch.float16)
+    kept = torch.empty((2, m, width), dtype=torch.float16, device="cuda")
+    got = mlp(x.cuda(), mid=kept)
+    assert torch.equal(linear.Exl3Stack.of(layers[:2])(x.cuda()), kept)
+    f16 = lambda a: a.astype(np.float16)
+    g = f16(native.exl3_linear(x.numpy(), tg.numpy(), sug.numpy(), svg.numpy(), 6, 0))
+    u = f16(native.exl3_linear(x.numpy(), tu.numpy(), suu.numpy(), svu.numpy(), 6, 0))
+    assert rel_l2(kept[0].float().cpu().numpy(), g.astype(np.float64)) <= 2e-3
+    assert rel_l2(kept[1].float().cpu().numpy(), u.astype(np.float64)) <= 2e-3
+    g32 = g.astype(np.float32)
+    act = f16(f16(g32 / (1.0 + np.exp(-g32))).astype(np.float32) * u.astype(np.float32))
+    assert np.isfinite(act).all() and float(np.abs(act).max()) > 1.0
+    want = native.exl3_linear(act, td.numpy()[:, :64], sud.numpy(), svd.numpy()[:1024], 6, 0)
+    out = got[:, :1024].float().cpu().numpy()
+    err = rel_l2(out, want)
+    print(f"config 4 MLP M={m}: rel-L2 {err:.2e}, max-abs {max_abs(out, want):.3e}")
+    assert err <= 2e-3
+
+
 def test_what_the_layer_refuses():
     g = Group.draw("3inst", 3)
     with pytest.raises(ValueError):                                  # no such codebook

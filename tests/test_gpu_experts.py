@@ -21,7 +21,10 @@ def build(case, seed):
     gs, swiglu, limit, e, d, ni, _ = case
     up = [synthetic.affine_general(ni, d, gs, seed + i, (e,)) for i in range(2 if swiglu else 1)]
     down = synthetic.affine_general(d, ni, gs, seed + 7, (e,))
-    ex = experts.make([tuple(t.to(DEV) for t in m) for m in up], tuple(t.to(DEV) for t in down), gs, limit=limit)
+    # a relu^2 layer is made for the bf16 prompt form unless told (its activations' range is not the tables' to
+    # know); these cases' activations are small, and the fp16 form is the one they pin
+    ex = experts.make([tuple(t.to(DEV) for t in m) for m in up], tuple(t.to(DEV) for t in down), gs, limit=limit,
+                      arith=experts.ARITH_F16)
     return ex, up, down
 
 
@@ -303,8 +306,11 @@ def test_prompt_experts_beyond_the_range_of_fp16():
     up, down = [table(ni, d, 150.0)], table(d, ni, 0.01)                 # only the up table is out of range
     ex = experts.make([tuple(t.to(DEV) for t in m) for m in up], tuple(t.to(DEV) for t in down), gs)
     assert ex.arith == experts.ARITH_BF16
-    fits = experts.make([tuple(t.to(DEV) for t in down)], tuple(t.to(DEV) for t in table(ni, ni, 0.01)), gs)
+    small = tuple(t.to(DEV) for t in down)
+    fits = experts.make([small, small], tuple(t.to(DEV) for t in table(ni, ni, 0.01)), gs)
     assert fits.arith == experts.ARITH_F16
+    # the same tables as a relu^2 layer: the bf16 form, whatever the tables (its activations are unbounded)
+    assert experts.make([small], tuple(t.to(DEV) for t in table(ni, ni, 0.01)), gs).arith == experts.ARITH_BF16
     x = (synthetic.activations(rows, d, 18).float() * 300).bfloat16()
     picks = torch.stack([torch.randperm(e, generator=g)[:3] for _ in range(rows)]).to(torch.int32)
     wts = torch.full((rows, 3), 1 / 3)
@@ -320,3 +326,76 @@ def test_prompt_experts_beyond_the_range_of_fp16():
     assert rel_l2(f32(y), y_ref) <= 2e-3
     print(f"bf16 prompt form: act rel-L2 {rel_l2(f32(act), ora.bf16_from_bits(act_ref)):.2e}, "
           f"y rel-L2 {rel_l2(f32(y), y_ref):.2e}, max-abs {max_abs(f32(y), y_ref):.3e}")
+
+
+def test_a_group_whose_weights_pass_256_takes_the_bf16_form():
+    """The fp16 prompt form holds fp16(256 (q s + b)): scales of 20 to 100 with small biases pass every test of the
+    scales and biases alone, but 15 s + b reaches 1,500 and 256 times that is past fp16.  Such a table must be made
+    for the bf16 form and its prompt outputs must be finite and the oracle's."""
+
+    from oracle import native
+    from tests.helpers import bits16
+
+    gs, e, d, ni, rows = 32, 5, 256, 128, 70
+    g = torch.Generator().manual_seed(29)
+
+    def table(n, k, lo, hi):
+        words = synthetic.affine_general(n, k, gs, n + k + 1, (e,))[0]
+        scales = (torch.rand((e, n, k // gs), generator=g) * (hi - lo) + lo).bfloat16()
+        return words, scales, (torch.rand((e, n, k // gs), generator=g) - 0.5).bfloat16()
+
+    wide, small = table(ni, d, 20.0, 100.0), table(d, ni, 0.002, 0.02)
+    assert not experts.fits_f16(wide[1], wide[2]) and experts.fits_f16(small[1], small[2])
+    assert not experts.fits_f16(torch.tensor([30.0]), torch.tensor([-100.0]))          # 15 s + b = 350
+    assert experts.fits_f16(torch.tensor([30.0]), torch.tensor([-240.0]))              # weights in [-240, 210]
+    dev = lambda m: tuple(t.to(DEV) for t in m)
+    ex = experts.make([dev(wide), dev(wide)], dev(small), gs)
+    assert ex.arith == experts.ARITH_BF16
+    from tensorfold_amd import qmm
+    q = qmm.pack(wide[0][0].to(DEV), wide[1][0].to(DEV), wide[2][0].to(DEV), gs)
+    assert q.arith == experts.ARITH_BF16
+    x = synthetic.activations(rows, d, 5, 0.02)
+    yq = qmm.prefill_matmul(x.to(DEV), q, f32=True)
+    assert torch.isfinite(yq).all()
+    picks = torch.stack([torch.randperm(e, generator=g)[:2] for _ in range(rows)]).to(torch.int32)
+    act, y, _ = run(ex, x.to(DEV), picks, prefill=True)
+    assert torch.isfinite(y).all() and torch.isfinite(act.float()).all()
+    tab = lambda m: (u32(m[0]), bits16(m[1]), bits16(m[2]))
+    wts = torch.full((rows, 2), 0.5)
+    _, act_ref, y_ref = native.moe_layer(bits16(x), picks.numpy(), wts.numpy(), tab(wide), tab(wide), tab(small), gs,
+                                         prefill=2, want_pairs=True)
+    assert rel_l2(f32(y), y_ref) <= 2e-3
+
+
+def test_relu2_prompt_activations_past_fp16():
+    """A relu^2 layer made without a word about its arithmetic (as the loader makes Nemotron-H's): up outputs beyond
+    256 square to activations beyond fp16's 65,504, and the prompt layer must carry them unclamped through the down
+    projection and the pair outputs: ``moe.run(prefill=True)`` against the oracle's bf16 prompt form."""
+
+    from oracle import native
+    from tensorfold_amd import moe
+    from tests.helpers import bits16
+
+    gs, ne, d, ni, rows, k = 64, 8, 256, 128, 48, 2
+    up = synthetic.affine(ni, d, gs, 41, (ne + 1,))               # expert `ne` is the shared one
+    down = synthetic.affine(d, ni, gs, 42, (ne + 1,))
+    dev = lambda m: tuple(t.to(DEV) for t in m)
+    ex = experts.make([dev(up)], dev(down), gs)
+    assert ex.arith == experts.ARITH_BF16
+    g = torch.Generator().manual_seed(43)
+    rr = (torch.randn((ne + 1, d), generator=g) * 0.0005).bfloat16()
+    x = (synthetic.activations(rows, d, 44).float() * 4000).bfloat16()
+    layer = moe.Routed(rr.to(DEV), ex, k)
+    out = moe.run(x.to(DEV), layer, prefill=True)
+    assert torch.isfinite(out.float()).all()
+    logits = moe.router(x.to(DEV), rr.to(DEV)).cpu().numpy()
+    picks, wts = orr.topk_rows(logits, ne, k, shared=True)
+    tab = lambda m: (u32(m[0]), bits16(m[1]), bits16(m[2]))
+    want, act_ref, y_ref = native.moe_layer(bits16(x), picks, wts, None, tab(up), tab(down), gs, prefill=2,
+                                            want_pairs=True)
+    big = float(ora.bf16_from_bits(act_ref).max())
+    assert big > 4 * 65504, big                                   # the case is the one the test is named for
+    assert float(np.abs(y_ref).max()) > 65504                     # and pair outputs that fp16 could not hold either
+    err = rel_l2(f32(out), ora.bf16_from_bits(want))
+    print(f"relu^2 prompt layer past fp16: largest activation {big:.3g}, rel-L2 {err:.2e}")
+    assert err <= 2e-3

@@ -63,3 +63,41 @@ def test_static_scratch_host_wrapper_and_limit():
     rc = so.tf_qmm_static(_lib.ptr(xb), xb.stride(0), _lib.ptr(xs), _lib.ptr(q.weight), _lib.ptr(q.scales),
                           _lib.ptr(q.biases), q.scales.stride(0), _lib.ptr(out), big, n, k, 16, gs, 64, 0, _lib.stream())
     assert rc != 0 and b"exceed" in so.tf_last_error()
+
+
+def test_static_scratch_allocates_nothing():
+    """What the entry point is for: calls of both paths (more than eight rows: split launch + reduce; up to eight:
+    one launch on the built-in counters) leave the device's free memory and torch's pools exactly where they were.
+    The built-in counters being back at zero shows in the runs of few-row calls above, which would sum wrongly
+    otherwise."""
+
+    n, k, gs = 1536, 4096, 64
+    q = qmm.pack(*(t.to(DEV) for t in synthetic.affine_general(n, k, gs, 78)), gs)
+    sk = qmm.split_k(n, k, gs)
+    so = _lib.lib()
+    cases = []
+    for rows in (40, 5):
+        x = synthetic.activations(rows, k, rows).to(DEV)
+        xs = qmm.group_sums(x, gs)
+        out = torch.empty((rows, n), device=DEV, dtype=torch.bfloat16)
+        cases.append((x, xs, out, rows, qmm.matmul(x, q, xs)))
+    stream = _lib.stream()
+
+    def run(x, xs, out, rows, _):
+        rc = so.tf_qmm_static(_lib.ptr(x), x.stride(0), _lib.ptr(xs), _lib.ptr(q.weight), _lib.ptr(q.scales),
+                              _lib.ptr(q.biases), q.scales.stride(0), _lib.ptr(out), rows, n, k, sk, gs,
+                              qmm.bucket(rows), 0, stream)
+        assert rc == 0, so.tf_last_error()
+
+    for c in cases:                      # first calls on this device: the array's address is looked up here
+        run(*c)
+    torch.cuda.synchronize()
+    before = (torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved())
+    for _ in range(20):
+        for c in cases:
+            run(*c)
+    torch.cuda.synchronize()
+    after = (torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved())
+    assert before == after, (before, after)
+    for c in cases:
+        assert torch.equal(c[2], c[4]), c[3]
