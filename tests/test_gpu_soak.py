@@ -54,24 +54,27 @@ def test_decode_layer_two_thousand_replays():
             with torch.cuda.graph(g):
                 fn()
             graphs.append(g)
-        layers.append((graphs, buf, ref, got, want))
+        # the graphs hold addresses, not references: everything they read or write lives as long as they do (entering
+        # a capture empties the allocator's cache, which would unmap a table freed before it)
+        layers.append((graphs, buf, ref, got, want, ex))
     for i in range(ROUNDS):
         x.copy_(xs[i % 16])
         l.copy_(ls[i % 17])
-        (g_fused, g_sep), buf, ref, got, want = layers[i % tables]
+        (g_fused, g_sep), buf, ref, got, want, _ = layers[i % tables]
         g_fused.replay()
         g_sep.replay()
         if not (torch.equal(got, want) and torch.equal(buf.y, ref.y) and torch.equal(buf.pick, ref.pick)):
             pytest.fail(f"replay {i}: the decode layer's bits differ from the separate kernels'")
     torch.cuda.synchronize()
-    for _, buf, _, _, _ in layers:
+    for _, buf, _, _, _, _ in layers:
         buf.check()
         assert not buf.fused(shape.gs)["counters"].any()          # every arrival counter is back at zero
 
 
 def test_dense_matmul_two_thousand_arrivals():
     """``tf_qmm`` on 1 to 8 rows with the weight's arrival counters (the last workgroup of a column tile adds the K
-    slices) against the split launch followed by its reduce launch, two weights in turn, new rows every call."""
+    slices) against the same call without counters, whose forms pass nothing between workgroups, two weights in
+    turn, new rows every call."""
 
     n, k, gs = 4096, 4096, 64
     qs = [qmm.pack(*(t.to(DEV) for t in synthetic.affine_general(n, k, gs, 7300 + i)), gs) for i in range(2)]
@@ -89,5 +92,5 @@ def test_dense_matmul_two_thousand_arrivals():
                   _lib.ptr(q.biases), q.scales.stride(0), _lib.ptr(want), _lib.ptr(part), None, 0, m, n, k, sk, gs,
                   qmm.bucket(m), 0, 1)
         if not torch.equal(got, want):
-            pytest.fail(f"call {i} ({m} rows): the arriving form's bits differ from the reduce launch's")
+            pytest.fail(f"call {i} ({m} rows): the arriving form's bits differ from the counter-less form's")
     assert not qs[0].counters.any() and not qs[1].counters.any()
