@@ -168,6 +168,17 @@ def run_batch(tokens: int, tables, steps: int, warmup: int, dev: str) -> dict:
     other_us = graph_us(other_path)
     fused_layer_us, split_layer_us = (layer_us, other_us) if moe.FUSED_DECODE else (other_us, layer_us)
 
+    def sliced_path(i: int) -> None:
+        saved = moe.SLICED_DECODE, moe.FUSED_DECODE
+        moe.SLICED_DECODE, moe.FUSED_DECODE = True, False
+        try:
+            layer.step(i)
+        finally:
+            moe.SLICED_DECODE, moe.FUSED_DECODE = saved
+
+    # the layer as ONE launch cut along the intermediate width (what moe.SLICED_DECODE selects)
+    sliced_layer_us = layer_us if moe.SLICED_DECODE and not moe.FUSED_DECODE else graph_us(sliced_path)
+
     # the two expert kernels by themselves: HIP events around back-to-back launches on the launch stream
     def kernel_us(fn) -> float:
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -198,7 +209,7 @@ def run_batch(tokens: int, tables, steps: int, warmup: int, dev: str) -> dict:
     return {
         "tokens": tokens, "layer_us": layer_us, "us_per_token": layer_us / tokens, "unique_experts": mean_u,
         "layer_bytes": algo, "layer_gbs": algo / layer_us * 1e-3, "layer_frac": algo / layer_us * 1e-3 / HBM_PEAK_GBS,
-        "fused_layer_us": fused_layer_us, "split_layer_us": split_layer_us, "up_kernel_us": up_us, "down_kernel_us": down_us, "fused_kernel_us": fused_us,
+        "fused_layer_us": fused_layer_us, "split_layer_us": split_layer_us, "sliced_layer_us": sliced_layer_us, "up_kernel_us": up_us, "down_kernel_us": down_us, "fused_kernel_us": fused_us,
         "fused_gbs": (u0 * 2 * half + act_bytes) / fused_us * 1e-3,
         "up_gbs": (u0 * half + act_bytes / 2) / up_us * 1e-3, "down_gbs": (u0 * half + act_bytes / 2) / down_us * 1e-3,
         "kernel_unique_experts": u0, "kernel_bytes": u0 * half,

@@ -226,6 +226,21 @@ int tf_moe_route_up(const float* logits, int64_t ldl, int rows, int experts, int
 int tf_moe_down_combine(int gs, const uint16_t* act, int rows, int slots, const uint32_t* down, int d, int ni,
                         const int32_t* desc, const float* wts, float* y, uint16_t* out, int32_t* arrive,
                         int max_items, tf_stream_t stream);
+/* The whole decode layer in ONE launch, cut along the intermediate width: tf_moe_route_up followed by
+ * tf_moe_down_combine, same outputs (pick, wts, members, items, counts, desc, act, y, out) and the same bits.  A
+ * workgroup takes (item of one or two pairs, 64 columns of ni): the up unit, then the part of the down projection those
+ * 64 activations feed, for all d columns; it leaves each group's term fp32 in `part` [pairs, d / 64, ni / gs, 64], and
+ * the workgroup that brings a (pair, 64 columns of d) cell its last group adds the terms in the down launch's order,
+ * the one that then completes a (token, 64 columns) cell adds the slots (nobody waits).  d and ni multiples of 64;
+ * `arrive` int32 [(pairs + rows) * (d / 64) * TF_ARRIVE_STRIDE], zero on entry and left at zero.  With logits the
+ * weights of a combine are taken from the token's logits again; with logits NULL pick and wts are inputs.  No
+ * counterpart in the reference, which splits a layer's intermediate width only across GPUs
+ * (families/nemotron_h/cuda/tp.py:38-51). */
+int tf_moe_decode_sliced(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared, int gs,
+                         int swiglu, const uint16_t* x, int64_t x_stride, const uint32_t* up, const uint32_t* down,
+                         int d, int ni, int32_t* pick, float* wts, int32_t* members, int32_t* items, int32_t* counts,
+                         int32_t* desc, uint16_t* act, float* y, uint16_t* out, float* part, int32_t* arrive,
+                         float limit, int max_items, tf_stream_t stream);
 /* The decode layer's routing in one launch (two past 16 rows: the top-k then runs a workgroup a row first), for
  * rows * (top_k + shared) <= 1024: tf_moe_topk and tf_experts_plan (tile 16), plus the item descriptors and the
  * zeroing of `zero` (n_zero ints: the counters of tf_moe_down_combine or tf_moe_decode_experts).  No counterpart in

@@ -33,6 +33,7 @@ PROTOTYPES = {
     "tf_experts_prefill": [I, I, P, L, I, P, I, I, P, P, P, P, I, F, L, I, I, P],
     "tf_moe_route_up": [P, L, I, I, I, I, I, I, P, L, P, I, I, P, P, P, P, P, P, P, F, I, P, I, P],
     "tf_moe_down_combine": [I, P, I, I, P, I, I, P, P, P, P, P, I, P],
+    "tf_moe_decode_sliced": [P, L, I, I, I, I, I, I, P, L, P, P, I, I, P, P, P, P, P, P, P, P, P, P, P, F, I, P],
     "tf_moe_route_decode": [P, L, I, I, I, I, P, P, P, P, P, P, P, I, P],
     "tf_moe_decode_experts": [I, I, P, L, I, I, P, P, I, I, P, P, P, P, P, P, P, P, P, F, I, P],
     "tf_moe_router": [P, L, P, P, I, I, I, P],

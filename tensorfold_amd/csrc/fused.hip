@@ -25,6 +25,8 @@ namespace {
 // loads in flight; past about 1,300 workgroups of the routing launch (about 1,700 of the down launch) eight waves
 // each no longer fit the chip at once and four are faster.
 int fused_waves(int64_t grid) { return grid < 768 ? 16 : grid < 2560 ? 8 : 4; }
+// the same for the one-launch layer cut along the intermediate width, whose units stream an up and a down part
+int sliced_waves(int64_t grid) { return grid < 384 ? 16 : grid < 1280 ? 8 : 4; }
 
 // An item's arrival counter sits alone in 256 bytes.  The 42 down units of an item poll it, and with the counters of
 // all items side by side (two cache lines for 48 items) a thousand polling workgroups queued on one memory channel,
@@ -156,6 +158,277 @@ __global__ void __launch_bounds__(WAVES * 64)
 }
 
 
+// ---- the whole layer in one launch, cut along the intermediate width --------------------------------------------------
+//
+// A unit = (item of one or two pairs, 64 columns of NI).  It runs the up unit as route_up_kernel does, keeps the 64
+// activations of its rows in LDS, and goes straight on to the part of the down projection those activations feed:
+// one group of inputs (two at groups of 32) of all of the expert's D columns, whose weights depend on nothing the
+// unit computes and are on their way before its up projection has been summed.  What it leaves is each group's term
+// t = fma(xs, b, P s) for every column of D: fp32 `part` [pair][64 columns of D][group][64], written through to
+// memory.  The unit that brings a (pair, 64 columns of D) cell its last group adds the terms up in the order the down
+// launch adds them (the groups of a K slice in turn, then the slices: gemv_stream with SEPG) and stores the pair's
+// output; the one that then completes a (token, 64 columns) cell adds the token's slots in slot order and writes
+// bf16: the bits of tf_moe_route_up + tf_moe_down_combine.  Nobody waits for anybody.
+//
+// Hand-offs are the last-arriver scheme of combine_cells.  To spread the adding-up over the units of an item instead
+// of leaving it all to whichever ends last, a unit starts its walk over the D columns at a place of its own and counts
+// each 64 columns in as it goes: the count for the columns of step k - 2 is issued at step k, after the wave has
+// waited for step k's weights, which it requested after the stores of step k - 2 (vector memory operations of a wave
+// complete in the order they were issued, so those stores have been acknowledged).
+
+struct SliceArgs {
+  const uint32_t* Wdown;
+  float* part;          // [pairs][D / 64][NI / gs][64]
+  float* y;             // [pairs][D]
+  uint16_t* out;        // [rows][D]
+  int* c1;              // arrival counts a (pair, 64 columns of D), TF_ARRIVE_STRIDE ints apart, zero between launches
+  int* c2;              // arrival counts a (token, 64 columns of D), likewise
+  const float* wts;     // the pairs' weights when the picks were given (no logits)
+};
+
+// The unit's inputs of one (64 columns of D): 64 / GS groups of one matrix.
+template <int GS>
+struct DownStage {
+  Stage<GS, 1> g[64 / GS];
+};
+
+// A wave's walk over the 64-column blocks of D: step k takes block (rot + wave + WAVES k) mod NBD2.
+template <int GS, int WAVES>
+struct DownWalk {
+  static constexpr int G1 = 64 / GS, BW = block_words(GS);
+  const uint32_t* wexp;        // the expert's down matrix
+  int NBd, NBD2, KGd, g0, ng, rot, wave, lane, n;
+  __device__ __forceinline__ int db(int k) const {
+    const int q = rot + wave + WAVES * k;
+    return q >= NBD2 ? q - NBD2 : q;
+  }
+  __device__ __forceinline__ bool col_ok(int k) const { return 2 * db(k) + (lane >> 5) < NBd; }
+  __device__ __forceinline__ void load(DownStage<GS>& s, int k) const {
+    const int nb = min(2 * db(k) + (lane >> 5), NBd - 1), c = lane & 31;
+    const uint32_t* blk = wexp + ((size_t)nb * KGd + g0) * BW;
+#pragma unroll
+    for (int gi = 0; gi < G1; ++gi) {
+      const uint32_t* b = blk + (size_t)(gi < ng ? gi : 0) * BW;
+#pragma unroll
+      for (int i = 0; i < GS / 32; ++i) s.g[gi].w[0][i] = ldg16(b + i * 128 + c * 4);
+      s.g[gi].s[0] = s.g[gi].b[0] = __builtin_nontemporal_load(b + 32 * GS / 8 + c);
+    }
+  }
+};
+
+// The terms of one step: t[r][gi] = fma(xs, b, P s) of row r and group gi for the lane's column.
+template <int GS, int RB>
+__device__ __forceinline__ void down_terms(const DownStage<GS>& s, const float (&sc)[RB][64 / GS],
+                                           float (&t)[RB][64 / GS]) {
+#pragma unroll
+  for (int gi = 0; gi < 64 / GS; ++gi) {
+    float p[1][RB];
+#pragma unroll
+    for (int r = 0; r < RB; ++r) p[0][r] = 0.f;
+#pragma unroll
+    for (int i = 0; i < GS / 32; ++i) chunk_dot<GS, 1, RB>(p, s.g[gi], i);
+#pragma unroll
+    for (int r = 0; r < RB; ++r) asm volatile("s_nop 2" : "+v"(p[0][r]));
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+      const float pq = fmaf(-128.f, sc[r][gi], p[0][r]);
+      const float scale = __uint_as_float(s.g[gi].s[0] << 16);
+      const float bias = __uint_as_float(s.g[gi].b[0] & 0xFFFF0000u);
+      t[r][gi] = group_term(pq, scale, sc[r][gi], bias);
+    }
+  }
+}
+
+// The groups' terms of one (pair, 64 columns) cell added up as the down launch adds them: the groups of a K slice in
+// turn from zero, then the slices in slice order.  src: the cell's terms [KG][64], already offset by the lane.
+__device__ __forceinline__ float slice_tree(const float* src, int KG) {
+  float total = 0.f, sacc = 0.f;
+  bool first = true;
+  int q = 0;
+  while (q < SLICES && slice_begin(q + 1, KG) == slice_begin(q, KG)) ++q;
+  int end = q < SLICES ? slice_begin(q + 1, KG) : -1;
+  for (int g0 = 0; g0 < KG; g0 += 16) {
+    float v[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) v[j] = ld_agent(src + (size_t)min(g0 + j, KG - 1) * 64);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      if (g0 + j >= KG) break;
+      sacc = __fadd_rn(sacc, v[j]);
+      if (g0 + j + 1 == end) {
+        total = first ? sacc : __fadd_rn(total, sacc);
+        first = false;
+        sacc = 0.f;
+        ++q;
+        while (q < SLICES && slice_begin(q + 1, KG) == slice_begin(q, KG)) ++q;
+        end = q < SLICES ? slice_begin(q + 1, KG) : -1;
+      }
+    }
+  }
+  return total;
+}
+
+// A unit's second half: every wave walks its share of D's 64-column blocks.
+template <int GS, int WAVES, int RB>
+__device__ __forceinline__ void down_slices(const DownWalk<GS, WAVES>& walk, DownStage<GS> (&st)[DEPTH], const int* pairs,
+                                            const uint32_t* actw, int slots, int D, int NU, const SliceArgs& sa,
+                                            const float* __restrict__ L, int64_t ldl, int NE, int TOPK, int shared) {
+  constexpr int G1 = 64 / GS, CH = GS / 32;
+  const int lane = walk.lane, n = walk.n, KG = walk.KGd, NBD2 = walk.NBD2;
+  int pr[RB];
+#pragma unroll
+  for (int r = 0; r < RB; ++r) pr[r] = pairs[r];
+  const int pr_lane = lane == 0 ? pr[0] : pr[RB - 1];
+  // the rows' 64 activations as the dot products want them, and their sums a group
+  float sc[RB][G1];
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d)
+#pragma unroll
+    for (int gi = 0; gi < G1; ++gi)
+#pragma unroll
+      for (int r = 0; r < RB; ++r)
+#pragma unroll
+        for (int i = 0; i < CH; ++i) st[d].g[gi].x[r][i] = actw[r * 32 + (gi * CH + i) * 16 + (lane & 15)];
+#pragma unroll
+  for (int r = 0; r < RB; ++r)
+#pragma unroll
+    for (int gi = 0; gi < G1; ++gi) sc[r][gi] = stage_row_sum<GS, 1>(st[0].g[gi], r);
+
+  auto bump = [&](int k) {
+    int v = 0;
+    if (lane < RB)
+      v = __hip_atomic_fetch_add(sa.c1 + ((size_t)pr_lane * NBD2 + walk.db(k)) * TF_ARRIVE_STRIDE, 1, __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_AGENT);
+    return v;
+  };
+  // bit RB k + r of `mine`: this wave's count completed the cell (pair r, block of step k).  The cells are added up
+  // after the walk, when the walk's registers are free.
+  unsigned long long mine = 0;
+  auto settle = [&](int k, int oldv) {
+#pragma unroll
+    for (int r = 0; r < RB; ++r)
+      if (__builtin_amdgcn_readlane(oldv, r) == NU - 1) mine |= 1ull << (RB * k + r);
+  };
+  int old[DEPTH] = {0, 0};
+  for (int k0 = 0; k0 < n; k0 += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      const int k = k0 + d;
+      if (k < n) {
+        float t[RB][G1];
+        down_terms<GS, RB>(st[d], sc, t);
+        // step k's weights are here, so everything this wave issued before requesting them is complete: the terms of
+        // step k - 2 are acknowledged and its count may go; the count issued at step k - 2 (for step k - 4) is back
+        asm volatile("" : "+v"(t[0][0]) : : "memory");
+        if (k >= 2 * DEPTH) settle(k - 2 * DEPTH, old[d]);
+        if (k >= DEPTH) old[d] = bump(k - DEPTH);
+        const int db = walk.db(k);
+        if (walk.col_ok(k)) {
+#pragma unroll
+          for (int r = 0; r < RB; ++r)
+#pragma unroll
+            for (int gi = 0; gi < G1; ++gi)
+              if (gi < walk.ng)
+                st_agent(sa.part + (((size_t)pr[r] * NBD2 + db) * KG + walk.g0 + gi) * 64 + lane, t[r][gi]);
+        }
+        __atomic_signal_fence(__ATOMIC_SEQ_CST);        // the refill below stays behind these stores
+        if (k + DEPTH < n) walk.load(st[d], k + DEPTH);
+      }
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0);
+  // what is still open: the counts issued at the last two steps, and the last two steps' own
+  for (int k = max(n - DEPTH, DEPTH); k < n; ++k) settle(k - DEPTH, (k & 1) ? old[1] : old[0]);
+  for (int k = max(n - DEPTH, 0); k < n; ++k) settle(k, bump(k));
+
+  // The cells this wave completed.  (pair p, block db) has all its groups: the pair's output; and if that completes
+  // the token's cell too, the token's.
+  while (mine) {
+    const int bit = __builtin_ctzll(mine);
+    mine &= mine - 1;
+    const int p = (RB == 2 && (bit & 1)) ? pr[RB - 1] : pr[0], db = walk.db(bit / RB);
+    const int col = db * 64 + lane;
+    const size_t cell = (size_t)p * NBD2 + db;
+    if (lane == 0) __hip_atomic_store(sa.c1 + cell * TF_ARRIVE_STRIDE, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const float yv = slice_tree(sa.part + cell * KG * 64 + lane, KG);
+    if (col < D) st_agent(sa.y + (size_t)p * D + col, yv);
+    __builtin_amdgcn_s_waitcnt(0);                    // the pair's output is acknowledged, then it counts
+    const int token = p / slots;
+    int done = 0;
+    if (lane == 0) {
+      int* c = sa.c2 + ((size_t)token * NBD2 + db) * TF_ARRIVE_STRIDE;
+      done = __hip_atomic_fetch_add(c, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == slots - 1;
+      if (done) __hip_atomic_store(c, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (!__builtin_amdgcn_readfirstlane(done)) continue;
+    // the token's weights: lane k holds slot k's
+    float w = 0.f;
+    if (L) {
+      int id;
+      topk_lane(L + (size_t)token * ldl, NE, TOPK, shared, lane, id, w);
+    } else if (lane < slots) {
+      w = sa.wts[(size_t)token * slots + lane];
+    }
+    float a = 0.f;
+    for (int k0 = 0; k0 < slots; k0 += 8) {
+      float v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int k = k0 + j < slots ? k0 + j : slots - 1;
+        v[j] = col < D ? ld_agent(sa.y + ((size_t)token * slots + k) * D + col) : 0.f;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (k0 + j < slots) a = fmaf(__shfl(w, k0 + j), v[j], a);
+    }
+    if (col < D) sa.out[(size_t)token * D + col] = (uint16_t)f32_bf16_bits(a);
+  }
+}
+
+// Up unit, then its part of the down projection (see above).  Every thread of the workgroup calls this.
+template <int GS, int NM, int EPI, int WAVES>
+__device__ __forceinline__ void sliced_unit(const uint16_t* __restrict__ X, int64_t x_stride, int slots,
+                                            const uint32_t* __restrict__ Wup, int D, int NI, int e, int cnt,
+                                            const int* pairs, int cb2, uint16_t* __restrict__ act, float limit, float* lds,
+                                            const SliceArgs& sa, const float* __restrict__ L, int64_t ldl, int NE,
+                                            int TOPK, int shared) {
+  __shared__ uint32_t actw[RBMAX * 32];
+  const int tid = threadIdx.x;
+  DownWalk<GS, WAVES> walk;
+  walk.NBd = D / 32;
+  walk.NBD2 = (walk.NBd + 1) >> 1;
+  walk.KGd = NI / GS;
+  walk.g0 = cb2 * (64 / GS);
+  walk.ng = min(64 / GS, walk.KGd - walk.g0);
+  const int NU = (NI / 32 + 1) >> 1;
+  walk.rot = (int)((long long)cb2 * walk.NBD2 / NU);
+  walk.wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  walk.lane = tid & 63;
+  walk.n = walk.wave < walk.NBD2 ? (walk.NBD2 - walk.wave + WAVES - 1) / WAVES : 0;
+  walk.wexp = sa.Wdown + (size_t)e * walk.NBd * walk.KGd * block_words(GS);
+  DownStage<GS> st[DEPTH];
+  struct Sink {
+    const DownWalk<GS, WAVES>& walk;
+    DownStage<GS> (&st)[DEPTH];
+    uint32_t* actw;
+    // the first steps of the down walk are requested before the up projection's sums meet
+    __device__ __forceinline__ void streamed() const {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d)
+        if (d < walk.n) walk.load(st[d], d);
+    }
+    __device__ __forceinline__ void act(int r, int l, uint32_t bits) const {
+      reinterpret_cast<uint16_t*>(actw)[r * 64 + l] = (uint16_t)bits;
+    }
+  } sink{walk, st, actw};
+  NoHook none;
+  expert_unit<GS, NM, EPI, WAVES, 0>(X, x_stride, slots, Wup, D / GS, NI / 32, e, cnt, pairs, cb2, act, NI, limit, lds, none,
+                                     sink);
+  __syncthreads();          // the rows' activations are in LDS
+  if (cnt == 2) down_slices<GS, WAVES, 2>(walk, st, pairs, actw, slots, D, NU, sa, L, ldl, NE, TOPK, shared);
+  else down_slices<GS, WAVES, 1>(walk, st, pairs, actw, slots, D, NU, sa, L, ldl, NE, TOPK, shared);
+}
+
 // ---- routing and the up projection in one launch -------------------------------------------------------------------
 //
 // Workgroup 0 writes the routing's outputs (picks, weights, members, items, counts, item descriptors) for the kernels
@@ -163,13 +436,13 @@ __global__ void __launch_bounds__(WAVES * 64)
 // to learn which expert and which pairs its item holds, then runs the up unit.  The routing's launch and its trip
 // through memory are gone; the price is about a microsecond of arithmetic at the head of each workgroup.
 
-template <int GS, int NM, int EPI, int WAVES>
+template <int GS, int NM, int EPI, int WAVES, bool SLICED = false>
 __global__ void __launch_bounds__(WAVES * 64)
     route_up_kernel(const float* __restrict__ L, int64_t ldl, int R, int NE, int TOPK, int shared,
                     const uint16_t* __restrict__ X, int64_t x_stride, const uint32_t* __restrict__ Wup, int D, int NI,
                     int* __restrict__ pick, float* __restrict__ wts, int* __restrict__ members,
                     int* __restrict__ items, int* __restrict__ counts, int* __restrict__ desc,
-                    uint16_t* __restrict__ act, float limit, int* __restrict__ zero, int n_zero) {
+                    uint16_t* __restrict__ act, float limit, int* __restrict__ zero, int n_zero, SliceArgs sa) {
   extern __shared__ float lds[];
   __shared__ int pk[PLAN_THREADS];
   __shared__ ItemLds item;
@@ -178,6 +451,17 @@ __global__ void __launch_bounds__(WAVES * 64)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, threads = WAVES * 64;
   const int slots = TOPK + (shared ? 1 : 0), P = R * slots, E = NE + (shared ? 1 : 0);
   const bool writer = blockIdx.x == 0;
+  // the workgroup's unit: the up projection alone, or (SLICED) with its part of the down projection behind it
+  auto unit = [&](int e, int cnt, const int* pairs, int cb2) {
+    if constexpr (SLICED) {
+      sliced_unit<GS, NM, EPI, WAVES>(X, x_stride, slots, Wup, D, NI, e, cnt, pairs, cb2, act, limit, lds, sa, L, ldl, NE,
+                                      TOPK, shared);
+    } else {
+      NoHook none;
+      expert_unit<GS, NM, EPI, WAVES, 0>(X, x_stride, slots, Wup, D / GS, NI / 32, e, cnt, pairs, cb2, act, NI, limit, lds,
+                                         none);
+    }
+  };
   auto keep = [&](int r, int id, float w) {
     if (lane < slots) {
       pk[r * slots + lane] = (unsigned)id < (unsigned)E ? id : -1;
@@ -219,9 +503,7 @@ __global__ void __launch_bounds__(WAVES * 64)
     }
     __syncthreads();
     if (item.sel[0] < 0) return;
-    NoHook none;
-    expert_unit<GS, NM, EPI, WAVES, 0>(X, x_stride, slots, Wup, D / GS, NI / 32, item.sel[0], 1, item.pairs, cb2,
-                                              act, NI, limit, lds, none);
+    unit(item.sel[0], 1, item.pairs, cb2);
     return;
   }
   if (L && !writer && R <= 64) {
@@ -234,9 +516,7 @@ __global__ void __launch_bounds__(WAVES * 64)
         : NE <= 512 ? pair_item<8, WAVES>(L, ldl, R, NE, TOPK, shared, slots, it, pk, item.sel, wavepairs[wave], e, cnt)
                     : pair_item<TOPK_VPL, WAVES>(L, ldl, R, NE, TOPK, shared, slots, it, pk, item.sel, wavepairs[wave], e, cnt);
     if (!live) return;
-    NoHook none;
-    expert_unit<GS, NM, EPI, WAVES, 0>(X, x_stride, slots, Wup, D / GS, NI / 32, e, cnt, wavepairs[wave], cb2, act,
-                                              NI, limit, lds, none);
+    unit(e, cnt, wavepairs[wave], cb2);
     return;
   }
   if (!L && !writer) {
@@ -245,9 +525,7 @@ __global__ void __launch_bounds__(WAVES * 64)
     if (it >= P) return;
     int e = 0, cnt = 0;
     if (!pair_item_given(pick, P, E, it, wavepairs[wave], e, cnt)) return;
-    NoHook none;
-    expert_unit<GS, NM, EPI, WAVES, 0>(X, x_stride, slots, Wup, D / GS, NI / 32, e, cnt, wavepairs[wave], cb2, act,
-                                              NI, limit, lds, none);
+    unit(e, cnt, wavepairs[wave], cb2);
     return;
   }
   for (int e = tid; e < E; e += threads) item.cnt[e] = 0;
@@ -359,17 +637,15 @@ __global__ void __launch_bounds__(WAVES * 64)
     return;
   }
   if (!find_item<DTILE, true>(item, pk, P, E, it)) return;
-  NoHook none;
   // the item's rows are summed group by group inside the unit (a pass at a time), under its first weight loads
-  expert_unit<GS, NM, EPI, WAVES, 0>(X, x_stride, slots, Wup, D / GS, NI / 32, item.sel[0], item.sel[2],
-                                            item.pairs, cb2, act, NI, limit, lds, none);
+  unit(item.sel[0], item.sel[2], item.pairs, cb2);
 }
 
-template <int GS, int NM, int EPI>
+template <int GS, int NM, int EPI, bool SLICED = false>
 int launch_route_up(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared, const uint16_t* x,
                     int64_t x_stride, const uint32_t* wup, int d, int ni, int* pick, float* wts, int* members,
                     int* items, int* counts, int* desc, uint16_t* act, float limit, int max_items, int* zero,
-                    int n_zero, hipStream_t stream) {
+                    int n_zero, hipStream_t stream, const SliceArgs& sa = SliceArgs{}) {
   const int nb2 = (ni / 32 + 1) / 2;
   // with the picks given, or logits of 2 to 64 rows, the workgroups go a pair (route_up_kernel), else an item
   const int64_t pairs = (int64_t)rows * (top_k + (shared ? 1 : 0));
@@ -380,17 +656,18 @@ int launch_route_up(const float* logits, int64_t ldl, int rows, int experts, int
   const size_t smem = sizeof(float) * (floats > 4 * EMAX ? floats : 4 * EMAX);
   TF_REQUIRE(smem <= 48 * 1024, "moe: %d input groups need %zu bytes of LDS", d / GS, smem);
   const dim3 g((unsigned)grid);
-#define TF_GO(W_)                                                                                                  \
-  route_up_kernel<GS, NM, EPI, W_><<<g, W_ * 64, smem, stream>>>(logits, ldl, rows, experts, top_k, shared, x, x_stride, \
-                                                                 wup, d, ni, pick, wts, members, items, counts, desc,  \
-                                                                 act, limit, zero, n_zero)
-  switch (fused_waves(2 * grid)) {
+#define TF_GO(W_)                                                                                              \
+  route_up_kernel<GS, NM, EPI, W_, SLICED><<<g, W_ * 64, smem, stream>>>(logits, ldl, rows, experts, top_k, shared, x, \
+                                                                         x_stride, wup, d, ni, pick, wts, members,    \
+                                                                         items, counts, desc, act, limit, zero,       \
+                                                                         n_zero, sa)
+  switch (SLICED ? sliced_waves(grid) : fused_waves(2 * grid)) {
     case 16: TF_GO(16); break;
     case 8: TF_GO(8); break;
     default: TF_GO(4);
   }
 #undef TF_GO
-  TF_LAUNCH_OK("tf_moe_route_up");
+  TF_LAUNCH_OK(SLICED ? "tf_moe_decode_sliced" : "tf_moe_route_up");
   return 0;
 }
 
@@ -482,6 +759,46 @@ extern "C" int tf_moe_route_up(const float* logits, int64_t ldl, int rows, int e
                                             members, items, counts, desc, act, limit, max_items, zero, n_zero, s)
                 : launch_route_up<32, 1, 1>(logits, ldl, rows, experts, top_k, shared, x, x_stride, up, d, ni, pick, wts,
                                             members, items, counts, desc, act, limit, max_items, zero, n_zero, s);
+}
+
+extern "C" int tf_moe_decode_sliced(const float* logits, int64_t ldl, int rows, int experts, int top_k, int shared, int gs,
+                                    int swiglu, const uint16_t* x, int64_t x_stride, const uint32_t* up,
+                                    const uint32_t* down, int d, int ni, int32_t* pick, float* wts, int32_t* members,
+                                    int32_t* items, int32_t* counts, int32_t* desc, uint16_t* act, float* y,
+                                    uint16_t* out, float* part, int32_t* arrive, float limit, int max_items,
+                                    tf_stream_t stream) {
+  clear_error();
+  TF_REQUIRE(gs == 32 || gs == 64, "moe: groups of 32 or 64 inputs, not %d", gs);
+  TF_REQUIRE(x && up && down && pick && wts && members && items && counts && desc && act && y && out && part && arrive,
+             "moe: null pointer argument");
+  TF_REQUIRE(experts >= 1 && experts + (shared ? 1 : 0) <= EMAX && experts <= 64 * TOPK_VPL,
+             "route: at most %d experts", EMAX - 1);
+  TF_REQUIRE(top_k >= 1 && top_k + (shared ? 1 : 0) <= 64 && top_k <= experts, "route: 1 to 64 slots a row, not %d",
+             top_k);
+  TF_REQUIRE(rows >= 1 && (int64_t)rows * (top_k + (shared ? 1 : 0)) <= PLAN_THREADS,
+             "route: the decode routing takes at most %d pairs", PLAN_THREADS);
+  TF_REQUIRE(!logits || ldl >= experts + (shared ? 1 : 0), "route: logits rows are too short");
+  TF_REQUIRE(d % 64 == 0 && ni % 64 == 0 && d % gs == 0 && ni % gs == 0 && d >= gs && max_items >= 1,
+             "moe: the sliced decode layer takes hidden and intermediate sizes that are multiples of 64");
+  TF_REQUIRE(d <= 8192, "moe: the sliced decode layer takes a hidden size of at most 8192, not %d", d);
+  TF_REQUIRE(aligned16(x) && x_stride % 8 == 0 && aligned16(up) && aligned16(down) && aligned16(act),
+             "x: rows of K = groups * group size inputs, 16-byte aligned");
+  hipStream_t s = as_stream(stream);
+  const int pairs = rows * (top_k + (shared ? 1 : 0));
+  SliceArgs sa;
+  sa.Wdown = down;
+  sa.part = part;
+  sa.y = y;
+  sa.out = out;
+  sa.c1 = arrive;
+  sa.c2 = arrive + (size_t)pairs * (d / 64) * TF_ARRIVE_STRIDE;
+  sa.wts = wts;
+#define TF_SL(GS_, NM_, EPI_)                                                                                          \
+  launch_route_up<GS_, NM_, EPI_, true>(logits, ldl, rows, experts, top_k, shared, x, x_stride, up, d, ni, pick, wts, \
+                                        members, items, counts, desc, act, limit, max_items, nullptr, 0, s, sa)
+  if (gs == 64) return swiglu ? TF_SL(64, 2, 2) : TF_SL(64, 1, 1);
+  return swiglu ? TF_SL(32, 2, 2) : TF_SL(32, 1, 1);
+#undef TF_SL
 }
 
 extern "C" int tf_moe_down_combine(int gs, const uint16_t* act, int rows, int slots, const uint32_t* down, int d, int ni,

@@ -169,6 +169,11 @@ __device__ __forceinline__ void chunk_dot(float (&p)[NM][RB], const Stage<GS, NM
 #undef TF_WORD
 }
 
+// A group's term by itself: fma(xs, b, P s), the product rounded once before the bias term joins it.
+__device__ __forceinline__ float group_term(float pq, float scale, float sc, float bias) {
+  return fmaf(sc, bias, __fmul_rn(pq, scale));
+}
+
 // One wave's share of a GEMV: groups [gA, gB) of NM matrices against RB rows.
 //   wq(g, m, i)     -> the lane's 16 bytes of chunk i of group g of matrix m
 //   sb(g, m, s, b)  -> the lane's column's scale and bias of that group, as loaded (see Stage)
@@ -176,8 +181,12 @@ __device__ __forceinline__ void chunk_dot(float (&p)[NM][RB], const Stage<GS, NM
 //   xsum(r, g)      -> row r's sum over group g (wave-uniform); with XIN the sums are taken from the staged inputs
 //   flush(g, acc)   -> called after group g has been added (wave-uniform); may park and clear acc
 // `st` holds the weights of groups gA .. gA + DEPTH - 1 on entry when `loaded`.
-template <int GS, int NM, int RB, int COH, bool XIN = false, bool BHI = false, int RBM, class WQ, class SB, class XS,
-          class FLUSH>
+// SEPG: a group's term is rounded by itself, t = fma(xs, b, P s), and added to the running sum (acc + t) instead of
+// being chained through it.  The down projection of the routed experts sums this way, so that a kernel that holds one
+// group of an expert's inputs (the decode layer cut along the intermediate width) can leave t for another workgroup
+// to add and arrive at the same bits.
+template <int GS, int NM, int RB, int COH, bool XIN = false, bool BHI = false, bool SEPG = false, int RBM, class WQ,
+          class SB, class XS, class FLUSH>
 __device__ __forceinline__ void gemv_stream(float (&acc)[NM][RB], Stage<GS, NM, RBM> (&st)[DEPTH], bool loaded,
                                             const WQ& wq, const SB& sb, const uint32_t* const (&xl)[RB],
                                             const XS& xsum, int gA, int gB, FLUSH& flush) {
@@ -219,7 +228,8 @@ __device__ __forceinline__ void gemv_stream(float (&acc)[NM][RB], Stage<GS, NM, 
             const float pq = fmaf(-128.f, sc, p[m][r]);
             const float scale = __uint_as_float(st[d].s[m] << 16);
             const float bias = __uint_as_float(BHI ? st[d].b[m] & 0xFFFF0000u : st[d].b[m] << 16);
-            acc[m][r] = fmaf(sc, bias, fmaf(pq, scale, acc[m][r]));
+            if constexpr (SEPG) acc[m][r] = __fadd_rn(acc[m][r], group_term(pq, scale, sc, bias));
+            else acc[m][r] = fmaf(sc, bias, fmaf(pq, scale, acc[m][r]));
           }
         }
         flush(g, acc);
@@ -236,13 +246,21 @@ __device__ __forceinline__ void gemv_stream(float (&acc)[NM][RB], Stage<GS, NM, 
 
 __device__ __forceinline__ int slice_begin(int s, int KG) { return (int)((long long)s * KG / SLICES); }
 
+// What a caller may hang on a unit (see expert_unit): `streamed()` runs in every wave once it has issued the last of
+// its own loads and before the workgroup meets to add the slices up; `act(r, l, bits)` receives the bf16 bits of
+// activation column l (of the unit's 64) of row r when the epilogue makes activations.
+struct NoSink {
+  __device__ __forceinline__ void streamed() const {}
+  __device__ __forceinline__ void act(int, int, uint32_t) const {}
+};
+
 // One pass of an item: RB of its rows (pairs[0 ..]) against the workgroup's 64 columns.
 // Each wave takes the sums of its groups' inputs from the dwords it reads for the dot products.
-template <int GS, int NM, int EPI, int WAVES, int RB, int COH, class WQ, class SB>
+template <int GS, int NM, int EPI, int WAVES, int RB, int COH, class WQ, class SB, class SINK>
 __device__ __forceinline__ void expert_pass(const uint16_t* __restrict__ X, int64_t x_stride, int slots, const WQ& wq,
                                             const SB& sb, int KG, int NB, int cb2, const int* pairs,
                                             void* __restrict__ out, int N, float limit, float* part,
-                                            Stage<GS, NM> (&st)[DEPTH], bool loaded, bool first_pass) {
+                                            Stage<GS, NM> (&st)[DEPTH], bool loaded, bool first_pass, SINK& sink) {
   constexpr int SPW = SLICES / WAVES;               // slices a wave
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   int pr[RB];
@@ -290,8 +308,10 @@ __device__ __forceinline__ void expert_pass(const uint16_t* __restrict__ X, int6
   const int gA = slice_begin(wave * SPW, KG), gB = slice_begin((wave + 1) * SPW, KG);
   auto no_sums = [](int, int) { return 0.f; };
   if (first_pass) TF_MARK(2);
-  gemv_stream<GS, NM, RB, COH, true, true>(acc, st, loaded, wq, sb, xl, no_sums, gA, gB, flush);
+  // the down projection (EPI 0) adds each group's term by itself: see gemv_stream
+  gemv_stream<GS, NM, RB, COH, true, true, EPI == 0>(acc, st, loaded, wq, sb, xl, no_sums, gA, gB, flush);
   TF_MARK(3);
+  sink.streamed();
   __syncthreads();
   TF_MARK(4);
   // a wave a row, a lane a column: the slices' sums in slice order, then the epilogue
@@ -319,6 +339,7 @@ __device__ __forceinline__ void expert_pass(const uint16_t* __restrict__ X, int6
     } else {
       const float o = round_bf16(EPI == 1 ? relu2(v[0]) : swiglu(v[0], v[NM - 1], limit));
       const uint32_t bits = __float_as_uint(o) >> 16;
+      sink.act(r, l, ok ? bits : 0u);
       if (COH & COH_OUT) {
         // two columns a dword, written by the even lane (N is even, rows are dword-aligned)
         const uint32_t hi = __shfl_down(bits, 1);
@@ -340,11 +361,11 @@ struct NoHook {
 // lands in.  `ready()` runs after the wave's first weights have been requested and before any activation is read
 // (the fused layer waits there for the item's activations); returning false abandons the unit.
 // lds: the slices' sums [SLICES][NM][RBMAX][64].
-template <int GS, int NM, int EPI, int WAVES, int COH, class HOOK>
+template <int GS, int NM, int EPI, int WAVES, int COH, class HOOK, class SINK = NoSink>
 __device__ __forceinline__ bool expert_unit(const uint16_t* __restrict__ X, int64_t x_stride, int slots,
                                             const uint32_t* __restrict__ W, int KG, int NB, int e, int cnt,
                                             const int* pairs, int cb2, void* __restrict__ out, int N, float limit,
-                                            float* lds, HOOK& ready) {
+                                            float* lds, HOOK& ready, SINK&& sink = SINK()) {
   constexpr int BW = block_words(GS);
   constexpr int SPW = SLICES / WAVES;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -370,7 +391,7 @@ __device__ __forceinline__ bool expert_unit(const uint16_t* __restrict__ X, int6
   int r0 = 0;
 #define TF_PASS(RB_)                                                                                                \
   expert_pass<GS, NM, EPI, WAVES, RB_, COH>(X, x_stride, slots, wq, sb, KG, NB, cb2, pairs + r0, out, N, limit, part, \
-                                            st, loaded, first_pass);                                                \
+                                            st, loaded, first_pass, sink);                                          \
   first_pass = false;                                                                                               \
   loaded = gB - gA <= DEPTH   /* a run that fits the stages stays in registers for the next pass */
   for (; r0 + 2 <= cnt; r0 += 2) {

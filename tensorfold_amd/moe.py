@@ -25,6 +25,10 @@ ROUTE_UP_LOGITS = 2048
 # With this set ``decode`` makes the whole routing (top-k, plan, group sums, descriptors) in launches of its own and
 # runs the up projection from its descriptors: one launch more, for callers that want the plan before the experts.
 ROUTING_LAUNCH = False
+# With this set ``decode`` runs the layer as ONE launch cut along the intermediate width (``tf_moe_decode_sliced``) when
+# the call has at most SLICED_ROWS rows (its scratch holds a term for every pair, input group and column); same bits.
+SLICED_DECODE = False
+SLICED_ROWS = 16
 # Item descriptors the routing launches leave for the decode expert kernels: rows of DESC_INTS int32, row 0 the
 # count; items of at most DESC_TILE pairs (TF_DESC_INTS / TF_DESC_TILE of the C header).
 DESC_INTS, DESC_TILE = 8, 2
@@ -94,10 +98,24 @@ class MoEBuffers:
                 out=torch.empty((self.rows, cfg.hidden_size), dtype=torch.bfloat16, device=dev))
         return self._fused[gs]
 
+    def sliced(self, gs: int) -> dict:
+        """Scratch of the one-launch form cut along the intermediate width, made on first use, for up to SLICED_ROWS
+        rows: a term for every (pair, 64 columns, input group, column) and the two levels of arrival counters."""
+
+        key = ("sliced", gs)
+        if key not in self._fused:
+            cfg, rows, blocks = self.cfg, min(self.rows, SLICED_ROWS), self.cfg.hidden_size // 64
+            self._fused[key] = dict(
+                part=torch.empty((rows * self.slots, blocks, cfg.moe_intermediate_size // gs, 64), dtype=torch.float32,
+                                 device=self.device),
+                arrive=torch.zeros(((rows * self.slots + rows) * blocks * ARRIVE_STRIDE,), dtype=torch.int32,
+                                   device=self.device))
+        return self._fused[key]
+
     def check(self) -> None:
         """Host-side look at the fused layer's status flag (synchronises): raises if a bounded wait ran out."""
 
-        if any(int(f["counters"][0]) for f in self._fused.values()):
+        if any(int(f["counters"][0]) for f in self._fused.values() if "counters" in f):
             raise RuntimeError("tensorfold-amd: the fused decode layer timed out waiting for its activations")
 
 
@@ -175,6 +193,17 @@ def decode(x: torch.Tensor, logits: torch.Tensor, ex: grouped.Experts, buf: MoEB
                   items)
         return out
     act = buf.act.view(-1, ex.width)
+    if SLICED_DECODE and n <= min(SLICED_ROWS, buf.rows):
+        sl = buf.sliced(ex.gs)
+        given = n * (experts + int(buf.shared)) > ROUTE_UP_LOGITS
+        if given:
+            select_rows(logits, buf, top_k, experts)
+        _lib.call("tf_moe_decode_sliced", None if given else _lib.ptr(logits), logits.stride(0), n, experts, top_k,
+                  int(buf.shared), ex.gs, int(ex.swiglu), _lib.ptr(x), x.stride(0), _lib.ptr(ex.up), _lib.ptr(ex.down),
+                  ex.dims, ex.width, _lib.ptr(buf.pick), _lib.ptr(buf.wts), _lib.ptr(plan.members), _lib.ptr(plan.items),
+                  _lib.ptr(plan.counts), _lib.ptr(f["desc"]), _lib.ptr(act), _lib.ptr(buf.y), _lib.ptr(out),
+                  _lib.ptr(sl["part"]), _lib.ptr(sl["arrive"]), ex.limit, items)
+        return out
     arrive = ctr.data_ptr() + 4 * (1 + f["items"])        # one arrival counter a (token, 64 columns) cell
     if ROUTING_LAUNCH:
         # the routing in a launch of its own, then up, down and combine from its item descriptors

@@ -266,7 +266,7 @@ def test_a_prompts_pair_outputs_in_fp16():
                                            # number of column pairs; 8 groups of 64
                                            (synthetic.MoEShape("short32", 448, 16, 192, 6, 32, True, True), 16, 64),
                                            (synthetic.MoEShape("short64", 1024, 40, 512, 8, 64, False, False), 40, 24)])
-@pytest.mark.parametrize("path", ["route_up", "topk_then_up", "route_then_up", "one_launch"])
+@pytest.mark.parametrize("path", ["route_up", "topk_then_up", "route_then_up", "one_launch", "sliced", "topk_then_sliced"])
 def test_the_fused_decode_layer_equals_the_separate_kernels(shape, ne, rows, path, monkeypatch):
     """The forms of ``decode`` (routing inside the up launch; a top-k launch, then the plan inside the up launch; a
     routing launch, then up, down, combine from its item descriptors; a routing launch and one launch for up + down +
@@ -275,7 +275,9 @@ def test_the_fused_decode_layer_equals_the_separate_kernels(shape, ne, rows, pat
 
     monkeypatch.setattr(moe, "FUSED_DECODE", path == "one_launch")
     monkeypatch.setattr(moe, "ROUTING_LAUNCH", path == "route_then_up")
-    monkeypatch.setattr(moe, "ROUTE_UP_LOGITS", 0 if path == "topk_then_up" else 1 << 30)
+    monkeypatch.setattr(moe, "ROUTE_UP_LOGITS", 0 if path.startswith("topk_then") else 1 << 30)
+    monkeypatch.setattr(moe, "SLICED_DECODE", path.endswith("sliced"))
+    monkeypatch.setattr(moe, "SLICED_ROWS", 64)
 
     up, down = layer_tables(shape, 1500, ne)
     ex = experts.make([tuple(t.to(DEV) for t in m) for m in up], tuple(t.to(DEV) for t in down), shape.gs)
@@ -352,12 +354,13 @@ def check_decode_forms(shape, ne, rows, seed, oracle=True, levels=0):
     experts.gate_up(x, ex, ref.plan, ref.act.view(-1, ex.width), rows)
     experts.down(ref.act.view(-1, ex.width), ex, ref.plan, ref.y.view(-1, ex.dims), rows)
     want = moe.combine(ref.y, ref.wts)
-    saved = moe.FUSED_DECODE, moe.ROUTE_UP_LOGITS, moe.ROUTING_LAUNCH
+    saved = moe.FUSED_DECODE, moe.ROUTE_UP_LOGITS, moe.ROUTING_LAUNCH, moe.SLICED_DECODE, moe.SLICED_ROWS
     try:
-        for path in ("route_up", "topk_then_up", "route_then_up", "one_launch"):
+        for path in ("route_up", "topk_then_up", "route_then_up", "one_launch", "sliced", "topk_then_sliced"):
             moe.FUSED_DECODE = path == "one_launch"
             moe.ROUTING_LAUNCH = path == "route_then_up"
-            moe.ROUTE_UP_LOGITS = 0 if path == "topk_then_up" else 1 << 30
+            moe.ROUTE_UP_LOGITS = 0 if path.startswith("topk_then") else 1 << 30
+            moe.SLICED_DECODE, moe.SLICED_ROWS = path.endswith("sliced"), 1024
             buf = moe.MoEBuffers(rows, cfg, DEV, shared=shared)
             for _ in range(2):
                 got = moe.decode(x, l, ex, buf, top_k, ne)
@@ -368,7 +371,7 @@ def check_decode_forms(shape, ne, rows, seed, oracle=True, levels=0):
                 assert torch.equal(buf.act, ref.act) and torch.equal(buf.y, ref.y), path
                 assert torch.equal(got, want), path
     finally:
-        moe.FUSED_DECODE, moe.ROUTE_UP_LOGITS, moe.ROUTING_LAUNCH = saved
+        moe.FUSED_DECODE, moe.ROUTE_UP_LOGITS, moe.ROUTING_LAUNCH, moe.SLICED_DECODE, moe.SLICED_ROWS = saved
     picks, _ = orr.topk_rows(l.cpu().numpy(), ne, top_k, shared=shared)
     assert np.array_equal(ref.pick.cpu().numpy(), picks)
     if oracle:
