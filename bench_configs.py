@@ -78,6 +78,9 @@ def c0() -> dict:
     us = graph_us(lambda i: qmm.prefill_matmul(x, copies[i % len(copies)], out=y), 12)
     flop = 2.0 * m * n * k
     prompt = {"rows": m, "us": us, "tflops": flop / us * 1e-6, "frac_mfma": flop / us * 1e-6 / MFMA}
+    # the reference's own prompt arithmetic on the same kernel: w = bf16(fma(q, s, b)), bf16 matrix instruction
+    us_b = graph_us(lambda i: qmm.prefill_matmul(x, copies[i % len(copies)], out=y, arith=1), 12)
+    prompt["bf16_arithmetic"] = {"us": us_b, "tflops": flop / us_b * 1e-6, "frac_mfma": flop / us_b * 1e-6 / MFMA}
     # the FP8 prompt path on the same weight: the rows quantized to e4m3 (a launch of its own), then the matmul; and
     # at groups of 32, where the per-group fma weighs twice as much
     xq = qmm.quantize_rows(x, 64)
@@ -158,10 +161,14 @@ def c2() -> dict:
             "down_gbs": uniq[0] * per_expert / 3 / down_us * 1e-3}
 
 
-def c3(tiles=((64, torch.float32), (128, torch.float32), ("128_y_bf16", torch.bfloat16), ("128_y_f16", torch.float16))) -> dict:
+def c3(tiles=((64, torch.float32), (128, torch.float32), ("128_y_bf16", torch.bfloat16), ("128_y_f16", torch.float16),
+             ("128_bf16_arithmetic", torch.bfloat16))) -> dict:
     s, rows = synthetic.C2, 4096
     gen = torch.Generator(device=DEV).manual_seed(3)
-    ex = moe_tables(s, 1, gen)[0]
+    ex_f16 = moe_tables(s, 1, gen)[0]
+    import dataclasses
+    # the same tables on the reference's prompt arithmetic (bf16 weights, bf16 pair outputs: cuda/moe.py:99)
+    ex_bf16 = dataclasses.replace(ex_f16, arith=experts.ARITH_BF16)
     x = synthetic.activations(rows, s.hidden, 1301).to(DEV)
     ids = synthetic.zipf_picks(rows, s.experts, s.top_k, 1302)
     picks = torch.cat([ids, torch.full((rows, 1), s.experts, dtype=torch.int32)], 1).contiguous().to(DEV)
@@ -174,6 +181,7 @@ def c3(tiles=((64, torch.float32), (128, torch.float32), ("128_y_bf16", torch.bf
     # with fp16 ones: the same bytes at an eighth of the rounding
     for tile, ydt in tiles:
         key, tile = tile, 128 if isinstance(tile, str) else tile
+        ex = ex_bf16 if key == "128_bf16_arithmetic" else ex_f16
         plan = experts.Plan(rows, slots, s.experts + 1, DEV, prefill=True)
         act = torch.empty((rows * slots, s.width), dtype=torch.bfloat16, device=DEV)
         y = torch.empty((rows * slots, s.hidden), dtype=ydt, device=DEV)

@@ -100,14 +100,14 @@ int tf_qmm_group(const uint16_t* x, int64_t ldx, const float* xs, int count, con
  *     holds 2e-3 relative L2 against dequant-then-matmul in fp32, and the fast one.
  *   TF_ARITH_BF16: the reference's own arithmetic - w = bf16(fma(q, s, b)) (round to nearest even), bf16 activations
  *     untouched, bf16 MFMA (kernels/qmm_prefill.cu:116-117, experts_prefill.cu:130-131).  bf16's range on both
- *     operands; runs on the four-wave kernel at every size, about half the speed.
+ *     operands; the same kernels (twice the vector instructions a weight: each is an fp32 fma rounded to bf16).
  * The Python wrappers choose TF_ARITH_BF16 by themselves for a table whose scales or biases do not fit the fp16 form. */
 enum { TF_ARITH_F16 = 0, TF_ARITH_BF16 = 1 };
 
 /* Prompt-form matmul on MFMA: each weight rounded once (see TF_ARITH_*), one fp32 chain over K.
  * tile: 0 = chosen from the row count (what kernels/qmm.py:202-205 `prompt_tile` stands for); 1, 4, 8 = the four-wave
- * kernel on 16, 64 or 128 rows a workgroup; 9 = the eight-wave kernel (128 rows x 512 columns; fp16 arithmetic and K
- * in whole steps of 64 only).  A row's bits are the same whatever the tile.
+ * kernel on 16, 64 or 128 rows a workgroup; 9 = the eight-wave kernel (128 rows x 512 columns; K in whole steps of
+ * 64 only).  A row's bits are the same whatever the tile.
  * Replaces kernels/qmm.cpp:83-102 `qmm_prefill`. */
 int tf_qmm_prefill(const uint16_t* x, int64_t ldx, const uint32_t* weight, const uint16_t* scales,
                    const uint16_t* biases, void* out, int m, int n, int k, int gs, int f32, int tile, int arith,

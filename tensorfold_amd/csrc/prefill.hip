@@ -379,7 +379,13 @@ struct DenseSource {
   }
 };
 
-template <int GS, int NM, int EPI, int RT, class WS, int TJ = 4, int NTHREADS = BIG_THREADS>
+// a column's stored (scale | bias << 16), from either source's form
+__device__ __forceinline__ uint32_t sb_raw(uint32_t v) { return v; }
+__device__ __forceinline__ uint32_t sb_raw(uint2 v) { return (v.x & 0xFFFFu) | (v.y << 16); }
+
+// AR: TF_ARITH_F16 (fp16 operands, weights scaled by 2^8) or TF_ARITH_BF16 (the reference's bf16(fma(q, s, b)) weights
+// and untouched bf16 activations on the bf16 matrix instruction): the operand bits of mfma_body's two forms.
+template <int GS, int NM, int EPI, int RT, int AR, class WS, int TJ = 4, int NTHREADS = BIG_THREADS>
 __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t x_stride, const WS& ws,
                                          const int (&ocol)[TJ], const bool (&jok)[TJ],
                                          int K, const int* src_rows, const int* dst_rows, int cnt,
@@ -411,9 +417,22 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
     for (int j = 0; j < PPT; ++j) {
       const int q = tid + j * NTHREADS;
       if (PIECES % NTHREADS == 0 || q < PIECES)
-        *reinterpret_cast<uint4*>(smem + buf * STAGE + (q >> 3) * AROW + (q & 7) * 16) = stage8(v[j]);
+        *reinterpret_cast<uint4*>(smem + buf * STAGE + (q >> 3) * AROW + (q & 7) * 16) =
+            AR ? stage8_bf16(v[j]) : stage8(v[j]);
     }
   };
+  // one packed word and its column's scale and bias -> the B operand's eight values, as bits
+  auto dequant = [](uint32_t w, SB sb) {
+    if constexpr (AR) return __builtin_bit_cast(u32x4_t, dequant8b(w, sb_raw(sb)));
+    else return __builtin_bit_cast(u32x4_t, dequant8h(w, sb_half2(sb)));
+  };
+  auto mfma = [](u32x4_t a, u32x4_t b, f32x4_t c) {
+    if constexpr (AR)
+      return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    else
+      return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  };
+  constexpr float UNSCALE = AR ? 1.f : WUNSCALE;
 
   f32x4_t acc[TJ][RT];
 #pragma unroll
@@ -430,9 +449,9 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
   load_w(min(1, last), wr[1], sr[1]);
   store_a(0, ar);
   // Software pipeline: the operands of the NEXT 32 inputs are dequantized under the MFMAs of these 32.
-  f16x8_t bcur[TJ];
+  u32x4_t bcur[TJ];
 #pragma unroll
-  for (int j = 0; j < TJ; ++j) bcur[j] = dequant8h(wr[0][j][0], sb_half2(sr[0][j][0]));
+  for (int j = 0; j < TJ; ++j) bcur[j] = dequant(wr[0][j][0], sr[0][j][0]);
   __syncthreads();
   for (int step0 = 0; step0 < steps; step0 += 2) {
 #pragma unroll
@@ -446,20 +465,20 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
         // activation operands are requested two row tiles before their MFMAs (an LDS read takes about as long as
         // one row tile's four MFMAs): operand t of the step is (chunk t / RT, row tile t % RT)
         auto read_a = [&](int t) {
-          return *reinterpret_cast<const f16x8_t*>(abuf + 16 * (t % RT) * AROW + (t / RT) * 64);
+          return *reinterpret_cast<const u32x4_t*>(abuf + 16 * (t % RT) * AROW + (t / RT) * 64);
         };
-        f16x8_t a = read_a(0), a1 = read_a(1);
+        u32x4_t a = read_a(0), a1 = read_a(1);
 #pragma unroll
         for (int i = 0; i < CPS; ++i) {
-          f16x8_t bnext[TJ];
+          u32x4_t bnext[TJ];
 #pragma unroll
           for (int r = 0; r < RT; ++r) {
             const int t = i * RT + r;
-            f16x8_t a2 = a1;
+            u32x4_t a2 = a1;
             if (t + 2 < CPS * RT) a2 = read_a(t + 2);
 #pragma unroll
             for (int j = 0; j < TJ; ++j)
-              acc[j][r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bcur[j], acc[j][r], 0, 0, 0);
+              acc[j][r] = mfma(a, bcur[j], acc[j][r]);
             a = a1;
             a1 = a2;
             // a share of the next chunk's dequantization rides along with each row tile
@@ -468,8 +487,8 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
             for (int jj = 0; jj < JPR; ++jj) {
               const int j = r * JPR + jj;
               if (j < TJ) {
-                if (i + 1 < CPS) bnext[j] = dequant8h(wr[u][j][i + 1], sb_half2(sr[u][j][(32 * (i + 1)) / GS]));
-                else bnext[j] = dequant8h(wr[1 - u][j][0], sb_half2(sr[1 - u][j][0]));
+                if (i + 1 < CPS) bnext[j] = dequant(wr[u][j][i + 1], sr[u][j][(32 * (i + 1)) / GS]);
+                else bnext[j] = dequant(wr[1 - u][j][0], sr[1 - u][j][0]);
               }
             }
             if (i + 2 == CPS && r * JPR + JPR >= TJ && (r - 1) * JPR + JPR < TJ)
@@ -496,11 +515,11 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
 #pragma unroll
         for (int j = 0; j < TJ / 2; ++j)
           if (jok[j])
-            store_out<EPI>(out, base + ocol[j], acc[j][r][i] * WUNSCALE, acc[j + TJ / 2][r][i] * WUNSCALE, limit);
+            store_out<EPI>(out, base + ocol[j], acc[j][r][i] * UNSCALE, acc[j + TJ / 2][r][i] * UNSCALE, limit);
       } else {
 #pragma unroll
         for (int j = 0; j < TJ; ++j)
-          if (jok[j]) store_out<EPI>(out, base + ocol[j], acc[j][r][i] * WUNSCALE, 0.f, limit);
+          if (jok[j]) store_out<EPI>(out, base + ocol[j], acc[j][r][i] * UNSCALE, 0.f, limit);
       }
     }
   }
@@ -509,7 +528,7 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
 // 32-column blocks a workgroup of the big kernel covers
 constexpr int big_blocks(int nm) { return nm == 2 ? BIG_WAVES : 2 * BIG_WAVES; }
 
-template <int GS, int NM, int EPI>
+template <int GS, int NM, int EPI, int AR>
 __global__ void __launch_bounds__(BIG_THREADS, 1)
     experts_prefill_big_kernel(const uint16_t* __restrict__ X, int64_t x_stride, int slots,
                                const uint32_t* __restrict__ W, int KG, int NB, const int* __restrict__ items,
@@ -548,13 +567,13 @@ __global__ void __launch_bounds__(BIG_THREADS, 1)
     ocol[j] = nb * 32 + toff + c;
   }
   const int K = KG * GS;
-  if (cnt <= 32) big_body<GS, NM, EPI, 2>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
-  else if (cnt <= 64) big_body<GS, NM, EPI, 4>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
-  else big_body<GS, NM, EPI, 8>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
+  if (cnt <= 32) big_body<GS, NM, EPI, 2, AR>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
+  else if (cnt <= 64) big_body<GS, NM, EPI, 4, AR>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
+  else big_body<GS, NM, EPI, 8, AR>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
 }
 
 // The dense prompt matmul on the same pipeline: 128 rows x 512 columns a workgroup, a wave a 64-column tile.
-template <int GS, int EPI>
+template <int GS, int EPI, int AR>
 __global__ void __launch_bounds__(BIG_THREADS, 1)
     qmm_prefill_big_kernel(const uint16_t* __restrict__ X, int64_t ldx, const uint32_t* __restrict__ W,
                            const uint16_t* __restrict__ S, const uint16_t* __restrict__ B, void* __restrict__ out,
@@ -585,9 +604,9 @@ __global__ void __launch_bounds__(BIG_THREADS, 1)
     jok[j] = ok && col < N;
   }
   const int K = KG * GS;
-  if (cnt <= 32) big_body<GS, 1, EPI, 2>(X, ldx, ws, ocol, jok, K, rows, rows, cnt, out, N, 0.f, smem);
-  else if (cnt <= 64) big_body<GS, 1, EPI, 4>(X, ldx, ws, ocol, jok, K, rows, rows, cnt, out, N, 0.f, smem);
-  else big_body<GS, 1, EPI, 8>(X, ldx, ws, ocol, jok, K, rows, rows, cnt, out, N, 0.f, smem);
+  if (cnt <= 32) big_body<GS, 1, EPI, 2, AR>(X, ldx, ws, ocol, jok, K, rows, rows, cnt, out, N, 0.f, smem);
+  else if (cnt <= 64) big_body<GS, 1, EPI, 4, AR>(X, ldx, ws, ocol, jok, K, rows, rows, cnt, out, N, 0.f, smem);
+  else big_body<GS, 1, EPI, 8, AR>(X, ldx, ws, ocol, jok, K, rows, rows, cnt, out, N, 0.f, smem);
 }
 
 // ---- dense prompt matmul --------------------------------------------------------------------------------------------
@@ -648,23 +667,29 @@ int launch_experts_prefill(int tile, int arith, const uint16_t* x, int64_t x_str
 #define TF_SMALL(RT_, AR_)                                                                                              \
   experts_prefill_kernel<GS, NM, EPI, RT_, AR_><<<g, b, stage_bytes<RT_>(), s>>>(x, x_stride, slots, w, kg, nb, items, \
                                                                                counts, members, out, n, limit)
-  if (arith) {
-    // the bf16 form runs on the four-wave kernel at every item size
-    if (tile == 16) TF_SMALL(1, 1);
-    else if (tile == 64) TF_SMALL(4, 1);
-    else TF_SMALL(8, 1);
-  } else if (tile == 16) {
-    TF_SMALL(1, 0);
+  if (tile == 16) {
+    if (arith) TF_SMALL(1, 1);
+    else TF_SMALL(1, 0);
   } else if ((kg * GS) % KSTEP) {
     // a K that is not whole steps of 64 (odd group counts at g32): the small kernel's tail handling
-    if (tile == 64) TF_SMALL(4, 0);
-    else TF_SMALL(8, 0);
+    if (tile == 64) {
+      if (arith) TF_SMALL(4, 1);
+      else TF_SMALL(4, 0);
+    } else {
+      if (arith) TF_SMALL(8, 1);
+      else TF_SMALL(8, 0);
+    }
   } else {
     constexpr int NBW = big_blocks(NM);
     const int64_t big = max_items * ((nb + NBW - 1) / NBW);
     TF_REQUIRE(big <= 0x7FFFFFFF, "experts: %lld workgroups exceed the grid limit", (long long)big);
-    experts_prefill_big_kernel<GS, NM, EPI><<<dim3((unsigned)big), BIG_THREADS, 2 * BIG_ROWS * AROW, s>>>(
-        x, x_stride, slots, w, kg, nb, items, counts, members, out, n, limit);
+    const dim3 bg((unsigned)big);
+    if (arith)
+      experts_prefill_big_kernel<GS, NM, EPI, 1><<<bg, BIG_THREADS, 2 * BIG_ROWS * AROW, s>>>(
+          x, x_stride, slots, w, kg, nb, items, counts, members, out, n, limit);
+    else
+      experts_prefill_big_kernel<GS, NM, EPI, 0><<<bg, BIG_THREADS, 2 * BIG_ROWS * AROW, s>>>(
+          x, x_stride, slots, w, kg, nb, items, counts, members, out, n, limit);
   }
 #undef TF_SMALL
   TF_LAUNCH_OK("tf_experts_prefill");
@@ -682,21 +707,23 @@ int launch_qmm_prefill(int arith, int tile, const uint16_t* x, int64_t ldx, cons
   qmm_prefill_kernel<GS, EPI, RT_, AR_><<<(unsigned)(((m + 16 * RT_ - 1) / (16 * RT_)) * ct), 256, stage_bytes<RT_>(), \
                                           st>>>(x, ldx, w, s, b, out, m, n, kg, npad)
   TF_REQUIRE((int64_t)((m + 15) / 16) * ct <= 0x7FFFFFFF, "qmm_prefill: grid too large");
-  const bool big_ok = !arith && (kg * GS) % KSTEP == 0 && (int64_t)npad * kg * GS / 2 < (1ll << 32);
-  TF_REQUIRE(tile != 9 || big_ok, "qmm_prefill: tile 9 (the eight-wave kernel) takes the fp16 arithmetic and K in whole steps of 64");
+  const bool big_ok = (kg * GS) % KSTEP == 0 && (int64_t)npad * kg * GS / 2 < (1ll << 32);
+  TF_REQUIRE(tile != 9 || big_ok, "qmm_prefill: tile 9 (the eight-wave kernel) takes K in whole steps of 64");
   const int rows = tile == 1 ? 16 : tile == 4 ? 64 : tile == 8 ? 128 : tile == 9 ? 129 : m;     // as if this many rows
-  if (arith) {
-    if (rows <= 16) TF_SMALL(1, 1);
-    else if (rows <= 64) TF_SMALL(4, 1);
-    else TF_SMALL(8, 1);
-  } else if (rows <= 16) {
-    TF_SMALL(1, 0);
+  if (rows <= 16) {
+    if (arith) TF_SMALL(1, 1);
+    else TF_SMALL(1, 0);
   } else if (rows <= 64) {
-    TF_SMALL(4, 0);
+    if (arith) TF_SMALL(4, 1);
+    else TF_SMALL(4, 0);
   } else if (big_ok && tile != 8) {
-    const int64_t grid = (int64_t)((m + BIG_ROWS - 1) / BIG_ROWS) * ((n + 511) / 512);
-    qmm_prefill_big_kernel<GS, EPI><<<(unsigned)grid, BIG_THREADS, 2 * BIG_ROWS * AROW, st>>>(x, ldx, w, s, b, out, m, n,
-                                                                                            kg, npad);
+    const unsigned grid = (unsigned)((int64_t)((m + BIG_ROWS - 1) / BIG_ROWS) * ((n + 511) / 512));
+    if (arith)
+      qmm_prefill_big_kernel<GS, EPI, 1><<<grid, BIG_THREADS, 2 * BIG_ROWS * AROW, st>>>(x, ldx, w, s, b, out, m, n, kg, npad);
+    else
+      qmm_prefill_big_kernel<GS, EPI, 0><<<grid, BIG_THREADS, 2 * BIG_ROWS * AROW, st>>>(x, ldx, w, s, b, out, m, n, kg, npad);
+  } else if (arith) {
+    TF_SMALL(8, 1);
   } else {
     TF_SMALL(8, 0);
   }

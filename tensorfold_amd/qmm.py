@@ -287,16 +287,16 @@ def matmul_group(x: torch.Tensor, qs: list[Q4], xs: torch.Tensor | None = None, 
     return outs
 
 
-def prompt_tile(m: int, n: int, k: int = 64, arith: int = 0) -> int:
+def prompt_tile(m: int, n: int, k: int = 64) -> int:
     """The prompt matmul's tile for ``m`` rows (cuda/kernels/qmm.py:202-205 names the reference's one tile, tuned for
     its chip): 1, 4 or 8 = a four-wave workgroup on 16, 64 or 128 rows x 128 columns; 9 = eight waves on 128 rows x
-    512 columns, from 65 rows on, for the fp16 arithmetic and K in whole steps of 64.  What ``tile=0`` picks."""
+    512 columns, from 65 rows on, for K in whole steps of 64.  What ``tile=0`` picks."""
 
     if m <= 16:
         return 1
     if m <= 64:
         return 4
-    return 9 if not arith and k % 64 == 0 else 8
+    return 9 if k % 64 == 0 else 8
 
 
 def prefill_matmul(x: torch.Tensor, q: Q4, *, f32: bool = False, tile: int = 0,
