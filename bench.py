@@ -296,6 +296,11 @@ def other_configs() -> dict:
     out["c4"] = {"workload": r["config"], "bound": "hbm", "roofline_valu": rnd(r["rows"][1]["valu"]),
                  "rows": {str(m): {k: rnd(v) for k, v in d.items()} for m, d in r["rows"].items()}}
     torch.cuda.empty_cache()
+    # what the vendor's tuned plain GEMM reaches on this box at the prompt kernels' sizes, same timing method: the
+    # ceiling the two prompt fractions above can be read against beside the data sheet's peak
+    r = bc.cal()
+    out["calibration"] = {"workload": r["config"], "sizes": rnd(r["sizes"])}
+    torch.cuda.empty_cache()
     return out
 
 

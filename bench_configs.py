@@ -1,7 +1,7 @@
 """Kernel timings of the benchmark configurations that are not bench.py's headline: 0 (dense 4-bit projection),
 2 (verify-window MoE layer), 3 (prompt chunk, grouped MFMA) and 4 (EXL3 projections).
 
-    python bench_configs.py [c0] [c2] [c3] [c4] [c4p] [glue] [c4x] [cal] [timeline] [timeline_c2]
+    python bench_configs.py [c0] [c2] [c3] [c4] [c4p] [glue] [c4x] [cal] [timeline] [timeline_c2] [timeline_c3]
 
 One JSON line a configuration: time of one pass (hipGraph of back-to-back passes cycling over enough weight copies to
 miss the 256 MB Infinity Cache, HIP events around the replay), algorithmic bytes or flops, and the fraction of the
@@ -589,11 +589,90 @@ def timeline_c2() -> dict:
     return res
 
 
+def timeline_c3() -> dict:
+    """Per-workgroup marks of configuration 3's two expert launches (the eight-wave prompt kernel, items of 128, fp16
+    pair outputs) through the timeline build: 0 entry, 1 the item's rows known, 2 first operands staged (the loop
+    begins), 3 the loop over K done, 4 results issued, 5 results written.  By the item's rows: how long a workgroup
+    lives and where; by compute unit: the gap between one workgroup's end and the next one's entry, and when each
+    unit went idle for good (the launch's tail)."""
+
+    import ctypes
+
+    import numpy as np
+
+    from tensorfold_amd import _lib, build
+
+    s, rows = synthetic.C2, 4096
+    gen = torch.Generator(device=DEV).manual_seed(3)
+    ex = moe_tables(s, 1, gen)[0]
+    x = synthetic.activations(rows, s.hidden, 1301).to(DEV)
+    ids = synthetic.zipf_picks(rows, s.experts, s.top_k, 1302)
+    picks = torch.cat([ids, torch.full((rows, 1), s.experts, dtype=torch.int32)], 1).contiguous().to(DEV)
+    slots = s.top_k + 1
+    plan = experts.Plan(rows, slots, s.experts + 1, DEV, prefill=True)
+    act = torch.empty((rows * slots, s.width), dtype=torch.bfloat16, device=DEV)
+    y = torch.empty((rows * slots, s.hidden), dtype=torch.float16, device=DEV)
+    experts.route(picks, plan, 128)
+    experts.gate_up(x, ex, plan, act, rows)
+    torch.cuda.synchronize()
+    n_items = int(plan.counts[0])
+    counts = plan.items[:n_items, 2].cpu().numpy()
+    res = {"config": "timeline_c3: the prompt chunk's two expert launches, workgroup by workgroup", "items": n_items,
+           "marks": ["entry", "rows_known", "loop_begins", "loop_done", "results_issued", "results_written"],
+           "unit": "us", "launches": {}}
+    with _lib.through(build.timeline_lib()) as tl:
+        for name, fn, per_item in (("up", lambda: experts.gate_up(x, ex, plan, act, rows), 2),
+                                   ("down", lambda: experts.down(act, ex, plan, y, rows), 4)):
+            fn()
+            torch.cuda.synchronize()
+            if tl.tf_timeline_clear_prefill():
+                raise RuntimeError(tl.tf_last_error().decode())
+            fn()
+            torch.cuda.synchronize()
+            h = np.zeros((7, 16384), dtype=np.uint64)
+            if tl.tf_timeline_read_prefill(h.ctypes.data_as(ctypes.c_void_p), h.shape[0], h.shape[1]):
+                raise RuntimeError(tl.tf_last_error().decode())
+            hw, t = h[6], h[:6].astype(np.int64)
+            live = t[5] > 0
+            t0 = t[0][live].min()
+            us = (t[:, live] - t0) / 100.0
+            group = np.nonzero(live)[0]
+            item_rows = counts[np.minimum(group // per_item, n_items - 1)]
+            cu = ((hw[live] >> np.uint64(32)) << np.uint64(8)) | ((hw[live] >> np.uint64(8)) & np.uint64(0xFF))
+            row = {"workgroups": int(live.sum()), "span_us": float(us[5].max())}
+            med = lambda v: round(float(np.median(v)), 2)
+            by_rows = {}
+            for lo, hi in ((1, 16), (17, 32), (33, 64), (65, 127), (128, 128)):
+                m = (item_rows >= lo) & (item_rows <= hi)
+                if m.any():
+                    by_rows[f"{lo}-{hi}"] = {"workgroups": int(m.sum()), "life": med(us[5][m] - us[0][m]),
+                                             "head": med(us[2][m] - us[0][m]), "loop": med(us[3][m] - us[2][m]),
+                                             "issue_results": med(us[4][m] - us[3][m]),
+                                             "results_acknowledged": med(us[5][m] - us[4][m])}
+            row["by_item_rows"] = by_rows
+            gaps, idle_from, per_cu = [], [], []
+            for u in np.unique(cu):
+                m = cu == u
+                order = np.argsort(us[0][m])
+                begin, end = us[0][m][order], us[5][m][order]
+                gaps += list(begin[1:] - end[:-1])
+                idle_from.append(end.max())
+                per_cu.append(int(m.sum()))
+            row["gap_between_workgroups_on_a_unit"] = {"median": med(gaps), "p90": round(float(np.percentile(gaps, 90)), 2)}
+            idle = np.array(idle_from)
+            row["units"] = len(idle_from)
+            row["workgroups_a_unit"] = [min(per_cu), round(float(np.mean(per_cu)), 2), max(per_cu)]
+            row["unit_idle_before_the_end_us"] = {"mean": round(float((idle.max() - idle).mean()), 2),
+                                                   "p90": round(float(np.percentile(idle.max() - idle, 90)), 2)}
+            res["launches"][name] = row
+    return res
+
+
 def main() -> int:
     torch.cuda.set_device(0)
     which = sys.argv[1:] or ["c0", "c2", "c3", "c4"]
     for name in which:
-        res = {"c0": c0, "c2": c2, "c3": c3, "c4": c4, "c4p": c4p, "glue": glue_, "c4x": c4x, "cal": cal, "timeline": timeline, "timeline_c2": timeline_c2}[name]()
+        res = {"c0": c0, "c2": c2, "c3": c3, "c4": c4, "c4p": c4p, "glue": glue_, "c4x": c4x, "cal": cal, "timeline": timeline, "timeline_c2": timeline_c2, "timeline_c3": timeline_c3}[name]()
         torch.cuda.empty_cache()
         print(json.dumps(res, default=lambda v: round(v, 4)), flush=True)
     return 0

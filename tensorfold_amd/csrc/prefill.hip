@@ -122,11 +122,48 @@ __device__ __forceinline__ void store_out(void* out, size_t at, float a, float u
   else reinterpret_cast<uint16_t*>(out)[at] = (uint16_t)f32_bf16_bits(a);
 }
 
+// Which way round a tile comes out of the matrix instruction.  Activations first: D[row 4 kq + i][column c], a lane
+// holds one column of four rows.  Weights first (SWAP): D[column 4 kq + i][row c], a lane holds four consecutive
+// columns of one row, which leave as one 8- or 16-byte store and cost a quarter of the address arithmetic.  The
+// products and their order along K are the same.  Which form is faster is a matter of what the compiler makes of the
+// loop around it, so it is a parameter of the body and each kernel family takes what it measured best with: the dense
+// prompt matmul SWAP (4096 cubed: 149 -> 144 us with the fp16 arithmetic, 176 -> 141 us with the bf16 one), the
+// grouped expert kernels not (their pair outputs lose 7 % with it, the activation launch gains nothing).
+
+// Four consecutive columns of one row (a SWAP lane's share of a tile): one store where the row's length allows
+// (n a multiple of 4: the columns are whole and aligned), else element by element.  `at`: index of the first of the
+// four; `left`: columns from it to the row's end.
+template <int EPI>
+__device__ __forceinline__ void store4(void* out, size_t at, const float (&a)[4], const float (&u)[4], float limit,
+                                       int left, bool whole) {
+  if (left <= 0) return;
+  if (!whole) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (i < left) store_out<EPI>(out, at + i, a[i], u[i], limit);
+    return;
+  }
+  if constexpr (EPI == 0) {
+    *reinterpret_cast<float4*>(reinterpret_cast<float*>(out) + at) = make_float4(a[0], a[1], a[2], a[3]);
+  } else if constexpr (EPI == 4) {
+    auto h = [](float lo, float hi) {
+      const _Float16 l = (_Float16)fminf(fmaxf(lo, -65504.f), 65504.f), g = (_Float16)fminf(fmaxf(hi, -65504.f), 65504.f);
+      return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, g) << 16);
+    };
+    *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(out) + at) = make_uint2(h(a[0], a[1]), h(a[2], a[3]));
+  } else {
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = EPI == 1 ? relu2(a[i]) : EPI == 2 ? swiglu(a[i], u[i], limit) : a[i];
+    *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(out) + at) = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
+  }
+}
+
 // The shared body.  SRC gives, for the workgroup's item: rows(), src_row(r), dst_row(r); WSRC gives the lane's
 // packed word and its column's scale and bias.
 //   word(g, m, i, t): group g, matrix m, chunk i (32 inputs) of the group, column tile t (16 columns) of the wave
 //   sb(g, m, t): that column's stored (scale | bias << 16) pair of group g
-template <int GS, int NM, int EPI, int RT, int AR, class WSRC>
+template <int GS, int NM, int EPI, int RT, int AR, bool SWAP, class WSRC>
 __device__ __forceinline__ void mfma_body(const uint16_t* __restrict__ X, int64_t x_stride, int K, const WSRC& ws,
                                           const int* src_rows, int cnt, void* out, int N, int col0, int wave_cols_ok,
                                           const int* dst_rows, float limit, unsigned char* smem) {
@@ -227,12 +264,13 @@ __device__ __forceinline__ void mfma_body(const uint16_t* __restrict__ X, int64_
         for (int m = 0; m < NM; ++m)
 #pragma unroll
           for (int t = 0; t < 2; ++t) {
+            const u32x4_t first = SWAP ? bfrag[m][t] : a, second = SWAP ? a : bfrag[m][t];
             if constexpr (AR)
               acc[m][r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                  __builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, bfrag[m][t]), acc[m][r][t], 0, 0, 0);
+                  __builtin_bit_cast(bf16x8_t, first), __builtin_bit_cast(bf16x8_t, second), acc[m][r][t], 0, 0, 0);
             else
               acc[m][r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                  __builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, bfrag[m][t]), acc[m][r][t], 0, 0, 0);
+                  __builtin_bit_cast(f16x8_t, first), __builtin_bit_cast(f16x8_t, second), acc[m][r][t], 0, 0, 0);
           }
       }
     }
@@ -253,6 +291,29 @@ __device__ __forceinline__ void mfma_body(const uint16_t* __restrict__ X, int64_
     __syncthreads();
   }
   if (!wave_cols_ok) return;
+  if constexpr (SWAP) {
+    // a lane holds row 16 r + c, columns 16 t + 4 kq + (0..3) of each 16 x 16 tile
+    const bool whole = N % 4 == 0;
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+      if (r >= nt) break;
+      const int row = 16 * r + c;
+      if (row >= cnt) continue;
+      const size_t base = (size_t)dst_rows[row] * N;
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const int col = col0 + 16 * t + 4 * kq;
+        float a4[4], u4[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          a4[i] = acc[0][r][t][i] * (AR ? 1.f : WUNSCALE);
+          u4[i] = acc[NM - 1][r][t][i] * (AR ? 1.f : WUNSCALE);
+        }
+        store4<EPI>(out, base + col, a4, u4, limit, N - col, whole);
+      }
+    }
+    return;
+  }
   // D[row 4 kq + i][column c] of each 16 x 16 tile
 #pragma unroll
   for (int r = 0; r < RT; ++r) {
@@ -311,7 +372,7 @@ __global__ void __launch_bounds__(256)
   const uint32_t* blk = W + (((size_t)e * NB + (ok ? nb : NB - 1)) * KG) * (size_t)(NM * block_words(GS));
   ws.base = blk + c * 4 + kq;
   ws.sbase = blk + 32 * GS / 8 + c;
-  mfma_body<GS, NM, EPI, RT, AR>(X, x_stride, KG * GS, ws, src_rows, cnt, out, N, nb * 32, ok, dst_rows, limit, smem);
+  mfma_body<GS, NM, EPI, RT, AR, false>(X, x_stride, KG * GS, ws, src_rows, cnt, out, N, nb * 32, ok, dst_rows, limit, smem);
 }
 
 // ---- routed experts, big items ---------------------------------------------------------------------------------------
@@ -385,7 +446,7 @@ __device__ __forceinline__ uint32_t sb_raw(uint2 v) { return (v.x & 0xFFFFu) | (
 
 // AR: TF_ARITH_F16 (fp16 operands, weights scaled by 2^8) or TF_ARITH_BF16 (the reference's bf16(fma(q, s, b)) weights
 // and untouched bf16 activations on the bf16 matrix instruction): the operand bits of mfma_body's two forms.
-template <int GS, int NM, int EPI, int RT, int AR, class WS, int TJ = 4, int NTHREADS = BIG_THREADS>
+template <int GS, int NM, int EPI, int RT, int AR, bool SWAP, class WS, int TJ = 4, int NTHREADS = BIG_THREADS>
 __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t x_stride, const WS& ws,
                                          const int (&ocol)[TJ], const bool (&jok)[TJ],
                                          int K, const int* src_rows, const int* dst_rows, int cnt,
@@ -398,6 +459,9 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
   const int tid = threadIdx.x, lane = tid & 63, c = lane & 15, kq = lane >> 4;
   const int steps = K / KSTEP;
   typedef typename WS::SB SB;
+  bool tile_ok[TJ];          // the lane's tile j exists at all (lane 0 of the tile's row of 16 says)
+#pragma unroll
+  for (int j = 0; j < TJ; ++j) tile_ok[j] = SWAP ? __shfl(jok[j] ? 1 : 0, lane & 48) != 0 : jok[j];
   auto load_w = [&](int step, uint32_t (&w)[TJ][CPS], SB (&sb)[TJ][GPS]) { ws.load(step, w, sb); };
   // this thread's pieces of the activation tile: piece q = (row q / 8, 16 bytes q % 8)
   const uint16_t* asrc[PPT];
@@ -427,10 +491,11 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
     else return __builtin_bit_cast(u32x4_t, dequant8h(w, sb_half2(sb)));
   };
   auto mfma = [](u32x4_t a, u32x4_t b, f32x4_t c) {
+    const u32x4_t first = SWAP ? b : a, second = SWAP ? a : b;
     if constexpr (AR)
-      return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+      return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, first), __builtin_bit_cast(bf16x8_t, second), c, 0, 0, 0);
     else
-      return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+      return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, first), __builtin_bit_cast(f16x8_t, second), c, 0, 0, 0);
   };
   constexpr float UNSCALE = AR ? 1.f : WUNSCALE;
 
@@ -453,6 +518,7 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
 #pragma unroll
   for (int j = 0; j < TJ; ++j) bcur[j] = dequant(wr[0][j][0], sr[0][j][0]);
   __syncthreads();
+  TF_MARK(2);
   for (int step0 = 0; step0 < steps; step0 += 2) {
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
@@ -503,6 +569,32 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
       }
     }
   }
+  TF_MARK(3);
+  if constexpr (SWAP) {
+    // a lane holds row 16 r + c, columns 4 kq + (0..3) of each of the wave's 16-column tiles (ocol: the lane's column c
+    // of the tile, so the tile begins at ocol - c; for the dense weight jok says the lane's column exists, and with N a
+    // multiple of 4 the tile's columns from 4 kq on exist or not together)
+    const bool whole = N % 4 == 0;
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+      const int row = 16 * r + c;
+      if (row >= cnt) continue;
+      const size_t base = (size_t)dst_rows[row] * N;
+#pragma unroll
+      for (int j = 0; j < (NM == 2 ? TJ / 2 : TJ); ++j) {
+        const int col = ocol[j] - c + 4 * kq;
+        if (!tile_ok[j]) continue;
+        float a4[4], u4[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          a4[i] = acc[j][r][i] * UNSCALE;
+          u4[i] = NM == 2 ? acc[j + TJ / 2][r][i] * UNSCALE : 0.f;
+        }
+        store4<EPI>(out, base + col, a4, u4, limit, N - col, whole);
+      }
+    }
+    return;
+  }
   // D[row 4 kq + i][column c] of each 16 x 16 tile
 #pragma unroll
   for (int r = 0; r < RT; ++r) {
@@ -540,6 +632,7 @@ __global__ void __launch_bounds__(BIG_THREADS, 1)
   __shared__ int src_rows[BIG_ROWS], dst_rows[BIG_ROWS];
   const int nbt = (NB + NBW - 1) / NBW;
   const int it = blockIdx.x / nbt, cbt = blockIdx.x - it * nbt;
+  TF_MARK(0);
   if (it >= counts[0]) return;
   const int e = items[3 * it], first = items[3 * it + 1], cnt = min(items[3 * it + 2], BIG_ROWS);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, kq = lane >> 4;
@@ -549,6 +642,7 @@ __global__ void __launch_bounds__(BIG_THREADS, 1)
     src_rows[tid] = slots ? p / slots : p;
   }
   __syncthreads();
+  TF_MARK(1);
   // the wave's four B operands: (matrix, 32-column block, 16-column half)
   const uint32_t* We = W + (size_t)e * NB * KG * (size_t)(NM * BW);      // the expert's matrices (wave-uniform)
   ExpertSource<GS, NM> ws;
@@ -567,9 +661,14 @@ __global__ void __launch_bounds__(BIG_THREADS, 1)
     ocol[j] = nb * 32 + toff + c;
   }
   const int K = KG * GS;
-  if (cnt <= 32) big_body<GS, NM, EPI, 2, AR>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
-  else if (cnt <= 64) big_body<GS, NM, EPI, 4, AR>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
-  else big_body<GS, NM, EPI, 8, AR>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
+  if (cnt <= 32) big_body<GS, NM, EPI, 2, AR, false>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
+  else if (cnt <= 64) big_body<GS, NM, EPI, 4, AR, false>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
+  else big_body<GS, NM, EPI, 8, AR, false>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
+  TF_MARK(4);
+#ifdef TF_TIMELINE
+  __builtin_amdgcn_s_waitcnt(0);         // mark 5 is the results written, not only issued
+#endif
+  TF_MARK(5);
 }
 
 // The dense prompt matmul on the same pipeline: 128 rows x 512 columns a workgroup, a wave a 64-column tile.
@@ -604,9 +703,9 @@ __global__ void __launch_bounds__(BIG_THREADS, 1)
     jok[j] = ok && col < N;
   }
   const int K = KG * GS;
-  if (cnt <= 32) big_body<GS, 1, EPI, 2, AR>(X, ldx, ws, ocol, jok, K, rows, rows, cnt, out, N, 0.f, smem);
-  else if (cnt <= 64) big_body<GS, 1, EPI, 4, AR>(X, ldx, ws, ocol, jok, K, rows, rows, cnt, out, N, 0.f, smem);
-  else big_body<GS, 1, EPI, 8, AR>(X, ldx, ws, ocol, jok, K, rows, rows, cnt, out, N, 0.f, smem);
+  if (cnt <= 32) big_body<GS, 1, EPI, 2, AR, true>(X, ldx, ws, ocol, jok, K, rows, rows, cnt, out, N, 0.f, smem);
+  else if (cnt <= 64) big_body<GS, 1, EPI, 4, AR, true>(X, ldx, ws, ocol, jok, K, rows, rows, cnt, out, N, 0.f, smem);
+  else big_body<GS, 1, EPI, 8, AR, true>(X, ldx, ws, ocol, jok, K, rows, rows, cnt, out, N, 0.f, smem);
 }
 
 // ---- dense prompt matmul --------------------------------------------------------------------------------------------
@@ -648,7 +747,7 @@ __global__ void __launch_bounds__(256)
   ws.B = B + (ok ? col0 : 0) + c;
   ws.stride = npad;
   ws.KG = KG;
-  mfma_body<GS, 1, EPI, RT, AR>(X, ldx, KG * GS, ws, rows, cnt, out, N, col0, ok, rows, 0.f, smem);
+  mfma_body<GS, 1, EPI, RT, AR, true>(X, ldx, KG * GS, ws, rows, cnt, out, N, col0, ok, rows, 0.f, smem);
 }
 
 template <int RT>
@@ -736,6 +835,8 @@ int launch_qmm_prefill(int arith, int tile, const uint16_t* x, int64_t ldx, cons
 }  // namespace tf
 
 using namespace tf;
+
+TF_TIMELINE_EXPORT(prefill)
 
 extern "C" int tf_experts_prefill(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w,
                                   int kg, int nb, const int32_t* items, const int32_t* counts, const int32_t* members,
