@@ -124,11 +124,13 @@ __device__ __forceinline__ void store_out(void* out, size_t at, float a, float u
 
 // Which way round a tile comes out of the matrix instruction.  Activations first: D[row 4 kq + i][column c], a lane
 // holds one column of four rows.  Weights first (SWAP): D[column 4 kq + i][row c], a lane holds four consecutive
-// columns of one row, which leave as one 8- or 16-byte store and cost a quarter of the address arithmetic.  The
-// products and their order along K are the same.  Which form is faster is a matter of what the compiler makes of the
-// loop around it, so it is a parameter of the body and each kernel family takes what it measured best with: the dense
-// prompt matmul SWAP (4096 cubed: 149 -> 144 us with the fp16 arithmetic, 176 -> 141 us with the bf16 one), the
-// grouped expert kernels not (their pair outputs lose 7 % with it, the activation launch gains nothing).
+// columns of one row, which leave as one 8- or 16-byte store (or, STAGE_OUT, go to LDS as one write so that whole
+// rows leave side by side).  The products and their order along K are the same, and so are the bits (the kernels
+// of one family are tested equal across the forms).  Which form is faster is a matter of what the compiler makes of
+// the loop around it, so it is a parameter of the body and each instance takes what it measured best with, side by
+// side on one box: the dense prompt matmul SWAP (4096 cubed: 177 -> 141 us with the bf16 arithmetic, 144 -> 143 with
+// the fp16 one), the experts' down projection SWAP with STAGE_OUT (config 3: 232 -> 222 us), the experts' gate and up
+// neither (342 -> 350 us with them).
 
 // Four consecutive columns of one row (a SWAP lane's share of a tile): one store where the row's length allows
 // (n a multiple of 4: the columns are whole and aligned), else element by element.  `at`: index of the first of the
@@ -446,7 +448,8 @@ __device__ __forceinline__ uint32_t sb_raw(uint2 v) { return (v.x & 0xFFFFu) | (
 
 // AR: TF_ARITH_F16 (fp16 operands, weights scaled by 2^8) or TF_ARITH_BF16 (the reference's bf16(fma(q, s, b)) weights
 // and untouched bf16 activations on the bf16 matrix instruction): the operand bits of mfma_body's two forms.
-template <int GS, int NM, int EPI, int RT, int AR, bool SWAP, class WS, int TJ = 4, int NTHREADS = BIG_THREADS>
+template <int GS, int NM, int EPI, int RT, int AR, bool SWAP, class WS, int TJ = 4, int NTHREADS = BIG_THREADS,
+          bool STAGE_OUT = false>
 __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t x_stride, const WS& ws,
                                          const int (&ocol)[TJ], const bool (&jok)[TJ],
                                          int K, const int* src_rows, const int* dst_rows, int cnt,
@@ -571,6 +574,57 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
   }
   TF_MARK(3);
   if constexpr (SWAP) {
+    if (N % 32 == 0 && STAGE_OUT) {
+      // Whole lines out: a lane's four columns of each tile go to the wave's own corner of LDS (free now: the loop
+      // ended on a barrier) as one 8- or 16-byte write, and a row tile leaves as 16-byte pieces, a row's 32 or 64
+      // columns side by side.  What the element-wise stores cost is the lines they touch (64 a row tile and wave, 32
+      // bytes of each; a wave's stores take about 19 cycles a line): this way it is 8 or 16.
+      constexpr int ES = EPI == 0 ? 4 : 2;                       // bytes an element
+      constexpr int OJ = NM == 2 ? TJ / 2 : TJ;                  // 16-column tiles of output a wave
+      constexpr int OROW = 16 * OJ * ES + 16;                    // bytes of a staged row (padded against bank conflicts)
+      constexpr int CPR = 16 * OJ * ES / 16;                     // 16-byte pieces a row
+      static_assert(BIG_WAVES * 16 * OROW <= 2 * STAGE, "the output tiles of a workgroup's waves fit the activation stages");
+      unsigned char* mine = smem + (tid >> 6) * (16 * OROW);
+      const int col0 = ocol[0] - c;                              // the wave's first output column (its tiles are neighbours)
+      unsigned okmask = 0;
+#pragma unroll
+      for (int j = 0; j < OJ; ++j) okmask |= (tile_ok[j] ? 1u : 0u) << j;
+      unsigned char* obytes = reinterpret_cast<unsigned char*>(out);
+#pragma unroll
+      for (int r = 0; r < RT; ++r) {
+        if (16 * r >= cnt) break;
+#pragma unroll
+        for (int j = 0; j < OJ; ++j) {
+          unsigned char* at = mine + c * OROW + (16 * j + 4 * kq) * ES;
+          float v[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float a = acc[j][r][i] * UNSCALE, u = NM == 2 ? acc[j + TJ / 2][r][i] * UNSCALE : 0.f;
+            v[i] = EPI == 1 ? relu2(a) : EPI == 2 ? swiglu(a, u, limit) : EPI == 4 ? fminf(fmaxf(a, -65504.f), 65504.f) : a;
+          }
+          if constexpr (EPI == 0) {
+            *reinterpret_cast<float4*>(at) = make_float4(v[0], v[1], v[2], v[3]);
+          } else if constexpr (EPI == 4) {
+            auto h = [](float lo, float hi) {
+              return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lo) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)hi) << 16);
+            };
+            *reinterpret_cast<uint2*>(at) = make_uint2(h(v[0], v[1]), h(v[2], v[3]));
+          } else {
+            *reinterpret_cast<uint2*>(at) = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
+          }
+        }
+        // a wave's LDS operations run in the order it issued them: the reads below see the writes above
+#pragma unroll
+        for (int q0 = 0; q0 < 16 * CPR; q0 += 64) {
+          const int q = q0 + lane, rl = q / CPR, ch = q - rl * CPR, row = 16 * r + rl;
+          if (q < 16 * CPR && row < cnt && ((okmask >> ((ch * (16 / ES)) >> 4)) & 1u)) {
+            const uint4 v = *reinterpret_cast<const uint4*>(mine + rl * OROW + ch * 16);
+            *reinterpret_cast<uint4*>(obytes + ((size_t)dst_rows[row] * N + col0 + ch * (16 / ES)) * ES) = v;
+          }
+        }
+      }
+      return;
+    }
     // a lane holds row 16 r + c, columns 4 kq + (0..3) of each of the wave's 16-column tiles (ocol: the lane's column c
     // of the tile, so the tile begins at ocol - c; for the dense weight jok says the lane's column exists, and with N a
     // multiple of 4 the tile's columns from 4 kq on exist or not together)
@@ -660,10 +714,13 @@ __global__ void __launch_bounds__(BIG_THREADS, 1)
     ws.sp[j] = blk + 32 * GS / 8 + toff + c;
     ocol[j] = nb * 32 + toff + c;
   }
+  // one matrix (the down projection, whose outputs are the bulk of a chunk's stores): tiles weights-first and whole
+  // lines out through LDS (4 % of the launch); gate and up with the SwiGLU between them: neither (3 % the other way)
+  constexpr bool OUT_LINES = NM == 1;
   const int K = KG * GS;
-  if (cnt <= 32) big_body<GS, NM, EPI, 2, AR, false>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
-  else if (cnt <= 64) big_body<GS, NM, EPI, 4, AR, false>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
-  else big_body<GS, NM, EPI, 8, AR, false>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
+  if (cnt <= 32) big_body<GS, NM, EPI, 2, AR, OUT_LINES, ExpertSource<GS, NM>, 4, BIG_THREADS, OUT_LINES>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
+  else if (cnt <= 64) big_body<GS, NM, EPI, 4, AR, OUT_LINES, ExpertSource<GS, NM>, 4, BIG_THREADS, OUT_LINES>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
+  else big_body<GS, NM, EPI, 8, AR, OUT_LINES, ExpertSource<GS, NM>, 4, BIG_THREADS, OUT_LINES>(X, x_stride, ws, ocol, jok, K, src_rows, dst_rows, cnt, out, N, limit, smem);
   TF_MARK(4);
 #ifdef TF_TIMELINE
   __builtin_amdgcn_s_waitcnt(0);         // mark 5 is the results written, not only issued
