@@ -171,7 +171,7 @@ int tf_experts_run_desc(int gs, int epi, const uint16_t* x, int64_t x_stride, in
 /* Prompt form on MFMA, each weight rounded once as in tf_qmm_prefill (arith: TF_ARITH_*); epi 3: bf16 out; epi 4: fp16 out, values beyond fp16's range stored as +-65504.  `tile` is
  * the plan's item size (16, 64 or 128).  Replaces experts.cpp:50-55 `prefill`. */
 int tf_experts_prefill(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg,
-                       int nb, const int32_t* items, const int32_t* counts, const int32_t* members, void* out, int n,
+                       int nb, const int32_t* items, int32_t* counts, const int32_t* members, void* out, int n,
                        float limit, int64_t max_items, int tile, int arith, tf_stream_t stream);
 
 /* ---- MoE glue (moe.py:23-151; Triton kernels in the reference) ------------------------------------------------------ */

@@ -448,18 +448,26 @@ __device__ __forceinline__ uint32_t sb_raw(uint2 v) { return (v.x & 0xFFFFu) | (
 
 // AR: TF_ARITH_F16 (fp16 operands, weights scaled by 2^8) or TF_ARITH_BF16 (the reference's bf16(fma(q, s, b)) weights
 // and untouched bf16 activations on the bf16 matrix instruction): the operand bits of mfma_body's two forms.
+struct NoStaged {
+  __device__ __forceinline__ void operator()() const {}
+};
+
+// `staged()` runs in every thread right after the barrier that ends the prologue: the first operands have arrived by
+// then, and with them (a wave's vector memory operations complete in issue order) whatever the caller requested
+// before calling, which it can put away there without a wait of its own.
 template <int GS, int NM, int EPI, int RT, int AR, bool SWAP, class WS, int TJ = 4, int NTHREADS = BIG_THREADS,
-          bool STAGE_OUT = false>
+          bool STAGE_OUT = false, class STAGED = NoStaged>
 __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t x_stride, const WS& ws,
                                          const int (&ocol)[TJ], const bool (&jok)[TJ],
                                          int K, const int* src_rows, const int* dst_rows, int cnt,
-                                         void* __restrict__ out, int N, float limit, unsigned char* smem) {
+                                         void* __restrict__ out, int N, float limit, unsigned char* smem,
+                                         STAGED&& staged = STAGED(), int thread = -1) {
   constexpr int CPS = KSTEP / 32, GPS = KSTEP / GS;
   constexpr int ROWS = 16 * RT;
   constexpr int PIECES = ROWS * 8;                // 16-byte pieces of a staged tile
   constexpr int PPT = (PIECES + NTHREADS - 1) / NTHREADS;
   constexpr int STAGE = BIG_ROWS * AROW;
-  const int tid = threadIdx.x, lane = tid & 63, c = lane & 15, kq = lane >> 4;
+  const int tid = thread < 0 ? (int)threadIdx.x : thread, lane = tid & 63, c = lane & 15, kq = lane >> 4;
   const int steps = K / KSTEP;
   typedef typename WS::SB SB;
   bool tile_ok[TJ];          // the lane's tile j exists at all (lane 0 of the tile's row of 16 says)
@@ -521,6 +529,7 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
 #pragma unroll
   for (int j = 0; j < TJ; ++j) bcur[j] = dequant(wr[0][j][0], sr[0][j][0]);
   __syncthreads();
+  staged();
   TF_MARK(2);
   for (int step0 = 0; step0 < steps; step0 += 2) {
 #pragma unroll
@@ -728,6 +737,145 @@ __global__ void __launch_bounds__(BIG_THREADS, 1)
   TF_MARK(5);
 }
 
+// The same units taken by workgroups that stay, one a compute unit (a unit = an item's 512 weight columns, as a
+// workgroup of experts_prefill_big_kernel takes).  A workgroup has a compute unit to itself (the body's registers), so
+// in the kernel above nothing runs under a unit's head (the item's rows looked up through two dependent reads, then
+// the first operands' trip), its results' drain, and the dispatch of the next workgroup; and with five or six
+// workgroups of 47 to 67 us to a compute unit, those that got five sit idle for the last tenth of the launch.  Here
+//   * the units are walked in one order, place q = 0, 1, 2, ...: workgroup w of G takes places w and w + G, then
+//     whichever place is next on a ticket counter in memory (an atomic add that returns: ticket t is place 2 G + t),
+//     so a compute unit that finishes early takes more and the launch ends within a unit's time of the moment the
+//     work runs out;
+//   * the walk alternates between the plan's front (the full items, bound by the matrix cores) and its back (the
+//     short items, which mostly stream their expert's tables), so both kinds run all through the launch;
+//   * everything a unit needs to begin is fetched under the units before it: at a unit's top the workgroup requests
+//     the next unit's row list and the ticket for the unit after that; both have arrived (for nothing: a wave's
+//     memory operations complete in issue order) when the first operands have, where the rows go to LDS and wave 0
+//     requests the ticket's item, which it holds through the loop over K and puts into LDS at the unit's end.
+// The ticket counter is zero between launches: F = max(total - 2 G, 0) + clamp(total - G, 0, G) tickets are drawn in a
+// launch over `total` units (every workgroup whose second unit exists draws until its first ticket past the end),
+// and the thread that draws ticket F - 1 puts the counter back.  Launches that share a counter must not overlap.
+// Same units, same body, same bits.
+//
+// The rows' lists and the next item live behind the activation stages in the dynamic LDS:
+// [unit parity][source row, pair][row of the item], then (expert, first member, rows, unit).
+constexpr int RESIDENT_LDS = 2 * BIG_ROWS * AROW + 2 * 2 * BIG_ROWS * 4 + 16;
+
+__device__ __forceinline__ int* resident_rows(int parity, int which) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  return reinterpret_cast<int*>(smem + 2 * BIG_ROWS * AROW) + (parity * 2 + which) * BIG_ROWS;
+}
+
+template <int GS, int NM, int EPI, int AR, int RT, class STAGED>
+__device__ __forceinline__ void resident_unit(const uint16_t* __restrict__ X, int64_t x_stride,
+                                              const uint32_t* __restrict__ We, int KG, int NB, int cbt, int cnt,
+                                              void* __restrict__ out, int N, float limit, int parity, int tid,
+                                              STAGED& staged) {
+  constexpr int BW = block_words(GS);
+  constexpr int NBW = big_blocks(NM);
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int lane = tid & 63, wave = tid >> 6, c = lane & 15, kq = lane >> 4;
+  ExpertSource<GS, NM> ws;
+  ws.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(We), 0, (uint32_t)NB * KG * (NM * BW) * 4u, 0x00020000);
+  int ocol[4];
+  bool jok[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int m = NM == 2 ? j >> 1 : 0;
+    const int nb = NM == 2 ? cbt * NBW + wave : cbt * NBW + wave * 2 + (j >> 1);
+    const int toff = (j & 1) * 16;
+    jok[j] = nb < NB;
+    const uint32_t blk = (uint32_t)((jok[j] ? nb : NB - 1) * KG) * (uint32_t)(NM * BW) + m * BW;
+    ws.wp[j] = blk + (toff + c) * 4 + kq;
+    ws.sp[j] = blk + 32 * GS / 8 + toff + c;
+    ocol[j] = nb * 32 + toff + c;
+  }
+  constexpr bool OUT_LINES = NM == 1;
+  big_body<GS, NM, EPI, RT, AR, OUT_LINES, ExpertSource<GS, NM>, 4, BIG_THREADS, OUT_LINES>(
+      X, x_stride, ws, ocol, jok, KG * GS, resident_rows(parity, 0), resident_rows(parity, 1), cnt, out, N, limit, smem,
+      staged, tid);
+}
+
+template <int GS, int NM, int EPI, int AR>
+__global__ void __launch_bounds__(BIG_THREADS, 1)
+    experts_prefill_resident_kernel(const uint16_t* __restrict__ X, int64_t x_stride, int slots,
+                                    const uint32_t* __restrict__ W, int KG, int NB, const int* __restrict__ items,
+                                    const int* __restrict__ counts, int* __restrict__ ticket,
+                                    const int* __restrict__ members, void* __restrict__ out, int N, float limit) {
+  constexpr int BW = block_words(GS);
+  constexpr int NBW = big_blocks(NM);
+  const int nbt = (NB + NBW - 1) / NBW;
+  const int total = counts[0] * nbt, G = gridDim.x;
+  // place q of the walk -> unit: alternately from the front of the plan (full items: matrix work) and from its back
+  // (the experts' short last items: mostly their tables' trip from memory), so that the two kinds run side by side
+  // all through the launch instead of one after the other
+  auto unit_at = [&](int q) { return (q & 1) ? total - 1 - (q >> 1) : q >> 1; };
+  const int tickets = max(total - 2 * G, 0) + min(max(total - G, 0), G);
+  int tid = threadIdx.x;
+  int unit = blockIdx.x;
+  if (unit >= total) return;
+  int* next_item = resident_rows(2, 0);
+  // an item's (expert, first member, rows): the same for every thread
+  auto item_of = [&](int u, int& e, int& first, int& cnt) {
+    const int it = unit_at(min(u, total - 1)) / nbt;
+    e = __builtin_amdgcn_readfirstlane(items[3 * it]);
+    first = __builtin_amdgcn_readfirstlane(items[3 * it + 1]);
+    cnt = min(__builtin_amdgcn_readfirstlane(items[3 * it + 2]), BIG_ROWS);
+  };
+  int unit1 = unit + G, e, first, cnt, e1, first1, cnt1;
+  item_of(unit, e, first, cnt);
+  item_of(unit1, e1, first1, cnt1);
+  if (tid < BIG_ROWS) {
+    const int p = members[first + (tid < cnt ? tid : 0)];
+    resident_rows(0, 1)[tid] = p;
+    resident_rows(0, 0)[tid] = slots ? p / slots : p;
+  }
+  __syncthreads();
+  for (int k = 0;; ++k) {
+    // what a unit derives from the thread's number is derived again for every unit: kept across units instead, it
+    // would crowd the body's registers
+    asm volatile("" : "+v"(tid));
+    TF_MARK(0);
+    TF_MARK(1);
+    const int it = unit_at(unit) / nbt, cbt = unit_at(unit) - it * nbt;
+    const int more = unit1 < total;
+    // requested now, used once this unit's first operands are here: the next unit's rows, the ticket after it
+    int p1 = 0, held = 0;
+    if (more && tid < BIG_ROWS) p1 = members[first1 + (tid < cnt1 ? tid : 0)];
+    if (more && tid == 0) held = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    auto staged = [&]() {
+      if (!more) return;
+      if (tid < BIG_ROWS) {
+        resident_rows(1 - (k & 1), 1)[tid] = p1;
+        resident_rows(1 - (k & 1), 0)[tid] = slots ? p1 / slots : p1;
+      }
+      if (tid < 64) {
+        // wave 0: the ticket's unit and its item, three ints on their way through the loop over K
+        if (tid == 0 && held == tickets - 1) __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int u2 = 2 * G + __builtin_amdgcn_readfirstlane(held);
+        held = tid < 3 ? items[3 * (unit_at(min(u2, total - 1)) / nbt) + tid] : u2;
+      }
+    };
+    const uint32_t* We = W + (size_t)e * NB * KG * (size_t)(NM * BW);
+    if (cnt <= 32) resident_unit<GS, NM, EPI, AR, 2>(X, x_stride, We, KG, NB, cbt, cnt, out, N, limit, k & 1, tid, staged);
+    else if (cnt <= 64) resident_unit<GS, NM, EPI, AR, 4>(X, x_stride, We, KG, NB, cbt, cnt, out, N, limit, k & 1, tid, staged);
+    else resident_unit<GS, NM, EPI, AR, 8>(X, x_stride, We, KG, NB, cbt, cnt, out, N, limit, k & 1, tid, staged);
+    TF_MARK(4);
+#ifdef TF_TIMELINE
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
+    TF_MARK_AS(5, unit_at(unit));
+    if (!more) break;
+    if (tid < 4) next_item[tid] = held;
+    __syncthreads();          // every wave is done with the stages (and its results' corner of them) and this unit's rows
+    unit = unit1, e = e1, first = first1, cnt = cnt1;
+    e1 = __builtin_amdgcn_readfirstlane(next_item[0]);
+    first1 = __builtin_amdgcn_readfirstlane(next_item[1]);
+    cnt1 = min(__builtin_amdgcn_readfirstlane(next_item[2]), BIG_ROWS);
+    unit1 = __builtin_amdgcn_readfirstlane(next_item[3]);
+  }
+}
+
 // The dense prompt matmul on the same pipeline: 128 rows x 512 columns a workgroup, a wave a 64-column tile.
 template <int GS, int EPI, int AR>
 __global__ void __launch_bounds__(BIG_THREADS, 1)
@@ -812,9 +960,21 @@ constexpr size_t stage_bytes() {
   return 2 * (size_t)(16 * RT) * AROW;
 }
 
+// compute units of the current device (looked up once a device)
+int compute_units() {
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (!cached[dev]) {
+    hipDeviceProp_t prop;
+    cached[dev] = hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+  }
+  return cached[dev];
+}
+
 template <int GS, int NM, int EPI>
 int launch_experts_prefill(int tile, int arith, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w,
-                           int kg, int nb, const int* items, const int* counts, const int* members, void* out, int n,
+                           int kg, int nb, const int* items, int* counts, const int* members, void* out, int n,
                            float limit, int64_t max_items, hipStream_t s) {
   const int64_t grid = max_items * ((nb + 3) / 4);
   if (grid < 1) return 0;
@@ -839,6 +999,19 @@ int launch_experts_prefill(int tile, int arith, const uint16_t* x, int64_t x_str
     constexpr int NBW = big_blocks(NM);
     const int64_t big = max_items * ((nb + NBW - 1) / NBW);
     TF_REQUIRE(big <= 0x7FFFFFFF, "experts: %lld workgroups exceed the grid limit", (long long)big);
+    // workgroups that stay and walk the units by stride, one a compute unit, once there are units to walk
+    const int cus = compute_units();
+    if (big > 2 * cus) {
+      const dim3 rg((unsigned)cus);
+      if (arith)
+        experts_prefill_resident_kernel<GS, NM, EPI, 1><<<rg, BIG_THREADS, RESIDENT_LDS, s>>>(
+            x, x_stride, slots, w, kg, nb, items, counts, counts + 2, members, out, n, limit);
+      else
+        experts_prefill_resident_kernel<GS, NM, EPI, 0><<<rg, BIG_THREADS, RESIDENT_LDS, s>>>(
+            x, x_stride, slots, w, kg, nb, items, counts, counts + 2, members, out, n, limit);
+      TF_LAUNCH_OK("tf_experts_prefill");
+      return 0;
+    }
     const dim3 bg((unsigned)big);
     if (arith)
       experts_prefill_big_kernel<GS, NM, EPI, 1><<<bg, BIG_THREADS, 2 * BIG_ROWS * AROW, s>>>(
@@ -896,7 +1069,7 @@ using namespace tf;
 TF_TIMELINE_EXPORT(prefill)
 
 extern "C" int tf_experts_prefill(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w,
-                                  int kg, int nb, const int32_t* items, const int32_t* counts, const int32_t* members,
+                                  int kg, int nb, const int32_t* items, int32_t* counts, const int32_t* members,
                                   void* out, int n, float limit, int64_t max_items, int tile, int arith,
                                   tf_stream_t stream) {
   clear_error();

@@ -110,13 +110,15 @@ __device__ __forceinline__ unsigned long long* timeline_lds() {
   __shared__ unsigned long long t[TIMELINE_MARKS];
   return t;
 }
-__device__ __forceinline__ void timeline_mark(int k) {
+// `as` >= 0: the row of the table to write at the last mark (a workgroup that takes several units one after another
+// marks each under the unit's number); otherwise the workgroup's own number
+__device__ __forceinline__ void timeline_mark(int k, int as = -1) {
   if (threadIdx.x != 0) return;
   unsigned long long* t = timeline_lds();
   if (k == 0)
     for (int i = 1; i < TIMELINE_MARKS; ++i) t[i] = 0;
   t[k] = wall_clock64();
-  const unsigned group = blockIdx.x + (blockIdx.y + blockIdx.z * gridDim.y) * gridDim.x;
+  const unsigned group = as >= 0 ? (unsigned)as : blockIdx.x + (blockIdx.y + blockIdx.z * gridDim.y) * gridDim.x;
   if (k == TIMELINE_MARKS - 1 && group < TIMELINE_GROUPS) {
     for (int i = 0; i < TIMELINE_MARKS; ++i) tf_timeline_marks[i][group] = t[i];
     // where it ran: the XCC id above the hardware id word (compute unit in bits 8-11, shader array 12, engine 13-15)
@@ -145,9 +147,13 @@ __device__ __forceinline__ void timeline_mark(int k) {
     return 0;                                                                                                       \
   }
 #define TF_MARK(K_) timeline_mark(K_)
+#define TF_MARK_AS(K_, AS_) timeline_mark(K_, AS_)
 #else
 #define TF_MARK(K_) \
   do {              \
+  } while (0)
+#define TF_MARK_AS(K_, AS_) \
+  do {                      \
   } while (0)
 #define TF_TIMELINE_EXPORT(NAME_)
 #endif

@@ -159,7 +159,9 @@ def max_items(pairs: int, experts: int, tile: int = TILE) -> int:
 
 class Plan:
     """Device scratch of the pair sort: ``members`` (pairs ordered by expert), ``items`` rows of
-    (expert, first member, count) and ``counts`` = (items, distinct experts).  Sized once for ``rows`` x ``slots``."""
+    (expert, first member, count) and ``counts`` = (items, distinct experts, the prompt kernels' ticket word, spare).
+    The ticket word hands an item's units to the prompt kernels' workgroups; it is zero whenever no prompt launch on
+    this plan is running, so launches that share a plan must not overlap.  Sized once for ``rows`` x ``slots``."""
 
     def __init__(self, rows: int, slots: int, experts: int, device: torch.device | str, *,
                  prefill: bool = False) -> None:
@@ -172,7 +174,7 @@ class Plan:
 
         self.members = ints(pairs)
         self.items = ints(max_items(pairs, experts, TILE), 3)     # sized for the narrowest item any consumer takes
-        self.counts = ints(2)
+        self.counts = ints(4)
         blocks = -(-pairs // SMALL)
         self.rank = ints(pairs if pairs > SMALL else 1)            # the multi-workgroup sort's scratch
         self.hist = ints(blocks * experts if pairs > SMALL else 1)

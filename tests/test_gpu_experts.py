@@ -275,6 +275,31 @@ def test_many_units_keep_the_bits():
         assert torch.equal(run(ex, x[r:r + 1], picks[r:r + 1])[1], y[9 * r:9 * r + 9]), r
 
 
+@pytest.mark.parametrize("used,rows", [(3, 80), (400, 96), (600, 640)])
+def test_prompt_units_walked_by_workgroups_that_stay(used, rows):
+    """Past two units a compute unit (by the host's bound on the items) the prompt form is one workgroup a compute
+    unit walking the units by ticket: with fewer units than workgroups, with between one and two each, and with
+    several each, the bits are those of the 16-row items (one workgroup a unit, never walked), and the plan's ticket
+    word is back at zero after every launch."""
+
+    case = (32, True, 0.0, 601, 512, 256, 1)
+    ex, _, _ = build(case, 91)
+    x = synthetic.activations(rows, ex.dims, 5, 0.5).to(DEV)
+    g = torch.Generator().manual_seed(13)
+    picks = torch.stack([torch.cat([torch.randperm(used, generator=g)[:6], torch.tensor([600])])
+                         for _ in range(rows)]).to(torch.int32)
+    assert experts.max_items(rows * 7, ex.count, 128) > 2 * torch.cuda.get_device_properties(0).multi_processor_count
+    act, y, plan = run(ex, x, picks, prefill=True, tile=128)
+    units = int(plan.counts[0])                       # the up launch: an item is one unit of 256 columns a matrix
+    assert plan.counts.cpu().tolist()[2:] == [0, 0]
+    want_act, want, _ = run(ex, x, picks, prefill=True, tile=16)
+    assert torch.equal(act, want_act) and torch.equal(y, want), units
+    # again on the same plan: the ticket word was left ready
+    experts.gate_up(x, ex, plan, act.zero_(), rows)
+    experts.down(act, ex, plan, y.zero_(), rows)
+    assert torch.equal(act, want_act) and torch.equal(y, want) and plan.counts.cpu().tolist()[2:] == [0, 0]
+
+
 def test_bad_arguments_raise():
     w = tuple(t.to(DEV) for t in synthetic.affine_general(96, 256, 64, 1, (2,)))
     with pytest.raises(ValueError):
