@@ -17,6 +17,10 @@
 // scale 2^9 turns two nibble-bytes into the fp16 pair (q0, q1); the operand order this gives, inputs
 // (0, 4, 1, 5, 2, 6, 3, 7) of the eight, is applied to the activations when they are staged.
 
+#include <mutex>
+#include <set>
+#include <utility>
+
 #include "tf_common.h"
 
 namespace tf {
@@ -388,63 +392,71 @@ __global__ void __launch_bounds__(256)
 constexpr int BIG_ROWS = 128;
 constexpr int BIG_WAVES = 8;
 constexpr int BIG_THREADS = BIG_WAVES * 64;
+// LDS of a workgroup: two stages of activations, then for each wave two stages of its own step of weights (the
+// packed words of its 64 columns, 1 KB a chunk of 32 inputs, then a word a column and group for scale and bias)
+constexpr int WSTAGE = (KSTEP / 32) * 1024 + 512;
+constexpr int BIG_LDS = 2 * BIG_ROWS * AROW + BIG_WAVES * 2 * WSTAGE;
 
 // The pipeline for an item of at most 16 * RT rows (RT = 2, 4 or 8).  K is a multiple of KSTEP and nothing inside a
 // step is conditional (prefetches past the end re-read the last step, rows past the item read its first row), so the
 // compiler is free to keep the LDS reads of the next row tile in flight under the MFMAs of this one.
-// Where a wave's weights come from.  load(step, w, sb): the lane's packed word of each of the four operands and two
-// chunks of the step, and the stored (scale | bias << 16) pair of each operand and group of the step.  Buffer loads:
-// the base in scalar registers, the step as the scalar offset, the lane's part as the vector offset and the chunk or
-// group as the immediate, so no address arithmetic is left on the vector unit.
-template <int GS, int NM, int TJ = 4>
+// Where a wave's weights come from.  A wave takes 64 weight columns (four operands of 16), and for loading them lane L
+// owns column L: load(step, raw) requests the column's four packed words of each 32-input chunk of the step as ONE
+// 16-byte load (both layouts keep a column's four words of 32 inputs side by side) and its scale and bias of each
+// group of the step, i.e. 4 to 6 load instructions a wave and step where a word a lane and operand took 16.  (A
+// wave's load instruction keeps the compute unit's address unit busy for about 16 cycles whatever its width: with a
+// word a lane the short items, which mostly stream their tables, ran at 3 TB/s with that unit busy 60 % of the time.)
+// The lane that multiplies is another one (lane (c, kq) takes words kq of columns 16 j + c), so the words change
+// lanes through a corner of LDS that is the wave's own: no barrier, a wave's LDS operations run in order.
+// Buffer loads: the base in scalar registers, the step as the scalar offset, the lane's part as the vector offset and
+// the chunk or group as the immediate, so no address arithmetic is left on the vector unit.
+template <int GS, int NM>
 struct ExpertSource {
   static constexpr int CPS = KSTEP / 32, GPS = KSTEP / GS;
   static constexpr uint32_t GSTRIDE = NM * block_words(GS);      // words from one group to the next
-  typedef uint32_t SB;                                            // a column's stored (scale | bias << 16)
+  struct Raw {
+    u32x4_t q[CPS];
+    uint32_t sb[GPS];
+  };
   __amdgpu_buffer_rsrc_t rsrc;                                    // one expert's matrices
-  uint32_t wp[TJ], sp[TJ];                                        // word offsets inside the expert: below 2^32
-  __device__ __forceinline__ void load(int step, uint32_t (&w)[TJ][CPS], uint32_t (&sb)[TJ][GPS]) const {
+  uint32_t qp, sp;      // byte offsets inside the expert (below 2^32): the column's words of group 0; its (scale | bias << 16)
+  __device__ __forceinline__ void load(int step, Raw& r) const {
     const int soff = step * (int)(GPS * GSTRIDE * 4);
 #pragma unroll
-    for (int j = 0; j < TJ; ++j) {
+    for (int i = 0; i < CPS; ++i)
+      r.q[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, qp + (((32 * i) / GS) * GSTRIDE + (((32 * i) % GS) / 32) * 128) * 4,
+                                                     soff, 0);
 #pragma unroll
-      for (int i = 0; i < CPS; ++i)
-        w[j][i] = __builtin_amdgcn_raw_buffer_load_b32(
-            rsrc, (wp[j] + ((32 * i) / GS) * GSTRIDE + (((32 * i) % GS) / 32) * 128) * 4, soff, 0);
-#pragma unroll
-      for (int gi = 0; gi < GPS; ++gi)
-        sb[j][gi] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (sp[j] + gi * GSTRIDE) * 4, soff, 0);
-    }
+    for (int gi = 0; gi < GPS; ++gi) r.sb[gi] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, sp + gi * GSTRIDE * 4, soff, 0);
   }
+  // the column's stored (scale | bias << 16) of group gi of the step
+  static __device__ __forceinline__ uint32_t sb_word(const Raw& r, int gi) { return r.sb[gi]; }
 };
 
 // The dense layout: codes [n / 64][K / gs][gs / 32][64][4] words, scales and biases bf16 [K / gs][npad].
-template <int GS, int TJ = 4>
+template <int GS>
 struct DenseSource {
   static constexpr int CPS = KSTEP / 32, GPS = KSTEP / GS;
-  typedef uint2 SB;                                               // a column's scale and bias, joined where they are used
+  struct Raw {
+    u32x4_t q[CPS];
+    uint32_t s[GPS], b[GPS];          // each a bf16 in the low half, joined when the words go to LDS (not when they
+  };                                  // are requested: that would wait for loads just issued)
   __amdgpu_buffer_rsrc_t codes, scales, biases;
-  uint32_t wp[TJ], cp[TJ];                                        // byte offsets: the lane's word; its column's bf16
+  uint32_t qp, cp;                                                // byte offsets: the column's four words; its bf16
   int row_bytes;                                                  // bytes from one group's scales to the next
-  __device__ __forceinline__ void load(int step, uint32_t (&w)[TJ][CPS], SB (&sb)[TJ][GPS]) const {
+  __device__ __forceinline__ void load(int step, Raw& r) const {
     const int soff = step * (KSTEP / 32) * 1024;                  // 32 inputs of a 64-column tile are 1 KB of codes
 #pragma unroll
-    for (int j = 0; j < TJ; ++j) {
+    for (int i = 0; i < CPS; ++i) r.q[i] = __builtin_amdgcn_raw_buffer_load_b128(codes, qp + i * 1024, soff, 0);
 #pragma unroll
-      for (int i = 0; i < CPS; ++i) w[j][i] = __builtin_amdgcn_raw_buffer_load_b32(codes, wp[j] + i * 1024, soff, 0);
-#pragma unroll
-      for (int gi = 0; gi < GPS; ++gi) {
-        const int goff = (step * GPS + gi) * row_bytes;
-        sb[j][gi].x = __builtin_amdgcn_raw_buffer_load_b16(scales, cp[j], goff, 0);
-        sb[j][gi].y = __builtin_amdgcn_raw_buffer_load_b16(biases, cp[j], goff, 0);
-      }
+    for (int gi = 0; gi < GPS; ++gi) {
+      const int goff = (step * GPS + gi) * row_bytes;
+      r.s[gi] = __builtin_amdgcn_raw_buffer_load_b16(scales, cp, goff, 0);
+      r.b[gi] = __builtin_amdgcn_raw_buffer_load_b16(biases, cp, goff, 0);
     }
   }
+  static __device__ __forceinline__ uint32_t sb_word(const Raw& r, int gi) { return (r.s[gi] & 0xFFFFu) | (r.b[gi] << 16); }
 };
-
-// a column's stored (scale | bias << 16), from either source's form
-__device__ __forceinline__ uint32_t sb_raw(uint32_t v) { return v; }
-__device__ __forceinline__ uint32_t sb_raw(uint2 v) { return (v.x & 0xFFFFu) | (v.y << 16); }
 
 // AR: TF_ARITH_F16 (fp16 operands, weights scaled by 2^8) or TF_ARITH_BF16 (the reference's bf16(fma(q, s, b)) weights
 // and untouched bf16 activations on the bf16 matrix instruction): the operand bits of mfma_body's two forms.
@@ -469,11 +481,31 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
   constexpr int STAGE = BIG_ROWS * AROW;
   const int tid = thread < 0 ? (int)threadIdx.x : thread, lane = tid & 63, c = lane & 15, kq = lane >> 4;
   const int steps = K / KSTEP;
-  typedef typename WS::SB SB;
+  typedef typename WS::Raw Raw;
+  static_assert(TJ == 4, "a wave takes 64 weight columns: four operands of 16");
   bool tile_ok[TJ];          // the lane's tile j exists at all (lane 0 of the tile's row of 16 says)
 #pragma unroll
   for (int j = 0; j < TJ; ++j) tile_ok[j] = SWAP ? __shfl(jok[j] ? 1 : 0, lane & 48) != 0 : jok[j];
-  auto load_w = [&](int step, uint32_t (&w)[TJ][CPS], SB (&sb)[TJ][GPS]) { ws.load(step, w, sb); };
+  // the wave's two weight stages.  put: lane L's column (its words of each chunk, its scale and bias of each group,
+  // the latter as the fp16 pair the fp16 form multiplies by: converted once a column here, not once an operand and
+  // lane there).  get: the words of the lane's four operands for chunk i, and their columns' scale and bias.
+  unsigned char* wl = smem + 2 * STAGE + (tid >> 6) * (2 * WSTAGE);
+  auto put = [&](int stage, const Raw& r) {
+    unsigned char* at = wl + stage * WSTAGE;
+#pragma unroll
+    for (int i = 0; i < CPS; ++i) *reinterpret_cast<u32x4_t*>(at + i * 1024 + lane * 16) = r.q[i];
+#pragma unroll
+    for (int gi = 0; gi < GPS; ++gi)
+      *reinterpret_cast<uint32_t*>(at + CPS * 1024 + gi * 256 + lane * 4) = AR ? WS::sb_word(r, gi) : sb_half2(WS::sb_word(r, gi));
+  };
+  auto get = [&](int stage, int i, uint32_t (&w)[TJ], uint32_t (&sb)[TJ]) {
+    const unsigned char* at = wl + stage * WSTAGE;
+#pragma unroll
+    for (int j = 0; j < TJ; ++j) w[j] = *reinterpret_cast<const uint32_t*>(at + i * 1024 + (64 * j + 4 * c + kq) * 4);
+#pragma unroll
+    for (int j = 0; j < TJ; ++j)
+      sb[j] = *reinterpret_cast<const uint32_t*>(at + CPS * 1024 + ((32 * i) / GS) * 256 + (16 * j + c) * 4);
+  };
   // this thread's pieces of the activation tile: piece q = (row q / 8, 16 bytes q % 8)
   const uint16_t* asrc[PPT];
 #pragma unroll
@@ -497,9 +529,9 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
     }
   };
   // one packed word and its column's scale and bias -> the B operand's eight values, as bits
-  auto dequant = [](uint32_t w, SB sb) {
-    if constexpr (AR) return __builtin_bit_cast(u32x4_t, dequant8b(w, sb_raw(sb)));
-    else return __builtin_bit_cast(u32x4_t, dequant8h(w, sb_half2(sb)));
+  auto dequant = [](uint32_t w, uint32_t sb) {
+    if constexpr (AR) return __builtin_bit_cast(u32x4_t, dequant8b(w, sb));
+    else return __builtin_bit_cast(u32x4_t, dequant8h(w, sb));
   };
   auto mfma = [](u32x4_t a, u32x4_t b, f32x4_t c) {
     const u32x4_t first = SWAP ? b : a, second = SWAP ? a : b;
@@ -516,18 +548,27 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
 #pragma unroll
     for (int r = 0; r < RT; ++r) acc[j][r] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
-  uint32_t wr[2][TJ][CPS];
-  SB sr[2][TJ][GPS];
+  // The weights of step t are requested at the head of step t - RD - 1 into one of RD landing sets of registers, put
+  // into the wave's LDS stage t & 1 at the head of step t - 1, and taken from there a chunk ahead of their MFMAs.
+  // With 128 rows the accumulators leave room for one landing set; with fewer, for two.
+  constexpr int RD = RT <= 4 ? 2 : 1;
+  Raw raw[RD];
   uint4 ar[PPT];
   const int last = steps - 1;
-  load_w(0, wr[0], sr[0]);
+  ws.load(0, raw[0]);
   load_a(0, ar);
-  load_w(min(1, last), wr[1], sr[1]);
+  if constexpr (RD == 2) ws.load(min(1, last), raw[1]);
+  put(0, raw[0]);
+  ws.load(min(RD, last), raw[0]);
   store_a(0, ar);
   // Software pipeline: the operands of the NEXT 32 inputs are dequantized under the MFMAs of these 32.
   u32x4_t bcur[TJ];
+  {
+    uint32_t wn[TJ], sn[TJ];
+    get(0, 0, wn, sn);
 #pragma unroll
-  for (int j = 0; j < TJ; ++j) bcur[j] = dequant(wr[0][j][0], sr[0][j][0]);
+    for (int j = 0; j < TJ; ++j) bcur[j] = dequant(wn[j], sn[j]);
+  }
   __syncthreads();
   staged();
   TF_MARK(2);
@@ -536,9 +577,13 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
     for (int u = 0; u < 2; ++u) {
       const int step = step0 + u;
       if (step < steps) {
-        // stage `u` of LDS holds this step's activations, wr[u] its weights (wr[1 - u] the next step's); the next
-        // step's activations are requested now and staged at the end of the step
+        // stage `u` of LDS holds this step's activations and (the wave's own) weights; the next step's activations
+        // are requested now and staged at the end of the step, its weights have landed and go to stage 1 - u, and
+        // the landing set they leave takes the request for step + 1 + RD
         load_a(min(step + 1, last), ar);
+        Raw& landed = raw[RD == 2 ? 1 - u : 0];
+        put(1 - u, landed);
+        ws.load(min(step + 1 + RD, last), landed);
         const unsigned char* abuf = smem + u * STAGE + c * AROW + kq * 16;
         // activation operands are requested two row tiles before their MFMAs (an LDS read takes about as long as
         // one row tile's four MFMAs): operand t of the step is (chunk t / RT, row tile t % RT)
@@ -549,6 +594,9 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
 #pragma unroll
         for (int i = 0; i < CPS; ++i) {
           u32x4_t bnext[TJ];
+          uint32_t wn[TJ], sn[TJ];                      // the next chunk's words: this step's, or the next step's first
+          if (i + 1 < CPS) get(u, i + 1, wn, sn);
+          else get(1 - u, 0, wn, sn);
 #pragma unroll
           for (int r = 0; r < RT; ++r) {
             const int t = i * RT + r;
@@ -564,15 +612,9 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
 #pragma unroll
             for (int jj = 0; jj < JPR; ++jj) {
               const int j = r * JPR + jj;
-              if (j < TJ) {
-                if (i + 1 < CPS) bnext[j] = dequant(wr[u][j][i + 1], sr[u][j][(32 * (i + 1)) / GS]);
-                else bnext[j] = dequant(wr[1 - u][j][0], sr[1 - u][j][0]);
-              }
+              if (j < TJ) bnext[j] = dequant(wn[j], sn[j]);
             }
-            if (i + 2 == CPS && r * JPR + JPR >= TJ && (r - 1) * JPR + JPR < TJ)
-              load_w(min(step + 2, last), wr[u], sr[u]);     // wr[u] has just been used for the last time
           }
-          if (CPS == 1) load_w(min(step + 2, last), wr[u], sr[u]);
 #pragma unroll
           for (int j = 0; j < TJ; ++j) bcur[j] = bnext[j];
         }
@@ -714,14 +756,17 @@ __global__ void __launch_bounds__(BIG_THREADS, 1)
   bool jok[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int m = NM == 2 ? j >> 1 : 0;
     const int nb = NM == 2 ? cbt * NBW + wave : cbt * NBW + wave * 2 + (j >> 1);
-    const int toff = (j & 1) * 16;
     jok[j] = nb < NB;
-    const uint32_t blk = (uint32_t)((jok[j] ? nb : NB - 1) * KG) * (uint32_t)(NM * BW) + m * BW;
-    ws.wp[j] = blk + (toff + c) * 4 + kq;
-    ws.sp[j] = blk + 32 * GS / 8 + toff + c;
-    ocol[j] = nb * 32 + toff + c;
+    ocol[j] = nb * 32 + (j & 1) * 16 + c;
+  }
+  {
+    // the column this lane loads: column lane & 31 of block (matrix or neighbour) lane >> 5
+    const int m = NM == 2 ? lane >> 5 : 0;
+    const int nb = min(NM == 2 ? cbt * NBW + wave : cbt * NBW + wave * 2 + (lane >> 5), NB - 1);
+    const uint32_t blk = (uint32_t)(nb * KG) * (uint32_t)(NM * BW) + m * BW;
+    ws.qp = (blk + (lane & 31) * 4) * 4u;
+    ws.sp = (blk + 32 * GS / 8 + (lane & 31)) * 4u;
   }
   // one matrix (the down projection, whose outputs are the bulk of a chunk's stores): tiles weights-first and whole
   // lines out through LDS (4 % of the launch); gate and up with the SwiGLU between them: neither (3 % the other way)
@@ -759,11 +804,11 @@ __global__ void __launch_bounds__(BIG_THREADS, 1)
 //
 // The rows' lists and the next item live behind the activation stages in the dynamic LDS:
 // [unit parity][source row, pair][row of the item], then (expert, first member, rows, unit).
-constexpr int RESIDENT_LDS = 2 * BIG_ROWS * AROW + 2 * 2 * BIG_ROWS * 4 + 16;
+constexpr int RESIDENT_LDS = BIG_LDS + 2 * 2 * BIG_ROWS * 4 + 16;
 
 __device__ __forceinline__ int* resident_rows(int parity, int which) {
   extern __shared__ __align__(16) unsigned char smem[];
-  return reinterpret_cast<int*>(smem + 2 * BIG_ROWS * AROW) + (parity * 2 + which) * BIG_ROWS;
+  return reinterpret_cast<int*>(smem + BIG_LDS) + (parity * 2 + which) * BIG_ROWS;
 }
 
 template <int GS, int NM, int EPI, int AR, int RT, class STAGED>
@@ -781,14 +826,17 @@ __device__ __forceinline__ void resident_unit(const uint16_t* __restrict__ X, in
   bool jok[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int m = NM == 2 ? j >> 1 : 0;
     const int nb = NM == 2 ? cbt * NBW + wave : cbt * NBW + wave * 2 + (j >> 1);
-    const int toff = (j & 1) * 16;
     jok[j] = nb < NB;
-    const uint32_t blk = (uint32_t)((jok[j] ? nb : NB - 1) * KG) * (uint32_t)(NM * BW) + m * BW;
-    ws.wp[j] = blk + (toff + c) * 4 + kq;
-    ws.sp[j] = blk + 32 * GS / 8 + toff + c;
-    ocol[j] = nb * 32 + toff + c;
+    ocol[j] = nb * 32 + (j & 1) * 16 + c;
+  }
+  {
+    // the column this lane loads: column lane & 31 of block (matrix or neighbour) lane >> 5
+    const int m = NM == 2 ? lane >> 5 : 0;
+    const int nb = min(NM == 2 ? cbt * NBW + wave : cbt * NBW + wave * 2 + (lane >> 5), NB - 1);
+    const uint32_t blk = (uint32_t)(nb * KG) * (uint32_t)(NM * BW) + m * BW;
+    ws.qp = (blk + (lane & 31) * 4) * 4u;
+    ws.sp = (blk + 32 * GS / 8 + (lane & 31)) * 4u;
   }
   constexpr bool OUT_LINES = NM == 1;
   big_body<GS, NM, EPI, RT, AR, OUT_LINES, ExpertSource<GS, NM>, 4, BIG_THREADS, OUT_LINES>(
@@ -901,12 +949,12 @@ __global__ void __launch_bounds__(BIG_THREADS, 1)
   bool jok[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int col = (ok ? tile : 0) * 64 + 32 * (j >> 1) + 16 * (j & 1) + c;      // columns up to npad are stored zeros
-    ws.wp[j] = ((uint32_t)(ok ? tile : 0) * KG * (GS / 32) * 256u + (32 * (j >> 1) + 16 * (j & 1) + c) * 4 + kq) * 4u;
-    ws.cp[j] = col * 2;
+    const int col = (ok ? tile : 0) * 64 + 16 * j + c;      // columns up to npad are stored zeros
     ocol[j] = col;
     jok[j] = ok && col < N;
   }
+  ws.qp = ((uint32_t)(ok ? tile : 0) * KG * (GS / 32) * 256u + lane * 4) * 4u;      // the column this lane loads: lane
+  ws.cp = ((ok ? tile : 0) * 64 + lane) * 2;
   const int K = KG * GS;
   if (cnt <= 32) big_body<GS, 1, EPI, 2, AR, true>(X, ldx, ws, ocol, jok, K, rows, rows, cnt, out, N, 0.f, smem);
   else if (cnt <= 64) big_body<GS, 1, EPI, 4, AR, true>(X, ldx, ws, ocol, jok, K, rows, rows, cnt, out, N, 0.f, smem);
@@ -960,6 +1008,20 @@ constexpr size_t stage_bytes() {
   return 2 * (size_t)(16 * RT) * AROW;
 }
 
+// The eight-wave kernels ask for more dynamic LDS than a launch gets unasked (64 KB of the compute unit's 160): the
+// attribute is set once a kernel and device.
+bool allow_lds(const void* kernel, int bytes) {
+  static std::mutex guard;
+  static std::set<std::pair<const void*, int>> done;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return false;
+  std::lock_guard<std::mutex> hold(guard);
+  if (done.count({kernel, dev})) return true;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return false;
+  done.insert({kernel, dev});
+  return true;
+}
+
 // compute units of the current device (looked up once a device)
 int compute_units() {
   static int cached[64] = {};
@@ -1003,6 +1065,9 @@ int launch_experts_prefill(int tile, int arith, const uint16_t* x, int64_t x_str
     const int cus = compute_units();
     if (big > 2 * cus) {
       const dim3 rg((unsigned)cus);
+      TF_REQUIRE(allow_lds(arith ? (const void*)experts_prefill_resident_kernel<GS, NM, EPI, 1>
+                                 : (const void*)experts_prefill_resident_kernel<GS, NM, EPI, 0>, RESIDENT_LDS),
+                 "experts: %d bytes of LDS a workgroup were refused", RESIDENT_LDS);
       if (arith)
         experts_prefill_resident_kernel<GS, NM, EPI, 1><<<rg, BIG_THREADS, RESIDENT_LDS, s>>>(
             x, x_stride, slots, w, kg, nb, items, counts, counts + 2, members, out, n, limit);
@@ -1013,11 +1078,14 @@ int launch_experts_prefill(int tile, int arith, const uint16_t* x, int64_t x_str
       return 0;
     }
     const dim3 bg((unsigned)big);
+    TF_REQUIRE(allow_lds(arith ? (const void*)experts_prefill_big_kernel<GS, NM, EPI, 1>
+                               : (const void*)experts_prefill_big_kernel<GS, NM, EPI, 0>, BIG_LDS),
+               "experts: %d bytes of LDS a workgroup were refused", BIG_LDS);
     if (arith)
-      experts_prefill_big_kernel<GS, NM, EPI, 1><<<bg, BIG_THREADS, 2 * BIG_ROWS * AROW, s>>>(
+      experts_prefill_big_kernel<GS, NM, EPI, 1><<<bg, BIG_THREADS, BIG_LDS, s>>>(
           x, x_stride, slots, w, kg, nb, items, counts, members, out, n, limit);
     else
-      experts_prefill_big_kernel<GS, NM, EPI, 0><<<bg, BIG_THREADS, 2 * BIG_ROWS * AROW, s>>>(
+      experts_prefill_big_kernel<GS, NM, EPI, 0><<<bg, BIG_THREADS, BIG_LDS, s>>>(
           x, x_stride, slots, w, kg, nb, items, counts, members, out, n, limit);
   }
 #undef TF_SMALL
@@ -1047,10 +1115,13 @@ int launch_qmm_prefill(int arith, int tile, const uint16_t* x, int64_t ldx, cons
     else TF_SMALL(4, 0);
   } else if (big_ok && tile != 8) {
     const unsigned grid = (unsigned)((int64_t)((m + BIG_ROWS - 1) / BIG_ROWS) * ((n + 511) / 512));
+    TF_REQUIRE(allow_lds(arith ? (const void*)qmm_prefill_big_kernel<GS, EPI, 1> : (const void*)qmm_prefill_big_kernel<GS, EPI, 0>,
+                         BIG_LDS),
+               "qmm_prefill: %d bytes of LDS a workgroup were refused", BIG_LDS);
     if (arith)
-      qmm_prefill_big_kernel<GS, EPI, 1><<<grid, BIG_THREADS, 2 * BIG_ROWS * AROW, st>>>(x, ldx, w, s, b, out, m, n, kg, npad);
+      qmm_prefill_big_kernel<GS, EPI, 1><<<grid, BIG_THREADS, BIG_LDS, st>>>(x, ldx, w, s, b, out, m, n, kg, npad);
     else
-      qmm_prefill_big_kernel<GS, EPI, 0><<<grid, BIG_THREADS, 2 * BIG_ROWS * AROW, st>>>(x, ldx, w, s, b, out, m, n, kg, npad);
+      qmm_prefill_big_kernel<GS, EPI, 0><<<grid, BIG_THREADS, BIG_LDS, st>>>(x, ldx, w, s, b, out, m, n, kg, npad);
   } else if (arith) {
     TF_SMALL(8, 1);
   } else {
