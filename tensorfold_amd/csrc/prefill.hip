@@ -10,10 +10,10 @@
 // bf16, an eighth of the rounding error, and the packed fp16 fma dequantizes two weights an instruction.
 //
 // A workgroup of four waves takes (item of up to 16*RT rows) x (128 columns); each wave owns 32 columns and all the
-// item's rows.  The gathered activation rows are staged through LDS (64 inputs a step, double-buffered); the
-// weights never touch LDS: lane (column c, quarter kq) of the MFMA's B operand needs the eight
-// inputs 8 kq .. 8 kq + 7 of column c, which is exactly one packed word, so each lane loads its word and
-// dequantizes it in registers.  A nibble in a byte is the e4m3 number q * 2^-9, so v_cvt_scalef32_pk_f16_fp8 with
+// item's rows.  The gathered activation rows are staged through LDS (64 inputs a step, double-buffered).  Lane
+// (column c, quarter kq) of the MFMA's B operand needs the eight inputs 8 kq .. 8 kq + 7 of column c, which is
+// exactly one packed word, and dequantizes it in registers; in the four-wave kernels each lane loads its own word,
+// in the eight-wave ones a lane loads a column's four words at once and they change lanes in LDS.  A nibble in a byte is the e4m3 number q * 2^-9, so v_cvt_scalef32_pk_f16_fp8 with
 // scale 2^9 turns two nibble-bytes into the fp16 pair (q0, q1); the operand order this gives, inputs
 // (0, 4, 1, 5, 2, 6, 3, 7) of the eight, is applied to the activations when they are staged.
 
@@ -386,8 +386,9 @@ __global__ void __launch_bounds__(256)
 // An item of up to 128 pairs against 512 weight columns (NM = 1: 512 output columns; NM = 2: 256 output columns of
 // gate and of up).  Each of the eight waves owns 64 weight columns = four B operands and all eight 16-row tiles, so
 // one dequantized operand feeds eight MFMAs and one LDS read of the activations feeds four: per 32 inputs a wave
-// issues 32 MFMAs against 8 LDS reads and 4 dequantizations.  Weights are requested two steps (128 inputs) ahead
-// into registers, activations one step ahead through registers into LDS (two stages), one barrier a step.  The arithmetic of a row (operand values, MFMA, K order) is the small kernel's, so the bits are too.
+// issues 32 MFMAs against 8 LDS reads and 4 dequantizations.  Weights are requested two or three steps (128 or 192
+// inputs) ahead into registers and pass through the wave's own LDS stages, activations one step ahead through
+// registers into the workgroup's two LDS stages, one barrier a step.  The arithmetic of a row (operand values, MFMA, K order) is the small kernel's, so the bits are too.
 
 constexpr int BIG_ROWS = 128;
 constexpr int BIG_WAVES = 8;
@@ -602,9 +603,14 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
             const int t = i * RT + r;
             u32x4_t a2 = a1;
             if (t + 2 < CPS * RT) a2 = read_a(t + 2);
+            // the matrix instructions go first among the SIMD's waves: the other wave's vector work fills the cycles
+            // between them, instead of both waves taking turns at the same kind of work (3 % on the fp16 form; the
+            // bf16 form, with twice the vector work an operand, lost 4 % to it)
+            if constexpr (!AR) __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int j = 0; j < TJ; ++j)
               acc[j][r] = mfma(a, bcur[j], acc[j][r]);
+            if constexpr (!AR) __builtin_amdgcn_s_setprio(0);
             a = a1;
             a1 = a2;
             // a share of the next chunk's dequantization rides along with each row tile
