@@ -208,6 +208,12 @@ def c3(tiles=((64, torch.float32), (128, torch.float32), ("128_y_bf16", torch.bf
                       "(flops count the shared expert's 4,096 pairs)", "bound": "mfma", "tiles": out}
 
 
+def c3d() -> dict:
+    """Configuration 3 with the default pair outputs only (items of 128, fp16): the leg counters are collected on."""
+
+    return c3(tiles=(("128_y_f16", torch.float16),))
+
+
 def c4() -> dict:
     gen = torch.Generator(device=DEV).manual_seed(4)
 
@@ -590,11 +596,12 @@ def timeline_c2() -> dict:
 
 
 def timeline_c3() -> dict:
-    """Per-workgroup marks of configuration 3's two expert launches (the eight-wave prompt kernel, items of 128, fp16
-    pair outputs) through the timeline build: 0 entry, 1 the item's rows known, 2 first operands staged (the loop
-    begins), 3 the loop over K done, 4 results issued, 5 results written.  By the item's rows: how long a workgroup
-    lives and where; by compute unit: the gap between one workgroup's end and the next one's entry, and when each
-    unit went idle for good (the launch's tail)."""
+    """Per-unit marks of configuration 3's two expert launches (the eight-wave prompt kernel, items of 128, fp16 pair
+    outputs) through the timeline build; a unit is an item's 512 weight columns, taken one after another by the
+    workgroup that stays on a compute unit ("workgroups" below counts units): 0 the unit begins, 1 its rows are known
+    (at once: they were fetched under the unit before), 2 first operands staged (the loop begins), 3 the loop over K
+    done, 4 results issued, 5 results written.  By the item's rows: how long a unit takes and where; by compute unit:
+    the gap between one unit's end and the next one's start, and when each went idle for good (the launch's tail)."""
 
     import ctypes
 
@@ -672,7 +679,7 @@ def main() -> int:
     torch.cuda.set_device(0)
     which = sys.argv[1:] or ["c0", "c2", "c3", "c4"]
     for name in which:
-        res = {"c0": c0, "c2": c2, "c3": c3, "c4": c4, "c4p": c4p, "glue": glue_, "c4x": c4x, "cal": cal, "timeline": timeline, "timeline_c2": timeline_c2, "timeline_c3": timeline_c3}[name]()
+        res = {"c0": c0, "c2": c2, "c3": c3, "c3d": c3d, "c4": c4, "c4p": c4p, "glue": glue_, "c4x": c4x, "cal": cal, "timeline": timeline, "timeline_c2": timeline_c2, "timeline_c3": timeline_c3}[name]()
         torch.cuda.empty_cache()
         print(json.dumps(res, default=lambda v: round(v, 4)), flush=True)
     return 0
