@@ -138,8 +138,9 @@ int tf_experts_pack(const uint32_t* words, const uint16_t* scales, const uint16_
 int tf_experts_unpack(const uint32_t* blocks, int64_t block_stride, int e, int n, int k, int gs, uint32_t* words,
                       uint16_t* scales, uint16_t* biases, tf_stream_t stream);
 /* Stable grouping of pairs p = row*slots + slot by expert: members [pairs], items [(expert, first, count<=tile)],
- * counts = {items, distinct experts}.  rank [pairs] and hist [ceil(pairs/1024) * experts] are scratch, used when
- * pairs > 1024.  tile is 16 (decode), 64 or 128 (prefill).  Replaces experts.cpp:33-41 `plan`. */
+ * counts = {items, distinct experts} (four int32 where the plan goes to tf_experts_prefill, see there).  rank [pairs]
+ * and hist [ceil(pairs/1024) * experts] are scratch, used when pairs > 1024.  tile is 16 (decode), 64 or 128
+ * (prefill).  Replaces experts.cpp:33-41 `plan`. */
 int tf_experts_plan(const int32_t* picks, int64_t pairs, int experts, int tile, int32_t* members, int32_t* items,
                     int32_t* counts, int32_t* rank, int32_t* hist, tf_stream_t stream);
 /* Decode form.  epi 0: fp32 out; 1: bf16 relu(bf16 a)^2; 2: bf16 SwiGLU(matrix 0, matrix 1) with clip `limit`.
@@ -168,8 +169,13 @@ int tf_experts_run(int gs, int epi, const uint16_t* x, int64_t x_stride, int slo
 int tf_experts_run_desc(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg,
                         int nb, const int32_t* desc, const int32_t* counts, void* out, int n, float limit,
                         int64_t max_items, tf_stream_t stream);
-/* Prompt form on MFMA, each weight rounded once as in tf_qmm_prefill (arith: TF_ARITH_*); epi 3: bf16 out; epi 4: fp16 out, values beyond fp16's range stored as +-65504.  `tile` is
- * the plan's item size (16, 64 or 128).  Replaces experts.cpp:50-55 `prefill`. */
+/* Prompt form on MFMA, each weight rounded once as in tf_qmm_prefill (arith: TF_ARITH_*); epi 3: bf16 out; epi 4: fp16
+ * out, values beyond fp16's range stored as +-65504.  `tile` is the plan's item size (16, 64 or 128).
+ * `counts` holds FOUR int32 here: {items, distinct experts} as tf_experts_plan left them, then a ticket word and a
+ * spare, both zero when the buffer is made.  Large plans run on one workgroup a compute unit, and the workgroups
+ * draw their work from the ticket word; the launch leaves it at zero again, so nothing has to clear it between
+ * launches, and launches that share a `counts` buffer must not overlap (one stream, or one after the other).
+ * Replaces experts.cpp:50-55 `prefill`. */
 int tf_experts_prefill(int gs, int epi, const uint16_t* x, int64_t x_stride, int slots, const uint32_t* w, int kg,
                        int nb, const int32_t* items, int32_t* counts, const int32_t* members, void* out, int n,
                        float limit, int64_t max_items, int tile, int arith, tf_stream_t stream);
