@@ -809,7 +809,7 @@ __global__ void __launch_bounds__(BIG_THREADS, 1)
 // and the thread that draws ticket F - 1 puts the counter back.  Launches that share a counter must not overlap.
 // Same units, same body, same bits.
 //
-// The rows' lists and the next item live behind the activation stages in the dynamic LDS:
+// The rows' lists and the next item live behind the activation and weight stages in the dynamic LDS:
 // [unit parity][source row, pair][row of the item], then (expert, first member, rows, unit).
 constexpr int RESIDENT_LDS = BIG_LDS + 2 * 2 * BIG_ROWS * 4 + 16;
 
