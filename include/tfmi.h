@@ -34,7 +34,7 @@ enum { TF_F16 = 0, TF_BF16 = 1, TF_F32 = 2 };
 
 /* The message of the last failing call on this thread ("" if none). */
 const char* tf_last_error(void);
-/* ABI version of this header. */
+/* ABI version of this header: 3 (tf_moe_decode_sliced added; tf_experts_prefill's `counts` holds four int32). */
 int tf_version(void);
 /* Digest of the sources and compiler flags the library was built from (16 hex digits), "unknown" when the build gave
  * none.  The Python loader compares it with the sources beside it before it loads the file. */

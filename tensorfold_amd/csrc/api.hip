@@ -23,7 +23,7 @@ void clear_error() { g_error.clear(); }
 
 extern "C" const char* tf_last_error(void) { return tf::g_error.c_str(); }
 
-extern "C" int tf_version(void) { return 2; }
+extern "C" int tf_version(void) { return 3; }
 
 // A digest of the sources and flags this library was built from, given by the build (tensorfold_amd/build.py); the
 // loader compares it with the sources it sees and rebuilds or refuses a library that is out of date.

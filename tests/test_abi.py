@@ -24,7 +24,7 @@ def test_library_exports_the_header():
     for name in DECLARED:
         assert hasattr(so, name), name
     so.tf_version.restype = ctypes.c_int
-    assert so.tf_version() == 2
+    assert so.tf_version() == 3
     # the library says which sources it was built from, and the loader only hands out one built from these
     so.tf_build_id.restype = ctypes.c_char_p
     assert so.tf_build_id().decode() == build.source_id() == build.built_id() and not build.stale()
