@@ -275,14 +275,16 @@ def test_many_units_keep_the_bits():
         assert torch.equal(run(ex, x[r:r + 1], picks[r:r + 1])[1], y[9 * r:9 * r + 9]), r
 
 
-@pytest.mark.parametrize("used,rows", [(3, 80), (400, 96), (600, 640)])
-def test_prompt_units_walked_by_workgroups_that_stay(used, rows):
+@pytest.mark.parametrize("used,rows,d,ni", [(3, 80, 512, 256), (400, 96, 512, 256), (600, 640, 512, 256),
+                                            (600, 200, 576, 320)])
+def test_prompt_units_walked_by_workgroups_that_stay(used, rows, d, ni):
     """Past two units a compute unit (by the host's bound on the items) the prompt form is one workgroup a compute
     unit walking the units by ticket: with fewer units than workgroups, with between one and two each, and with
     several each, the bits are those of the 16-row items (one workgroup a unit, never walked), and the plan's ticket
-    word is back at zero after every launch."""
+    word is back at zero after every launch.  The last case has an odd number of 64-input steps (576 inputs) and
+    part-filled last units (320 and 576 columns: 10 and 18 blocks of 32 where a unit holds 8 or 16)."""
 
-    case = (32, True, 0.0, 601, 512, 256, 1)
+    case = (32, True, 0.0, 601, d, ni, 1)
     ex, _, _ = build(case, 91)
     x = synthetic.activations(rows, ex.dims, 5, 0.5).to(DEV)
     g = torch.Generator().manual_seed(13)
