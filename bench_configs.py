@@ -1,7 +1,7 @@
 """Kernel timings of the benchmark configurations that are not bench.py's headline: 0 (dense 4-bit projection),
 2 (verify-window MoE layer), 3 (prompt chunk, grouped MFMA) and 4 (EXL3 projections).
 
-    python bench_configs.py [c0] [c2] [c3] [c4] [c4p] [glue] [c4x] [cal] [timeline] [timeline_c2] [timeline_c3]
+    python bench_configs.py [c0] [c2] [c3] [c3d] [c4] [c4p] [glue] [c4x] [cal] [timeline] [timeline_c2] [timeline_c3]
 
 One JSON line a configuration: time of one pass (hipGraph of back-to-back passes cycling over enough weight copies to
 miss the 256 MB Infinity Cache, HIP events around the replay), algorithmic bytes or flops, and the fraction of the
