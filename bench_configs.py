@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import json
 import sys
+import time
 
 import torch
 
@@ -28,8 +29,12 @@ VALU = 256 * 4 * 16 * 2.4e9
 EXL3_VALU_PER_WEIGHT = 310 / 64
 
 
-def graph_us(step, reps: int) -> float:
-    """Mean time of ``step(i)`` over a replayed graph of ``reps`` calls."""
+def graph_us(step, reps: int, window_ms: float = 25.0) -> float:
+    """Mean time of ``step(i)`` over a replayed graph of ``reps`` calls, at the clock the card settles at under that
+    load: the graph is replayed back to back for ``window_ms`` untimed, then for ``window_ms`` between two events
+    with no synchronization inside, three times over (the median counts).  The shader clock follows the load with a
+    delay of some milliseconds: a 2 ms burst between two idle waits runs at 1.7-1.8 GHz where the same kernels back
+    to back run at 2.2 GHz (cycles a launch the same), and a prompt pass or a decode loop is the latter."""
 
     for i in range(3):
         step(i)
@@ -38,17 +43,47 @@ def graph_us(step, reps: int) -> float:
     with torch.cuda.graph(g):
         for i in range(reps):
             step(i)
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    g.replay()
+    b.record()
+    torch.cuda.synchronize()
+    n = max(1, min(2000, int(window_ms / max(a.elapsed_time(b), 1e-3) + 0.5)))
+    times = []
+    for _ in range(3):
+        for _ in range(n):
+            g.replay()
+        a.record()
+        for _ in range(n):
+            g.replay()
+        b.record()
+        torch.cuda.synchronize()
+        times.append(a.elapsed_time(b) * 1e3 / (n * reps))
+    return sorted(times)[1]
+
+
+def burst_us(step, reps: int) -> float:
+    """The same graph timed as one replay between two idle waits (the median of five): a burst of a millisecond or
+    two, which the card runs at the clock of an idle card woken up.  Reported beside ``graph_us`` where the difference
+    matters (the matrix-bound legs), so that both regimes can be read from one run."""
+
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for i in range(reps):
+            step(i)
     g.replay()
     torch.cuda.synchronize()
-    best = []
+    times = []
     for _ in range(5):
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        time.sleep(0.02)
         a.record()
         g.replay()
         b.record()
         torch.cuda.synchronize()
-        best.append(a.elapsed_time(b) * 1e3 / reps)
-    return sorted(best)[len(best) // 2]
+        times.append(a.elapsed_time(b) * 1e3 / reps)
+    return sorted(times)[2]
 
 
 def rand_affine(n: int, k: int, gs: int, gen, lead=()):
@@ -77,7 +112,8 @@ def c0() -> dict:
     y = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
     us = graph_us(lambda i: qmm.prefill_matmul(x, copies[i % len(copies)], out=y), 12)
     flop = 2.0 * m * n * k
-    prompt = {"rows": m, "us": us, "tflops": flop / us * 1e-6, "frac_mfma": flop / us * 1e-6 / MFMA}
+    prompt = {"rows": m, "us": us, "tflops": flop / us * 1e-6, "frac_mfma": flop / us * 1e-6 / MFMA,
+              "burst_us": burst_us(lambda i: qmm.prefill_matmul(x, copies[i % len(copies)], out=y), 12)}
     # the reference's own prompt arithmetic on the same kernel: w = bf16(fma(q, s, b)), bf16 matrix instruction
     us_b = graph_us(lambda i: qmm.prefill_matmul(x, copies[i % len(copies)], out=y, arith=1), 12)
     prompt["bf16_arithmetic"] = {"us": us_b, "tflops": flop / us_b * 1e-6, "frac_mfma": flop / us_b * 1e-6 / MFMA}
@@ -379,7 +415,8 @@ def cal() -> dict:
             y = torch.empty((m, n), dtype=dtype, device=DEV)
             us = graph_us(lambda i: torch.matmul(a, ws[i % len(ws)].t(), out=y), 12)
             flop = 2.0 * m * n * k
-            row[str(dtype).split(".")[-1]] = {"us": us, "tflops": flop / us * 1e-6, "frac_mfma": flop / us * 1e-6 / MFMA}
+            row[str(dtype).split(".")[-1]] = {"us": us, "tflops": flop / us * 1e-6, "frac_mfma": flop / us * 1e-6 / MFMA,
+                                              "burst_us": burst_us(lambda i: torch.matmul(a, ws[i % len(ws)].t(), out=y), 12)}
             del ws
             torch.cuda.empty_cache()
         out[name] = row
