@@ -106,7 +106,11 @@ __device__ __forceinline__ uint32_t pack_bf16_rn(float lo, float hi) {
 // values: round to nearest even, as the reference's __float2bfloat16_rn
 __device__ __forceinline__ bf16x8_t dequant8b(uint32_t w, uint32_t sb) {
   const float s = bf16_lo(sb), b = bf16_hi(sb);
-  const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
+  uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
+  // the compiler is not to know that these are w's nibbles: knowing it, it extracts each of the eight from w and
+  // converts that (16 instructions), where a byte of lo or hi converts as it lies (v_cvt_f32_ubyte0..3: 8)
+  asm("" : "+v"(lo));
+  asm("" : "+v"(hi));
   auto q = [](uint32_t v, int byte) { return (float)((v >> (8 * byte)) & 0xFFu); };
   const u32x4_t r = {pack_bf16_rn(fmaf(q(lo, 0), s, b), fmaf(q(lo, 1), s, b)),
                      pack_bf16_rn(fmaf(q(lo, 2), s, b), fmaf(q(lo, 3), s, b)),
