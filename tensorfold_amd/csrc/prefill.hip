@@ -13,13 +13,9 @@
 // item's rows.  The gathered activation rows are staged through LDS (64 inputs a step, double-buffered).  Lane
 // (column c, quarter kq) of the MFMA's B operand needs the eight inputs 8 kq .. 8 kq + 7 of column c, which is
 // exactly one packed word, and dequantizes it in registers; in the four-wave kernels each lane loads its own word,
-// in the eight-wave ones a lane loads a column's four words at once and they change lanes in LDS.  A nibble in a byte is the e4m3 number q * 2^-9, so v_cvt_scalef32_pk_f16_fp8 with
+// in the eight-wave ones a lane loads a column's four words at once and they change lanes by swaps.  A nibble in a byte is the e4m3 number q * 2^-9, so v_cvt_scalef32_pk_f16_fp8 with
 // scale 2^9 turns two nibble-bytes into the fp16 pair (q0, q1); the operand order this gives, inputs
 // (0, 4, 1, 5, 2, 6, 3, 7) of the eight, is applied to the activations when they are staged.
-
-#include <mutex>
-#include <set>
-#include <utility>
 
 #include "tf_common.h"
 
@@ -390,17 +386,16 @@ __global__ void __launch_bounds__(256)
 // An item of up to 128 pairs against 512 weight columns (NM = 1: 512 output columns; NM = 2: 256 output columns of
 // gate and of up).  Each of the eight waves owns 64 weight columns = four B operands and all eight 16-row tiles, so
 // one dequantized operand feeds eight MFMAs and one LDS read of the activations feeds four: per 32 inputs a wave
-// issues 32 MFMAs against 8 LDS reads and 4 dequantizations.  Weights are requested two or three steps (128 or 192
-// inputs) ahead into registers and pass through the wave's own LDS stages, activations one step ahead through
-// registers into the workgroup's two LDS stages, one barrier a step.  The arithmetic of a row (operand values, MFMA, K order) is the small kernel's, so the bits are too.
+// issues 32 MFMAs against 8 LDS reads and 4 dequantizations.  Weights are requested a step and a half (96 inputs)
+// ahead into registers and change lanes there, activations one step ahead through registers into the workgroup's
+// two LDS stages, one barrier a step.  The arithmetic of a row (operand values, MFMA, K order) is the small kernel's, so the bits are too.
 
 constexpr int BIG_ROWS = 128;
 constexpr int BIG_WAVES = 8;
 constexpr int BIG_THREADS = BIG_WAVES * 64;
-// LDS of a workgroup: two stages of activations, then for each wave two stages of its own step of weights (the
-// packed words of its 64 columns, 1 KB a chunk of 32 inputs, then a word a column and group for scale and bias)
-constexpr int WSTAGE = (KSTEP / 32) * 1024 + 512;
-constexpr int BIG_LDS = 2 * BIG_ROWS * AROW + BIG_WAVES * 2 * WSTAGE;
+// LDS of a workgroup: two stages of activations
+constexpr int BIG_LDS = 2 * BIG_ROWS * AROW;
+static_assert(BIG_LDS + 2 * 2 * BIG_ROWS * 4 + 16 <= 64 * 1024, "within what a launch gets without asking");
 
 // The pipeline for an item of at most 16 * RT rows (RT = 2, 4 or 8).  K is a multiple of KSTEP and nothing inside a
 // step is conditional (prefetches past the end re-read the last step, rows past the item read its first row), so the
@@ -412,7 +407,7 @@ constexpr int BIG_LDS = 2 * BIG_ROWS * AROW + BIG_WAVES * 2 * WSTAGE;
 // wave's load instruction keeps the compute unit's address unit busy for about 16 cycles whatever its width: with a
 // word a lane the short items, which mostly stream their tables, ran at 3 TB/s with that unit busy 60 % of the time.)
 // The lane that multiplies is another one (lane (c, kq) takes words kq of columns 16 j + c), so the words change
-// lanes through a corner of LDS that is the wave's own: no barrier, a wave's LDS operations run in order.
+// lanes on their way: by the chip's lane-swap instructions, in registers (big_body's `across`).
 // Buffer loads: the base in scalar registers, the step as the scalar offset, the lane's part as the vector offset and
 // the chunk or group as the immediate, so no address arithmetic is left on the vector unit.
 template <int GS, int NM>
@@ -444,7 +439,7 @@ struct DenseSource {
   static constexpr int CPS = KSTEP / 32, GPS = KSTEP / GS;
   struct Raw {
     u32x4_t q[CPS];
-    uint32_t s[GPS], b[GPS];          // each a bf16 in the low half, joined when the words go to LDS (not when they
+    uint32_t s[GPS], b[GPS];          // each a bf16 in the low half, joined when a chunk is taken (not when they
   };                                  // are requested: that would wait for loads just issued)
   __amdgpu_buffer_rsrc_t codes, scales, biases;
   uint32_t qp, cp;                                                // byte offsets: the column's four words; its bf16
@@ -491,25 +486,36 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
   bool tile_ok[TJ];          // the lane's tile j exists at all (lane 0 of the tile's row of 16 says)
 #pragma unroll
   for (int j = 0; j < TJ; ++j) tile_ok[j] = SWAP ? __shfl(jok[j] ? 1 : 0, lane & 48) != 0 : jok[j];
-  // the wave's two weight stages.  put: lane L's column (its words of each chunk, its scale and bias of each group,
-  // the latter as the fp16 pair the fp16 form multiplies by: converted once a column here, not once an operand and
-  // lane there).  get: the words of the lane's four operands for chunk i, and their columns' scale and bias.
-  unsigned char* wl = smem + 2 * STAGE + (tid >> 6) * (2 * WSTAGE);
-  auto put = [&](int stage, const Raw& r) {
-    unsigned char* at = wl + stage * WSTAGE;
-#pragma unroll
-    for (int i = 0; i < CPS; ++i) *reinterpret_cast<u32x4_t*>(at + i * 1024 + lane * 16) = r.q[i];
-#pragma unroll
-    for (int gi = 0; gi < GPS; ++gi)
-      *reinterpret_cast<uint32_t*>(at + CPS * 1024 + gi * 256 + lane * 4) = AR ? WS::sb_word(r, gi) : sb_half2(WS::sb_word(r, gi));
+  // Lane L loads column L's four packed words of a chunk as one 16-byte load (a load instruction costs the address
+  // unit the same 16 cycles whatever its width); the matrix instruction wants lane (column c, quarter kq) to hold
+  // word kq of columns c, 16 + c, 32 + c, 48 + c.  That is the transpose of a 4 x 4 matrix whose rows are the wave's
+  // four rows of 16 lanes and whose columns are the four registers, which this chip's two swap instructions do in
+  // four steps (rows 2, 3 of one register against rows 0, 1 of another, then odd rows against even ones).  Four
+  // copies of the column's scale and bias word transposed the same way are the four columns' words in every row;
+  // for the fp16 form the word is made the fp16 pair first, once a column and group instead of once an operand.
+  auto across = [](uint32_t (&v)[TJ]) {
+    auto swap32 = [](uint32_t& x, uint32_t& y) {
+      const auto r = __builtin_amdgcn_permlane32_swap(x, y, false, false);
+      x = r[0], y = r[1];
+    };
+    auto swap16 = [](uint32_t& x, uint32_t& y) {
+      const auto r = __builtin_amdgcn_permlane16_swap(x, y, false, false);
+      x = r[0], y = r[1];
+    };
+    swap32(v[0], v[2]);
+    swap32(v[1], v[3]);
+    swap16(v[0], v[1]);
+    swap16(v[2], v[3]);
   };
-  auto get = [&](int stage, int i, uint32_t (&w)[TJ], uint32_t (&sb)[TJ]) {
-    const unsigned char* at = wl + stage * WSTAGE;
+  auto take = [&](const Raw& r, int i, uint32_t (&w)[TJ], uint32_t (&sb)[TJ]) {
 #pragma unroll
-    for (int j = 0; j < TJ; ++j) w[j] = *reinterpret_cast<const uint32_t*>(at + i * 1024 + (64 * j + 4 * c + kq) * 4);
+    for (int j = 0; j < TJ; ++j) w[j] = r.q[i][j];
+    across(w);
+    const uint32_t word = WS::sb_word(r, (32 * i) / GS);
+    const uint32_t mine = AR ? word : sb_half2(word);
 #pragma unroll
-    for (int j = 0; j < TJ; ++j)
-      sb[j] = *reinterpret_cast<const uint32_t*>(at + CPS * 1024 + ((32 * i) / GS) * 256 + (16 * j + c) * 4);
+    for (int j = 0; j < TJ; ++j) sb[j] = mine;
+    across(sb);
   };
   // this thread's pieces of the activation tile: piece q = (row q / 8, 16 bytes q % 8)
   const uint16_t* asrc[PPT];
@@ -553,24 +559,22 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
 #pragma unroll
     for (int r = 0; r < RT; ++r) acc[j][r] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
-  // The weights of step t are requested at the head of step t - RD - 1 into one of RD landing sets of registers, put
-  // into the wave's LDS stage t & 1 at the head of step t - 1, and taken from there a chunk ahead of their MFMAs.
-  // With 128 rows the accumulators leave room for one landing set; with fewer, for two.
-  constexpr int RD = RT <= 4 ? 2 : 1;
-  Raw raw[RD];
+  // Two landing sets of registers: step t's words are requested into set t & 1 in the middle of step t - 2, a moment
+  // after that set's last chunk has been taken, and are taken a chunk ahead of their MFMAs (the first in the last
+  // chunk of step t - 1).
+  static_assert(CPS == 2, "a step is two chunks: the landing set is free after the first");
+  Raw raw[2];
   uint4 ar[PPT];
   const int last = steps - 1;
   ws.load(0, raw[0]);
   load_a(0, ar);
-  if constexpr (RD == 2) ws.load(min(1, last), raw[1]);
-  put(0, raw[0]);
-  ws.load(min(RD, last), raw[0]);
+  ws.load(min(1, last), raw[1]);
   store_a(0, ar);
   // Software pipeline: the operands of the NEXT 32 inputs are dequantized under the MFMAs of these 32.
   u32x4_t bcur[TJ];
   {
     uint32_t wn[TJ], sn[TJ];
-    get(0, 0, wn, sn);
+    take(raw[0], 0, wn, sn);
 #pragma unroll
     for (int j = 0; j < TJ; ++j) bcur[j] = dequant(wn[j], sn[j]);
   }
@@ -582,13 +586,9 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
     for (int u = 0; u < 2; ++u) {
       const int step = step0 + u;
       if (step < steps) {
-        // stage `u` of LDS holds this step's activations and (the wave's own) weights; the next step's activations
-        // are requested now and staged at the end of the step, its weights have landed and go to stage 1 - u, and
-        // the landing set they leave takes the request for step + 1 + RD
+        // stage `u` of LDS holds this step's activations; the next step's are requested now and staged at the end
+        // of the step
         load_a(min(step + 1, last), ar);
-        Raw& landed = raw[RD == 2 ? 1 - u : 0];
-        put(1 - u, landed);
-        ws.load(min(step + 1 + RD, last), landed);
         const unsigned char* abuf = smem + u * STAGE + c * AROW + kq * 16;
         // activation operands are requested two row tiles before their MFMAs (an LDS read takes about as long as
         // one row tile's four MFMAs): operand t of the step is (chunk t / RT, row tile t % RT)
@@ -600,8 +600,8 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
         for (int i = 0; i < CPS; ++i) {
           u32x4_t bnext[TJ];
           uint32_t wn[TJ], sn[TJ];                      // the next chunk's words: this step's, or the next step's first
-          if (i + 1 < CPS) get(u, i + 1, wn, sn);
-          else get(1 - u, 0, wn, sn);
+          if (i + 1 < CPS) take(raw[u], i + 1, wn, sn);
+          else take(raw[1 - u], 0, wn, sn);
 #pragma unroll
           for (int r = 0; r < RT; ++r) {
             const int t = i * RT + r;
@@ -627,6 +627,8 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
           }
 #pragma unroll
           for (int j = 0; j < TJ; ++j) bcur[j] = bnext[j];
+          // this step's last words have been taken: their landing set takes the request for the step after next
+          if (i == CPS - 2) ws.load(min(step + 2, last), raw[u]);
         }
         store_a(1 - u, ar);
         __syncthreads();
@@ -1019,20 +1021,6 @@ constexpr size_t stage_bytes() {
   return 2 * (size_t)(16 * RT) * AROW;
 }
 
-// The eight-wave kernels ask for more dynamic LDS than a launch gets unasked (64 KB of the compute unit's 160): the
-// attribute is set once a kernel and device.
-bool allow_lds(const void* kernel, int bytes) {
-  static std::mutex guard;
-  static std::set<std::pair<const void*, int>> done;
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return false;
-  std::lock_guard<std::mutex> hold(guard);
-  if (done.count({kernel, dev})) return true;
-  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return false;
-  done.insert({kernel, dev});
-  return true;
-}
-
 // compute units of the current device (looked up once a device)
 int compute_units() {
   static int cached[64] = {};
@@ -1076,9 +1064,6 @@ int launch_experts_prefill(int tile, int arith, const uint16_t* x, int64_t x_str
     const int cus = compute_units();
     if (big > 2 * cus) {
       const dim3 rg((unsigned)cus);
-      TF_REQUIRE(allow_lds(arith ? (const void*)experts_prefill_resident_kernel<GS, NM, EPI, 1>
-                                 : (const void*)experts_prefill_resident_kernel<GS, NM, EPI, 0>, RESIDENT_LDS),
-                 "experts: %d bytes of LDS a workgroup were refused", RESIDENT_LDS);
       if (arith)
         experts_prefill_resident_kernel<GS, NM, EPI, 1><<<rg, BIG_THREADS, RESIDENT_LDS, s>>>(
             x, x_stride, slots, w, kg, nb, items, counts, counts + 2, members, out, n, limit);
@@ -1089,9 +1074,6 @@ int launch_experts_prefill(int tile, int arith, const uint16_t* x, int64_t x_str
       return 0;
     }
     const dim3 bg((unsigned)big);
-    TF_REQUIRE(allow_lds(arith ? (const void*)experts_prefill_big_kernel<GS, NM, EPI, 1>
-                               : (const void*)experts_prefill_big_kernel<GS, NM, EPI, 0>, BIG_LDS),
-               "experts: %d bytes of LDS a workgroup were refused", BIG_LDS);
     if (arith)
       experts_prefill_big_kernel<GS, NM, EPI, 1><<<bg, BIG_THREADS, BIG_LDS, s>>>(
           x, x_stride, slots, w, kg, nb, items, counts, members, out, n, limit);
@@ -1126,9 +1108,6 @@ int launch_qmm_prefill(int arith, int tile, const uint16_t* x, int64_t ldx, cons
     else TF_SMALL(4, 0);
   } else if (big_ok && tile != 8) {
     const unsigned grid = (unsigned)((int64_t)((m + BIG_ROWS - 1) / BIG_ROWS) * ((n + 511) / 512));
-    TF_REQUIRE(allow_lds(arith ? (const void*)qmm_prefill_big_kernel<GS, EPI, 1> : (const void*)qmm_prefill_big_kernel<GS, EPI, 0>,
-                         BIG_LDS),
-               "qmm_prefill: %d bytes of LDS a workgroup were refused", BIG_LDS);
     if (arith)
       qmm_prefill_big_kernel<GS, EPI, 1><<<grid, BIG_THREADS, BIG_LDS, st>>>(x, ldx, w, s, b, out, m, n, kg, npad);
     else
