@@ -570,14 +570,28 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
   load_a(0, ar);
   ws.load(min(1, last), raw[1]);
   store_a(0, ar);
-  // Software pipeline: the operands of the NEXT 32 inputs are dequantized under the MFMAs of these 32.
-  u32x4_t bcur[TJ];
+  // Software pipeline: the operands of the NEXT 32 inputs are dequantized under the MFMAs of these 32 (chunk i's are
+  // bb[i], and it makes bb[1 - i]).  And a step's last row tile waits until the barrier is behind: its four MFMAs run
+  // at the head of the next step, while that step's first activation operands are on their way from LDS (before
+  // the first step they multiply zeros).
+  u32x4_t bb[2][TJ], alast = {0u, 0u, 0u, 0u};
   {
     uint32_t wn[TJ], sn[TJ];
     take(raw[0], 0, wn, sn);
 #pragma unroll
-    for (int j = 0; j < TJ; ++j) bcur[j] = dequant(wn[j], sn[j]);
+    for (int j = 0; j < TJ; ++j) {
+      bb[0][j] = dequant(wn[j], sn[j]);
+      bb[1][j] = (u32x4_t){0u, 0u, 0u, 0u};
+    }
   }
+  constexpr bool DEFER = RT == 8;          // with fewer row tiles a step the tile put off is too large a part of it
+  auto last_tile = [&]() {
+    if constexpr (!DEFER) return;
+    if constexpr (!AR) __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+    for (int j = 0; j < TJ; ++j) acc[j][RT - 1] = mfma(alast, bb[1][j], acc[j][RT - 1]);
+    if constexpr (!AR) __builtin_amdgcn_s_setprio(0);
+  };
   __syncthreads();
   staged();
   TF_MARK(2);
@@ -596,9 +610,9 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
           return *reinterpret_cast<const u32x4_t*>(abuf + 16 * (t % RT) * AROW + (t / RT) * 64);
         };
         u32x4_t a = read_a(0), a1 = read_a(1);
+        last_tile();
 #pragma unroll
         for (int i = 0; i < CPS; ++i) {
-          u32x4_t bnext[TJ];
           uint32_t wn[TJ], sn[TJ];                      // the next chunk's words: this step's, or the next step's first
           if (i + 1 < CPS) take(raw[u], i + 1, wn, sn);
           else take(raw[1 - u], 0, wn, sn);
@@ -610,11 +624,15 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
             // the matrix instructions go first among the SIMD's waves: the other wave's vector work fills the cycles
             // between them, instead of both waves taking turns at the same kind of work (3 % on the fp16 form; the
             // bf16 form, with twice the vector work an operand, lost 4 % to it)
-            if constexpr (!AR) __builtin_amdgcn_s_setprio(1);
+            if (DEFER && t == CPS * RT - 1) {
+              alast = a;
+            } else {
+              if constexpr (!AR) __builtin_amdgcn_s_setprio(1);
 #pragma unroll
-            for (int j = 0; j < TJ; ++j)
-              acc[j][r] = mfma(a, bcur[j], acc[j][r]);
-            if constexpr (!AR) __builtin_amdgcn_s_setprio(0);
+              for (int j = 0; j < TJ; ++j)
+                acc[j][r] = mfma(a, bb[i][j], acc[j][r]);
+              if constexpr (!AR) __builtin_amdgcn_s_setprio(0);
+            }
             a = a1;
             a1 = a2;
             // a share of the next chunk's dequantization rides along with each row tile
@@ -622,11 +640,9 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
 #pragma unroll
             for (int jj = 0; jj < JPR; ++jj) {
               const int j = r * JPR + jj;
-              if (j < TJ) bnext[j] = dequant(wn[j], sn[j]);
+              if (j < TJ) bb[1 - i][j] = dequant(wn[j], sn[j]);
             }
           }
-#pragma unroll
-          for (int j = 0; j < TJ; ++j) bcur[j] = bnext[j];
           // this step's last words have been taken: their landing set takes the request for the step after next
           if (i == CPS - 2) ws.load(min(step + 2, last), raw[u]);
         }
@@ -635,6 +651,7 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
       }
     }
   }
+  last_tile();
   TF_MARK(3);
   if constexpr (SWAP) {
     if (N % 32 == 0 && STAGE_OUT) {
