@@ -587,10 +587,8 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
   constexpr bool DEFER = RT == 8;          // with fewer row tiles a step the tile put off is too large a part of it
   auto last_tile = [&]() {
     if constexpr (!DEFER) return;
-    if constexpr (!AR) __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int j = 0; j < TJ; ++j) acc[j][RT - 1] = mfma(alast, bb[1][j], acc[j][RT - 1]);
-    if constexpr (!AR) __builtin_amdgcn_s_setprio(0);
   };
   __syncthreads();
   staged();
@@ -621,17 +619,12 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
             const int t = i * RT + r;
             u32x4_t a2 = a1;
             if (t + 2 < CPS * RT) a2 = read_a(t + 2);
-            // the matrix instructions go first among the SIMD's waves: the other wave's vector work fills the cycles
-            // between them, instead of both waves taking turns at the same kind of work (3 % on the fp16 form; the
-            // bf16 form, with twice the vector work an operand, lost 4 % to it)
             if (DEFER && t == CPS * RT - 1) {
               alast = a;
             } else {
-              if constexpr (!AR) __builtin_amdgcn_s_setprio(1);
 #pragma unroll
               for (int j = 0; j < TJ; ++j)
                 acc[j][r] = mfma(a, bb[i][j], acc[j][r]);
-              if constexpr (!AR) __builtin_amdgcn_s_setprio(0);
             }
             a = a1;
             a1 = a2;
