@@ -413,6 +413,7 @@ static_assert(BIG_LDS + 2 * 2 * BIG_ROWS * 4 + 16 <= 64 * 1024, "within what a l
 template <int GS, int NM>
 struct ExpertSource {
   static constexpr int CPS = KSTEP / 32, GPS = KSTEP / GS;
+  static constexpr bool KEEPS_GROUP_WORDS = false;
   static constexpr uint32_t GSTRIDE = NM * block_words(GS);      // words from one group to the next
   struct Raw {
     u32x4_t q[CPS];
@@ -437,6 +438,7 @@ struct ExpertSource {
 template <int GS>
 struct DenseSource {
   static constexpr int CPS = KSTEP / 32, GPS = KSTEP / GS;
+  static constexpr bool KEEPS_GROUP_WORDS = true;
   struct Raw {
     u32x4_t q[CPS];
     uint32_t s[GPS], b[GPS];          // each a bf16 in the low half, joined when a chunk is taken (not when they
@@ -493,6 +495,9 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
   // four steps (rows 2, 3 of one register against rows 0, 1 of another, then odd rows against even ones).  Four
   // copies of the column's scale and bias word transposed the same way are the four columns' words in every row;
   // for the fp16 form the word is made the fp16 pair first, once a column and group instead of once an operand.
+  // With groups of 64 a step's two chunks share their scale and bias words; the dense kernel keeps them across the two
+  // (2 % of its time).  The experts' kernels, a few registers fuller, would spill for it and transpose them again.
+  constexpr bool KEEP_SB = WS::KEEPS_GROUP_WORDS && GS == 64;
   auto across = [](uint32_t (&v)[TJ]) {
     auto swap32 = [](uint32_t& x, uint32_t& y) {
       const auto r = __builtin_amdgcn_permlane32_swap(x, y, false, false);
@@ -511,6 +516,7 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
 #pragma unroll
     for (int j = 0; j < TJ; ++j) w[j] = r.q[i][j];
     across(w);
+    if (KEEP_SB && i % 2 == 1) return;          // the group of the chunk before: its columns' words are in sb still
     const uint32_t word = WS::sb_word(r, (32 * i) / GS);
     const uint32_t mine = AR ? word : sb_half2(word);
 #pragma unroll
@@ -575,8 +581,10 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
   // at the head of the next step, while that step's first activation operands are on their way from LDS (before
   // the first step they multiply zeros).
   u32x4_t bb[2][TJ], alast = {0u, 0u, 0u, 0u};
+  uint32_t sn_step[TJ];          // KEEP_SB: the four columns' scale and bias words of the group last taken
   {
-    uint32_t wn[TJ], sn[TJ];
+    uint32_t wn[TJ];
+    uint32_t (&sn)[TJ] = sn_step;
     take(raw[0], 0, wn, sn);
 #pragma unroll
     for (int j = 0; j < TJ; ++j) {
@@ -611,7 +619,8 @@ __device__ __forceinline__ void big_body(const uint16_t* __restrict__ X, int64_t
         last_tile();
 #pragma unroll
         for (int i = 0; i < CPS; ++i) {
-          uint32_t wn[TJ], sn[TJ];                      // the next chunk's words: this step's, or the next step's first
+          uint32_t wn[TJ], sn_chunk[TJ];
+          uint32_t (&sn)[TJ] = KEEP_SB ? sn_step : sn_chunk;                      // the next chunk's words: this step's, or the next step's first
           if (i + 1 < CPS) take(raw[u], i + 1, wn, sn);
           else take(raw[1 - u], 0, wn, sn);
 #pragma unroll
