@@ -1,7 +1,7 @@
 """Kernel timings of the benchmark configurations that are not bench.py's headline: 0 (dense 4-bit projection),
 2 (verify-window MoE layer), 3 (prompt chunk, grouped MFMA) and 4 (EXL3 projections).
 
-    python bench_configs.py [c0] [c2] [c3] [c3d] [c4] [c4p] [glue] [c4x] [cal] [timeline] [timeline_c2] [timeline_c3]
+    python bench_configs.py [c0] [c2] [c3] [c3d] [c4] [c4p] [glue] [c4x] [cal] [timeline] [timeline_c0] [timeline_c2] [timeline_c3]
 
 One JSON line a configuration: time of one pass (hipGraph of back-to-back passes cycling over enough weight copies to
 miss the 256 MB Infinity Cache, HIP events around the replay), algorithmic bytes or flops, and the fraction of the
@@ -459,7 +459,7 @@ def timeline() -> dict:
                 g.replay()
                 g.replay()
                 torch.cuda.synchronize()
-                h = np.zeros((len(marks) + 1, 16384), dtype=np.uint64)
+                h = np.zeros((len(marks) + 2, 16384), dtype=np.uint64)
                 if tl.tf_timeline_read_moe(h.ctypes.data_as(ctypes.c_void_p), h.shape[0], h.shape[1]):
                     raise RuntimeError(tl.tf_last_error().decode())
                 where = h[len(marks)]
@@ -522,7 +522,7 @@ def timeline() -> dict:
             g.replay()
             g.replay()
             torch.cuda.synchronize()
-            h = np.zeros((len(names) + 1, 16384), dtype=np.uint64)
+            h = np.zeros((len(names) + 2, 16384), dtype=np.uint64)
             if tl.tf_timeline_read_exl3(h.ctypes.data_as(ctypes.c_void_p), h.shape[0], h.shape[1]):
                 raise RuntimeError(tl.tf_last_error().decode())
         where = h[len(names)]
@@ -606,7 +606,7 @@ def timeline_c2() -> dict:
             g.replay()
             g.replay()
             torch.cuda.synchronize()
-            h = np.zeros((marks + 1, 16384), dtype=np.uint64)
+            h = np.zeros((marks + 2, 16384), dtype=np.uint64)
             if tl.tf_timeline_read_moe(h.ctypes.data_as(ctypes.c_void_p), h.shape[0], h.shape[1]):
                 raise RuntimeError(tl.tf_last_error().decode())
             where, h = h[marks], h[:marks].astype(np.int64)
@@ -630,6 +630,57 @@ def timeline_c2() -> dict:
             row["alive_at_us"] = {str(t): int((begin <= t).sum() - (done <= t).sum()) for t in (5, 15, 25, 35, 45, 55)}
             res["launches"][name] = row
     return res
+
+
+def timeline_c0() -> dict:
+    """The clock the dense prompt kernel runs at, read inside it through the timeline build: every workgroup counts the
+    shader cycles (s_memtime) of its loop over K between two of its 100 MHz marks, and cycles over time is the clock of
+    its compute unit.  The same launch (4096 cubed, 64 steps of 64 inputs) in a short burst after an idle wait, after
+    hundreds of launches back to back, and on activations of zeros: the cycles a step stay, the clock does not."""
+
+    import ctypes
+
+    import numpy as np
+
+    from tensorfold_amd import _lib, build
+
+    n = k = m = 4096
+    gen = torch.Generator(device=DEV).manual_seed(1)
+    q = qmm.pack(*rand_affine(n, k, 64, gen), 64)
+    x = synthetic.activations(m, k, 8).to(DEV)
+    y = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+    cases = []
+    with _lib.through(build.timeline_lib()) as tl:
+        def run(what, xin, launches, idle_s):
+            torch.cuda.synchronize()
+            time.sleep(idle_s)
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(launches):
+                qmm.prefill_matmul(xin, q, out=y)
+            b.record()
+            torch.cuda.synchronize()
+            h = np.zeros((8, 16384), dtype=np.uint64)
+            if tl.tf_timeline_read_prefill(h.ctypes.data_as(ctypes.c_void_p), h.shape[0], h.shape[1]):
+                raise RuntimeError(tl.tf_last_error().decode())
+            t = h.astype(np.int64)
+            live = (t[5] > 0) & (t[3] > t[2])
+            ghz = t[7][live] / ((t[3][live] - t[2][live]) * 10.0)
+            cases.append({"case": what, "launches": launches, "us_a_launch": a.elapsed_time(b) * 1e3 / launches,
+                          "clock_ghz": [round(float(v), 3) for v in np.percentile(ghz, [0, 50, 100])],
+                          "cycles_a_step": round(float(np.median(t[7][live])) / (k // 64), 1),
+                          "loop_us": round(float(np.median(t[3][live] - t[2][live])) / 100.0, 1)})
+
+        for _ in range(3):
+            qmm.prefill_matmul(x, q, out=y)
+        run("a burst after 50 ms of idling", x, 12, 0.05)
+        run("back to back", x, 100, 0.0)
+        run("back to back", x, 500, 0.0)
+        run("back to back", x, 2000, 0.0)
+        run("zero activations, back to back", torch.zeros_like(x), 500, 0.0)
+        run("a burst after 50 ms of idling", x, 12, 0.05)
+    return {"config": "timeline_c0: the dense prompt kernel's clock and cycles, read inside the kernel (marks of each "
+                      "case's last launch; clock as min / median / max over its 256 workgroups)", "cases": cases}
 
 
 def timeline_c3() -> dict:
@@ -673,7 +724,7 @@ def timeline_c3() -> dict:
                 raise RuntimeError(tl.tf_last_error().decode())
             fn()
             torch.cuda.synchronize()
-            h = np.zeros((7, 16384), dtype=np.uint64)
+            h = np.zeros((8, 16384), dtype=np.uint64)
             if tl.tf_timeline_read_prefill(h.ctypes.data_as(ctypes.c_void_p), h.shape[0], h.shape[1]):
                 raise RuntimeError(tl.tf_last_error().decode())
             hw, t = h[6], h[:6].astype(np.int64)
@@ -716,7 +767,7 @@ def main() -> int:
     torch.cuda.set_device(0)
     which = sys.argv[1:] or ["c0", "c2", "c3", "c4"]
     for name in which:
-        res = {"c0": c0, "c2": c2, "c3": c3, "c3d": c3d, "c4": c4, "c4p": c4p, "glue": glue_, "c4x": c4x, "cal": cal, "timeline": timeline, "timeline_c2": timeline_c2, "timeline_c3": timeline_c3}[name]()
+        res = {"c0": c0, "c2": c2, "c3": c3, "c3d": c3d, "c4": c4, "c4p": c4p, "glue": glue_, "c4x": c4x, "cal": cal, "timeline": timeline, "timeline_c2": timeline_c2, "timeline_c0": timeline_c0, "timeline_c3": timeline_c3}[name]()
         torch.cuda.empty_cache()
         print(json.dumps(res, default=lambda v: round(v, 4)), flush=True)
     return 0

@@ -968,8 +968,10 @@ __global__ void __launch_bounds__(BIG_THREADS, 1)
   const int rt = blockIdx.x / ct, cbt = blockIdx.x - rt * ct;
   const int m0 = rt * BIG_ROWS, cnt = min(BIG_ROWS, M - m0);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, kq = lane >> 4;
+  TF_MARK(0);
   if (tid < BIG_ROWS) rows[tid] = m0 + (tid < cnt ? tid : 0);
   __syncthreads();
+  TF_MARK(1);
   const int tiles = npad >> 6, tile = cbt * 8 + wave;
   const bool ok = tile < tiles;
   DenseSource<GS> ws;
@@ -991,6 +993,11 @@ __global__ void __launch_bounds__(BIG_THREADS, 1)
   if (cnt <= 32) big_body<GS, 1, EPI, 2, AR, true>(X, ldx, ws, ocol, jok, K, rows, rows, cnt, out, N, 0.f, smem);
   else if (cnt <= 64) big_body<GS, 1, EPI, 4, AR, true>(X, ldx, ws, ocol, jok, K, rows, rows, cnt, out, N, 0.f, smem);
   else big_body<GS, 1, EPI, 8, AR, true>(X, ldx, ws, ocol, jok, K, rows, rows, cnt, out, N, 0.f, smem);
+  TF_MARK(4);
+#ifdef TF_TIMELINE
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
+  TF_MARK(5);
 }
 
 // ---- dense prompt matmul --------------------------------------------------------------------------------------------

@@ -99,15 +99,16 @@ __device__ __forceinline__ void prio_by_progress(int left, int n) {
 // Compiled with -DTF_TIMELINE (libtfmi_timeline.so) the decode expert kernels note when thread 0 of each workgroup
 // passes a few marks, on the 100 MHz clock every compute unit reads alike: 0 kernel entry, 1 the workgroup knows its
 // item, 2 its first weights and inputs are requested, 3 wave 0 has streamed its share, 4 every wave has, 5 the unit
-// has stored its output (and combined what it completed); a seventh row says which compute unit ran the workgroup.
-// The marks are kept in LDS and written out once, at mark
+// has stored its output (and combined what it completed); a seventh row says which compute unit ran the workgroup,
+// an eighth how many shader cycles (s_memtime) passed between marks 2 and 3, which against the marks' own 10 ns
+// ticks is the clock the compute unit ran at.  The marks are kept in LDS and written out once, at mark
 // 5 (a store to memory at each mark would put its round trip into the waits that follow it).  The ordinary build
 // compiles the marks away.
 #ifdef TF_TIMELINE
-constexpr int TIMELINE_MARKS = 6, TIMELINE_ROWS = TIMELINE_MARKS + 1, TIMELINE_GROUPS = 16384;
+constexpr int TIMELINE_MARKS = 6, TIMELINE_ROWS = TIMELINE_MARKS + 2, TIMELINE_GROUPS = 16384;
 static __device__ unsigned long long tf_timeline_marks[TIMELINE_ROWS][TIMELINE_GROUPS];
 __device__ __forceinline__ unsigned long long* timeline_lds() {
-  __shared__ unsigned long long t[TIMELINE_MARKS];
+  __shared__ unsigned long long t[TIMELINE_MARKS + 1];
   return t;
 }
 // `as` >= 0: the row of the table to write at the last mark (a workgroup that takes several units one after another
@@ -116,19 +117,22 @@ __device__ __forceinline__ void timeline_mark(int k, int as = -1) {
   if (threadIdx.x != 0) return;
   unsigned long long* t = timeline_lds();
   if (k == 0)
-    for (int i = 1; i < TIMELINE_MARKS; ++i) t[i] = 0;
+    for (int i = 1; i <= TIMELINE_MARKS; ++i) t[i] = 0;
   t[k] = wall_clock64();
+  if (k == 2) t[TIMELINE_MARKS] = __builtin_readcyclecounter();
+  if (k == 3) t[TIMELINE_MARKS] = __builtin_readcyclecounter() - t[TIMELINE_MARKS];
   const unsigned group = as >= 0 ? (unsigned)as : blockIdx.x + (blockIdx.y + blockIdx.z * gridDim.y) * gridDim.x;
   if (k == TIMELINE_MARKS - 1 && group < TIMELINE_GROUPS) {
     for (int i = 0; i < TIMELINE_MARKS; ++i) tf_timeline_marks[i][group] = t[i];
     // where it ran: the XCC id above the hardware id word (compute unit in bits 8-11, shader array 12, engine 13-15)
     tf_timeline_marks[TIMELINE_MARKS][group] =
         ((unsigned long long)__builtin_amdgcn_s_getreg((31 << 11) | 20) << 32) | __builtin_amdgcn_s_getreg((31 << 11) | 4);
+    tf_timeline_marks[TIMELINE_MARKS + 1][group] = t[TIMELINE_MARKS];
   }
 }
 // The timeline build's two extra entry points of a source file that places marks: the marks of that file's last
 // launches, [TIMELINE_ROWS][TIMELINE_GROUPS]: six rows of 64-bit ticks of 10 ns (0: never passed), then the row of
-// hardware ids (each source file has its own table).
+// hardware ids and the row of shader cycles between marks 2 and 3 (each source file has its own table).
 #define TF_TIMELINE_EXPORT(NAME_)                                                                                   \
   extern "C" int tf_timeline_read_##NAME_(unsigned long long* host, int rows, int groups) {                         \
     ::tf::clear_error();                                                                                            \
